@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused Leech-lattice dequant-GEMV on one MI355X.
+
+Workload (BASELINE config 1 at the scale the metric is quoted on): the seven
+projections of a Qwen3-4B decoder layer at batch 1, over `--layers` distinct
+layers (default 36 = every LLVQ matrix of the 4B model, 252 matrices, 981 MB of
+encoded weights — larger than the 256 MB Infinity Cache, so HBM is what is
+measured).  One step = one token's worth of projection GEMVs: for every layer
+q/k/v on the hidden activation, o_proj, gate/up, down_proj.
+
+Prints ONE JSON line.  `value` = encoded-weight GB/s over the timed steps with
+all inputs resident in HBM.  `roofline` is for the GEMV kernel; `cpu_baseline`
+is the CPU oracle (a C port of the reference's decode + reconstruct + f32 dot)
+timed on the host cores on one layer of the same workload.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_layers(n_layers, seed):
+    from llvq_amd import synth
+
+    t0 = time.time()
+    layers = []
+    for layer in range(n_layers):
+        layers.append(synth.layer_matrices(layer, seed))
+        if layer % 6 == 5:
+            log(f"[bench] generated {layer + 1}/{n_layers} layers ({time.time() - t0:.1f}s)")
+    return layers
+
+
+def cpu_baseline(layer_mats, acts, threads):
+    """CPU oracle on one layer (4 185 600 blocks): 2 discarded + 5 kept rounds, median
+    (protocol of llvq-cuda/src/bin/matvec.rs:64-65)."""
+    from oracle import pyoracle as orc
+
+    total_bytes = sum(m.encoded_bytes() for m in layer_mats)
+    total_blocks = sum(m.d_out * m.nblocks for m in layer_mats)
+    times = []
+    for rnd in range(7):
+        t0 = time.perf_counter()
+        for m in layer_mats:
+            x = acts[m.d_in]
+            orc.cpu_gemv(m.codes, m.d_out, m.d_in, m.centroids, m.row_scales, m.tail, x.view(np.uint16), threads)
+        dt = time.perf_counter() - t0
+        if rnd >= 2:
+            times.append(dt)
+    med = statistics.median(times)
+    # decode-only cost per block on one core, as llvq-bench's decfull measures it
+    m = layer_mats[1]
+    nb = min(m.d_out * m.nblocks, 200_000)
+    t0 = time.perf_counter()
+    orc.cpu_decode_only(m.codes, nb)
+    ns_per_block = (time.perf_counter() - t0) / nb * 1e9
+    return {
+        "value": round(total_bytes / med / 1e9, 4),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"one Qwen3-4B layer (7 projections, {total_blocks} blocks, {total_bytes} encoded bytes), "
+                  f"median of 5 rounds after 2 discarded [{min(times) * 1e3:.1f}-{max(times) * 1e3:.1f} ms]",
+        "ms_per_layer": round(med * 1e3, 3),
+        "decode_only_ns_per_block_per_core": round(ns_per_block, 1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--layers", type=int, default=36)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: this build has no multi-GPU path (rows shard trivially; see DESIGN.md). "
+            "Run with --gpus 1.")
+        sys.exit(2)
+
+    import torch
+
+    import llvq_amd
+    from llvq_amd import synth
+
+    if not torch.cuda.is_available():
+        log("bench.py needs a GPU (there is no CPU fallback for the product path)")
+        sys.exit(1)
+    dev = torch.device("cuda", 0)
+    layers = build_layers(args.layers, args.seed)
+    acts_np = {d: synth.make_activation(d, args.seed)[0] for d in (2560, 4096, 9728)}
+    acts = {d: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16).to(dev) for d, a in acts_np.items()}
+
+    rt = llvq_amd.FusedRuntime(device=0)
+    t0 = time.time()
+    projs = [[rt.upload(m) for m in layer] for layer in layers]
+    log(f"[bench] uploaded {sum(len(p) for p in projs)} matrices in {time.time() - t0:.1f}s")
+    enc_bytes = sum(m.encoded_bytes() for layer in layers for m in layer)
+    code_bytes = sum(m.codes.size for layer in layers for m in layer)
+    n_blocks = code_bytes // 6
+    n_launch = sum(len(p) for p in projs)
+
+    def step():
+        for lp in projs:
+            q, k, v, o, gate, up, down = lp
+            rt.forward_group([q, k, v], acts[2560])
+            rt.forward_rotated(o, acts[4096])
+            rt.forward_group([gate, up], acts[2560])
+            rt.forward_rotated(down, acts[9728])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = ev0.elapsed_time(ev1)
+    ms_per_step = wall * 1e3 / args.steps
+    gbps = enc_bytes * args.steps / wall / 1e9
+
+    # cache-resident figure: the same seven projections of layer 0 over and over
+    lp = projs[0]
+    one_layer_bytes = sum(m.encoded_bytes() for m in layers[0])
+    reps = max(20, args.steps * 4)
+    torch.cuda.synchronize()
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    for _ in range(reps):
+        q, k, v, o, gate, up, down = lp
+        rt.forward_group([q, k, v], acts[2560])
+        rt.forward_rotated(o, acts[4096])
+        rt.forward_group([gate, up], acts[2560])
+        rt.forward_rotated(down, acts[9728])
+    c1.record()
+    torch.cuda.synchronize()
+    cache_gbps = one_layer_bytes * reps / (c0.elapsed_time(c1) * 1e-3) / 1e9
+
+    avg_launch_us = dev_ms * 1e3 / (args.steps * n_launch)
+    achieved = enc_bytes * args.steps / (dev_ms * 1e-3) / 1e9
+    out = {
+        "metric": "dequant_gemv_encoded_weight_GBps",
+        "value": round(gbps, 3),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"Qwen3-4B decoder-layer projections at batch 1 (BASELINE config 1 shapes), "
+                        f"{args.layers} distinct layers = {n_launch} LLVQ matrices, {n_blocks} blocks, "
+                        f"{enc_bytes} encoded bytes per step",
+            "layers": args.layers,
+            "seed": args.seed,
+        },
+        "hbm_peak_frac": round(gbps / HBM_PEAK_GBPS, 5),
+        "codes_only_GBps": round(code_bytes * args.steps / wall / 1e9, 3),
+        "blocks_per_s": round(n_blocks * args.steps / wall, 1),
+        "projection_tokens_per_s": round(args.steps / wall * (36 / args.layers), 2),
+        "cache_resident_one_layer_GBps": round(cache_gbps, 3),
+        "roofline": {
+            "kernel": "gemv_rows_kernel",
+            "bound": "hbm",
+            "achieved": round(achieved, 3),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 5),
+            "traffic": None,
+            "avg_launch_us": round(avg_launch_us, 3),
+            "launches_per_step": n_launch,
+            "algorithmic_bytes_per_launch": round(enc_bytes / n_launch, 1),
+        },
+    }
+    if not args.no_cpu:
+        threads = min(16, os.cpu_count() or 1)
+        out["cpu_baseline"] = cpu_baseline(layers[0], acts_np, threads)
+    rt.close()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,132 @@
+/* llvq_hip.h — C ABI of the MI355X (gfx950) fused Leech-lattice dequant-GEMV/GEMM.
+ *
+ * This is the boundary a host program binds in place of the reference's
+ * quantized-linear operator (llvq-llm/src/fused.rs + fused_cuda.rs).  Plain
+ * pointers and sizes only.  Every call returns LLVQ_OK or an llvq_status; the
+ * text of the last failure on the calling thread is llvq_hip_last_error().
+ *
+ * Conventions kept from the reference operator:
+ *   - never abort on data: a malformed record is a status code
+ *     (llvq-artifact/src/error.rs:11-45, tests/hostile_files.rs);
+ *   - exactly two gain centroids / one gain bit (llvq-llm/src/fused.rs:1168-1177);
+ *   - every output row is stored, nothing is accumulated into
+ *     (llvq-llm/src/fused_cuda.rs:789-797);
+ *   - work is enqueued on the runtime's stream and the call returns without
+ *     synchronising (fused_cuda.rs:28-34);
+ *   - runtime and matrices are immutable after construction; launches are
+ *     issued from one thread at a time.
+ * Device pointers passed in are caller-owned; llvq_rt and llvq_mat are owned
+ * by the library.
+ */
+#ifndef LLVQ_HIP_H
+#define LLVQ_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Mirrors llvq_artifact::Error (llvq-artifact/src/error.rs:11-45) for the
+ * variants that can arise on this path, plus device-side failures. */
+typedef enum llvq_status {
+  LLVQ_OK = 0,
+  LLVQ_ERR_NOT_AN_ARTIFACT = 1,   /* Error::NotAnArtifact */
+  LLVQ_ERR_TRUNCATED = 2,         /* Error::Truncated { reading } */
+  LLVQ_ERR_BAD_NAME = 3,          /* Error::BadName */
+  LLVQ_ERR_INCONSISTENT = 5,      /* Error::Inconsistent */
+  LLVQ_ERR_INDEX_TOO_WIDE = 7,    /* Error::IndexTooWide */
+  LLVQ_ERR_INDEX_OUT_OF_RANGE = 8,/* Error::IndexOutOfRange */
+  LLVQ_ERR_CODEBOOK_MISMATCH = 10,/* Error::CodebookMismatch */
+  LLVQ_ERR_UNKNOWN_VERSION = 11,  /* Error::UnknownVersion */
+  LLVQ_ERR_INVALID_ARGUMENT = 32, /* null pointer, wrong shape, unsupported dtype */
+  LLVQ_ERR_UNSUPPORTED = 33,      /* e.g. centroid count != 2, rotated matrix */
+  LLVQ_ERR_DEVICE = 34            /* a HIP call failed; message carries hipGetErrorString */
+} llvq_status;
+
+typedef enum llvq_dtype { LLVQ_F32 = 0, LLVQ_F16 = 1 } llvq_dtype;
+
+typedef struct llvq_rt llvq_rt;   /* replaces FusedRuntime  (fused_cuda.rs:145-180) */
+typedef struct llvq_mat llvq_mat; /* replaces FusedProj     (fused_cuda.rs:119-134) */
+
+/* One projection as the file stores it: the fields of RawMatrix
+ * (llvq-artifact/src/format.rs:215-229) with the code stream left packed
+ * (format.rs:185-203: per block index_bits(cap) bits of index then the gain
+ * bit, MSB first — 6 bytes per block at cap 12). All pointers are host memory. */
+typedef struct llvq_matrix_desc {
+  const char* name;          /* may be NULL */
+  uint32_t d_out, d_in;
+  uint32_t shell_cap;        /* 12 is the only cap with a 6-byte record */
+  uint32_t n_centroids;      /* must be 2 */
+  const double* centroids;   /* [n_centroids] */
+  const double* row_scales;  /* [d_out] */
+  const float* tail;         /* [d_out * (d_in % 24)], row-major; may be NULL when d_in % 24 == 0 */
+  const uint8_t* codes;      /* packed stream, >= 6 * d_out * (d_in / 24) bytes */
+  size_t code_bytes;
+  uint64_t rotation_seed;
+  uint32_t has_rotation;     /* rotated matrices are refused (LLVQ_ERR_UNSUPPORTED) */
+} llvq_matrix_desc;
+
+/* FusedRuntime::new (fused_cuda.rs:182): builds the Golay / class tables on the
+ * host, checks them against the pinned codebook fingerprint, uploads them.
+ * `hip_stream` is a hipStream_t (NULL = the device's default stream). */
+int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out);
+void llvq_hip_runtime_destroy(llvq_rt* rt);
+
+/* codebook_fingerprint (llvq-artifact/src/codebook.rs:182), computed from this
+ * library's own tables and host decoder.  Needs no GPU.
+ * The published value is 0x338f420f11866319. */
+uint64_t llvq_hip_codebook_fingerprint(void);
+
+/* Host-side decode of one index with the library's own tables (the same
+ * arithmetic the kernels run).  Returns 1, or 0 for idx > N(13).  Needs no GPU. */
+int llvq_hip_host_decode(uint64_t idx, int8_t point[24], int* shell);
+
+/* upload_matrix (fused_cuda.rs:1058): validates, range-checks every index
+ * (IndexOutOfRange, format.rs:389-392) and copies the record to the device. */
+int llvq_hip_matrix_upload(llvq_rt* rt, const llvq_matrix_desc* desc, llvq_mat** out);
+
+/* read_header (format.rs:588): parses magic, count and, for LVQ4, the
+ * fingerprint.  *pos is advanced past the header. */
+int llvq_hip_read_header(const uint8_t* buf, size_t len, size_t* pos, uint32_t* version,
+                         uint32_t* n_matrices);
+/* read_matrix_raw (format.rs:301) fused with upload: parses one on-disk matrix
+ * record at buf[*pos..] and uploads it; the code stream is copied verbatim.
+ * *pos is advanced past the record. */
+int llvq_hip_matrix_from_record(llvq_rt* rt, const uint8_t* buf, size_t len, size_t* pos,
+                                llvq_mat** out);
+void llvq_hip_matrix_free(llvq_rt* rt, llvq_mat* m);
+
+/* Shape and accounting of an uploaded matrix (FusedMatrix fields, fused.rs:566-588). */
+int llvq_hip_matrix_info(const llvq_mat* m, uint32_t* d_out, uint32_t* d_in, uint32_t* nblocks,
+                         uint32_t* tail_w, uint64_t* device_bytes);
+const char* llvq_hip_matrix_name(const llvq_mat* m);
+
+/* forward_rotated (fused_cuda.rs:384) for one activation: y = W x.
+ * x: d_in binary16 values on the device; y: d_out values of y_dtype. */
+int llvq_hip_gemv(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, void* y_dev, int y_dtype);
+
+/* group_forward (llvq-llm/src/model.rs:497-536) for projections that share an
+ * activation (q/k/v, gate/up): one launch over the concatenated rows. */
+int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x_f16_dev,
+                        void* const* y_dev, int y_dtype);
+
+/* The row loop of group_forward (model.rs:521-529) as one batched product:
+ * Y[M, d_out] = X[M, d_in] W^T, X row-major binary16. */
+int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, int M, void* y_dev,
+                  int y_dtype);
+
+/* Parity probe (the role of decode_probe, llvq-cuda/kernels/preflight.cu:39):
+ * unrank packed 6-byte records on the device.  points: 24 int8 per block;
+ * gains: one byte per block; shells (may be NULL): one byte per block. */
+int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks,
+                           int8_t* points_dev, uint8_t* gains_dev, uint8_t* shells_dev);
+
+int llvq_hip_synchronize(llvq_rt* rt);
+const char* llvq_hip_last_error(void);
+const char* llvq_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

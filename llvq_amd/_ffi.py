@@ -1,0 +1,87 @@
+"""ctypes binding of include/llvq_hip.h.  There is no fallback: if the HIP
+library is missing every entry point raises."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "csrc", "libllvq_hip.so")
+
+STATUS = {
+    0: "Ok", 1: "NotAnArtifact", 2: "Truncated", 3: "BadName", 5: "Inconsistent", 7: "IndexTooWide",
+    8: "IndexOutOfRange", 10: "CodebookMismatch", 11: "UnknownVersion", 32: "InvalidArgument",
+    33: "Unsupported", 34: "Device",
+}
+F32, F16 = 0, 1
+FINGERPRINT = 0x338F420F11866319
+
+
+class LlvqError(RuntimeError):
+    def __init__(self, code, message):
+        self.code = code
+        self.kind = STATUS.get(code, str(code))
+        super().__init__(f"{self.kind}: {message}")
+
+
+class MatrixDesc(C.Structure):
+    _fields_ = [
+        ("name", C.c_char_p),
+        ("d_out", C.c_uint32), ("d_in", C.c_uint32), ("shell_cap", C.c_uint32), ("n_centroids", C.c_uint32),
+        ("centroids", C.c_void_p), ("row_scales", C.c_void_p), ("tail", C.c_void_p),
+        ("codes", C.c_void_p), ("code_bytes", C.c_size_t),
+        ("rotation_seed", C.c_uint64), ("has_rotation", C.c_uint32),
+    ]
+
+
+def lib_path():
+    return _LIB
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB):
+        raise RuntimeError(
+            f"{_LIB} is missing: build it with `make -C {os.path.dirname(_LIB)}` "
+            "(or __graft_entry__.build()); there is no CPU fallback")
+    L = C.CDLL(_LIB)
+    vp, sz = C.c_void_p, C.c_size_t
+    L.llvq_hip_runtime_create.argtypes = [C.c_int, vp, C.POINTER(vp)]
+    L.llvq_hip_runtime_destroy.argtypes = [vp]
+    L.llvq_hip_runtime_destroy.restype = None
+    L.llvq_hip_codebook_fingerprint.restype = C.c_uint64
+    L.llvq_hip_host_decode.argtypes = [C.c_uint64, vp, C.POINTER(C.c_int)]
+    L.llvq_hip_matrix_upload.argtypes = [vp, C.POINTER(MatrixDesc), C.POINTER(vp)]
+    L.llvq_hip_read_header.argtypes = [C.c_char_p, sz, C.POINTER(sz), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+    L.llvq_hip_matrix_from_record.argtypes = [vp, C.c_char_p, sz, C.POINTER(sz), C.POINTER(vp)]
+    L.llvq_hip_matrix_free.argtypes = [vp, vp]
+    L.llvq_hip_matrix_free.restype = None
+    L.llvq_hip_matrix_info.argtypes = [vp] + [C.POINTER(C.c_uint32)] * 4 + [C.POINTER(C.c_uint64)]
+    L.llvq_hip_matrix_name.argtypes = [vp]
+    L.llvq_hip_matrix_name.restype = C.c_char_p
+    L.llvq_hip_gemv.argtypes = [vp, vp, vp, vp, C.c_int]
+    L.llvq_hip_gemv_group.argtypes = [vp, C.POINTER(vp), C.c_int, vp, C.POINTER(vp), C.c_int]
+    L.llvq_hip_gemm.argtypes = [vp, vp, vp, C.c_int, vp, C.c_int]
+    L.llvq_hip_decode_blocks.argtypes = [vp, vp, sz, vp, vp, vp]
+    L.llvq_hip_synchronize.argtypes = [vp]
+    L.llvq_hip_last_error.restype = C.c_char_p
+    L.llvq_hip_version.restype = C.c_char_p
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != 0:
+        raise LlvqError(rc, (lib().llvq_hip_last_error() or b"").decode("utf-8", "replace"))
+
+
+EXPORTS = [
+    "llvq_hip_runtime_create", "llvq_hip_runtime_destroy", "llvq_hip_codebook_fingerprint",
+    "llvq_hip_host_decode", "llvq_hip_matrix_upload", "llvq_hip_read_header", "llvq_hip_matrix_from_record",
+    "llvq_hip_matrix_free", "llvq_hip_matrix_info", "llvq_hip_matrix_name", "llvq_hip_gemv",
+    "llvq_hip_gemv_group", "llvq_hip_gemm", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
+    "llvq_hip_last_error", "llvq_hip_version",
+]

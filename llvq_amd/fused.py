@@ -1,0 +1,215 @@
+"""The quantized-linear operator, host side.
+
+Mirrors the reference's `FusedMatrix` / `fused::load` (llvq-llm/src/fused.rs:566-588,
+:1147) and `FusedProj` / `FusedRuntime::{new, rotate, forward_rotated}`
+(llvq-llm/src/fused_cuda.rs:119-134, :182, :362, :384) over the C ABI of
+include/llvq_hip.h.  torch is used for device buffers and the stream only.
+Refusals name the projection, as the reference's do; nothing here computes.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _ffi
+from .artifact import RawMatrix, read_header, read_matrix_raw
+
+
+class FusedMatrix:
+    """One projection ready to upload (fused.rs:566-588).  The payload is the
+    file's own code stream; there is no load-time transcode on this path."""
+
+    def __init__(self, raw: RawMatrix):
+        # one gain bit is compiled into the kernels (fused.rs:1168-1177)
+        if raw.centroids.size != 2:
+            raise ValueError(f"{raw.name}: {raw.centroids.size} centroids, but the kernels hard-code 1 gain bit")
+        self.raw = raw
+        self.name = raw.name
+        self.d_out, self.d_in = raw.d_out, raw.d_in
+        self.nblocks, self.tail_w = raw.nblocks, raw.tail_w
+        self.gscale = raw.centroids.astype(np.float32)
+        self.rscale = raw.row_scales.astype(np.float32)
+        self.tail = raw.tail
+        self.rotation = None if raw.rotation_seed is None else (raw.d_in, raw.rotation_seed)
+        self.bytes = raw.codes.size + 4 * raw.tail.size + 4 * raw.d_out + 8
+
+
+class FusedModel:
+    def __init__(self, matrices):
+        self.matrices = list(matrices)
+        self.runtime_bytes = sum(m.bytes for m in self.matrices)
+
+
+def load(path: str) -> FusedModel:
+    """fused::load (fused.rs:1147): header, then every matrix record, host only."""
+    with open(path, "rb") as f:
+        buf = f.read()
+    return load_bytes(buf)
+
+
+def load_bytes(buf) -> FusedModel:
+    _version, n, pos = read_header(buf)
+    mats = []
+    for _ in range(n):
+        raw, pos = read_matrix_raw(buf, pos)
+        mats.append(FusedMatrix(raw))
+    return FusedModel(mats)
+
+
+class FusedProj:
+    """One projection's weights on the device (fused_cuda.rs:119-134)."""
+
+    def __init__(self, rt, handle, fm: FusedMatrix):
+        self._rt = rt
+        self.handle = handle
+        self.name = fm.name
+        self.d_out, self.d_in = fm.d_out, fm.d_in
+        self.nblocks, self.tail_w = fm.nblocks, fm.tail_w
+        self._rotation = fm.rotation
+        self.encoded_bytes = fm.raw.encoded_bytes()
+
+    def rotation(self):
+        return self._rotation
+
+
+class FusedRuntime:
+    """Tables and stream (fused_cuda.rs:145-180).  `FusedRuntime(model, device)`
+    is `FusedRuntime::new`: it returns with every projection uploaded in `projs`."""
+
+    def __init__(self, model: FusedModel = None, device: int = 0, stream=None):
+        import torch
+
+        self._torch = torch
+        self.device = torch.device("cuda", device)
+        L = _ffi.lib()
+        if stream is None:
+            stream = torch.cuda.current_stream(self.device)
+        self._stream = stream
+        h = C.c_void_p()
+        _ffi.check(L.llvq_hip_runtime_create(device, C.c_void_p(stream.cuda_stream), C.byref(h)))
+        self.handle = h
+        self.projs = []
+        if model is not None:
+            for fm in model.matrices:
+                self.projs.append(self.upload(fm))
+
+    def upload(self, fm) -> FusedProj:
+        if isinstance(fm, RawMatrix):
+            fm = FusedMatrix(fm)
+        raw = fm.raw
+        d = _ffi.MatrixDesc()
+        d.name = raw.name.encode()
+        d.d_out, d.d_in, d.shell_cap, d.n_centroids = raw.d_out, raw.d_in, raw.shell_cap, raw.centroids.size
+        d.centroids = raw.centroids.ctypes.data
+        d.row_scales = raw.row_scales.ctypes.data
+        d.tail = raw.tail.ctypes.data if raw.tail.size else None
+        codes = np.ascontiguousarray(raw.codes)
+        d.codes = codes.ctypes.data
+        d.code_bytes = codes.size
+        d.rotation_seed = raw.rotation_seed or 0
+        d.has_rotation = 1 if raw.rotation_seed is not None else 0
+        h = C.c_void_p()
+        _ffi.check(_ffi.lib().llvq_hip_matrix_upload(self.handle, C.byref(d), C.byref(h)))
+        return FusedProj(self, h, fm)
+
+    def upload_record(self, buf, pos=0):
+        """Parse one on-disk record with the library's own reader and upload it."""
+        p = C.c_size_t(pos)
+        h = C.c_void_p()
+        _ffi.check(_ffi.lib().llvq_hip_matrix_from_record(self.handle, bytes(buf), len(buf), C.byref(p), C.byref(h)))
+        raw, _ = read_matrix_raw(buf, pos)
+        return FusedProj(self, h, FusedMatrix(raw)), p.value
+
+    def free(self, proj: FusedProj):
+        if proj.handle:
+            _ffi.lib().llvq_hip_matrix_free(self.handle, proj.handle)
+            proj.handle = None
+
+    # -- the operator ---------------------------------------------------------------
+    def rotate(self, proj: FusedProj, x):
+        """FusedRuntime::rotate (fused_cuda.rs:362): one activation into the basis
+        the projection was quantized in.  Natural-basis matrices pass through."""
+        torch = self._torch
+        d_in = x.shape[-1]
+        if d_in != proj.d_in:
+            raise ValueError(f"{proj.name} expects d_in={proj.d_in}, got {d_in}")
+        rows = x.numel() // d_in
+        if rows != 1:
+            raise ValueError(f"{proj.name}: rotation asked for {rows} vectors; the row loop belongs to the caller")
+        if proj.rotation() is not None:
+            raise ValueError(f"{proj.name}: stored in a rotated basis; activation rotation is not built yet")
+        return x.to(torch.float16).contiguous()
+
+    def forward_rotated(self, proj: FusedProj, xr, out_dims=None, out_dtype=None):
+        """FusedRuntime::forward_rotated (fused_cuda.rs:384): y = W' xr, shaped like
+        the caller's tensor with the last dim replaced by d_out.  f16 out by default."""
+        torch = self._torch
+        if not xr.is_cuda:
+            raise ValueError("the fused LLVQ kernel has no CPU path")
+        if not xr.is_contiguous():
+            raise ValueError("activation is not contiguous")
+        if xr.dtype != torch.float16:
+            raise ValueError(f"{proj.name}: activation must be binary16, got {xr.dtype}")
+        if xr.numel() != proj.d_in:
+            raise ValueError(f"rotated activation of {xr.numel()} values for d_in={proj.d_in}")
+        out_dtype = out_dtype or torch.float16
+        dims = list(out_dims if out_dims is not None else xr.shape)
+        dims[-1] = proj.d_out
+        y = torch.empty(dims, dtype=out_dtype, device=xr.device)  # uninitialised: every row is stored
+        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        _ffi.check(_ffi.lib().llvq_hip_gemv(self.handle, proj.handle, xr.data_ptr(), y.data_ptr(), code))
+        return y
+
+    def forward(self, proj: FusedProj, x, out_dtype=None):
+        return self.forward_rotated(proj, self.rotate(proj, x), x.shape, out_dtype)
+
+    def forward_group(self, projs, x, out_dtype=None):
+        """group_forward (llvq-llm/src/model.rs:497-536) for projections sharing one activation."""
+        torch = self._torch
+        xr = self.rotate(projs[0], x)
+        out_dtype = out_dtype or torch.float16
+        ys = [torch.empty(list(x.shape[:-1]) + [p.d_out], dtype=out_dtype, device=xr.device) for p in projs]
+        mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
+        outs = (C.c_void_p * len(projs))(*[y.data_ptr() for y in ys])
+        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        _ffi.check(_ffi.lib().llvq_hip_gemv_group(self.handle, mats, len(projs), xr.data_ptr(), outs, code))
+        return ys
+
+    def forward_batched(self, proj: FusedProj, x, out_dtype=None):
+        """Rows of `x` [M, d_in] through one projection (the row loop of model.rs:521-529)."""
+        torch = self._torch
+        if x.dim() != 2 or x.shape[1] != proj.d_in:
+            raise ValueError(f"{proj.name} expects [M, {proj.d_in}], got {list(x.shape)}")
+        x = x.to(torch.float16).contiguous()
+        out_dtype = out_dtype or torch.float16
+        y = torch.empty((x.shape[0], proj.d_out), dtype=out_dtype, device=x.device)
+        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        _ffi.check(_ffi.lib().llvq_hip_gemm(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
+        return y
+
+    def decode_blocks(self, codes):
+        """Parity probe: packed 6-byte records (uint8 tensor on the device) →
+        (points int8 [n,24], gains uint8 [n], shells uint8 [n])."""
+        torch = self._torch
+        n = codes.numel() // 6
+        pts = torch.empty((n, 24), dtype=torch.int8, device=codes.device)
+        gains = torch.empty(n, dtype=torch.uint8, device=codes.device)
+        shells = torch.empty(n, dtype=torch.uint8, device=codes.device)
+        _ffi.check(_ffi.lib().llvq_hip_decode_blocks(self.handle, codes.data_ptr(), n, pts.data_ptr(),
+                                                      gains.data_ptr(), shells.data_ptr()))
+        return pts, gains, shells
+
+    def synchronize(self):
+        _ffi.check(_ffi.lib().llvq_hip_synchronize(self.handle))
+
+    def close(self):
+        if self.handle:
+            for p in self.projs:
+                self.free(p)
+            _ffi.lib().llvq_hip_runtime_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

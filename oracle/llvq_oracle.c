@@ -1027,7 +1027,7 @@ int orc_read_matrix_raw(const uint8_t* buf, size_t len, size_t* pos, orc_raw_mat
   if (tail_n * 4 > len - *pos) FAIL(ORC_TRUNCATED, "tail");
   m->tail = (double*)malloc(sizeof(double) * (tail_n ? tail_n : 1));
   for (uint64_t i = 0; i < tail_n; i++) {
-    uint32_t b;
+    uint32_t b = 0;
     float f;
     get_u32(buf, len, pos, &b);
     memcpy(&f, &b, 4);
@@ -1288,6 +1288,17 @@ int orc_cpu_gemv(const uint8_t* codes, size_t d_out, size_t d_in, const double* 
   }
   free(xf);
   return err;
+}
+
+int orc_decode_batch(const uint64_t* idx, size_t n, int8_t* out, int fast) {
+  ensure_init();
+  for (size_t k = 0; k < n; k++) {
+    int32_t p[ORC_DIM];
+    int ok = fast ? orc_fast_decode(idx[k], p) : orc_index_decode(idx[k], p);
+    if (!ok) return ORC_INDEX_OUT_OF_RANGE;
+    for (int q = 0; q < ORC_DIM; q++) out[k * ORC_DIM + q] = (int8_t)p[q];
+  }
+  return ORC_OK;
 }
 
 uint64_t orc_cpu_decode_only(const uint8_t* codes, size_t nblocks) {

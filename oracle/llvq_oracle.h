@@ -68,6 +68,8 @@ int orc_index_decode(uint64_t idx, int32_t out[ORC_DIM]);
 int orc_index_encode(const int32_t p[ORC_DIM], uint64_t* idx);
 /* fastdec.rs:321-399 (u64 recurrence).  Same contract as orc_index_decode. */
 int orc_fast_decode(uint64_t idx, int32_t out[ORC_DIM]);
+/* n indices -> n*24 int8 coordinates with either decoder; ORC_INDEX_OUT_OF_RANGE on a bad index. */
+int orc_decode_batch(const uint64_t* idx, size_t n, int8_t* out, int fast);
 int orc_class_of(uint64_t idx);                      /* fastdec.rs:293-298; -1 for 0 and > N13 */
 /* fastdec.rs:402-433 — canonical level table of a class. */
 void orc_class_levels(int ci, int32_t values[5], uint8_t counts[5], int* len,

@@ -107,6 +107,7 @@ def lib():
     L.orc_f32_to_f16.argtypes = [C.c_float]
     L.orc_cpu_gemv.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.POINTER(C.c_double), C.POINTER(C.c_double),
                                C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+    L.orc_decode_batch.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int]
     L.orc_cpu_decode_only.restype = C.c_uint64
     L.orc_cpu_decode_only.argtypes = [C.c_void_p, C.c_size_t]
     _lib = L
@@ -140,16 +141,12 @@ def fast_decode(idx):
 
 def decode_many(indices, fast=True):
     """Decode an array of indices to an int8 [n, 24] array (every index must be valid)."""
-    L = lib()
-    f = L.orc_fast_decode if fast else L.orc_index_decode
     idx = np.ascontiguousarray(indices, dtype=np.uint64)
-    out = np.zeros((idx.size, DIM), np.int32)
-    base = out.ctypes.data
-    i32p = C.POINTER(C.c_int32)
-    for k in range(idx.size):
-        if not f(int(idx[k]), C.cast(base + k * DIM * 4, i32p)):
-            raise OracleError(8, f"index {int(idx[k])}")
-    return out.astype(np.int8)
+    out = np.zeros((idx.size, DIM), np.int8)
+    rc = lib().orc_decode_batch(idx.ctypes.data, idx.size, out.ctypes.data, 1 if fast else 0)
+    if rc:
+        raise OracleError(rc)
+    return out
 
 
 def index_encode(p):

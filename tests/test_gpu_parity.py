@@ -1,0 +1,227 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI.
+
+Bars: lattice points and (index, gain) fields bit-exact; GEMV within 1e-3 of the
+f64 reference, measured as |y - y_ref| / sum|w_i x_i| (the reference's own V0
+metric, llvq-cuda/src/bin/matvec.rs:114-120) and as plain relative error where
+|y_ref| is not tiny.
+"""
+import numpy as np
+import pytest
+
+from llvq_amd import artifact, synth
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3  # north-star tolerance for GEMV/GEMM outputs (f32 accumulate)
+
+
+def _dev(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _x16(x):
+    import torch
+
+    return torch.from_numpy(x.view(np.int16).copy()).view(torch.float16).cuda()
+
+
+def _oracle_matrix(orc, raw):
+    m, _ = orc.read_matrix_raw(artifact.write_matrix_raw(raw))
+    return m
+
+
+def _check_gemv(orc, y, raw, x):
+    om = _oracle_matrix(orc, raw)
+    y_ref, a_ref = om.fused_product(x.astype(np.float64))
+    y = y.astype(np.float64)
+    e_norm = np.abs(y - y_ref) / np.maximum(a_ref, 1e-30)
+    assert e_norm.max() < TOL, f"max |dy|/sum|wx| = {e_norm.max():.3e}"
+    big = np.abs(y_ref) > 1e-2 * a_ref
+    if big.any():
+        rel = np.abs(y - y_ref)[big] / np.abs(y_ref)[big]
+        assert rel.max() < TOL, f"max relative error {rel.max():.3e}"
+    return e_norm.max()
+
+
+def test_decode_class_boundaries_bit_exact(gpu_rt, orc, boundary_indices):
+    idx = boundary_indices[boundary_indices < (1 << 47)]  # what a 47-bit field can hold
+    gains = (np.arange(idx.size) & 1).astype(np.uint8)
+    pts, g, shells = gpu_rt.decode_blocks(_dev(artifact.pack_codes(idx, gains)))
+    ref = orc.decode_many(idx, fast=False)
+    assert np.array_equal(pts.cpu().numpy(), ref)
+    assert np.array_equal(g.cpu().numpy(), gains)
+    ref_shell = (ref.astype(np.int64) ** 2).sum(1) // 16
+    assert np.array_equal(shells.cpu().numpy().astype(np.int64), ref_shell)
+
+
+def test_decode_zero_run_free_classes(gpu_rt, orc):
+    """Even classes with no zero coordinate: the case where 'last kind = zero run'
+    must be decided by value (llvq-metal/shaders/cascade_archive.metal:186-205)."""
+    picks = []
+    for ci in range(orc.lib().orc_n_classes()):
+        info = orc.class_info(ci)
+        vals, counts, _ = orc.class_levels(ci)
+        if not info["odd"] and 0 not in vals and info["lo"] < (1 << 47):
+            hi = min(info["hi"], (1 << 47) - 1)
+            picks += list(np.linspace(info["lo"], hi, 64, dtype=np.uint64))
+    assert len(picks) >= 6 * 64
+    idx = np.array(picks, dtype=np.uint64)
+    pts, _, _ = gpu_rt.decode_blocks(_dev(artifact.pack_codes(idx, np.zeros(idx.size, np.uint8))))
+    assert np.array_equal(pts.cpu().numpy(), orc.decode_many(idx))
+
+
+def test_decode_million_uniform_ranks_bit_exact(gpu_rt, orc):
+    rng = synth.SplitMix64(0x63_0001)
+    idx = rng.take(1_000_000) % np.uint64(orc.N12 + 1)
+    gains = (rng.take(idx.size) & np.uint64(1)).astype(np.uint8)
+    pts, g, _ = gpu_rt.decode_blocks(_dev(artifact.pack_codes(idx, gains)))
+    assert np.array_equal(pts.cpu().numpy(), orc.decode_many(idx))
+    assert np.array_equal(g.cpu().numpy(), gains)
+
+
+def test_decode_full_47bit_range(gpu_rt, orc):
+    """Indices in (N(12), 2^47) fit the field and decode as shell-13 points."""
+    rng = synth.SplitMix64(7)
+    idx = rng.take(200_000) % np.uint64(1 << 47)
+    pts, _, shells = gpu_rt.decode_blocks(_dev(artifact.pack_codes(idx, np.zeros(idx.size, np.uint8))))
+    assert np.array_equal(pts.cpu().numpy(), orc.decode_many(idx))
+    assert shells.max().item() == 13
+
+
+def test_decode_empty(gpu_rt):
+    import torch
+
+    pts, g, s = gpu_rt.decode_blocks(torch.empty(0, dtype=torch.uint8, device="cuda"))
+    assert pts.shape == (0, 24) and g.numel() == 0
+
+
+# (d_out, d_in) of llvq-artifact/tests/fused_path_matches_dense.rs:45-51 plus ragged shapes
+SMALL_SHAPES = [(8, 240), (8, 2560), (16, 9728), (8, 4096), (24, 96), (1, 24), (3, 47), (5, 2568), (7, 5120)]
+
+
+@pytest.mark.parametrize("d_out,d_in", SMALL_SHAPES)
+def test_gemv_small_shapes(gpu_rt, orc, d_out, d_in):
+    import torch
+
+    raw = synth.make_matrix(f"model.layers.0.test.{d_out}x{d_in}.weight", d_out, d_in, seed=d_out * 131 + d_in)
+    x = synth.make_activation(d_in, seed=d_in)[0]
+    proj = gpu_rt.upload(raw)
+    try:
+        y32 = gpu_rt.forward(proj, _x16(x), out_dtype=torch.float32).cpu().numpy()
+        y16 = gpu_rt.forward(proj, _x16(x)).cpu().numpy()
+    finally:
+        gpu_rt.free(proj)
+    e = _check_gemv(orc, y32, raw, x)
+    assert e < 1e-5  # f32 out: the reference's own threshold (docs/mesures/e1v-cuda-2026-08-16.txt:95-96)
+    _check_gemv(orc, y16.astype(np.float32), raw, x)
+
+
+def test_gemv_origin_and_shell13_blocks(gpu_rt, orc):
+    """A matrix whose blocks are origins (decode to zero whatever the gain) and
+    shell-13 indices above N(12)."""
+    import torch
+
+    d_out, d_in = 16, 24 * 8 + 5
+    rng = synth.SplitMix64(99)
+    idx = rng.take(d_out * 8) % np.uint64(1 << 47)
+    idx[::3] = 0
+    idx[1::7] = np.uint64((1 << 47) - 1)
+    gains = (rng.take(idx.size) & np.uint64(1)).astype(np.uint8)
+    raw = artifact.RawMatrix("model.layers.0.edge.weight", d_out, d_in, 12, [0.8, 1.25],
+                             np.exp(rng.gaussian(d_out)), rng.gaussian(d_out * 5).astype(np.float32),
+                             artifact.pack_codes(idx, gains))
+    x = synth.make_activation(d_in, seed=5)[0]
+    proj = gpu_rt.upload(raw)
+    y = gpu_rt.forward(proj, _x16(x), out_dtype=torch.float32).cpu().numpy()
+    gpu_rt.free(proj)
+    _check_gemv(orc, y, raw, x)
+
+
+def test_gemv_config0_full_size(gpu_rt, orc):
+    """BASELINE config 0: gate_proj 9728 x 2560, seed 0, against the oracle's f64 product."""
+    import torch
+
+    raw = synth.config0(seed=0)
+    assert raw.encoded_bytes() == 6_887_440
+    x = synth.make_activation(2560, seed=0)[0]
+    proj = gpu_rt.upload(raw)
+    y = gpu_rt.forward(proj, _x16(x), out_dtype=torch.float32).cpu().numpy()
+    gpu_rt.free(proj)
+    e = _check_gemv(orc, y, raw, x)
+    assert e < 1e-5
+
+
+def test_gemv_group_matches_single(gpu_rt, orc):
+    import torch
+
+    mats = [synth.make_matrix(f"model.layers.1.self_attn.{n}.weight", do, 2560, seed=3)
+            for n, do in (("q_proj", 96), ("k_proj", 32), ("v_proj", 32))]
+    x = synth.make_activation(2560, seed=11)[0]
+    projs = [gpu_rt.upload(m) for m in mats]
+    ys = gpu_rt.forward_group(projs, _x16(x), out_dtype=torch.float32)
+    for p, raw, y in zip(projs, mats, ys):
+        single = gpu_rt.forward(p, _x16(x), out_dtype=torch.float32)
+        assert torch.equal(single, y)
+        _check_gemv(orc, y.cpu().numpy(), raw, x)
+        gpu_rt.free(p)
+
+
+def test_batched_rows_match_oracle(gpu_rt, orc):
+    import torch
+
+    raw = synth.make_matrix("model.layers.2.mlp.up_proj.weight", 64, 2560, seed=4)
+    X = synth.make_activation(2560, seed=21, rows=16)
+    proj = gpu_rt.upload(raw)
+    Y = gpu_rt.forward_batched(proj, _x16(X), out_dtype=torch.float32).cpu().numpy()
+    gpu_rt.free(proj)
+    for r in range(X.shape[0]):
+        _check_gemv(orc, Y[r], raw, X[r])
+
+
+def test_record_upload_path(gpu_rt, orc):
+    """The library's own record reader: an on-disk LVQ4 file, parsed and uploaded through the C ABI."""
+    import ctypes as C
+
+    import torch
+
+    from llvq_amd import _ffi
+
+    mats = [synth.make_matrix(f"model.layers.0.self_attn.{n}.weight", 16, 2560, seed=8) for n in ("q_proj", "k_proj")]
+    buf = artifact.write_file(mats, version=4)
+    pos = C.c_size_t(0)
+    ver, n = C.c_uint32(), C.c_uint32()
+    _ffi.check(_ffi.lib().llvq_hip_read_header(buf, len(buf), C.byref(pos), C.byref(ver), C.byref(n)))
+    assert (ver.value, n.value) == (4, 2)
+    x = synth.make_activation(2560, seed=1)[0]
+    p = pos.value
+    for raw in mats:
+        proj, p = gpu_rt.upload_record(buf, p)
+        assert proj.name == raw.name
+        y = gpu_rt.forward(proj, _x16(x), out_dtype=torch.float32).cpu().numpy()
+        gpu_rt.free(proj)
+        _check_gemv(orc, y, raw, x)
+    assert p == len(buf) - 8
+
+
+def test_full_size_properties_linearity_and_scaling(gpu_rt):
+    """Size-independent properties at config-0 size: y(2x) = 2 y(x) exactly in
+    binary floating point, and y is linear in the activation to rounding."""
+    import torch
+
+    raw = synth.config0(seed=0)
+    proj = gpu_rt.upload(raw)
+    x = _x16(synth.make_activation(2560, seed=0)[0])
+    z = _x16(synth.make_activation(2560, seed=1)[0])
+    y1 = gpu_rt.forward(proj, x, out_dtype=torch.float32)
+    y2 = gpu_rt.forward(proj, (x * 2).contiguous(), out_dtype=torch.float32)
+    assert torch.equal(y2, 2 * y1)
+    half = torch.float16
+    xz = (x.float() * 0.5 + z.float() * 0.5).to(half)  # may round: compare against f32 products of the rounded sum
+    yz = gpu_rt.forward(proj, xz, out_dtype=torch.float32)
+    exact = (xz.float() == x.float() * 0.5 + z.float() * 0.5)
+    lin = 0.5 * y1 + 0.5 * gpu_rt.forward(proj, z, out_dtype=torch.float32)
+    if bool(exact.all()):
+        assert torch.allclose(yz, lin, rtol=1e-4, atol=1e-6)
+    gpu_rt.free(proj)
