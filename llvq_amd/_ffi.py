@@ -47,6 +47,13 @@ def lib():
         raise RuntimeError(
             f"{_LIB} is missing: build it with `make -C {os.path.dirname(_LIB)}` "
             "(or __graft_entry__.build()); there is no CPU fallback")
+    # torch ships its own HIP runtime; load it first so the process holds exactly
+    # one (libllvq_hip.so's libamdhip64 dependency then resolves to that one, and
+    # the two share devices, streams and allocations).
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(_LIB)
     vp, sz = C.c_void_p, C.c_size_t
     L.llvq_hip_runtime_create.argtypes = [C.c_int, vp, C.POINTER(vp)]

@@ -401,9 +401,9 @@ int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y,
 
 int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks, int8_t* points_dev,
                            uint8_t* gains_dev, uint8_t* shells_dev) {
-  if (!rt || !points_dev || (nblocks && !codes_dev))
-    return fail(LLVQ_ERR_INVALID_ARGUMENT, "decode_blocks: null argument");
-  if (nblocks == 0) return LLVQ_OK;
+  if (!rt) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decode_blocks: runtime is null");
+  if (nblocks == 0) return LLVQ_OK;  // an empty stream is valid and writes nothing
+  if (!points_dev || !codes_dev) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decode_blocks: null argument");
   HIP_TRY(hipSetDevice(rt->device));
   size_t grid = (nblocks + 255) / 256;
   const size_t cap = (size_t)(rt->cu_count > 0 ? rt->cu_count : 256) * 2;
