@@ -20,7 +20,10 @@ constexpr uint64_t kN13 = 280974212784720ULL;  // llvq-core/src/leech.rs:54
 constexpr uint64_t kFingerprint = 0x338f420f11866319ULL;  // llvq-artifact/tests/codebook_fingerprint.rs:58
 constexpr int kMaxShell = 13;
 constexpr int kClassSlots = 384;   // 383 classes + one sentinel, a power-of-two-friendly size
-constexpr int kEndsPadded = 512;   // class ends padded for a fixed-depth search
+constexpr int kStartsPadded = 512; // class starts, padded with UINT64_MAX past N(13)
+constexpr int kLutShift = 36;      // class-find table is keyed on the zero-based index >> 36
+constexpr int kOnLutSlots = 4352;  // LDS slots for the support-arrangement table (4322 entries used)
+constexpr int kLutSize = 4096;     // covers every zero-based index < N(13) < 2^48 (a 47-bit field uses the lower half)
 
 struct KindCount {
   int value;
@@ -69,15 +72,49 @@ constexpr int kMetaPreqShift = 6;          // bit 6       p_req
 constexpr int kMetaSfShift = 7;            // bits 7..11  free-sign bits
 constexpr int kMetaSwShift = 12;           // bits 12..16 support-sign bits (w-1, or 0)
 
+// LDS-resident class record of the two fast decode paths, 48 bytes.
+//   odd-coset walk:   inv0 = 1/m_arr, d1 = m_arr, u0 = packed thresholds, tab = signed value table
+//   even-coset table: inv0 = 1/a_off, d1 = 1/a_on, u0 = first on_lut entry | second free value << 16,
+//                     u1 = first off_lut entry, a_off/a_on as floats (both < 2^24), tab = signed value table
+// `tab` is the 8-byte table a byte-permute indexes with a 3-bit code per coordinate:
+//   odd:  code = (3 - kind) | (off-support ? 4 : 0); bytes 0..3 = a_kind, bytes 4..7 = -a_kind
+//   even: code = on-support | primary-kind << 1 | minus << 2
+struct alignas(16) FastClass {
+  double inv0;
+  double d1;
+  uint32_t u0, u1;
+  float inv_norm;
+  uint32_t meta;     // kMeta* fields, path in bits 17..18, golay_base in bits 20..31
+  float a_off, a_on;
+  uint32_t tab_lo, tab_hi;
+};
+static_assert(sizeof(FastClass) == 48, "FastClass must stay 48 bytes");
+
+constexpr int kMetaPathShift = 17;         // bits 17..18: which decoder a class takes
+constexpr int kMetaGolayShift = 20;        // bits 20..31: first codeword of the weight bucket
+enum : uint32_t { kPathOdd = 0, kPathEven = 1, kPathGeneric = 2 };
+
 struct Codebook {
   uint32_t golay[4096];
   int bucket_start[26];
   std::vector<ClassDef> classes;          // 383, format order
   // device-shaped tables
   DevClass dev_classes[kClassSlots];
-  uint64_t ends[kEndsPadded];             // offset + card per class, then UINT64_MAX
+  uint64_t starts[kStartsPadded];         // starts[c] = offset of class c, starts[383] = N(13), then UINT64_MAX
+  uint16_t lut[kLutSize];                 // class holding zero-based index (key << kLutShift), clamped to 382
   double rcp[32];                         // rcp[c] = 1/c, rcp[0] unused
   uint64_t n12 = 0;                       // points in the cap-12 ball (47-bit field)
+  // fast paths
+  FastClass fast[kClassSlots];
+  // Arrangement tables of the even coset, slot space: entry r of a problem is the
+  // r-th arrangement in lexicographic order (index.rs:97-117) as two 16-bit slot
+  // masks, kind 0 in the low half and kind 1 in the high half.
+  std::vector<uint32_t> on_lut;           // support problems (w in {8,12,16}, at most 2 word kinds)
+  std::vector<uint32_t> off_lut;          // off-support problems (24-w slots, free kinds then the zero run)
+  // Per codeword, the five move masks that deposit slot bits onto the set
+  // positions of the word (dwords 0..3) and onto its unset positions (4..7).
+  uint32_t expand[4096][8];
+  uint8_t pdep4[256];                     // pdep4[mask << 4 | bits]: low bits of `bits` onto the set bits of `mask`
 };
 
 const Codebook& codebook();

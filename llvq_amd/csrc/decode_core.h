@@ -12,22 +12,32 @@
 //    true quotient (x + 1/2)/d is at least 1/(2d) away from every integer,
 //    the computed one is off by at most q * 2^-52, and q * d <= x.
 //
-//  * Multiset-permutation unranking without ever forming an arrangement count.
-//    With M arrangements of the remaining multiset, n slots left and kind
-//    counts c_0.. (prefix sums T_0 = 0, T_1, ...), the reference picks the
-//    kind j with  M T_j / n <= rank < M T_{j+1} / n  and continues with
-//    rank' = rank - M T_j / n,  M' = M c_j / n  (fastdec.rs:173-194).  Writing
-//    rho = (rank + 1/2) / M  this is:  t = rho n;  j = the kind of sorted
-//    element floor(t);  rho' = (t - T_j) / c_j  — and rho' equals
+//  * Odd coset — multiset-permutation unranking without ever forming an
+//    arrangement count.  With M arrangements of the remaining multiset, n slots
+//    left and kind counts c_0.. (prefix sums T_0 = 0, T_1, ...), the reference
+//    picks the kind j with  M T_j / n <= rank < M T_{j+1} / n  and continues
+//    with rank' = rank - M T_j / n,  M' = M c_j / n  (fastdec.rs:173-194).
+//    Writing rho = (rank + 1/2) / M  this is:  t = rho n;  j = the kind of
+//    sorted element floor(t);  rho' = (t - T_j) / c_j  — and rho' equals
 //    (rank' + 1/2) / M' exactly, so the half-unit guard band travels with the
 //    recurrence.  A decision is wrong only if the accumulated error of rho,
-//    measured in units of 1/M, reaches 1/2; that error grows by about 2^-52 M_i
-//    per step and M <= 5 354 228 880 < 2^33, so FP64 leaves a factor > 2^10.
+//    measured in units of 1/M, reaches 1/2; that error grows by about
+//    2^-52 M_i per step and M <= 5 354 228 880 < 2^33, so FP64 leaves a factor
+//    > 2^10.  The k-1 comparisons of one step are done at once on thresholds
+//    packed into 6-bit fields of one register (a guard bit per field turns the
+//    per-field comparison into one subtraction).
 //
-//  * The k-1 comparisons of one step are done at once on thresholds packed
-//    into 6-bit fields of one register (a guard bit per field turns the
-//    per-field comparison into one subtraction), so a step costs the same for
-//    2 and for 5 kinds and needs no per-lane indexed registers.
+//  * Even coset (support weight 8, 12 or 16, at most two word kinds — all but
+//    0.04 % of uniformly drawn blocks) — no walk at all.  The two arrangement
+//    ranks index tables of slot masks; slot masks and sign bits are moved to
+//    coordinate positions by a five-step parallel bit deposit whose move masks
+//    are stored per codeword.
+//
+//  * Every path ends in a 3-bit code per coordinate, four codes per dword, that
+//    a byte permute turns into signed 8-bit lattice coordinates.
+//
+// Classes outside the fast paths (five magnitudes on the odd coset, support
+// weight 0 or 24, three word kinds) take the generic walk of both cosets.
 #pragma once
 #include <cstdint>
 
@@ -43,16 +53,25 @@
 namespace llvq {
 
 struct DecodeTables {
-  const uint32_t* golay;   // 4096 codewords, canonical order
-  const DevClass* cls;     // kClassSlots records
-  const uint64_t* ends;    // kEndsPadded class ends
-  const double* rcp;       // rcp[c] = 1/c for c in 1..24
+  const uint32_t* golay;    // 4096 codewords, canonical order
+  const DevClass* cls;      // generic-walk class records
+  const FastClass* fast;    // fast-path class records
+  const uint64_t* starts;   // starts[c] = first zero-based index of class c; starts[383] = N(13)
+  const uint16_t* lut;      // lut[i >> kLutShift] = class holding zero-based index (key << kLutShift)
+  const double* rcp;        // rcp[c] = 1/c for c in 1..24
+  const uint32_t* on_lut;   // even coset, support arrangements
+  const uint32_t* off_lut;  // even coset, off-support arrangements
+  const uint32_t* expand;   // 8 dwords per codeword: deposit masks for the word and for its complement
+  const uint8_t* pdep4;     // 4-bit deposit table
 };
 
 // Threshold packing: field f (bits 6f..6f+4) holds T_{4-f}; bit 6f+5 is the
 // field's guard bit.  Fields of kinds a problem does not have hold n.
 constexpr uint32_t kFieldOnes = 1u | (1u << 6) | (1u << 12) | (1u << 18);
 constexpr uint32_t kFieldGuard = kFieldOnes << 5;
+
+// bit k of a nibble -> bit 0 / 1 / 2 of byte k
+constexpr uint32_t kSpread0 = 0x00204081u, kSpread1 = 0x00408102u, kSpread2 = 0x00810204u;
 
 LLVQ_HD uint32_t popc32(uint32_t v) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -62,15 +81,15 @@ LLVQ_HD uint32_t popc32(uint32_t v) {
 #endif
 }
 
-LLVQ_HD double floor64(double v) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  return __builtin_floor(v);
-#else
-  return __builtin_floor(v);
-#endif
-}
-
+LLVQ_HD double floor64(double v) { return __builtin_floor(v); }
 LLVQ_HD double fma64(double a, double b, double c) { return __builtin_fma(a, b, c); }
+LLVQ_HD uint32_t bfi32(uint32_t mask, uint32_t a, uint32_t b) { return (a & mask) | (b & ~mask); }
+
+// signed byte `code` (0..7) of the 8-byte table {hi:lo}
+LLVQ_HD int table_byte(uint32_t lo, uint32_t hi, uint32_t code) {
+  const uint32_t w = code & 4u ? hi : lo;
+  return (int)(int8_t)(w >> (8u * (code & 3u)));
+}
 
 // One slot of the arrangement walk.  Returns jj = 4 - kind.
 LLVQ_HD uint32_t walk_step(double& rho, uint32_t& tg, uint32_t n, const double* rcp) {
@@ -87,52 +106,122 @@ LLVQ_HD uint32_t walk_step(double& rho, uint32_t& tg, uint32_t n, const double* 
   return jj;
 }
 
-// Count of class ends <= i over the padded table: fixed nine probes.
-LLVQ_HD uint32_t find_class(const uint64_t* ends, uint64_t i) {
-  uint32_t lo = 0;
-#pragma unroll
-  for (uint32_t step = 256; step >= 1; step >>= 1)
-    if (ends[lo + step - 1] <= i) lo += step;
-  return lo;
+// Class of the zero-based index i < N(13): one table probe on the top bits,
+// then a short forward scan (empty for 96 % of uniformly drawn indices).
+LLVQ_HD uint32_t find_class(const DecodeTables& T, uint64_t i) {
+  uint32_t ci = T.lut[(uint32_t)(i >> kLutShift)];
+  while (ci < 382u && T.starts[ci + 1] <= i) ++ci;
+  return ci;
 }
 
-// Decodes `idx` and calls emit(position, value) for positions 0..23 in order.
-// Returns the class index, -1 for the origin, -2 for an index past N(13)
-// (which emits zeros).
-template <class Emit>
-LLVQ_HD int decode_index(const DecodeTables& T, uint64_t idx, Emit&& emit) {
-  if (idx == 0 || idx > kN13) {
-    for (int p = 0; p < kDim; ++p) emit(p, 0);
-    return idx == 0 ? -1 : -2;
-  }
-  const uint64_t i = idx - 1;
-  uint32_t ci = find_class(T.ends, i);
-  if (ci > 382u) ci = 382u;
-  const uint64_t offset = ci ? T.ends[ci - 1] : 0;
-  const DevClass c = T.cls[ci];
-  uint64_t li = i - offset;
-
-  if (c.meta & kMetaOdd) {
-    // local = g * m_arr + r_arr  (index.rs:33-36)
-    const double local = (double)li;
-    const double g = floor64((local + 0.5) * c.inv0);
-    const double r = fma64(-g, c.m0, local);
-    double rho = (r + 0.5) * c.inv0;
-    const uint32_t cw = T.golay[(uint32_t)g & 4095u];
-    uint32_t tg = c.tg0;
+// ---- odd coset, fast path (at most four magnitudes) ------------------------------
+// local = g * m_arr + r_arr (index.rs:33-36).  Calls on_codes(q, sel) for q = 0..5:
+// byte j of sel is the table code of coordinate 4q + j,
+// code = (3 - kind) | (coordinate off the codeword's support ? 4 : 0).
+template <class OnCodes>
+LLVQ_HD void odd_codes(const DecodeTables& T, const FastClass& f, uint64_t li, OnCodes&& on_codes) {
+  const double local = (double)li;
+  const double g = floor64((local + 0.5) * f.inv0);
+  const double r = fma64(-g, f.d1, local);
+  double rho = (r + 0.5) * f.inv0;
+  const uint32_t ncw = ~T.golay[(uint32_t)g & 4095u];
+  uint32_t tg = f.u0;
 #pragma unroll
-    for (int p = 0; p < kDim; ++p) {
-      const uint32_t jj = walk_step(rho, tg, (uint32_t)(kDim - p), T.rcp);
-      const int v = (int)((c.vals0 >> (4u * jj)) & 15u);
-      // forced signs (index.rs:417-431): a = v if v = 3 mod 4 else -v; a on the
-      // codeword's support, -a off it.
-      const uint32_t neg = ((cw >> p) ^ ((uint32_t)v >> 1)) & 1u;
-      emit(p, neg ? -v : v);
+  for (int q = 0; q < 6; ++q) {
+    uint32_t sel = (((ncw >> (4 * q)) & 15u) * kSpread2) & 0x04040404u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t jj = walk_step(rho, tg, (uint32_t)(kDim - 4 * q - j), T.rcp);
+      sel |= (jj - 1u) << (8 * j);
     }
-    return (int)ci;
+    on_codes(q, sel);
   }
+}
 
-  // local = (((g A_on + r_on) A_off + r_off) S_w + r_sw) S_f + r_sf  (index.rs:24-32)
+// ---- even coset, fast path --------------------------------------------------------
+// Deposits bit k of x onto the k-th selected position; e = four packed move-mask
+// dwords.  Bits are copied, not moved: positions outside the selection hold
+// leftovers and must be masked off by the caller.
+LLVQ_HD uint32_t expand24(uint32_t x, const uint32_t* e) {
+  const uint32_t e0 = e[0];
+  x = bfi32((e0 >> 8) & 0x00FF0000u, x << 16, x);
+  x = bfi32(e[3], x << 8, x);
+  x = bfi32(e[2], x << 4, x);
+  x = bfi32(e[1], x << 2, x);
+  x = bfi32(e0, x << 1, x);
+  return x;
+}
+
+// local = (((g A_on + r_on) A_off + r_off) S_w + r_sw) S_f + r_sf  (index.rs:24-32).
+// Calls on_codes(q, sel, sel2) for q = 0..5: byte j of sel is
+// on-support | primary-kind << 1 | minus << 2 of coordinate 4q + j (FastClass::tab);
+// byte j of sel2 is second-free-kind | minus << 2.
+template <class OnCodes>
+LLVQ_HD void even_codes(const DecodeTables& T, const FastClass& f, uint64_t li, OnCodes&& on_codes) {
+  const uint32_t p_req = (f.meta >> kMetaPreqShift) & 1u;
+  const uint32_t sf = (f.meta >> kMetaSfShift) & 31u;
+  const uint32_t sw = (f.meta >> kMetaSwShift) & 31u;
+  const uint32_t r_sf = (uint32_t)li & ((1u << sf) - 1u);
+  li >>= sf;
+  const uint32_t r_sw = (uint32_t)li & ((1u << sw) - 1u);
+  li >>= sw;
+  const double rest = (double)li;
+  const double q1 = floor64((rest + 0.5) * f.inv0);
+  const uint32_t r_off = (uint32_t)fma64(-q1, (double)f.a_off, rest);
+  const double g = floor64((q1 + 0.5) * f.d1);
+  const uint32_t r_on = (uint32_t)fma64(-g, (double)f.a_on, q1);
+  const uint32_t gi = ((f.meta >> kMetaGolayShift) + (uint32_t)g) & 4095u;
+  const uint32_t cw = T.golay[gi];
+  const uint32_t* e_on = T.expand + 8u * gi;
+  const uint32_t* e_off = e_on + 4;
+  const uint32_t on_e = T.on_lut[(f.u0 & 0xFFFFu) + r_on];
+  const uint32_t off_e = T.off_lut[f.u1 + r_off];
+  // word signs: bit s of r_sw for support slot s < w-1, the last one forced by
+  // the parity rule (index.rs:375-388)
+  const uint32_t signs_on = r_sw | (((popc32(r_sw) & 1u) ^ p_req) << sw);
+  // free signs go to the nonzero off-support slots in slot order (index.rs:403-415)
+  const uint32_t nz = (off_e | (off_e >> 16)) & 0xFFFFu;
+  uint32_t signs_off = 0, r = r_sf;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t m4 = (nz >> (4 * k)) & 15u;
+    signs_off |= (uint32_t)T.pdep4[m4 * 16u + (r & 15u)] << (4 * k);
+    r >>= popc32(m4);
+  }
+  const uint32_t prim = bfi32(cw, expand24(on_e & 0xFFFFu, e_on), expand24(off_e & 0xFFFFu, e_off));
+  const uint32_t sec = expand24(off_e >> 16, e_off) & ~cw;
+  const uint32_t sign = bfi32(cw, expand24(signs_on, e_on), expand24(signs_off, e_off));
+#pragma unroll
+  for (int q = 0; q < 6; ++q) {
+    const uint32_t s2 = (((sign >> (4 * q)) & 15u) * kSpread2) & 0x04040404u;
+    const uint32_t sel = ((((cw >> (4 * q)) & 15u) * kSpread0) & 0x01010101u) |
+                         ((((prim >> (4 * q)) & 15u) * kSpread1) & 0x02020202u) | s2;
+    const uint32_t sel2 = ((((sec >> (4 * q)) & 15u) * kSpread0) & 0x01010101u) | s2;
+    on_codes(q, sel, sel2);
+  }
+}
+
+// ---- generic walk of both cosets (rare classes) -----------------------------------
+template <class Emit>
+LLVQ_HD void decode_odd(const DecodeTables& T, const DevClass& c, uint64_t li, Emit&& emit) {
+  const double local = (double)li;
+  const double g = floor64((local + 0.5) * c.inv0);
+  const double r = fma64(-g, c.m0, local);
+  double rho = (r + 0.5) * c.inv0;
+  const uint32_t cw = T.golay[(uint32_t)g & 4095u];
+  uint32_t tg = c.tg0;
+  for (int p = 0; p < kDim; ++p) {
+    const uint32_t jj = walk_step(rho, tg, (uint32_t)(kDim - p), T.rcp);
+    const int v = (int)((c.vals0 >> (4u * jj)) & 15u);
+    // forced signs (index.rs:417-431): a = v if v = 3 mod 4 else -v; a on the
+    // codeword's support, -a off it.
+    const uint32_t neg = ((cw >> p) ^ ((uint32_t)v >> 1)) & 1u;
+    emit(p, neg ? -v : v);
+  }
+}
+
+template <class Emit>
+LLVQ_HD void decode_even(const DecodeTables& T, const DevClass& c, uint64_t li, Emit&& emit) {
   const uint32_t w = (c.meta >> kMetaWShift) & 31u;
   const uint32_t p_req = (c.meta >> kMetaPreqShift) & 1u;
   const uint32_t sf = (c.meta >> kMetaSfShift) & 31u;
@@ -149,12 +238,9 @@ LLVQ_HD int decode_index(const DecodeTables& T, uint64_t idx, Emit&& emit) {
   double rho_off = (r_off + 0.5) * c.inv0;
   double rho_on = (r_on + 0.5) * c.inv1;
   const uint32_t cw = T.golay[(c.golay_base + (uint32_t)g) & 4095u];
-  // word signs: bit s of r_sw for support slot s < w-1, the last one forced by
-  // the parity rule (index.rs:375-388)
   uint32_t signs_on = r_sw | (((popc32(r_sw) & 1u) ^ p_req) << sw);
   uint32_t tg_on = c.tg1, tg_off = c.tg0;
   uint32_t n_on = w, n_off = kDim - w;
-#pragma unroll
   for (int p = 0; p < kDim; ++p) {
     int v;
     uint32_t neg;
@@ -168,12 +254,45 @@ LLVQ_HD int decode_index(const DecodeTables& T, uint64_t idx, Emit&& emit) {
       const uint32_t jj = walk_step(rho_off, tg_off, n_off, T.rcp);
       --n_off;
       v = (int)((c.vals0 >> (4u * jj)) & 15u);
-      // free signs are consumed by the nonzero off-support slots only
-      // (index.rs:403-415); the zero run is recognised by its value
+      // the zero run is recognised by its value, never by its kind index
       neg = v ? (r_sf & 1u) : 0u;
       r_sf >>= (v ? 1 : 0);
     }
     emit(p, neg ? -v : v);
+  }
+}
+
+// Decodes `idx` and calls emit(position, value) for positions 0..23 in order,
+// taking the same path the GEMV kernel takes for the index's class.  Returns
+// the class index, -1 for the origin, -2 for an index past N(13) (zeros).
+template <class Emit>
+LLVQ_HD int decode_index(const DecodeTables& T, uint64_t idx, Emit&& emit) {
+  if (idx == 0 || idx > kN13) {
+    for (int p = 0; p < kDim; ++p) emit(p, 0);
+    return idx == 0 ? -1 : -2;
+  }
+  const uint64_t i = idx - 1;
+  const uint32_t ci = find_class(T, i);
+  const uint64_t li = i - T.starts[ci];
+  const FastClass f = T.fast[ci];
+  const uint32_t path = (f.meta >> kMetaPathShift) & 3u;
+  if (path == kPathOdd) {
+    odd_codes(T, f, li, [&](int q, uint32_t sel) {
+      for (int j = 0; j < 4; ++j) emit(4 * q + j, table_byte(f.tab_lo, f.tab_hi, (sel >> (8 * j)) & 7u));
+    });
+  } else if (path == kPathEven) {
+    const int fv1 = (int)(f.u0 >> 16);
+    even_codes(T, f, li, [&](int q, uint32_t sel, uint32_t sel2) {
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t c2 = (sel2 >> (8 * j)) & 7u;
+        const int second = (c2 & 1u) ? ((c2 & 4u) ? -fv1 : fv1) : 0;
+        emit(4 * q + j, table_byte(f.tab_lo, f.tab_hi, (sel >> (8 * j)) & 7u) + second);
+      }
+    });
+  } else {
+    const DevClass c = T.cls[ci];
+    if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
+    else decode_even(T, c, li, emit);
   }
   return (int)ci;
 }

@@ -21,27 +21,43 @@
 namespace llvq {
 
 // ---- table image --------------------------------------------------------------
+// What every workgroup copies into LDS.  The rarely used generic class records
+// and the large even-coset tables stay in HBM (they live in L2).
 struct TableImage {
   uint32_t golay[4096];
-  DevClass cls[kClassSlots];
-  uint64_t ends[kEndsPadded];
+  FastClass fast[kClassSlots];
+  uint64_t starts[kClassSlots];
+  uint16_t lut[2048];        // a 47-bit field only reaches the lower half of the host table
   double rcp[32];
+  uint8_t pdep4[256];
+  uint32_t on_lut[kOnLutSlots];
 };
 static_assert(sizeof(TableImage) % 16 == 0, "table image is copied in 16-byte units");
 
-__device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const TableImage* g) {
-  const uint4* src = reinterpret_cast<const uint4*>(g);
+struct GlobalTables {
+  const TableImage* image;
+  const DevClass* cls;
+  const uint32_t* off_lut;
+  const uint32_t* expand;
+};
+
+__device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const GlobalTables& g) {
+  const uint4* src = reinterpret_cast<const uint4*>(g.image);
   uint4* dst = reinterpret_cast<uint4*>(smem);
   for (uint32_t i = threadIdx.x; i < sizeof(TableImage) / 16; i += blockDim.x) dst[i] = src[i];
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
-  return DecodeTables{s->golay, s->cls, s->ends, s->rcp};
+  return DecodeTables{s->golay, g.cls, s->fast, s->starts, s->lut, s->rcp, s->on_lut, g.off_lut, g.expand, s->pdep4};
 }
 
-__device__ __forceinline__ uint64_t load_record(const uint8_t* codes, size_t block) {
-  // 6-byte big-endian record; the stream is 2-byte aligned at every block.
-  const uint16_t* p = reinterpret_cast<const uint16_t*>(codes + 6 * block);
-  auto be16 = [](uint32_t h) { return ((h & 0xFFu) << 8) | (h >> 8); };
-  return ((uint64_t)be16(p[0]) << 32) | ((uint64_t)be16(p[1]) << 16) | (uint64_t)be16(p[2]);
+// 6-byte big-endian record at a 2-byte-aligned offset of a 4-byte-aligned buffer
+// (global or LDS): two dword reads, one funnel shift, two byte swaps.
+__device__ __forceinline__ uint64_t read_record(const uint8_t* buf, size_t byte) {
+  const uint32_t* w = reinterpret_cast<const uint32_t*>(buf + (byte & ~(size_t)3));
+  const uint32_t w0 = w[0], w1 = w[1];
+  const bool odd = (byte & 2) != 0;
+  const uint32_t first = odd ? __builtin_amdgcn_alignbit(w1, w0, 16) : w0;  // bytes 0..3
+  const uint32_t second = odd ? (w1 >> 16) : (w1 & 0xFFFFu);                // bytes 4..5
+  return ((uint64_t)__builtin_bswap32(first) << 16) | (uint64_t)(__builtin_bswap32(second) >> 16);
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -51,17 +67,16 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // ---- parity probe: unrank records to points -----------------------------------
-__global__ __launch_bounds__(256) void decode_blocks_kernel(const TableImage* __restrict__ tables,
-                                                            const uint8_t* __restrict__ codes,
+__global__ __launch_bounds__(256) void decode_blocks_kernel(GlobalTables g, const uint8_t* __restrict__ codes,
                                                             size_t nblocks, int8_t* __restrict__ points,
                                                             uint8_t* __restrict__ gains,
                                                             uint8_t* __restrict__ shells) {
   extern __shared__ __align__(16) uint8_t smem[];
-  const DecodeTables T = stage_tables(smem, tables);
+  const DecodeTables T = stage_tables(smem, g);
   __syncthreads();
   for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < nblocks;
        b += (size_t)gridDim.x * blockDim.x) {
-    const uint64_t rec = load_record(codes, b);
+    const uint64_t rec = read_record(codes, 6 * b);
     int8_t* out = points + b * kDim;
     const int ci = decode_index(T, rec >> 1, [&](int p, int v) { out[p] = (int8_t)v; });
     if (gains) gains[b] = (uint8_t)(rec & 1);
@@ -69,51 +84,257 @@ __global__ __launch_bounds__(256) void decode_blocks_kernel(const TableImage* __
   }
 }
 
-// ---- fused dequant-GEMV, one wavefront per output row -------------------------
-struct GemvArgs {
-  const TableImage* tables;
+// ---- fused dequant-GEMV ---------------------------------------------------------
+// One persistent 1024-lane workgroup per CU.  The rows of up to four matrices
+// that share an activation are cut into tiles of at most kTileBlocks blocks; a
+// workgroup takes tiles round-robin and runs four phases on each:
+//   P0  copy the tile's code bytes from HBM to LDS with 16-byte loads;
+//   P1  one lane per block: find the block's class and push the block onto the
+//       odd-coset or the even-coset queue (the two decoders are different
+//       straight-line programs; binning keeps every lane of a wavefront on the
+//       same one); blocks of the rare generic classes are decoded on the spot;
+//   P2  wavefronts take 64 queued blocks at a time, unrank them to 8-bit
+//       coordinates, reduce them against the activation with integer dot
+//       products and write one partial sum per block;
+//   P3  one wavefront per row adds the row's partial sums in a fixed order,
+//       applies the row scale and the tail columns, and stores y.
+// Results do not depend on the queue order, so they are reproducible.
+//
+// The activation is held in LDS as block-scaled fixed point: per 24-column
+// block a power-of-two scale and three signed byte planes (x = scale *
+// (65536 d2 + 256 d1 + d0), |65536 d2 + ...| <= 2^22), i.e. every binary16
+// value within 2^12 of its block's largest is exact and the rest round at
+// 2^-23 of that largest.  Integer sums of 24 products are exact; the three
+// plane sums are combined and scaled in f32.
+constexpr int kWgThreads = 1024;
+constexpr int kWaves = kWgThreads / 64;
+constexpr int kTileBlocks = 4096;
+constexpr int kRawBytes = kTileBlocks * 6 + 32;
+constexpr int kMaxGroup = 4;
+constexpr int kPlaneDwords = 18;  // 3 planes x 6 dwords per 24-column block
+
+struct MatArg {
   const uint8_t* codes;
   const float* rscale;
   const float* tail;
+  void* y;
   float g0, g1;
-  uint32_t d_out, nblocks, tail_w;
+  uint32_t d_out;
+  uint32_t tile_begin;  // first tile of this matrix in the launch
 };
 
-template <typename OutT>
-__device__ __forceinline__ void store_out(OutT* y, uint32_t r, float v);
-template <>
-__device__ __forceinline__ void store_out<float>(float* y, uint32_t r, float v) { y[r] = v; }
-template <>
-__device__ __forceinline__ void store_out<__half>(__half* y, uint32_t r, float v) { y[r] = __float2half_rn(v); }
+struct GroupArgs {
+  GlobalTables tables;
+  const __half* x;
+  uint32_t nblocks, tail_w, n_mats, rows_per_tile, n_tiles;
+  float inv_nblocks;  // 1 / nblocks, for the block -> column split
+  MatArg m[kMaxGroup];
+};
+
+__host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks) {
+  return sizeof(TableImage) + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + kRawBytes +
+         (size_t)kTileBlocks * 4 * 2 + 16;
+}
 
 template <typename OutT>
-__global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs a, const __half* __restrict__ x,
-                                                        OutT* __restrict__ y) {
+__device__ __forceinline__ void store_out(void* y, uint32_t r, float v);
+template <>
+__device__ __forceinline__ void store_out<float>(void* y, uint32_t r, float v) {
+  reinterpret_cast<float*>(y)[r] = v;
+}
+template <>
+__device__ __forceinline__ void store_out<__half>(void* y, uint32_t r, float v) {
+  reinterpret_cast<__half*>(y)[r] = __float2half_rn(v);
+}
+
+// queue entry: block slot in the tile (12 bits) | class (9 bits) << 16 | gain << 25
+__device__ __forceinline__ void queue_push(uint32_t* counter, uint32_t* queue, bool mine, uint32_t entry,
+                                           bool from_top) {
+  const uint64_t m = __ballot(mine);
+  if (m == 0) return;
+  const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
+  const int first = __ffsll((long long)m) - 1;
+  uint32_t base = 0;
+  if ((int)(threadIdx.x & 63u) == first) base = atomicAdd(counter, (uint32_t)__popcll(m));
+  base = __shfl(base, first, 64);
+  if (mine) queue[from_top ? (kTileBlocks - 1 - (base + rank)) : (base + rank)] = entry;
+}
+
+// One 24-column block of the activation -> scale and byte planes.
+__device__ __forceinline__ void quantize_block(const __half* x, uint32_t* planes, float* scale) {
+  float v[kDim];  // 2-byte loads: the activation of a batched row need not be 16-byte aligned
+#pragma unroll
+  for (int j = 0; j < kDim; ++j) v[j] = __half2float(x[j]);
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < kDim; ++j) amax = fmaxf(amax, fabsf(v[j]));
+  bool bad = false;
+#pragma unroll
+  for (int j = 0; j < kDim; ++j) bad |= !(fabsf(v[j]) <= 65504.f);  // inf or NaN
+  int e = 0;
+  (void)frexpf(amax, &e);  // amax = m 2^e, m in [0.5, 1)
+  const float up = ldexpf(1.f, 22 - e);
+  *scale = bad ? __builtin_nanf("") : (amax == 0.f ? 0.f : ldexpf(1.f, e - 22));
+  uint32_t p0[6], p1[6], p2[6];
+#pragma unroll
+  for (int q = 0; q < 6; ++q) p0[q] = p1[q] = p2[q] = 0;
+#pragma unroll
+  for (int j = 0; j < kDim; ++j) {
+    const int xq = (amax == 0.f || bad) ? 0 : (int)rintf(v[j] * up);  // |xq| <= 2^22
+    const int d0 = (int)(int8_t)(xq & 0xFF);
+    const int x1 = (xq - d0) >> 8;
+    const int d1 = (int)(int8_t)(x1 & 0xFF);
+    const int d2 = (x1 - d1) >> 8;
+    p0[j >> 2] |= (uint32_t)(d0 & 0xFF) << (8 * (j & 3));
+    p1[j >> 2] |= (uint32_t)(d1 & 0xFF) << (8 * (j & 3));
+    p2[j >> 2] |= (uint32_t)(d2 & 0xFF) << (8 * (j & 3));
+  }
+#pragma unroll
+  for (int q = 0; q < 6; ++q) {
+    planes[q] = p0[q];
+    planes[6 + q] = p1[q];
+    planes[12 + q] = p2[q];
+  }
+}
+
+__device__ __forceinline__ float planes_to_float(int d0, int d1, int d2) {
+  return fmaf((float)d2, 65536.f, fmaf((float)d1, 256.f, (float)d0));
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
   const DecodeTables T = stage_tables(smem, a.tables);
-  float* xs = reinterpret_cast<float*>(smem + sizeof(TableImage));
-  const uint32_t d_in = a.nblocks * kDim + a.tail_w;
-  for (uint32_t i = threadIdx.x; i < d_in; i += blockDim.x) xs[i] = __half2float(x[i]);
-  __syncthreads();
+  const uint32_t nb = a.nblocks;
+  uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + sizeof(TableImage));
+  float* xscale = reinterpret_cast<float*>(xplanes + (size_t)nb * kPlaneDwords);
+  float* xtail = xscale + nb;
+  uint8_t* raw = reinterpret_cast<uint8_t*>(xtail + 32);
+  uint32_t* queue = reinterpret_cast<uint32_t*>(raw + kRawBytes);
+  float* partial = reinterpret_cast<float*>(queue + kTileBlocks);
+  uint32_t* ctrl = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  for (uint32_t col = tid; col < nb; col += kWgThreads)
+    quantize_block(a.x + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+  if (tid < a.tail_w) xtail[tid] = __half2float(a.x[(size_t)nb * kDim + tid]);
 
-  const uint32_t lane = threadIdx.x & 63u;
-  const uint32_t wave = threadIdx.x >> 6;
-  const uint32_t waves = (blockDim.x >> 6) * gridDim.x;
-  for (uint32_t row = blockIdx.x * (blockDim.x >> 6) + wave; row < a.d_out; row += waves) {
-    float acc = 0.f;
-    for (uint32_t b = lane; b < a.nblocks; b += 64u) {
-      const uint64_t rec = load_record(a.codes, (size_t)row * a.nblocks + b);
-      const float* xb = xs + b * kDim;
-      float dot = 0.f;
-      const int ci = decode_index(T, rec >> 1, [&](int p, int v) { dot = fmaf((float)v, xb[p], dot); });
-      const float g = (rec & 1) ? a.g1 : a.g0;
-      const float s = ci >= 0 ? T.cls[ci].inv_norm * g : 0.f;
-      acc = fmaf(dot, s, acc);
+  for (uint32_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+    uint32_t mi = 0;
+#pragma unroll
+    for (uint32_t k = 1; k < kMaxGroup; ++k)
+      if (k < a.n_mats && tile >= a.m[k].tile_begin) mi = k;
+    const MatArg M = a.m[mi];
+    const uint32_t r0 = (tile - M.tile_begin) * a.rows_per_tile;
+    const uint32_t rows = min(a.rows_per_tile, M.d_out - r0);
+    const uint32_t nblk = rows * nb;
+    const size_t byte0 = (size_t)r0 * nb * 6;
+    const uint32_t off = (uint32_t)(byte0 & 15);
+
+    // P0: code bytes HBM -> LDS
+    if (tid < 2) ctrl[tid] = 0;
+    {
+      const uint4* src = reinterpret_cast<const uint4*>(M.codes + (byte0 - off));
+      const uint32_t n16 = (off + nblk * 6 + 15) >> 4;
+      for (uint32_t i = tid; i < n16; i += kWgThreads) reinterpret_cast<uint4*>(raw)[i] = src[i];
     }
-    float v = acc * a.rscale[row];
-    if (lane < a.tail_w) v = fmaf(a.tail[(size_t)row * a.tail_w + lane], xs[a.nblocks * kDim + lane], v);
-    v = wave_sum(v);
-    if (lane == 0) store_out<OutT>(y, row, v);
+    __syncthreads();
+
+    // P1: classify and bin
+    for (uint32_t base = 0; base < nblk; base += kWgThreads) {
+      const uint32_t f = base + tid;
+      uint32_t entry = 0;
+      bool is_odd = false, is_even = false;
+      if (f < nblk) {
+        const uint64_t rec = read_record(raw, off + 6 * f);
+        const uint64_t idx = rec >> 1;
+        if (idx == 0) {
+          partial[f] = 0.f;  // the origin decodes to zero whatever the gain (index.rs:335-337)
+        } else {
+          const uint32_t ci = find_class(T, idx - 1);
+          const uint32_t path = (T.fast[ci].meta >> kMetaPathShift) & 3u;
+          entry = f | (ci << 16) | ((uint32_t)(rec & 1) << 25);
+          is_odd = path == kPathOdd;
+          is_even = path == kPathEven;
+          if (path == kPathGeneric) {  // rare classes: generic walk, right here
+            const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
+            const uint32_t col = f - row * nb;
+            const uint8_t* xb = reinterpret_cast<const uint8_t*>(xplanes + (size_t)col * kPlaneDwords);
+            const DevClass c = T.cls[ci];
+            const uint64_t li = idx - 1 - T.starts[ci];
+            int d0 = 0, d1 = 0, d2 = 0;
+            auto emit = [&](int p, int v) {
+              d0 += v * (int)(int8_t)xb[p];
+              d1 += v * (int)(int8_t)xb[24 + p];
+              d2 += v * (int)(int8_t)xb[48 + p];
+            };
+            if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
+            else decode_even(T, c, li, emit);
+            partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (c.inv_norm * ((rec & 1) ? M.g1 : M.g0));
+          }
+        }
+      }
+      queue_push(&ctrl[0], queue, is_odd, entry, false);
+      queue_push(&ctrl[1], queue, is_even, entry, true);
+    }
+    __syncthreads();
+
+    // P2: unrank and reduce, odd queue then even queue
+    const uint32_t n_odd = ctrl[0], n_even = ctrl[1];
+    for (uint32_t k = tid; k < ((n_odd + 63u) & ~63u); k += kWgThreads) {
+      if (k < n_odd) {
+        const uint32_t entry = queue[k];
+        const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
+        const uint64_t rec = read_record(raw, off + 6 * f);
+        const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+        const FastClass fc = T.fast[ci];
+        const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
+        const uint32_t col = f - row * nb;
+        const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
+        int d0 = 0, d1 = 0, d2 = 0;
+        odd_codes(T, fc, li, [&](int q, uint32_t sel) {
+          const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+          d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+          d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+          d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+        });
+        partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+      }
+    }
+    for (uint32_t k = tid; k < ((n_even + 63u) & ~63u); k += kWgThreads) {
+      if (k < n_even) {
+        const uint32_t entry = queue[kTileBlocks - 1 - k];
+        const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
+        const uint64_t rec = read_record(raw, off + 6 * f);
+        const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+        const FastClass fc = T.fast[ci];
+        const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
+        const uint32_t col = f - row * nb;
+        const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
+        const uint32_t fv1 = fc.u0 >> 16;
+        const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
+        int d0 = 0, d1 = 0, d2 = 0;
+        even_codes(T, fc, li, [&](int q, uint32_t sel, uint32_t sel2) {
+          const int w = (int)(__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel) |
+                              __builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2));
+          d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+          d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+          d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+        });
+        partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+      }
+    }
+    __syncthreads();
+
+    // P3: fixed-order row sums, row scale, tail columns
+    for (uint32_t row = wave; row < rows; row += kWaves) {
+      float s = 0.f;
+      for (uint32_t b = lane; b < nb; b += 64u) s += partial[row * nb + b];
+      float v = s * M.rscale[r0 + row];
+      if (lane < a.tail_w) v = fmaf(M.tail[(size_t)(r0 + row) * a.tail_w + lane], xtail[lane], v);
+      v = wave_sum(v);
+      if (lane == 0) store_out<OutT>(M.y, r0 + row, v);
+    }
+    __syncthreads();
   }
 }
 
@@ -127,7 +348,8 @@ using namespace llvq;
 struct llvq_rt {
   int device = 0;
   hipStream_t stream = nullptr;
-  TableImage* tables = nullptr;  // device
+  uint8_t* blob = nullptr;  // one device allocation holding every table
+  GlobalTables tables{};
   int cu_count = 0;
 };
 
@@ -182,20 +404,36 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   hipError_t e = hipGetDeviceProperties(&prop, device);
   if (e != hipSuccess) { delete rt; return hip_fail(e, "hipGetDeviceProperties"); }
   rt->cu_count = prop.multiProcessorCount;
-  std::vector<uint8_t> host(sizeof(TableImage));
+  // one blob: LDS image | generic class records | off-support table | deposit masks
+  if (cb.on_lut.size() > (size_t)kOnLutSlots) { delete rt; return fail(LLVQ_ERR_UNSUPPORTED, "support-arrangement table outgrew its LDS slot"); }
+  const size_t off_cls = sizeof(TableImage);
+  const size_t off_lut = off_cls + sizeof(cb.dev_classes);
+  const size_t off_exp = (off_lut + cb.off_lut.size() * 4 + 15) & ~(size_t)15;
+  const size_t total = off_exp + sizeof(cb.expand);
+  std::vector<uint8_t> host(total, 0);
   auto* img = reinterpret_cast<TableImage*>(host.data());
   std::memcpy(img->golay, cb.golay, sizeof img->golay);
-  std::memcpy(img->cls, cb.dev_classes, sizeof img->cls);
-  std::memcpy(img->ends, cb.ends, sizeof img->ends);
+  std::memcpy(img->fast, cb.fast, sizeof img->fast);
+  std::memcpy(img->starts, cb.starts, sizeof img->starts);
+  std::memcpy(img->lut, cb.lut, sizeof img->lut);
   std::memcpy(img->rcp, cb.rcp, sizeof img->rcp);
-  e = hipMalloc(reinterpret_cast<void**>(&rt->tables), sizeof(TableImage));
+  std::memcpy(img->pdep4, cb.pdep4, sizeof img->pdep4);
+  std::memcpy(img->on_lut, cb.on_lut.data(), cb.on_lut.size() * 4);
+  std::memcpy(host.data() + off_cls, cb.dev_classes, sizeof(cb.dev_classes));
+  std::memcpy(host.data() + off_lut, cb.off_lut.data(), cb.off_lut.size() * 4);
+  std::memcpy(host.data() + off_exp, cb.expand, sizeof(cb.expand));
+  e = hipMalloc(reinterpret_cast<void**>(&rt->blob), total);
   if (e != hipSuccess) { delete rt; return hip_fail(e, "hipMalloc(tables)"); }
-  e = hipMemcpy(rt->tables, host.data(), sizeof(TableImage), hipMemcpyHostToDevice);
-  if (e != hipSuccess) { (void)hipFree(rt->tables); delete rt; return hip_fail(e, "hipMemcpy(tables)"); }
+  e = hipMemcpy(rt->blob, host.data(), total, hipMemcpyHostToDevice);
+  if (e != hipSuccess) { (void)hipFree(rt->blob); delete rt; return hip_fail(e, "hipMemcpy(tables)"); }
+  rt->tables.image = reinterpret_cast<const TableImage*>(rt->blob);
+  rt->tables.cls = reinterpret_cast<const DevClass*>(rt->blob + off_cls);
+  rt->tables.off_lut = reinterpret_cast<const uint32_t*>(rt->blob + off_lut);
+  rt->tables.expand = reinterpret_cast<const uint32_t*>(rt->blob + off_exp);
   // the activation tile of a wide matrix pushes dynamic LDS past the 64 KB default
   const int max_lds = 160 * 1024;
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_rows_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_rows_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   *out = rt;
   return LLVQ_OK;
 }
@@ -203,7 +441,7 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
 void llvq_hip_runtime_destroy(llvq_rt* rt) {
   if (!rt) return;
   (void)hipSetDevice(rt->device);
-  (void)hipFree(rt->tables);
+  (void)hipFree(rt->blob);
   delete rt;
 }
 
@@ -342,26 +580,56 @@ int llvq_hip_matrix_info(const llvq_mat* m, uint32_t* d_out, uint32_t* d_in, uin
 
 const char* llvq_hip_matrix_name(const llvq_mat* m) { return m ? m->name.c_str() : ""; }
 
-static int launch_gemv(llvq_rt* rt, const llvq_mat* m, const void* x, void* y, int y_dtype) {
-  GemvArgs a{rt->tables, m->codes, m->rscale, m->tail, m->g[0], m->g[1], m->d_out, m->nblocks, m->tail_w};
-  const size_t lds = sizeof(TableImage) + (size_t)m->d_in * sizeof(float);
-  if (lds > 160 * 1024)
-    return fail(LLVQ_ERR_UNSUPPORTED, m->name + ": d_in " + std::to_string(m->d_in) + " does not fit the LDS activation tile");
-  const uint32_t waves_per_wg = 4;
-  uint32_t grid = (m->d_out + waves_per_wg - 1) / waves_per_wg;
-  const uint32_t cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256) * 2;
-  if (grid > cap) grid = cap;
-  if (y_dtype == LLVQ_F32) {
-    hipLaunchKernelGGL(gemv_rows_kernel<float>, dim3(grid), dim3(256), lds, rt->stream, a,
-                       reinterpret_cast<const __half*>(x), reinterpret_cast<float*>(y));
-  } else if (y_dtype == LLVQ_F16) {
-    hipLaunchKernelGGL(gemv_rows_kernel<__half>, dim3(grid), dim3(256), lds, rt->stream, a,
-                       reinterpret_cast<const __half*>(x), reinterpret_cast<__half*>(y));
-  } else {
-    return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv: unknown output dtype");
+// Rows per tile: as even a split over the CUs as the tile capacity allows.
+static uint32_t pick_rows_per_tile(const llvq_mat* const* mats, int n, uint32_t nblocks, uint32_t grid) {
+  const uint32_t cap = nblocks ? (uint32_t)kTileBlocks / nblocks : 0xFFFFFFFFu;
+  uint64_t total = 0;
+  for (int i = 0; i < n; ++i) total += mats[i]->d_out;
+  uint32_t r = (uint32_t)((total + grid - 1) / grid);
+  if (r < 1) r = 1;
+  for (uint32_t tries = 0; tries < 64 && r < cap; ++tries, ++r) {
+    uint64_t tiles = 0;
+    for (int i = 0; i < n; ++i) tiles += (mats[i]->d_out + r - 1) / r;
+    if (tiles <= grid) break;
   }
+  if (r > cap) r = cap;
+  return r < 1 ? 1 : r;
+}
+
+static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, void* const* y,
+                        int y_dtype) {
+  const llvq_mat* m0 = mats[0];
+  if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv: unknown output dtype");
+  const size_t lds = gemv_lds_bytes(m0->nblocks);
+  if (lds > 160 * 1024 || m0->nblocks > (uint32_t)kTileBlocks)
+    return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": d_in " + std::to_string(m0->d_in) + " does not fit the LDS activation tile");
+  const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
+  GroupArgs a{};
+  a.tables = rt->tables;
+  a.x = reinterpret_cast<const __half*>(x);
+  a.nblocks = m0->nblocks;
+  a.tail_w = m0->tail_w;
+  a.n_mats = (uint32_t)n;
+  a.inv_nblocks = m0->nblocks ? 1.0f / (float)m0->nblocks : 0.f;
+  a.rows_per_tile = pick_rows_per_tile(mats, n, m0->nblocks, grid_cap);
+  uint32_t tiles = 0;
+  for (int i = 0; i < n; ++i) {
+    a.m[i] = MatArg{mats[i]->codes, mats[i]->rscale, mats[i]->tail, y[i], mats[i]->g[0], mats[i]->g[1],
+                    mats[i]->d_out, tiles};
+    tiles += (mats[i]->d_out + a.rows_per_tile - 1) / a.rows_per_tile;
+  }
+  a.n_tiles = tiles;
+  const uint32_t grid = tiles < grid_cap ? tiles : grid_cap;
+  if (y_dtype == LLVQ_F32)
+    hipLaunchKernelGGL(gemv_tiles_kernel<float>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
+  else
+    hipLaunchKernelGGL(gemv_tiles_kernel<__half>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
   HIP_TRY(hipGetLastError());
   return LLVQ_OK;
+}
+
+static int launch_gemv(llvq_rt* rt, const llvq_mat* m, const void* x, void* y, int y_dtype) {
+  return launch_group(rt, &m, 1, x, &y, y_dtype);
 }
 
 int llvq_hip_gemv(llvq_rt* rt, const llvq_mat* m, const void* x, void* y, int y_dtype) {
@@ -379,8 +647,9 @@ int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
       return fail(LLVQ_ERR_INVALID_ARGUMENT, mats[i]->name + ": projections of one group must share d_in");
   }
   HIP_TRY(hipSetDevice(rt->device));
-  for (int i = 0; i < n; ++i) {
-    const int rc = launch_gemv(rt, mats[i], x, y[i], y_dtype);
+  for (int i = 0; i < n; i += kMaxGroup) {
+    const int k = n - i < kMaxGroup ? n - i : kMaxGroup;
+    const int rc = launch_group(rt, mats + i, k, x, y + i, y_dtype);
     if (rc) return rc;
   }
   return LLVQ_OK;
