@@ -21,6 +21,7 @@ constexpr uint64_t kFingerprint = 0x338f420f11866319ULL;  // llvq-artifact/tests
 constexpr int kMaxShell = 13;
 constexpr int kClassSlots = 384;   // 383 classes + one sentinel, a power-of-two-friendly size
 constexpr int kStartsPadded = 512; // class starts, padded with UINT64_MAX past N(13)
+constexpr int kStartsLds = 448;    // what a bounded search from class <= 382 with k <= 6 can touch
 constexpr int kLutShift = 36;      // class-find table is keyed on the zero-based index >> 36
 constexpr int kOnLutSlots = 4352;  // LDS slots for the support-arrangement table (4322 entries used)
 constexpr int kLutSize = 4096;     // covers every zero-based index < N(13) < 2^48 (a 47-bit field uses the lower half)
@@ -101,7 +102,9 @@ struct Codebook {
   // device-shaped tables
   DevClass dev_classes[kClassSlots];
   uint64_t starts[kStartsPadded];         // starts[c] = offset of class c, starts[383] = N(13), then UINT64_MAX
-  uint16_t lut[kLutSize];                 // class holding zero-based index (key << kLutShift), clamped to 382
+  // lut[key]: low 9 bits = class holding zero-based index (key << kLutShift), clamped to 382;
+  // bits 9.. = k, where the class of any index of the bucket is at most 2^k - 1 classes further
+  uint16_t lut[kLutSize];
   double rcp[32];                         // rcp[c] = 1/c, rcp[0] unused
   uint64_t n12 = 0;                       // points in the cap-12 ball (47-bit field)
   // fast paths

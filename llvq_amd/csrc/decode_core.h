@@ -107,10 +107,13 @@ LLVQ_HD uint32_t walk_step(double& rho, uint32_t& tg, uint32_t n, const double* 
 }
 
 // Class of the zero-based index i < N(13): one table probe on the top bits,
-// then a short forward scan (empty for 96 % of uniformly drawn indices).
+// then a halving search over at most 2^k classes (k = 0 for 96 % of uniformly
+// drawn indices, k <= 6 always).  starts[] is padded with UINT64_MAX.
 LLVQ_HD uint32_t find_class(const DecodeTables& T, uint64_t i) {
-  uint32_t ci = T.lut[(uint32_t)(i >> kLutShift)];
-  while (ci < 382u && T.starts[ci + 1] <= i) ++ci;
+  const uint32_t e = T.lut[(uint32_t)(i >> kLutShift)];
+  uint32_t ci = e & 511u;
+  for (uint32_t step = (1u << (e >> 9)) >> 1; step; step >>= 1)
+    if (T.starts[ci + step] <= i) ci += step;
   return ci;
 }
 

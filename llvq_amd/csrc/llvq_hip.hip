@@ -26,7 +26,7 @@ namespace llvq {
 struct TableImage {
   uint32_t golay[4096];
   FastClass fast[kClassSlots];
-  uint64_t starts[kClassSlots];
+  uint64_t starts[kStartsLds];
   uint16_t lut[2048];        // a 47-bit field only reaches the lower half of the host table
   double rcp[32];
   uint8_t pdep4[256];
@@ -109,9 +109,11 @@ __global__ __launch_bounds__(256) void decode_blocks_kernel(GlobalTables g, cons
 constexpr int kWgThreads = 1024;
 constexpr int kWaves = kWgThreads / 64;
 constexpr int kTileBlocks = 4096;
+constexpr int kP1Blocks = kTileBlocks / kWgThreads;  // blocks one lane classifies per tile
 constexpr int kRawBytes = kTileBlocks * 6 + 32;
 constexpr int kMaxGroup = 4;
 constexpr int kPlaneDwords = 18;  // 3 planes x 6 dwords per 24-column block
+constexpr int kGenericSlots = 64; // queue for blocks of the rare generic classes
 
 struct MatArg {
   const uint8_t* codes;
@@ -133,7 +135,7 @@ struct GroupArgs {
 
 __host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks) {
   return sizeof(TableImage) + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + kRawBytes +
-         (size_t)kTileBlocks * 4 * 2 + 16;
+         (size_t)kTileBlocks * 4 * 2 + kGenericSlots * 4 + 16;
 }
 
 template <typename OutT>
@@ -201,6 +203,41 @@ __device__ __forceinline__ float planes_to_float(int d0, int d1, int d2) {
   return fmaf((float)d2, 65536.f, fmaf((float)d1, 256.f, (float)d0));
 }
 
+// One block of a class outside the fast paths: generic walk, scalar reduction
+// against the activation planes.
+__device__ __noinline__ void generic_block(const DecodeTables& T, const GroupArgs& a, const MatArg& M,
+                                           uint32_t entry, const uint8_t* raw, uint32_t off,
+                                           const uint32_t* xplanes, const float* xscale, float* partial) {
+  const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
+  const uint64_t rec = read_record(raw, off + 6 * f);
+  const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+  const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
+  const uint32_t col = f - row * a.nblocks;
+  const uint8_t* xb = reinterpret_cast<const uint8_t*>(xplanes + (size_t)col * kPlaneDwords);
+  const DevClass c = T.cls[ci];
+  int d0 = 0, d1 = 0, d2 = 0;
+  auto emit = [&](int p, int v) {
+    d0 += v * (int)(int8_t)xb[p];
+    d1 += v * (int)(int8_t)xb[24 + p];
+    d2 += v * (int)(int8_t)xb[48 + p];
+  };
+  if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
+  else decode_even(T, c, li, emit);
+  partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (c.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+}
+
+// Phase timestamps for tuning builds (-DLLVQ_PHASE_TIMING): wave 0 of each
+// workgroup stores the realtime counter at every phase boundary of its first tile.
+#ifdef LLVQ_PHASE_TIMING
+__device__ unsigned long long g_phase_stamps[1024 * 8];
+#define LLVQ_STAMP(k)                                                                     \
+  do {                                                                                    \
+    if (threadIdx.x == 0 && tile == blockIdx.x) g_phase_stamps[blockIdx.x * 8 + (k)] = wall_clock64(); \
+  } while (0)
+#else
+#define LLVQ_STAMP(k) do {} while (0)
+#endif
+
 template <typename OutT>
 __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
@@ -212,18 +249,22 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   uint8_t* raw = reinterpret_cast<uint8_t*>(xtail + 32);
   uint32_t* queue = reinterpret_cast<uint32_t*>(raw + kRawBytes);
   float* partial = reinterpret_cast<float*>(queue + kTileBlocks);
-  uint32_t* ctrl = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
+  uint32_t* gqueue = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
+  uint32_t* ctrl = gqueue + kGenericSlots;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   for (uint32_t col = tid; col < nb; col += kWgThreads)
     quantize_block(a.x + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
   if (tid < a.tail_w) xtail[tid] = __half2float(a.x[(size_t)nb * kDim + tid]);
 
+#ifdef LLVQ_PHASE_TIMING
+  if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 7] = wall_clock64();
+#endif
   for (uint32_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
-    uint32_t mi = 0;
+    LLVQ_STAMP(0);
+    MatArg M = a.m[0];  // constant indices only: a dynamic one would move the arguments to scratch
 #pragma unroll
     for (uint32_t k = 1; k < kMaxGroup; ++k)
-      if (k < a.n_mats && tile >= a.m[k].tile_begin) mi = k;
-    const MatArg M = a.m[mi];
+      if (k < a.n_mats && tile >= a.m[k].tile_begin) M = a.m[k];
     const uint32_t r0 = (tile - M.tile_begin) * a.rows_per_tile;
     const uint32_t rows = min(a.rows_per_tile, M.d_out - r0);
     const uint32_t nblk = rows * nb;
@@ -231,102 +272,174 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     const uint32_t off = (uint32_t)(byte0 & 15);
 
     // P0: code bytes HBM -> LDS
-    if (tid < 2) ctrl[tid] = 0;
+    if (tid < 4) ctrl[tid] = 0;
     {
       const uint4* src = reinterpret_cast<const uint4*>(M.codes + (byte0 - off));
       const uint32_t n16 = (off + nblk * 6 + 15) >> 4;
       for (uint32_t i = tid; i < n16; i += kWgThreads) reinterpret_cast<uint4*>(raw)[i] = src[i];
     }
     __syncthreads();
+    LLVQ_STAMP(1);
 
-    // P1: classify and bin
-    for (uint32_t base = 0; base < nblk; base += kWgThreads) {
-      const uint32_t f = base + tid;
-      uint32_t entry = 0;
-      bool is_odd = false, is_even = false;
-      if (f < nblk) {
-        const uint64_t rec = read_record(raw, off + 6 * f);
-        const uint64_t idx = rec >> 1;
-        if (idx == 0) {
-          partial[f] = 0.f;  // the origin decodes to zero whatever the gain (index.rs:335-337)
-        } else {
-          const uint32_t ci = find_class(T, idx - 1);
-          const uint32_t path = (T.fast[ci].meta >> kMetaPathShift) & 3u;
-          entry = f | (ci << 16) | ((uint32_t)(rec & 1) << 25);
-          is_odd = path == kPathOdd;
-          is_even = path == kPathEven;
-          if (path == kPathGeneric) {  // rare classes: generic walk, right here
-            const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
-            const uint32_t col = f - row * nb;
-            const uint8_t* xb = reinterpret_cast<const uint8_t*>(xplanes + (size_t)col * kPlaneDwords);
-            const DevClass c = T.cls[ci];
-            const uint64_t li = idx - 1 - T.starts[ci];
-            int d0 = 0, d1 = 0, d2 = 0;
-            auto emit = [&](int p, int v) {
-              d0 += v * (int)(int8_t)xb[p];
-              d1 += v * (int)(int8_t)xb[24 + p];
-              d2 += v * (int)(int8_t)xb[48 + p];
-            };
-            if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
-            else decode_even(T, c, li, emit);
-            partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (c.inv_norm * ((rec & 1) ? M.g1 : M.g0));
-          }
+    // P1: classify and bin.  Each lane owns up to kP1Blocks blocks and walks their
+    // class searches side by side (independent LDS chains); a wavefront then
+    // claims queue space with one atomic per queue.
+    {
+      uint32_t entry[kP1Blocks], ci[kP1Blocks];
+      uint64_t zi[kP1Blocks];  // zero-based index, ~0 when the lane has no block / an origin
+#pragma unroll
+      for (int i = 0; i < kP1Blocks; ++i) {
+        const uint32_t f = tid + (uint32_t)i * kWgThreads;
+        zi[i] = ~0ULL;
+        entry[i] = 0;
+        ci[i] = 0;
+        if (f < nblk) {
+          const uint64_t rec = read_record(raw, off + 6 * f);
+          entry[i] = f | ((uint32_t)(rec & 1) << 25);
+          if ((rec >> 1) == 0) partial[f] = 0.f;  // the origin decodes to zero whatever the gain (index.rs:335-337)
+          else zi[i] = (rec >> 1) - 1;
         }
       }
-      queue_push(&ctrl[0], queue, is_odd, entry, false);
-      queue_push(&ctrl[1], queue, is_even, entry, true);
+      uint32_t kmax = 0;
+#pragma unroll
+      for (int i = 0; i < kP1Blocks; ++i)
+        if (zi[i] != ~0ULL) {
+          const uint32_t e = T.lut[(uint32_t)(zi[i] >> kLutShift)];
+          ci[i] = e & 511u;
+          kmax = max(kmax, e >> 9);
+        }
+      // every chain of the wavefront runs the same number of halving steps: a
+      // search over a superset of the bucket's classes finds the same class
+      uint32_t kw = 0;
+#pragma unroll
+      for (uint32_t t = 1; t <= 6; ++t) kw = __any(kmax >= t) ? t : kw;
+      for (uint32_t step = (1u << kw) >> 1; step; step >>= 1) {
+#pragma unroll
+        for (int i = 0; i < kP1Blocks; ++i)
+          if (zi[i] != ~0ULL && T.starts[ci[i] + step] <= zi[i]) ci[i] += step;
+      }
+      uint32_t path[kP1Blocks];
+#pragma unroll
+      for (int i = 0; i < kP1Blocks; ++i) {
+        path[i] = zi[i] != ~0ULL ? ((T.fast[ci[i]].meta >> kMetaPathShift) & 3u) : 3u;
+        entry[i] |= ci[i] << 16;
+      }
+      uint32_t odd_rank[kP1Blocks], even_rank[kP1Blocks], n_o = 0, n_e = 0;
+#pragma unroll
+      for (int i = 0; i < kP1Blocks; ++i) {
+        const uint64_t mo = __ballot(path[i] == kPathOdd), me = __ballot(path[i] == kPathEven);
+        odd_rank[i] = n_o + __builtin_amdgcn_mbcnt_hi((uint32_t)(mo >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mo, 0));
+        even_rank[i] = n_e + __builtin_amdgcn_mbcnt_hi((uint32_t)(me >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)me, 0));
+        n_o += (uint32_t)__popcll(mo);
+        n_e += (uint32_t)__popcll(me);
+      }
+      uint32_t base_o = 0, base_e = 0;
+      if (lane == 0) {
+        base_o = atomicAdd(&ctrl[0], n_o);
+        base_e = atomicAdd(&ctrl[1], n_e);
+      }
+      base_o = __shfl(base_o, 0, 64);
+      base_e = __shfl(base_e, 0, 64);
+#pragma unroll
+      for (int i = 0; i < kP1Blocks; ++i) {
+        if (path[i] == kPathOdd) queue[base_o + odd_rank[i]] = entry[i];
+        if (path[i] == kPathEven) queue[kTileBlocks - 1 - (base_e + even_rank[i])] = entry[i];
+      }
+      // rare classes go to a small third queue; what does not fit is decoded here
+#pragma unroll
+      for (int i = 0; i < kP1Blocks; ++i) {
+        if (path[i] == kPathGeneric) {
+          const uint32_t slot = atomicAdd(&ctrl[2], 1u);
+          if (slot < (uint32_t)kGenericSlots) gqueue[slot] = entry[i];
+          else generic_block(T, a, M, entry[i], raw, off, xplanes, xscale, partial);
+        }
+      }
     }
     __syncthreads();
+    LLVQ_STAMP(2);
 
-    // P2: unrank and reduce, odd queue then even queue
-    const uint32_t n_odd = ctrl[0], n_even = ctrl[1];
-    for (uint32_t k = tid; k < ((n_odd + 63u) & ~63u); k += kWgThreads) {
-      if (k < n_odd) {
-        const uint32_t entry = queue[k];
-        const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
-        const uint64_t rec = read_record(raw, off + 6 * f);
-        const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
-        const FastClass fc = T.fast[ci];
-        const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
-        const uint32_t col = f - row * nb;
-        const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
-        int d0 = 0, d1 = 0, d2 = 0;
-        odd_codes(T, fc, li, [&](int q, uint32_t sel) {
-          const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
-          d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
-          d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-          d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
-        });
-        partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+    // P2: unrank and reduce.  Chunks of 64 queued blocks are handed out through a
+    // counter: the generic chunk first (longest), then odd, then even.
+    const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
+    const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
+    for (;;) {
+      uint32_t chunk = 0;
+      if (lane == 0) chunk = atomicAdd(&ctrl[3], 1u);
+      chunk = __shfl(chunk, 0, 64);
+      if (chunk >= c_gen + c_odd + c_even) break;
+      if (chunk < c_gen) {
+        if (lane < n_gen) generic_block(T, a, M, gqueue[lane], raw, off, xplanes, xscale, partial);
+      } else if (chunk < c_gen + c_odd) {
+        const uint32_t k = (chunk - c_gen) * 64u + lane;
+        if (k < n_odd) {
+          const uint32_t entry = queue[k];
+          const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
+          const uint64_t rec = read_record(raw, off + 6 * f);
+          const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+          const FastClass fc = T.fast[ci];
+          const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
+          const uint32_t col = f - row * nb;
+          const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
+          int d0 = 0, d1 = 0, d2 = 0;
+          odd_codes(T, fc, li, [&](int q, uint32_t sel) {
+            const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+            d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+            d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+            d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+          });
+          partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+        }
+      } else {
+        const uint32_t k = (chunk - c_gen - c_odd) * 64u + lane;
+        if (k < n_even) {
+          const uint32_t entry = queue[kTileBlocks - 1 - k];
+          const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
+          const uint64_t rec = read_record(raw, off + 6 * f);
+          const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+          const FastClass fc = T.fast[ci];
+          const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
+          const uint32_t col = f - row * nb;
+          const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
+          const uint32_t fv1 = fc.u0 >> 16;
+          const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
+          int d0 = 0, d1 = 0, d2 = 0;
+          even_codes(T, fc, li, [&](int q, uint32_t sel, uint32_t sel2) {
+            const int w = (int)(__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel) |
+                                __builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2));
+            d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+            d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+            d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+          });
+          partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+        }
       }
     }
-    for (uint32_t k = tid; k < ((n_even + 63u) & ~63u); k += kWgThreads) {
-      if (k < n_even) {
-        const uint32_t entry = queue[kTileBlocks - 1 - k];
-        const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
-        const uint64_t rec = read_record(raw, off + 6 * f);
-        const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
-        const FastClass fc = T.fast[ci];
-        const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
-        const uint32_t col = f - row * nb;
-        const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
-        const uint32_t fv1 = fc.u0 >> 16;
-        const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
-        int d0 = 0, d1 = 0, d2 = 0;
-        even_codes(T, fc, li, [&](int q, uint32_t sel, uint32_t sel2) {
-          const int w = (int)(__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel) |
-                              __builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2));
-          d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
-          d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-          d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
-        });
-        partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
-      }
+    // P3 operands are fetched before the barrier so their latency hides behind it
+    constexpr int kP3Rows = 4;
+    float rs_pre[kP3Rows], tl_pre[kP3Rows];
+#pragma unroll
+    for (int j = 0; j < kP3Rows; ++j) {
+      const uint32_t row = wave + (uint32_t)j * kWaves;
+      rs_pre[j] = row < rows ? M.rscale[r0 + row] : 0.f;
+      tl_pre[j] = (row < rows && lane < a.tail_w) ? M.tail[(size_t)(r0 + row) * a.tail_w + lane] : 0.f;
     }
+    LLVQ_STAMP(4);
     __syncthreads();
+    LLVQ_STAMP(5);
 
     // P3: fixed-order row sums, row scale, tail columns
-    for (uint32_t row = wave; row < rows; row += kWaves) {
+#pragma unroll
+    for (int j = 0; j < kP3Rows; ++j) {
+      const uint32_t row = wave + (uint32_t)j * kWaves;
+      if (row < rows) {
+        float s = 0.f;
+        for (uint32_t b = lane; b < nb; b += 64u) s += partial[row * nb + b];
+        float v = fmaf(tl_pre[j], lane < a.tail_w ? xtail[lane] : 0.f, s * rs_pre[j]);
+        v = wave_sum(v);
+        if (lane == 0) store_out<OutT>(M.y, r0 + row, v);
+      }
+    }
+    for (uint32_t row = wave + kP3Rows * kWaves; row < rows; row += kWaves) {
       float s = 0.f;
       for (uint32_t b = lane; b < nb; b += 64u) s += partial[row * nb + b];
       float v = s * M.rscale[r0 + row];
@@ -335,6 +448,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       if (lane == 0) store_out<OutT>(M.y, r0 + row, v);
     }
     __syncthreads();
+    LLVQ_STAMP(6);
   }
 }
 
@@ -444,6 +558,12 @@ void llvq_hip_runtime_destroy(llvq_rt* rt) {
   (void)hipFree(rt->blob);
   delete rt;
 }
+
+#ifdef LLVQ_PHASE_TIMING
+int llvq_hip_debug_phase_stamps(unsigned long long* out, size_t n) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_phase_stamps), n * sizeof(unsigned long long));
+}
+#endif
 
 int llvq_hip_synchronize(llvq_rt* rt) {
   if (!rt) return fail(LLVQ_ERR_INVALID_ARGUMENT, "synchronize: runtime is null");
