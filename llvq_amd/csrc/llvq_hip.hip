@@ -113,7 +113,6 @@ constexpr int kP1Blocks = kTileBlocks / kWgThreads;  // blocks one lane classifi
 constexpr int kRawBytes = kTileBlocks * 6 + 32;
 constexpr int kMaxGroup = 4;
 constexpr int kPlaneDwords = 18;  // 3 planes x 6 dwords per 24-column block
-constexpr int kGenericSlots = 64; // queue for blocks of the rare generic classes
 
 struct MatArg {
   const uint8_t* codes;
@@ -135,7 +134,7 @@ struct GroupArgs {
 
 __host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks) {
   return sizeof(TableImage) + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + kRawBytes +
-         (size_t)kTileBlocks * 4 * 2 + kGenericSlots * 4 + 16;
+         (size_t)kTileBlocks * 4 * 2 + 16;
 }
 
 template <typename OutT>
@@ -149,7 +148,7 @@ __device__ __forceinline__ void store_out<__half>(void* y, uint32_t r, float v) 
   reinterpret_cast<__half*>(y)[r] = __float2half_rn(v);
 }
 
-// queue entry: block slot in the tile (12 bits) | class (9 bits) << 16 | gain << 25
+// queue entry: block slot in the tile (12 bits) | class (9 bits) << 16 | gain << 25 | generic-walk << 31
 __device__ __forceinline__ void queue_push(uint32_t* counter, uint32_t* queue, bool mine, uint32_t entry,
                                            bool from_top) {
   const uint64_t m = __ballot(mine);
@@ -164,9 +163,23 @@ __device__ __forceinline__ void queue_push(uint32_t* counter, uint32_t* queue, b
 
 // One 24-column block of the activation -> scale and byte planes.
 __device__ __forceinline__ void quantize_block(const __half* x, uint32_t* planes, float* scale) {
-  float v[kDim];  // 2-byte loads: the activation of a batched row need not be 16-byte aligned
+  float v[kDim];
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const uint4* src = reinterpret_cast<const uint4*>(x);
 #pragma unroll
-  for (int j = 0; j < kDim; ++j) v[j] = __half2float(x[j]);
+    for (int k = 0; k < 3; ++k) {
+      const uint4 u = src[k];
+      const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[8 * k + 2 * j] = __half2float(__ushort_as_half((unsigned short)(w[j] & 0xFFFFu)));
+        v[8 * k + 2 * j + 1] = __half2float(__ushort_as_half((unsigned short)(w[j] >> 16)));
+      }
+    }
+  } else {  // the activation of a batched row need not be 16-byte aligned
+#pragma unroll
+    for (int j = 0; j < kDim; ++j) v[j] = __half2float(x[j]);
+  }
   float amax = 0.f;
 #pragma unroll
   for (int j = 0; j < kDim; ++j) amax = fmaxf(amax, fabsf(v[j]));
@@ -203,27 +216,28 @@ __device__ __forceinline__ float planes_to_float(int d0, int d1, int d2) {
   return fmaf((float)d2, 65536.f, fmaf((float)d1, 256.f, (float)d0));
 }
 
-// One block of a class outside the fast paths: generic walk, scalar reduction
-// against the activation planes.
-__device__ __noinline__ void generic_block(const DecodeTables& T, const GroupArgs& a, const MatArg& M,
-                                           uint32_t entry, const uint8_t* raw, uint32_t off,
-                                           const uint32_t* xplanes, const float* xscale, float* partial) {
-  const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
-  const uint64_t rec = read_record(raw, off + 6 * f);
-  const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
-  const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
-  const uint32_t col = f - row * a.nblocks;
-  const uint8_t* xb = reinterpret_cast<const uint8_t*>(xplanes + (size_t)col * kPlaneDwords);
-  const DevClass c = T.cls[ci];
-  int d0 = 0, d1 = 0, d2 = 0;
-  auto emit = [&](int p, int v) {
-    d0 += v * (int)(int8_t)xb[p];
-    d1 += v * (int)(int8_t)xb[24 + p];
-    d2 += v * (int)(int8_t)xb[48 + p];
-  };
-  if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
-  else decode_even(T, c, li, emit);
-  partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (c.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+__device__ __forceinline__ void tile_of(const GroupArgs& a, uint32_t tile, MatArg& M, uint32_t& r0, uint32_t& rows) {
+  M = a.m[0];  // constant indices only: a dynamic one would move the arguments to scratch
+#pragma unroll
+  for (uint32_t k = 1; k < kMaxGroup; ++k)
+    if (k < a.n_mats && tile >= a.m[k].tile_begin) M = a.m[k];
+  r0 = (tile - M.tile_begin) * a.rows_per_tile;
+  rows = min(a.rows_per_tile, M.d_out - r0);
+}
+
+// Issues the loads of a tile's code bytes (16-byte units, from the aligned
+// address at or below the tile's first byte) into two registers per lane.
+__device__ __forceinline__ void prefetch_tile(const GroupArgs& a, uint32_t tile, uint32_t tid, uint4& p0, uint4& p1) {
+  if (tile >= a.n_tiles) return;
+  MatArg M;
+  uint32_t r0, rows;
+  tile_of(a, tile, M, r0, rows);
+  const size_t byte0 = (size_t)r0 * a.nblocks * 6;
+  const uint32_t off = (uint32_t)(byte0 & 15);
+  const uint4* src = reinterpret_cast<const uint4*>(M.codes + (byte0 - off));
+  const uint32_t n16 = (off + rows * a.nblocks * 6 + 15) >> 4;
+  if (tid < n16) p0 = src[tid];
+  if (tid + kWgThreads < n16) p1 = src[tid + kWgThreads];
 }
 
 // Phase timestamps for tuning builds (-DLLVQ_PHASE_TIMING): wave 0 of each
@@ -249,9 +263,14 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   uint8_t* raw = reinterpret_cast<uint8_t*>(xtail + 32);
   uint32_t* queue = reinterpret_cast<uint32_t*>(raw + kRawBytes);
   float* partial = reinterpret_cast<float*>(queue + kTileBlocks);
-  uint32_t* gqueue = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
-  uint32_t* ctrl = gqueue + kGenericSlots;
+  uint32_t* ctrl = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  // The code bytes of a tile travel HBM -> registers -> LDS; the first tile's
+  // loads are issued before the tables and the activation are staged, the next
+  // tile's while the current one is being decoded.
+  static_assert(kRawBytes <= 2 * 16 * kWgThreads, "two 16-byte registers per lane hold a tile's code bytes");
+  uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0;
+  prefetch_tile(a, blockIdx.x, tid, pre0, pre1);
   for (uint32_t col = tid; col < nb; col += kWgThreads)
     quantize_block(a.x + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
   if (tid < a.tail_w) xtail[tid] = __half2float(a.x[(size_t)nb * kDim + tid]);
@@ -261,22 +280,31 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 #endif
   for (uint32_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
     LLVQ_STAMP(0);
-    MatArg M = a.m[0];  // constant indices only: a dynamic one would move the arguments to scratch
-#pragma unroll
-    for (uint32_t k = 1; k < kMaxGroup; ++k)
-      if (k < a.n_mats && tile >= a.m[k].tile_begin) M = a.m[k];
-    const uint32_t r0 = (tile - M.tile_begin) * a.rows_per_tile;
-    const uint32_t rows = min(a.rows_per_tile, M.d_out - r0);
+    MatArg M;
+    uint32_t r0, rows;
+    tile_of(a, tile, M, r0, rows);
     const uint32_t nblk = rows * nb;
     const size_t byte0 = (size_t)r0 * nb * 6;
     const uint32_t off = (uint32_t)(byte0 & 15);
 
-    // P0: code bytes HBM -> LDS
+    // P0: code bytes registers -> LDS
     if (tid < 4) ctrl[tid] = 0;
     {
-      const uint4* src = reinterpret_cast<const uint4*>(M.codes + (byte0 - off));
       const uint32_t n16 = (off + nblk * 6 + 15) >> 4;
-      for (uint32_t i = tid; i < n16; i += kWgThreads) reinterpret_cast<uint4*>(raw)[i] = src[i];
+      if (tid < n16) reinterpret_cast<uint4*>(raw)[tid] = pre0;
+      if (tid + kWgThreads < n16) reinterpret_cast<uint4*>(raw)[tid + kWgThreads] = pre1;
+    }
+    // P3 operands (row scales, tail weights): fetched now, used after the decode
+    const uint32_t sub = lane >> 4, l16 = lane & 15u;
+    constexpr int kP3Rounds = 2;  // 64 rows per round cover every tile of the usual shapes
+    float rs_pre[kP3Rounds], tl_pre[kP3Rounds][2];
+#pragma unroll
+    for (int j = 0; j < kP3Rounds; ++j) {
+      const uint32_t row = (wave * 4 + sub) + (uint32_t)j * (kWaves * 4);
+      const bool ok = row < rows;
+      rs_pre[j] = ok ? M.rscale[r0 + row] : 0.f;
+      tl_pre[j][0] = (ok && l16 < a.tail_w) ? M.tail[(size_t)(r0 + row) * a.tail_w + l16] : 0.f;
+      tl_pre[j][1] = (ok && l16 + 16 < a.tail_w) ? M.tail[(size_t)(r0 + row) * a.tail_w + l16 + 16] : 0.f;
     }
     __syncthreads();
     LLVQ_STAMP(1);
@@ -300,23 +328,26 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
           else zi[i] = (rec >> 1) - 1;
         }
       }
-      uint32_t kmax = 0;
+      uint32_t kbits[kP1Blocks], kmax = 0;  // kbits = 2^k: how many classes the bucket's search spans
 #pragma unroll
-      for (int i = 0; i < kP1Blocks; ++i)
+      for (int i = 0; i < kP1Blocks; ++i) {
+        kbits[i] = 0;
         if (zi[i] != ~0ULL) {
           const uint32_t e = T.lut[(uint32_t)(zi[i] >> kLutShift)];
           ci[i] = e & 511u;
-          kmax = max(kmax, e >> 9);
+          kbits[i] = 1u << (e >> 9);
+          kmax = max(kmax, kbits[i]);
         }
-      // every chain of the wavefront runs the same number of halving steps: a
-      // search over a superset of the bucket's classes finds the same class
-      uint32_t kw = 0;
+      }
+      // the wavefront runs as many halving steps as its widest bucket needs; a
+      // lane only reads the table on the steps its own bucket needs
+      uint32_t kw = 1;
 #pragma unroll
-      for (uint32_t t = 1; t <= 6; ++t) kw = __any(kmax >= t) ? t : kw;
-      for (uint32_t step = (1u << kw) >> 1; step; step >>= 1) {
+      for (uint32_t t = 1; t <= 6; ++t) kw = __any(kmax >= (1u << t)) ? (1u << t) : kw;
+      for (uint32_t step = kw >> 1; step; step >>= 1) {
 #pragma unroll
         for (int i = 0; i < kP1Blocks; ++i)
-          if (zi[i] != ~0ULL && T.starts[ci[i] + step] <= zi[i]) ci[i] += step;
+          if (step < kbits[i] && T.starts[ci[i] + step] <= zi[i]) ci[i] += step;
       }
       uint32_t path[kP1Blocks];
 #pragma unroll
@@ -324,10 +355,12 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
         path[i] = zi[i] != ~0ULL ? ((T.fast[ci[i]].meta >> kMetaPathShift) & 3u) : 3u;
         entry[i] |= ci[i] << 16;
       }
+      // blocks of the rare generic classes ride in the odd queue with bit 31 set
       uint32_t odd_rank[kP1Blocks], even_rank[kP1Blocks], n_o = 0, n_e = 0;
 #pragma unroll
       for (int i = 0; i < kP1Blocks; ++i) {
-        const uint64_t mo = __ballot(path[i] == kPathOdd), me = __ballot(path[i] == kPathEven);
+        if (path[i] == kPathGeneric) entry[i] |= 0x80000000u;
+        const uint64_t mo = __ballot(path[i] == kPathOdd || path[i] == kPathGeneric), me = __ballot(path[i] == kPathEven);
         odd_rank[i] = n_o + __builtin_amdgcn_mbcnt_hi((uint32_t)(mo >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mo, 0));
         even_rank[i] = n_e + __builtin_amdgcn_mbcnt_hi((uint32_t)(me >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)me, 0));
         n_o += (uint32_t)__popcll(mo);
@@ -342,55 +375,60 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       base_e = __shfl(base_e, 0, 64);
 #pragma unroll
       for (int i = 0; i < kP1Blocks; ++i) {
-        if (path[i] == kPathOdd) queue[base_o + odd_rank[i]] = entry[i];
+        if (path[i] == kPathOdd || path[i] == kPathGeneric) queue[base_o + odd_rank[i]] = entry[i];
         if (path[i] == kPathEven) queue[kTileBlocks - 1 - (base_e + even_rank[i])] = entry[i];
-      }
-      // rare classes go to a small third queue; what does not fit is decoded here
-#pragma unroll
-      for (int i = 0; i < kP1Blocks; ++i) {
-        if (path[i] == kPathGeneric) {
-          const uint32_t slot = atomicAdd(&ctrl[2], 1u);
-          if (slot < (uint32_t)kGenericSlots) gqueue[slot] = entry[i];
-          else generic_block(T, a, M, entry[i], raw, off, xplanes, xscale, partial);
-        }
       }
     }
     __syncthreads();
     LLVQ_STAMP(2);
+    prefetch_tile(a, tile + gridDim.x, tid, pre0, pre1);
 
     // P2: unrank and reduce.  Chunks of 64 queued blocks are handed out through a
     // counter: the generic chunk first (longest), then odd, then even.
-    const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
-    const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
+    const uint32_t n_odd = ctrl[0], n_even = ctrl[1];
+    const uint32_t c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
     for (;;) {
       uint32_t chunk = 0;
       if (lane == 0) chunk = atomicAdd(&ctrl[3], 1u);
       chunk = __shfl(chunk, 0, 64);
-      if (chunk >= c_gen + c_odd + c_even) break;
-      if (chunk < c_gen) {
-        if (lane < n_gen) generic_block(T, a, M, gqueue[lane], raw, off, xplanes, xscale, partial);
-      } else if (chunk < c_gen + c_odd) {
-        const uint32_t k = (chunk - c_gen) * 64u + lane;
+      if (chunk >= c_odd + c_even) break;
+      if (chunk < c_odd) {
+        const uint32_t k = chunk * 64u + lane;
         if (k < n_odd) {
           const uint32_t entry = queue[k];
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
           const uint64_t rec = read_record(raw, off + 6 * f);
           const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
-          const FastClass fc = T.fast[ci];
           const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
           const uint32_t col = f - row * nb;
           const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
-          int d0 = 0, d1 = 0, d2 = 0;
-          odd_codes(T, fc, li, [&](int q, uint32_t sel) {
-            const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
-            d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
-            d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-            d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
-          });
-          partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+          const float g = (entry >> 25) & 1u ? M.g1 : M.g0;
+          if (entry >> 31) {  // generic walk, scalar reduction against the planes
+            const uint8_t* xb = reinterpret_cast<const uint8_t*>(xp);
+            const DevClass c = T.cls[ci];
+            int d0 = 0, d1 = 0, d2 = 0;
+            auto emit = [&](int p, int v) {
+              d0 += v * (int)(int8_t)xb[p];
+              d1 += v * (int)(int8_t)xb[24 + p];
+              d2 += v * (int)(int8_t)xb[48 + p];
+            };
+            if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
+            else decode_even(T, c, li, emit);
+            partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (c.inv_norm * g);
+          } else {
+            const FastClass fc = T.fast[ci];
+            int d0 = 0, d1 = 0, d2 = 0;
+            odd_codes(T, fc, li, [&](int q, uint32_t sel) {
+              const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+              d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+              d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+              d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+            });
+            partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * g);
+          }
         }
       } else {
-        const uint32_t k = (chunk - c_gen - c_odd) * 64u + lane;
+        const uint32_t k = (chunk - c_odd) * 64u + lane;
         if (k < n_even) {
           const uint32_t entry = queue[kTileBlocks - 1 - k];
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
@@ -414,38 +452,33 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
         }
       }
     }
-    // P3 operands are fetched before the barrier so their latency hides behind it
-    constexpr int kP3Rows = 4;
-    float rs_pre[kP3Rows], tl_pre[kP3Rows];
-#pragma unroll
-    for (int j = 0; j < kP3Rows; ++j) {
-      const uint32_t row = wave + (uint32_t)j * kWaves;
-      rs_pre[j] = row < rows ? M.rscale[r0 + row] : 0.f;
-      tl_pre[j] = (row < rows && lane < a.tail_w) ? M.tail[(size_t)(r0 + row) * a.tail_w + lane] : 0.f;
-    }
     LLVQ_STAMP(4);
     __syncthreads();
     LLVQ_STAMP(5);
-
-    // P3: fixed-order row sums, row scale, tail columns
-#pragma unroll
-    for (int j = 0; j < kP3Rows; ++j) {
-      const uint32_t row = wave + (uint32_t)j * kWaves;
-      if (row < rows) {
-        float s = 0.f;
-        for (uint32_t b = lane; b < nb; b += 64u) s += partial[row * nb + b];
-        float v = fmaf(tl_pre[j], lane < a.tail_w ? xtail[lane] : 0.f, s * rs_pre[j]);
-        v = wave_sum(v);
-        if (lane == 0) store_out<OutT>(M.y, r0 + row, v);
-      }
-    }
-    for (uint32_t row = wave + kP3Rows * kWaves; row < rows; row += kWaves) {
+    // P3: 16 lanes per row, fixed summation order
+    for (uint32_t base = 0; base < rows; base += kWaves * 4) {
+      const uint32_t j = base / (kWaves * 4);
+      const uint32_t row = base + wave * 4 + sub;
+      const bool ok = row < rows;
       float s = 0.f;
-      for (uint32_t b = lane; b < nb; b += 64u) s += partial[row * nb + b];
-      float v = s * M.rscale[r0 + row];
-      if (lane < a.tail_w) v = fmaf(M.tail[(size_t)(r0 + row) * a.tail_w + lane], xtail[lane], v);
-      v = wave_sum(v);
-      if (lane == 0) store_out<OutT>(M.y, r0 + row, v);
+      if (ok)
+        for (uint32_t b = l16; b < nb; b += 16u) s += partial[row * nb + b];  // fixed order per lane
+      float rs, t0, t1;
+      if (j < (uint32_t)kP3Rounds) {
+        rs = j == 0 ? rs_pre[0] : rs_pre[1];
+        t0 = j == 0 ? tl_pre[0][0] : tl_pre[1][0];
+        t1 = j == 0 ? tl_pre[0][1] : tl_pre[1][1];
+      } else {
+        rs = ok ? M.rscale[r0 + row] : 0.f;
+        t0 = (ok && l16 < a.tail_w) ? M.tail[(size_t)(r0 + row) * a.tail_w + l16] : 0.f;
+        t1 = (ok && l16 + 16 < a.tail_w) ? M.tail[(size_t)(r0 + row) * a.tail_w + l16 + 16] : 0.f;
+      }
+      float v = s * rs;
+      v = fmaf(t0, l16 < a.tail_w ? xtail[l16] : 0.f, v);
+      v = fmaf(t1, l16 + 16 < a.tail_w ? xtail[l16 + 16] : 0.f, v);
+#pragma unroll
+      for (int o = 8; o >= 1; o >>= 1) v += __shfl_xor(v, o, 16);  // fixed tree inside each group of 16 lanes
+      if (ok && l16 == 0) store_out<OutT>(M.y, r0 + row, v);
     }
     __syncthreads();
     LLVQ_STAMP(6);

@@ -174,6 +174,28 @@ class FusedRuntime:
         _ffi.check(_ffi.lib().llvq_hip_gemv_group(self.handle, mats, len(projs), xr.data_ptr(), outs, code))
         return ys
 
+    def plan_group(self, projs, x, out_dtype=None):
+        """Pre-binds one launch: returns (launch, outputs).  `launch()` enqueues the
+        group's GEMV on the runtime's stream with no Python-side allocation or
+        argument marshalling — what a decode loop calls once per token."""
+        torch = self._torch
+        xr = self.rotate(projs[0], x)
+        out_dtype = out_dtype or torch.float16
+        ys = [torch.empty(list(x.shape[:-1]) + [p.d_out], dtype=out_dtype, device=xr.device) for p in projs]
+        mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
+        outs = (C.c_void_p * len(projs))(*[y.data_ptr() for y in ys])
+        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        fn = _ffi.lib().llvq_hip_gemv_group
+        rt, n, xp = self.handle, len(projs), C.c_void_p(xr.data_ptr())
+        keep = (xr, ys, mats, outs)
+
+        def launch(_keep=keep):
+            rc = fn(rt, mats, n, xp, outs, code)
+            if rc:
+                _ffi.check(rc)
+
+        return launch, ys
+
     def forward_batched(self, proj: FusedProj, x, out_dtype=None):
         """Rows of `x` [M, d_in] through one projection (the row loop of model.rs:521-529)."""
         torch = self._torch
