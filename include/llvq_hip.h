@@ -90,6 +90,19 @@ int llvq_hip_matrix_upload(llvq_rt* rt, const llvq_matrix_desc* desc, llvq_mat**
  * fingerprint.  *pos is advanced past the header. */
 int llvq_hip_read_header(const uint8_t* buf, size_t len, size_t* pos, uint32_t* version,
                          uint32_t* n_matrices);
+/* read_matrix_raw (format.rs:301) without decoding or uploading anything: the
+ * shape and byte ranges of the record at buf[*pos..], *pos advanced past it.
+ * Needs no GPU.  Offsets are relative to buf. */
+typedef struct llvq_record_info {
+  char name[256];            /* truncated to 255 bytes, NUL-terminated */
+  uint32_t d_out, d_in, shell_cap, n_centroids;
+  uint64_t rotation_seed;
+  uint32_t has_rotation;
+  size_t centroids_off, row_scales_off, tail_off, codes_off;
+  size_t code_bytes;
+} llvq_record_info;
+int llvq_hip_parse_matrix_record(const uint8_t* buf, size_t len, size_t* pos, llvq_record_info* out);
+
 /* read_matrix_raw (format.rs:301) fused with upload: parses one on-disk matrix
  * record at buf[*pos..] and uploads it; the code stream is copied verbatim.
  * *pos is advanced past the record. */

@@ -32,6 +32,16 @@ class MatrixDesc(C.Structure):
     ]
 
 
+class RecordInfo(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 256),
+        ("d_out", C.c_uint32), ("d_in", C.c_uint32), ("shell_cap", C.c_uint32), ("n_centroids", C.c_uint32),
+        ("rotation_seed", C.c_uint64), ("has_rotation", C.c_uint32),
+        ("centroids_off", C.c_size_t), ("row_scales_off", C.c_size_t), ("tail_off", C.c_size_t),
+        ("codes_off", C.c_size_t), ("code_bytes", C.c_size_t),
+    ]
+
+
 def lib_path():
     return _LIB
 
@@ -63,6 +73,7 @@ def lib():
     L.llvq_hip_host_decode.argtypes = [C.c_uint64, vp, C.POINTER(C.c_int)]
     L.llvq_hip_matrix_upload.argtypes = [vp, C.POINTER(MatrixDesc), C.POINTER(vp)]
     L.llvq_hip_read_header.argtypes = [C.c_char_p, sz, C.POINTER(sz), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+    L.llvq_hip_parse_matrix_record.argtypes = [C.c_char_p, sz, C.POINTER(sz), C.POINTER(RecordInfo)]
     L.llvq_hip_matrix_from_record.argtypes = [vp, C.c_char_p, sz, C.POINTER(sz), C.POINTER(vp)]
     L.llvq_hip_matrix_free.argtypes = [vp, vp]
     L.llvq_hip_matrix_free.restype = None
@@ -87,7 +98,8 @@ def check(rc):
 
 EXPORTS = [
     "llvq_hip_runtime_create", "llvq_hip_runtime_destroy", "llvq_hip_codebook_fingerprint",
-    "llvq_hip_host_decode", "llvq_hip_matrix_upload", "llvq_hip_read_header", "llvq_hip_matrix_from_record",
+    "llvq_hip_host_decode", "llvq_hip_matrix_upload", "llvq_hip_read_header", "llvq_hip_parse_matrix_record",
+    "llvq_hip_matrix_from_record",
     "llvq_hip_matrix_free", "llvq_hip_matrix_info", "llvq_hip_matrix_name", "llvq_hip_gemv",
     "llvq_hip_gemv_group", "llvq_hip_gemm", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
     "llvq_hip_last_error", "llvq_hip_version",

@@ -19,6 +19,7 @@ struct RecordView {
   std::vector<float> tail;      // d_out * (d_in % 24), as stored (f32)
   const uint8_t* codes = nullptr;
   size_t code_bytes = 0;
+  size_t centroids_off = 0, row_scales_off = 0, tail_off = 0, codes_off = 0;  // relative to the buffer
 };
 
 // Status codes are the llvq_status values of include/llvq_hip.h.

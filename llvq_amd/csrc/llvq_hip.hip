@@ -695,6 +695,30 @@ int llvq_hip_read_header(const uint8_t* buf, size_t len, size_t* pos, uint32_t* 
   return rc ? fail(rc, err) : LLVQ_OK;
 }
 
+int llvq_hip_parse_matrix_record(const uint8_t* buf, size_t len, size_t* pos, llvq_record_info* out) {
+  if (!buf || !pos || !out || *pos > len) return fail(LLVQ_ERR_INVALID_ARGUMENT, "parse_matrix_record: bad argument");
+  RecordView r;
+  std::string err;
+  size_t p = *pos;
+  const int rc = parse_matrix_record(buf, len, &p, &r, &err);
+  if (rc) return fail(rc, err);
+  std::memset(out, 0, sizeof *out);
+  std::strncpy(out->name, r.name.c_str(), sizeof out->name - 1);
+  out->d_out = r.d_out;
+  out->d_in = r.d_in;
+  out->shell_cap = r.shell_cap;
+  out->n_centroids = r.n_centroids;
+  out->rotation_seed = r.rotation_seed;
+  out->has_rotation = r.has_rotation ? 1 : 0;
+  out->centroids_off = r.centroids_off;
+  out->row_scales_off = r.row_scales_off;
+  out->tail_off = r.tail_off;
+  out->codes_off = r.codes_off;
+  out->code_bytes = r.code_bytes;
+  *pos = p;
+  return LLVQ_OK;
+}
+
 int llvq_hip_matrix_from_record(llvq_rt* rt, const uint8_t* buf, size_t len, size_t* pos,
                                 llvq_mat** out) {
   if (!rt || !buf || !pos || !out || *pos > len)

@@ -692,10 +692,30 @@ int orc_fast_decode(uint64_t idx, int32_t p[ORC_DIM]) { /* fastdec.rs:321-399 */
 typedef struct {
   int32_t* out;
   size_t cap, n;
+  /* streaming check (orc_shell_roundtrip_check) */
+  int check, shell, err;
+  size_t stride;
+  uint64_t lo, hi;
+  uint8_t* seen;
 } sink_t;
 
+static void check_point(sink_t* s, const int32_t* x) {
+  uint64_t idx;
+  int32_t back[ORC_DIM];
+  if (!orc_leech_contains(x) || orc_shell_index(x) != s->shell) { s->err = 1; return; }
+  if (!orc_index_encode(x, &idx) || idx < s->lo || idx > s->hi) { s->err = 2; return; }
+  if (s->seen[(idx - s->lo) >> 3] & (1u << ((idx - s->lo) & 7))) { s->err = 3; return; }
+  s->seen[(idx - s->lo) >> 3] |= (uint8_t)(1u << ((idx - s->lo) & 7));
+  if (!orc_index_decode(idx, back) || memcmp(back, x, sizeof back)) { s->err = 4; return; }
+  if (!orc_fast_decode(idx, back) || memcmp(back, x, sizeof back)) { s->err = 5; return; }
+}
+
 static void emit(sink_t* s, const int32_t* x) {
-  if (s->out && s->n < s->cap) memcpy(s->out + s->n * ORC_DIM, x, sizeof(int32_t) * ORC_DIM);
+  if (s->check) {
+    if (!s->err && s->n % s->stride == 0) check_point(s, x);
+  } else if (s->out && s->n < s->cap) {
+    memcpy(s->out + s->n * ORC_DIM, x, sizeof(int32_t) * ORC_DIM);
+  }
   s->n++;
 }
 static void ones_base(uint32_t c, int32_t* x) {
@@ -714,9 +734,40 @@ static void emit_two_support(sink_t* s, uint32_t support, int want_odd_minus, in
   }
 }
 
+static size_t enumerate_shell(int m, sink_t* sp);
+
 size_t orc_enumerate_shell(int m, int32_t* out, size_t cap_points) {
   ensure_init();
-  sink_t s = {out, cap_points, 0};
+  sink_t s;
+  memset(&s, 0, sizeof s);
+  s.out = out;
+  s.cap = cap_points;
+  return enumerate_shell(m, &s);
+}
+
+/* Every stride-th point of shell m (2 or 3) from the independent enumerator:
+ * member of the lattice on shell m, encodes into [lo, hi] with no collision,
+ * and both decoders return it.  Returns the number of points enumerated, or
+ * the negated code of the first failure (1 membership, 2 range, 3 collision,
+ * 4 Indexer round trip, 5 FastDecoder round trip). */
+long long orc_shell_roundtrip_check(int m, size_t stride, uint64_t lo, uint64_t hi) {
+  ensure_init();
+  sink_t s;
+  memset(&s, 0, sizeof s);
+  s.check = 1;
+  s.shell = m;
+  s.stride = stride ? stride : 1;
+  s.lo = lo;
+  s.hi = hi;
+  s.seen = (uint8_t*)calloc((size_t)((hi - lo) / 8 + 2), 1);
+  size_t n = enumerate_shell(m, &s);
+  free(s.seen);
+  return s.err ? -(long long)s.err : (long long)n;
+}
+
+static size_t enumerate_shell(int m, sink_t* sp) {
+  sink_t s = *sp;
+  size_t ret = 0;
   if (m == 2) { /* shells.rs:66-92 */
     for (int i = g_start[8]; i < g_start[9]; i++) emit_two_support(&s, g_words[i], 0, -1, 0);
     for (int i = 0; i < ORC_DIM; i++)
@@ -734,7 +785,9 @@ size_t orc_enumerate_shell(int m, int32_t* out, size_t cap_points) {
         x[p] = ((g_words[g] >> p) & 1) ? 3 : -3;
         emit(&s, x);
       }
-    return s.n;
+    ret = s.n;
+    *sp = s;
+    return ret;
   }
   if (m == 3) { /* shells.rs:94-143 */
     for (int i = g_start[12]; i < g_start[13]; i++) emit_two_support(&s, g_words[i], 0, -1, 0);
@@ -763,7 +816,9 @@ size_t orc_enumerate_shell(int m, int32_t* out, size_t cap_points) {
             x[k] = ((c >> k) & 1) ? 3 : -3;
             emit(&s, x);
           }
-    return s.n;
+    ret = s.n;
+    *sp = s;
+    return ret;
   }
   return 0;
 }

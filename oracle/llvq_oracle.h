@@ -48,6 +48,9 @@ int64_t orc_shell_index(const int32_t p[ORC_DIM]);   /* leech.rs:132-142; -1 whe
 /* shells.rs:66-143 — every point of shell 2 or 3 exactly once; returns count,
  * 0 for an unsupported shell.  `out` may be NULL (count only). */
 size_t orc_enumerate_shell(int m, int32_t* out /* count*24 */, size_t cap_points);
+/* llvq-search/tests/g3_index.rs:41-60 on every stride-th point of shell 2 or 3:
+ * count of enumerated points, or a negative failure code. */
+long long orc_shell_roundtrip_check(int m, size_t stride, uint64_t lo, uint64_t hi);
 
 /* rng.rs:21-40 */
 uint64_t orc_splitmix_next(uint64_t* state);

@@ -64,6 +64,8 @@ def lib():
     L.orc_shell_index.argtypes = [i32p]
     L.orc_enumerate_shell.restype = C.c_size_t
     L.orc_enumerate_shell.argtypes = [C.c_int, i32p, C.c_size_t]
+    L.orc_shell_roundtrip_check.restype = C.c_longlong
+    L.orc_shell_roundtrip_check.argtypes = [C.c_int, C.c_size_t, C.c_uint64, C.c_uint64]
     for f in (L.orc_splitmix_next,):
         f.restype = C.c_uint64
         f.argtypes = [C.POINTER(C.c_uint64)]

@@ -1,0 +1,121 @@
+"""The shipped library without a GPU: exported symbols, its own codebook tables
+and host decoder (the arithmetic the kernels run), its record reader."""
+import ctypes as C
+import os
+import re
+import struct
+
+import numpy as np
+import pytest
+
+from llvq_amd import _ffi, artifact, synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_every_declared_symbol_is_exported():
+    hdr = open(os.path.join(ROOT, "include", "llvq_hip.h")).read()
+    declared = sorted(set(re.findall(r"\b(llvq_hip_[a-z_0-9]+)\s*\(", hdr)))
+    assert declared == sorted(_ffi.EXPORTS)
+    L = _ffi.lib()
+    for name in declared:
+        assert hasattr(L, name), name
+
+
+def test_library_fingerprint_is_the_published_one():
+    assert _ffi.lib().llvq_hip_codebook_fingerprint() == 0x338F420F11866319
+
+
+def _host_decode(indices):
+    L = _ffi.lib()
+    out = np.zeros((len(indices), 24), np.int8)
+    shells = np.zeros(len(indices), np.int32)
+    s = C.c_int()
+    for k, i in enumerate(indices):
+        assert L.llvq_hip_host_decode(int(i), out[k].ctypes.data, C.byref(s)) == 1
+        shells[k] = s.value
+    return out, shells
+
+
+def test_host_decoder_matches_oracle_on_boundaries_and_draws(orc, boundary_indices):
+    """The library's decoder (table-driven even coset, FP64 walk of the odd coset) against
+    the reference algorithm restated in the oracle: every class boundary, 60 000 draws."""
+    got, shells = _host_decode(boundary_indices)
+    ref = orc.decode_many(boundary_indices, fast=False)
+    assert np.array_equal(got, ref)
+    assert np.array_equal(shells, (ref.astype(np.int64) ** 2).sum(1) // 16)
+    idx = synth.SplitMix64(0xBEEF).take(60_000) % np.uint64(orc.N13 + 1)
+    assert np.array_equal(_host_decode(idx)[0], orc.decode_many(idx))
+    out = np.zeros(24, np.int8)
+    assert _ffi.lib().llvq_hip_host_decode(orc.N13 + 1, out.ctypes.data, None) == 0
+
+
+def test_host_decoder_dense_sweep_of_small_classes(orc):
+    """Consecutive indices across the first classes (every arrangement and sign pattern of
+    shells 2 and 3's small classes), where a mixed-radix slip would show at once."""
+    idx = np.arange(0, 120_000, dtype=np.uint64)
+    assert np.array_equal(_host_decode(idx)[0], orc.decode_many(idx))
+
+
+def test_record_reader_happy_path_and_hostile_files():
+    L = _ffi.lib()
+    raw = synth.make_matrix("model.layers.3.mlp.up_proj.weight", 4, 77, seed=2)
+    buf = artifact.write_file([raw], version=4)
+    pos = C.c_size_t(0)
+    ver, n = C.c_uint32(), C.c_uint32()
+    assert L.llvq_hip_read_header(buf, len(buf), C.byref(pos), C.byref(ver), C.byref(n)) == 0
+    assert (ver.value, n.value, pos.value) == (4, 1, 16)
+    info = _ffi.RecordInfo()
+    assert L.llvq_hip_parse_matrix_record(buf, len(buf), C.byref(pos), C.byref(info)) == 0
+    assert info.name.decode() == raw.name and (info.d_out, info.d_in, info.shell_cap, info.n_centroids) == (4, 77, 12, 2)
+    assert buf[info.codes_off:info.codes_off + info.code_bytes] == raw.codes.tobytes()
+    assert np.array_equal(np.frombuffer(buf, "<f8", 4, info.row_scales_off), raw.row_scales)
+    assert pos.value == len(buf) - 8
+
+    from test_oracle_format import _hostile_cases
+
+    kinds = {"NotAnArtifact": 1, "Truncated": 2, "BadName": 3, "Inconsistent": 5}
+    for hbuf, what, kind, reading in _hostile_cases():
+        pos = C.c_size_t(0)
+        if what == "header":
+            rc = L.llvq_hip_read_header(hbuf, len(hbuf), C.byref(pos), C.byref(ver), C.byref(n))
+        else:
+            rc = L.llvq_hip_parse_matrix_record(hbuf, len(hbuf), C.byref(pos), C.byref(info))
+        assert rc == kinds[kind], (kind, rc)
+        msg = L.llvq_hip_last_error().decode()
+        if reading:
+            assert msg == f"file ends mid-{reading}"
+        if kind == "Inconsistent":
+            assert "shell cap 65535" in msg
+    bad = bytearray(artifact.write_header(4, 1))
+    bad[9] ^= 0x40
+    pos = C.c_size_t(0)
+    assert L.llvq_hip_read_header(bytes(bad), len(bad), C.byref(pos), C.byref(ver), C.byref(n)) == 10
+
+
+def test_python_operator_refusals():
+    from llvq_amd.fused import FusedMatrix
+
+    raw = synth.make_matrix("model.layers.0.mlp.gate_proj.weight", 2, 48, seed=1)
+    three = artifact.RawMatrix(raw.name, 2, 48, 12, [0.5, 1.0, 1.5], raw.row_scales, raw.tail, raw.codes)
+    with pytest.raises(ValueError, match="3 centroids"):
+        FusedMatrix(three)
+    assert artifact.split_name("model.layers.17.self_attn.q_proj.weight") == (17, "self_attn.q_proj")
+    with pytest.raises(artifact.ArtifactError):
+        artifact.split_name("lm_head.weight")
+
+
+def test_synthetic_configs():
+    raw = synth.make_matrix("model.layers.0.self_attn.k_proj.weight", 8, 2560, seed=0)
+    assert raw.nblocks == 106 and raw.tail_w == 16 and raw.codes.size == 8 * 106 * 6
+    idx, g = raw.unpack()
+    assert int(idx.max()) <= artifact.N12 and set(np.unique(g)) <= {0, 1}
+    assert raw.encoded_bytes() == 8 * 106 * 6 + 8 * 16 * 4 + 8 * 8 + 16
+    # BASELINE byte counts: config 0 = 6 887 440, one layer = 27 243 632
+    shapes = {n: (o, i) for n, o, i in synth.QWEN3_4B_LAYER}
+    total = sum(6 * o * (i // 24) + 4 * o * (i % 24) + 8 * o + 16 for o, i in shapes.values())
+    assert total == 27_243_632
+    o, i = shapes["mlp.gate_proj"]
+    assert 6 * o * (i // 24) + 4 * o * (i % 24) + 8 * o + 16 == 6_887_440
+    x = synth.make_activation(2560, 0)
+    assert x.dtype == np.float16 and x.shape == (1, 2560)
