@@ -23,16 +23,27 @@ namespace llvq {
 // ---- table image --------------------------------------------------------------
 // What every workgroup copies into LDS.  The rarely used generic class records
 // and the large even-coset tables stay in HBM (they live in L2).
+#ifndef LLVQ_WG_THREADS
+#define LLVQ_WG_THREADS 1024
+#endif
+#ifndef LLVQ_TILE_BLOCKS
+#define LLVQ_TILE_BLOCKS 4096
+#endif
+#ifndef LLVQ_LDS_GOLAY
+#define LLVQ_LDS_GOLAY 1   // 1: Golay words and the support-arrangement table live in LDS; 0: read through L2
+#endif
 struct TableImage {
-  uint32_t golay[4096];
   FastClass fast[kClassSlots];
   uint64_t starts[kStartsLds];
   uint16_t lut[2048];        // a 47-bit field only reaches the lower half of the host table
   double rcp[32];
   uint8_t pdep4[256];
+  uint32_t golay[4096];
   uint32_t on_lut[kOnLutSlots];
 };
 static_assert(sizeof(TableImage) % 16 == 0, "table image is copied in 16-byte units");
+constexpr size_t kLdsImageBytes = LLVQ_LDS_GOLAY ? sizeof(TableImage) : offsetof(TableImage, golay);
+static_assert(kLdsImageBytes % 16 == 0, "LDS part of the table image is copied in 16-byte units");
 
 struct GlobalTables {
   const TableImage* image;
@@ -44,9 +55,10 @@ struct GlobalTables {
 __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const GlobalTables& g) {
   const uint4* src = reinterpret_cast<const uint4*>(g.image);
   uint4* dst = reinterpret_cast<uint4*>(smem);
-  for (uint32_t i = threadIdx.x; i < sizeof(TableImage) / 16; i += blockDim.x) dst[i] = src[i];
+  for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) dst[i] = src[i];
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
-  return DecodeTables{s->golay, g.cls, s->fast, s->starts, s->lut, s->rcp, s->on_lut, g.off_lut, g.expand, s->pdep4};
+  const TableImage* far = LLVQ_LDS_GOLAY ? s : g.image;
+  return DecodeTables{far->golay, g.cls, s->fast, s->starts, s->lut, s->rcp, far->on_lut, g.off_lut, g.expand, s->pdep4};
 }
 
 // 6-byte big-endian record at a 2-byte-aligned offset of a 4-byte-aligned buffer
@@ -106,13 +118,14 @@ __global__ __launch_bounds__(256) void decode_blocks_kernel(GlobalTables g, cons
 // value within 2^12 of its block's largest is exact and the rest round at
 // 2^-23 of that largest.  Integer sums of 24 products are exact; the three
 // plane sums are combined and scaled in f32.
-constexpr int kWgThreads = 1024;
+constexpr int kWgThreads = LLVQ_WG_THREADS;
 constexpr int kWaves = kWgThreads / 64;
-constexpr int kTileBlocks = 4096;
+constexpr int kTileBlocks = LLVQ_TILE_BLOCKS;
 constexpr int kP1Blocks = kTileBlocks / kWgThreads;  // blocks one lane classifies per tile
 constexpr int kRawBytes = kTileBlocks * 6 + 32;
 constexpr int kMaxGroup = 4;
 constexpr int kPlaneDwords = 18;  // 3 planes x 6 dwords per 24-column block
+constexpr int kGenericSlots = 64; // queue of blocks that take the generic walk
 
 struct MatArg {
   const uint8_t* codes;
@@ -133,8 +146,8 @@ struct GroupArgs {
 };
 
 __host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks) {
-  return sizeof(TableImage) + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + kRawBytes +
-         (size_t)kTileBlocks * 4 * 2 + 16;
+  return kLdsImageBytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + kRawBytes +
+         (size_t)kTileBlocks * 4 * 2 + kGenericSlots * 4 + 16;
 }
 
 template <typename OutT>
@@ -257,13 +270,14 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
   const DecodeTables T = stage_tables(smem, a.tables);
   const uint32_t nb = a.nblocks;
-  uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + sizeof(TableImage));
+  uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + kLdsImageBytes);
   float* xscale = reinterpret_cast<float*>(xplanes + (size_t)nb * kPlaneDwords);
   float* xtail = xscale + nb;
   uint8_t* raw = reinterpret_cast<uint8_t*>(xtail + 32);
   uint32_t* queue = reinterpret_cast<uint32_t*>(raw + kRawBytes);
   float* partial = reinterpret_cast<float*>(queue + kTileBlocks);
-  uint32_t* ctrl = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
+  uint32_t* gqueue = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
+  uint32_t* ctrl = gqueue + kGenericSlots;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   // The code bytes of a tile travel HBM -> registers -> LDS; the first tile's
   // loads are issued before the tables and the activation are staged, the next
@@ -355,11 +369,20 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
         path[i] = zi[i] != ~0ULL ? ((T.fast[ci[i]].meta >> kMetaPathShift) & 3u) : 3u;
         entry[i] |= ci[i] << 16;
       }
-      // blocks of the rare generic classes ride in the odd queue with bit 31 set
+      // Blocks of the rare generic classes take ~2000 dependent instructions: they
+      // go to a small queue that P2 hands out first; what does not fit rides in the
+      // odd queue.  Either way bit 31 marks them.
       uint32_t odd_rank[kP1Blocks], even_rank[kP1Blocks], n_o = 0, n_e = 0;
 #pragma unroll
       for (int i = 0; i < kP1Blocks; ++i) {
-        if (path[i] == kPathGeneric) entry[i] |= 0x80000000u;
+        if (path[i] == kPathGeneric) {
+          entry[i] |= 0x80000000u;
+          const uint32_t slot = atomicAdd(&ctrl[2], 1u);
+          if (slot < (uint32_t)kGenericSlots) {
+            gqueue[slot] = entry[i];
+            path[i] = 3u;  // placed
+          }
+        }
         const uint64_t mo = __ballot(path[i] == kPathOdd || path[i] == kPathGeneric), me = __ballot(path[i] == kPathEven);
         odd_rank[i] = n_o + __builtin_amdgcn_mbcnt_hi((uint32_t)(mo >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mo, 0));
         even_rank[i] = n_e + __builtin_amdgcn_mbcnt_hi((uint32_t)(me >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)me, 0));
@@ -385,17 +408,18 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 
     // P2: unrank and reduce.  Chunks of 64 queued blocks are handed out through a
     // counter: the generic chunk first (longest), then odd, then even.
-    const uint32_t n_odd = ctrl[0], n_even = ctrl[1];
-    const uint32_t c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
+    const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
+    const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
     for (;;) {
       uint32_t chunk = 0;
       if (lane == 0) chunk = atomicAdd(&ctrl[3], 1u);
       chunk = __shfl(chunk, 0, 64);
-      if (chunk >= c_odd + c_even) break;
-      if (chunk < c_odd) {
-        const uint32_t k = chunk * 64u + lane;
-        if (k < n_odd) {
-          const uint32_t entry = queue[k];
+      if (chunk >= c_gen + c_odd + c_even) break;
+      if (chunk < c_gen + c_odd) {
+        const bool from_gen = chunk < c_gen;
+        const uint32_t k = from_gen ? lane : (chunk - c_gen) * 64u + lane;
+        if (k < (from_gen ? n_gen : n_odd)) {
+          const uint32_t entry = from_gen ? gqueue[k] : queue[k];
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
           const uint64_t rec = read_record(raw, off + 6 * f);
           const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
@@ -428,7 +452,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
           }
         }
       } else {
-        const uint32_t k = (chunk - c_odd) * 64u + lane;
+        const uint32_t k = (chunk - c_gen - c_odd) * 64u + lane;
         if (k < n_even) {
           const uint32_t entry = queue[kTileBlocks - 1 - k];
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
@@ -780,7 +804,10 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   const size_t lds = gemv_lds_bytes(m0->nblocks);
   if (lds > 160 * 1024 || m0->nblocks > (uint32_t)kTileBlocks)
     return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": d_in " + std::to_string(m0->d_in) + " does not fit the LDS activation tile");
-  const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
+  // as many workgroups as fit a CU's 160 KB of LDS side by side
+  const uint32_t per_cu = (uint32_t)((160 * 1024) / lds) < 1u ? 1u : (uint32_t)((160 * 1024) / lds);
+  const uint32_t wg_per_cu = per_cu > (uint32_t)(2048 / kWgThreads) ? (uint32_t)(2048 / kWgThreads) : per_cu;
+  const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256) * wg_per_cu;
   GroupArgs a{};
   a.tables = rt->tables;
   a.x = reinterpret_cast<const __half*>(x);
@@ -854,7 +881,7 @@ int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks
   size_t grid = (nblocks + 255) / 256;
   const size_t cap = (size_t)(rt->cu_count > 0 ? rt->cu_count : 256) * 2;
   if (grid > cap) grid = cap;
-  hipLaunchKernelGGL(decode_blocks_kernel, dim3((uint32_t)grid), dim3(256), sizeof(TableImage), rt->stream,
+  hipLaunchKernelGGL(decode_blocks_kernel, dim3((uint32_t)grid), dim3(256), kLdsImageBytes, rt->stream,
                      rt->tables, codes_dev, nblocks, points_dev, gains_dev, shells_dev);
   HIP_TRY(hipGetLastError());
   return LLVQ_OK;
