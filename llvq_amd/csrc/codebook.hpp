@@ -103,9 +103,13 @@ struct Codebook {
   DevClass dev_classes[kClassSlots];
   uint64_t starts[kStartsPadded];         // starts[c] = offset of class c, starts[383] = N(13), then UINT64_MAX
   // lut[key]: low 9 bits = class holding zero-based index (key << kLutShift), clamped to 382;
-  // bits 9.. = k, where the class of any index of the bucket is at most 2^k - 1 classes further
+  // bits 9..11 = k, where the class of any index of the bucket is at most 2^k - 1 classes further;
+  // bits 12..13 = decoder path of that class (meaningful when k = 0)
   uint16_t lut[kLutSize];
   double rcp[32];                         // rcp[c] = 1/c, rcp[0] unused
+  // step[(m * 25 + c) * 2 + {0,1}] = {m / c, 1 - m / c}: the odd-coset walk's per-slot
+  // update t' + 1 = (t + 1 - lo) * (m / c) + (1 - m / c), m = slots left after this one
+  double step[24 * 25 * 2];
   uint64_t n12 = 0;                       // points in the cap-12 ball (47-bit field)
   // fast paths
   FastClass fast[kClassSlots];

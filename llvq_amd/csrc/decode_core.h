@@ -63,6 +63,7 @@ struct DecodeTables {
   const uint32_t* off_lut;  // even coset, off-support arrangements
   const uint32_t* expand;   // 8 dwords per codeword: deposit masks for the word and for its complement
   const uint8_t* pdep4;     // 4-bit deposit table
+  const double* step;       // {m/c, 1 - m/c} pairs, see Codebook::step
 };
 
 // Threshold packing: field f (bits 6f..6f+4) holds T_{4-f}; bit 6f+5 is the
@@ -78,6 +79,17 @@ LLVQ_HD uint32_t popc32(uint32_t v) {
   return (uint32_t)__popc(v);
 #else
   return (uint32_t)__builtin_popcount(v);
+#endif
+}
+
+// a * b + c with 24-bit signed factors (one full-rate instruction on the device)
+LLVQ_HD int mad24(int a, int b, int c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  int r;  // the compiler would widen this to a 64-bit multiply-add
+  asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(b), "v"(c));
+  return r;
+#else
+  return a * b + c;
 #endif
 }
 
@@ -112,7 +124,7 @@ LLVQ_HD uint32_t walk_step(double& rho, uint32_t& tg, uint32_t n, const double* 
 LLVQ_HD uint32_t find_class(const DecodeTables& T, uint64_t i) {
   const uint32_t e = T.lut[(uint32_t)(i >> kLutShift)];
   uint32_t ci = e & 511u;
-  for (uint32_t step = (1u << (e >> 9)) >> 1; step; step >>= 1)
+  for (uint32_t step = (1u << ((e >> 9) & 7u)) >> 1; step; step >>= 1)
     if (T.starts[ci + step] <= i) ci += step;
   return ci;
 }
@@ -121,23 +133,39 @@ LLVQ_HD uint32_t find_class(const DecodeTables& T, uint64_t i) {
 // local = g * m_arr + r_arr (index.rs:33-36).  Calls on_codes(q, sel) for q = 0..5:
 // byte j of sel is the table code of coordinate 4q + j,
 // code = (3 - kind) | (coordinate off the codeword's support ? 4 : 0).
+// The walk carries t + 1 = rho n + 1 instead of rho: floor(t + 1) is the operand
+// of the packed comparison, and the next slot's value is one fused multiply-add,
+// (t + 1 - T_j) (m / c_j) + (1 - m / c_j) with m = n - 1, both factors from one
+// 16-byte table entry.
 template <class OnCodes>
 LLVQ_HD void odd_codes(const DecodeTables& T, const FastClass& f, uint64_t li, OnCodes&& on_codes) {
   const double local = (double)li;
   const double g = floor64((local + 0.5) * f.inv0);
   const double r = fma64(-g, f.d1, local);
-  double rho = (r + 0.5) * f.inv0;
+  double t1 = fma64((r + 0.5) * f.inv0, 24.0, 1.0);
   const uint32_t ncw = ~T.golay[(uint32_t)g & 4095u];
   uint32_t tg = f.u0;
 #pragma unroll
   for (int q = 0; q < 6; ++q) {
-    uint32_t sel = (((ncw >> (4 * q)) & 15u) * kSpread2) & 0x04040404u;
+    uint32_t sel = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t jj = walk_step(rho, tg, (uint32_t)(kDim - 4 * q - j), T.rcp);
-      sel |= (jj - 1u) << (8 * j);
+      const uint32_t n = (uint32_t)(kDim - 4 * q - j);
+      const uint32_t ti1 = (uint32_t)t1;                      // floor(t) + 1
+      const uint32_t ltg = (uint32_t)mad24(-(int)ti1, (int)kFieldOnes, (int)tg) & kFieldGuard;  // guard survives iff T_m > floor(t)
+      const uint32_t jj = popc32(ltg);                        // 4 - kind
+      const uint32_t sh = jj * 6u;
+      const uint32_t lo = (tg >> sh) & 31u;
+      const uint32_t hi = (((tg << 6) | n) >> sh) & 31u;
+      tg -= ltg >> 5;
+      if (n > 1u) {
+        const double* e = T.step + 2u * ((n - 1u) * 25u + (hi - lo));
+        t1 = fma64(t1 - (double)lo, e[0], e[1]);
+      }
+      sel |= jj << (8 * j);
     }
-    on_codes(q, sel);
+    // table index = jj - 1 (kinds 0..3 <-> jj 4..1), bit 2 = off the codeword's support
+    on_codes(q, (sel - 0x01010101u) | ((((ncw >> (4 * q)) & 15u) * kSpread2) & 0x04040404u));
   }
 }
 

@@ -37,6 +37,7 @@ struct TableImage {
   uint64_t starts[kStartsLds];
   uint16_t lut[2048];        // a 47-bit field only reaches the lower half of the host table
   double rcp[32];
+  double step[24 * 25 * 2];
   uint8_t pdep4[256];
   uint32_t golay[4096];
   uint32_t on_lut[kOnLutSlots];
@@ -58,7 +59,7 @@ __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const Global
   for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) dst[i] = src[i];
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
   const TableImage* far = LLVQ_LDS_GOLAY ? s : g.image;
-  return DecodeTables{far->golay, g.cls, s->fast, s->starts, s->lut, s->rcp, far->on_lut, g.off_lut, g.expand, s->pdep4};
+  return DecodeTables{far->golay, g.cls, s->fast, s->starts, s->lut, s->rcp, far->on_lut, g.off_lut, g.expand, s->pdep4, s->step};
 }
 
 // 6-byte big-endian record at a 2-byte-aligned offset of a 4-byte-aligned buffer
@@ -349,7 +350,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
         if (zi[i] != ~0ULL) {
           const uint32_t e = T.lut[(uint32_t)(zi[i] >> kLutShift)];
           ci[i] = e & 511u;
-          kbits[i] = 1u << (e >> 9);
+          kbits[i] = 1u << ((e >> 9) & 7u);
           kmax = max(kmax, kbits[i]);
         }
       }
@@ -588,6 +589,7 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   std::memcpy(img->starts, cb.starts, sizeof img->starts);
   std::memcpy(img->lut, cb.lut, sizeof img->lut);
   std::memcpy(img->rcp, cb.rcp, sizeof img->rcp);
+  std::memcpy(img->step, cb.step, sizeof img->step);
   std::memcpy(img->pdep4, cb.pdep4, sizeof img->pdep4);
   std::memcpy(img->on_lut, cb.on_lut.data(), cb.on_lut.size() * 4);
   std::memcpy(host.data() + off_cls, cb.dev_classes, sizeof(cb.dev_classes));
