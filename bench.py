@@ -28,6 +28,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 
+# (6311.0 KiB fetched x 2.000 + 23.8 KiB written) per gemv_tiles_kernel launch on the default workload
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = round((6311.0 * 2.000 + 23.8) * 1024)
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -87,6 +91,9 @@ def main():
     ap.add_argument("--layers", type=int, default=36)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB device copy three times: the known-size kernel that "
+                         "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (rows shard trivially; see DESIGN.md). "
@@ -189,12 +196,20 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 5),
-            "traffic": None,
+            # L2-miss bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command,
+            # each scaled by its reading for a 256 MiB device copy (x2.000 and x1.000); profiles/ holds both
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (args.layers, args.seed) == (36, 0) else None,
             "avg_launch_us": round(avg_launch_us, 3),
             "launches_per_step": n_kernels,
             "algorithmic_bytes_per_launch": round(enc_bytes / n_kernels, 1),
         },
     }
+    if args.copy_probe:
+        src = torch.arange(1 << 26, dtype=torch.int32, device=dev)  # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
         out["cpu_baseline"] = cpu_baseline(layers[0], acts_np, threads)
