@@ -512,6 +512,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 
 }  // namespace llvq
 
+#include "gemm_kernel.h"
+
 // =================================================================================
 // C ABI
 // =================================================================================
@@ -523,6 +525,11 @@ struct llvq_rt {
   uint8_t* blob = nullptr;  // one device allocation holding every table
   GlobalTables tables{};
   int cu_count = 0;
+  // split-K state of the batched kernel: partial sums and per-band arrival counters
+  float* gemm_ws = nullptr;
+  size_t gemm_ws_bytes = 0;
+  uint32_t* gemm_counters = nullptr;
+  size_t gemm_counter_slots = 0;
 };
 
 struct llvq_mat {
@@ -607,6 +614,12 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   const int max_lds = 160 * 1024;
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<2, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<4, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<2, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<4, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   *out = rt;
   return LLVQ_OK;
 }
@@ -615,6 +628,8 @@ void llvq_hip_runtime_destroy(llvq_rt* rt) {
   if (!rt) return;
   (void)hipSetDevice(rt->device);
   (void)hipFree(rt->blob);
+  (void)hipFree(rt->gemm_ws);
+  (void)hipFree(rt->gemm_counters);
   delete rt;
 }
 
@@ -861,14 +876,103 @@ int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   return LLVQ_OK;
 }
 
+// Split of a matrix's block range over work units: the count that minimises a
+// coarse time model (rounds of units over the CUs x per-unit time), so that a
+// matrix with few 64-row bands still occupies the chip.
+static void pick_gemm_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint32_t grid, uint32_t* S_out,
+                            uint32_t* bps_out) {
+  double best = 1e30;
+  uint32_t best_s = 1, best_bps = nblocks ? nblocks : 1;
+  for (uint32_t S = 1; S <= 64 && S <= (nblocks ? nblocks : 1); ++S) {
+    const uint32_t bps = (nblocks + S - 1) / S;
+    if ((uint64_t)(S - 1) * bps >= nblocks && S > 1) continue;  // an empty last split
+    const uint32_t slices = (bps + kGemmKb - 1) / kGemmKb;
+    const double unit_us = slices * (1.0 + 0.008 * M) + 64.0 * bps * 0.0042 + (S > 1 ? 0.5 + 0.002 * M * S : 0.0);
+    const uint64_t units = (uint64_t)n_bands * S;
+    const double t = (double)((units + grid - 1) / grid) * unit_us;
+    if (t < best * 0.999) { best = t; best_s = S; best_bps = bps; }
+  }
+  *S_out = best_s;
+  *bps_out = best_bps;
+}
+
+static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M, void* y, int y_dtype) {
+  const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
+  GemmArgs a{};
+  a.tables = rt->tables;
+  a.x = reinterpret_cast<const __half*>(x);
+  a.codes = m->codes;
+  a.rscale = m->rscale;
+  a.tail = m->tail;
+  a.y = y;
+  a.g0 = m->g[0];
+  a.g1 = m->g[1];
+  a.M = M;
+  a.ldx = m->d_in;
+  a.d_out = m->d_out;
+  a.nblocks = m->nblocks;
+  a.tail_w = m->tail_w;
+  a.n_bands = (m->d_out + kGemmRows - 1) / kGemmRows;
+  pick_gemm_split(a.n_bands, m->nblocks, M, grid_cap, &a.S, &a.bps);
+  if (a.S > 1) {
+    const size_t need = (size_t)a.S * M * m->d_out * sizeof(float);
+    if (need > rt->gemm_ws_bytes) {
+      (void)hipFree(rt->gemm_ws);  // waits for launches that still use it
+      rt->gemm_ws = nullptr;
+      rt->gemm_ws_bytes = 0;
+      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_ws), need));
+      rt->gemm_ws_bytes = need;
+    }
+    if (a.n_bands > rt->gemm_counter_slots) {
+      (void)hipFree(rt->gemm_counters);
+      rt->gemm_counters = nullptr;
+      rt->gemm_counter_slots = 0;
+      const size_t slots = (size_t)a.n_bands + 1024;
+      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_counters), slots * sizeof(uint32_t)));
+      HIP_TRY(hipMemset(rt->gemm_counters, 0, slots * sizeof(uint32_t)));
+      rt->gemm_counter_slots = slots;
+    }
+    a.ws = rt->gemm_ws;
+    a.counters = rt->gemm_counters;
+  }
+  const uint32_t units = a.n_bands * a.S;
+  const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
+  const size_t lds = gemm_lds_bytes();
+  const bool f32 = y_dtype == LLVQ_F32;
+  if (M <= 128) {
+    if (f32) hipLaunchKernelGGL((gemm_tiles_kernel<1, float>), grid, wg, lds, rt->stream, a);
+    else hipLaunchKernelGGL((gemm_tiles_kernel<1, __half>), grid, wg, lds, rt->stream, a);
+  } else if (M <= 256) {
+    if (f32) hipLaunchKernelGGL((gemm_tiles_kernel<2, float>), grid, wg, lds, rt->stream, a);
+    else hipLaunchKernelGGL((gemm_tiles_kernel<2, __half>), grid, wg, lds, rt->stream, a);
+  } else {
+    if (f32) hipLaunchKernelGGL((gemm_tiles_kernel<4, float>), grid, wg, lds, rt->stream, a);
+    else hipLaunchKernelGGL((gemm_tiles_kernel<4, __half>), grid, wg, lds, rt->stream, a);
+  }
+  HIP_TRY(hipGetLastError());
+  return LLVQ_OK;
+}
+
 int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y, int y_dtype) {
   if (!rt || !m || !x || !y || M < 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: bad argument");
+  if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: unknown output dtype");
   HIP_TRY(hipSetDevice(rt->device));
   const size_t esz = y_dtype == LLVQ_F32 ? 4 : 2;
-  if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: unknown output dtype");
-  for (int r = 0; r < M; ++r) {
-    const int rc = launch_gemv(rt, m, reinterpret_cast<const uint8_t*>(x) + (size_t)r * m->d_in * 2,
-                               reinterpret_cast<uint8_t*>(y) + (size_t)r * m->d_out * esz, y_dtype);
+  const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
+  uint8_t* yb = reinterpret_cast<uint8_t*>(y);
+  // The matrix-core kernel reads activations as 16-byte vectors; a single row,
+  // or a shape that breaks that alignment, runs as GEMV launches instead.
+  const bool mfma_ok = M >= 2 && m->d_in % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && m->nblocks > 0;
+  if (!mfma_ok) {
+    for (int r = 0; r < M; ++r) {
+      const int rc = launch_gemv(rt, m, xb + (size_t)r * m->d_in * 2, yb + (size_t)r * m->d_out * esz, y_dtype);
+      if (rc) return rc;
+    }
+    return LLVQ_OK;
+  }
+  for (int m0 = 0; m0 < M; m0 += kGemmMaxM) {
+    const uint32_t mc = (uint32_t)(M - m0 < kGemmMaxM ? M - m0 : kGemmMaxM);
+    const int rc = launch_gemm(rt, m, xb + (size_t)m0 * m->d_in * 2, mc, yb + (size_t)m0 * m->d_out * esz, y_dtype);
     if (rc) return rc;
   }
   return LLVQ_OK;

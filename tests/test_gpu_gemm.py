@@ -1,0 +1,135 @@
+"""Parity of the batched matrix-core path (llvq_hip_gemm, M >= 2) against the
+CPU oracle: Y = X W^T with W the oracle's decoded matrix, in f64.
+
+Bar: |y - y_ref| / sum|w_i x_i| < 1e-3 and plain relative error < 1e-3 where
+|y_ref| is not tiny.  Weights enter the matrix cores as binary16 (one rounding
+of value * centroid / sqrt(16 shell)), accumulation is f32; row scale and tail
+columns are applied in f32.
+"""
+import numpy as np
+import pytest
+
+from llvq_amd import artifact, synth
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+
+
+def _x16(x):
+    import torch
+
+    return torch.from_numpy(x.view(np.int16).copy()).view(torch.float16).cuda()
+
+
+def _reference(orc, raw, X):
+    om, _ = orc.read_matrix_raw(artifact.write_matrix_raw(raw))
+    W = om.decode_matrix().astype(np.float64)  # [d_out, d_in], tail columns included
+    X = X.astype(np.float64)
+    return X @ W.T, np.abs(X) @ np.abs(W).T
+
+
+def _check(Y, Y_ref, A_ref, tol=TOL):
+    Y = Y.astype(np.float64)
+    e = np.abs(Y - Y_ref) / np.maximum(A_ref, 1e-30)
+    assert e.max() < tol, f"max |dy|/sum|wx| = {e.max():.3e}"
+    big = np.abs(Y_ref) > 1e-2 * A_ref
+    if big.any():
+        rel = (np.abs(Y - Y_ref)[big] / np.abs(Y_ref)[big]).max()
+        assert rel < 0.1, f"max relative error {rel:.3e}"  # |y| >= 1e-2 sum|wx| turns the bound above into this one
+    return e.max()
+
+
+# d_in must keep activation rows 16-byte aligned (d_in % 8 == 0) for the matrix-core path
+CASES = [
+    # d_out, d_in, M
+    (64, 480, 16),      # one band, one full K-slice, no tail
+    (72, 184, 16),      # ragged band (72 = 64 + 8), 7 blocks + 16 tail columns
+    (8, 2560, 2),       # tiny band, smallest batch
+    (128, 2568, 17),    # ragged batch, tail
+    (256, 4096, 64),    # 8B hidden size: 170 blocks + 16 tail
+    (192, 976, 130),    # two column tiles per wavefront
+    (64, 1000, 256),
+    (128, 4096, 512),   # four column tiles per wavefront
+    (64, 488, 600),     # more rows than one launch holds
+]
+
+
+@pytest.mark.parametrize("d_out,d_in,M", CASES)
+def test_gemm_shapes(gpu_rt, orc, d_out, d_in, M):
+    import torch
+
+    raw = synth.make_matrix(f"model.layers.0.gemm.{d_out}x{d_in}.weight", d_out, d_in, seed=7 * d_out + d_in)
+    X = synth.make_activation(d_in, seed=M, rows=M)
+    Y_ref, A_ref = _reference(orc, raw, X)
+    proj = gpu_rt.upload(raw)
+    try:
+        Y32 = gpu_rt.forward_batched(proj, _x16(X), out_dtype=torch.float32).cpu().numpy()
+        Y16 = gpu_rt.forward_batched(proj, _x16(X)).cpu().numpy()
+        again = gpu_rt.forward_batched(proj, _x16(X), out_dtype=torch.float32).cpu().numpy()
+    finally:
+        gpu_rt.free(proj)
+    e = _check(Y32, Y_ref, A_ref)
+    assert e < 2e-4  # observed level of the binary16 weight rounding
+    _check(Y16.astype(np.float32), Y_ref, A_ref)
+    assert np.array_equal(Y32, again)  # fixed summation order, split or not
+
+
+def test_gemm_origin_shell13_and_generic_blocks(gpu_rt, orc, boundary_indices):
+    """Origins, shell-13 indices above N(12) and the class boundaries (which
+    include every class that takes the generic walk)."""
+    import torch
+
+    d_out, nb, tw = 64, 40, 8
+    d_in = 24 * nb + tw
+    rng = synth.SplitMix64(2024)
+    idx = rng.take(d_out * nb) % np.uint64(1 << 47)
+    b = boundary_indices[boundary_indices < (1 << 47)]
+    idx[: b.size] = b[: idx.size]
+    idx[::5] = 0
+    idx[1::11] = np.uint64((1 << 47) - 1)
+    gains = (rng.take(idx.size) & np.uint64(1)).astype(np.uint8)
+    raw = artifact.RawMatrix("model.layers.0.edge.weight", d_out, d_in, 12, [0.8, 1.25],
+                             np.exp(rng.gaussian(d_out)), rng.gaussian(d_out * tw).astype(np.float32),
+                             artifact.pack_codes(idx, gains))
+    X = synth.make_activation(d_in, seed=77, rows=32)
+    Y_ref, A_ref = _reference(orc, raw, X)
+    proj = gpu_rt.upload(raw)
+    Y = gpu_rt.forward_batched(proj, _x16(X), out_dtype=torch.float32).cpu().numpy()
+    gpu_rt.free(proj)
+    _check(Y, Y_ref, A_ref)
+
+
+def test_gemm_matches_gemv_rows(gpu_rt):
+    """The batched kernel against the single-row kernel of the same library."""
+    import torch
+
+    raw = synth.make_matrix("model.layers.3.self_attn.k_proj.weight", 1024, 4096, seed=3)
+    X = synth.make_activation(4096, seed=5, rows=16)
+    proj = gpu_rt.upload(raw)
+    Xd = _x16(X)
+    Y = gpu_rt.forward_batched(proj, Xd, out_dtype=torch.float32)
+    rows = torch.stack([gpu_rt.forward(proj, Xd[r], out_dtype=torch.float32).reshape(-1) for r in range(16)])
+    gpu_rt.free(proj)
+    scale = rows.abs().max().item()
+    assert (Y - rows).abs().max().item() < 2e-3 * scale
+
+
+@pytest.mark.parametrize("site,d_out,d_in,M", [
+    ("self_attn.k_proj", 1024, 4096, 64),     # few bands: the block range is split over units
+    ("mlp.down_proj", 4096, 12288, 16),
+    ("mlp.gate_proj", 12288, 4096, 256),
+])
+def test_gemm_qwen3_8b_shapes(gpu_rt, orc, site, d_out, d_in, M):
+    """BASELINE config 3 shapes; checked on a sample of activation rows to keep the f64 reference short."""
+    import torch
+
+    raw = synth.make_matrix(f"model.layers.0.{site}.weight", d_out, d_in, seed=8)
+    X = synth.make_activation(d_in, seed=M + 1, rows=M)
+    proj = gpu_rt.upload(raw)
+    Y = gpu_rt.forward_batched(proj, _x16(X), out_dtype=torch.float32).cpu().numpy()
+    gpu_rt.free(proj)
+    pick = sorted({0, 1, M // 2, M - 1})
+    Y_ref, A_ref = _reference(orc, raw, X[pick])
+    _check(Y[pick], Y_ref, A_ref)
+    assert np.isfinite(Y).all()
