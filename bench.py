@@ -83,6 +83,102 @@ def cpu_baseline(layer_mats, acts, threads):
     }
 
 
+QWEN3_8B_LAYER = [  # (site, d_out, d_in): hidden 4096, intermediate 12288, 32 query / 8 KV heads of 128
+    ("self_attn.q_proj", 4096, 4096),
+    ("self_attn.k_proj", 1024, 4096),
+    ("self_attn.v_proj", 1024, 4096),
+    ("self_attn.o_proj", 4096, 4096),
+    ("mlp.gate_proj", 12288, 4096),
+    ("mlp.up_proj", 12288, 4096),
+    ("mlp.down_proj", 4096, 12288),
+]
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def bench_gemm(args, torch, llvq_amd, synth, dev):
+    """Batched dequant-GEMM: the seven projections of `--layers` (default 4 here) Qwen3-8B-shaped
+    layers against M activation rows.  A step is one pass over all of them."""
+    n_layers = min(args.layers, 4)
+    M = args.M
+    rt = llvq_amd.FusedRuntime(device=0)
+    mats = [synth.layer_matrices(layer, args.seed, QWEN3_8B_LAYER) for layer in range(n_layers)]
+    projs = [[rt.upload(m) for m in layer] for layer in mats]
+    X = {d: torch.from_numpy(synth.make_activation(d, args.seed, rows=M).view(np.int16).copy()).view(torch.float16).to(dev)
+         for d in (4096, 12288)}
+    Y = {p.name: torch.empty((M, p.d_out), dtype=torch.float16, device=dev) for lp in projs for p in lp}
+    flops = sum(2.0 * M * p.d_out * p.d_in for lp in projs for p in lp)
+    enc_bytes = sum(m.encoded_bytes() for layer in mats for m in layer)
+    n_blocks = sum(m.codes.size for layer in mats for m in layer) // 6
+
+    def step():
+        for lp in projs:
+            for p in lp:
+                rt.forward_batched_into(p, X[p.d_in], Y[p.name])
+
+    per_shape = {}
+    for p in projs[0]:
+        for _ in range(2):
+            rt.forward_batched_into(p, X[p.d_in], Y[p.name])
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            rt.forward_batched_into(p, X[p.d_in], Y[p.name])
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / 5
+        per_shape[f"{p.d_out}x{p.d_in}"] = {"us": round(us, 1),
+                                            "TFLOPs": round(2.0 * M * p.d_out * p.d_in / us / 1e6, 1)}
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_s = ev0.elapsed_time(ev1) * 1e-3
+    tflops = flops * args.steps / wall / 1e12
+    n_launch = n_layers * 7
+    out = {
+        "metric": "dequant_gemm_TFLOPs",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3 / args.steps, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"Qwen3-8B decoder-layer projections (BASELINE config 3 shapes), {n_layers} distinct "
+                               f"layers = {n_launch} LLVQ matrices, M = {M} activation rows, f16 in / f16 out",
+                   "layers": n_layers, "M": M, "seed": args.seed},
+        "encoded_weight_GBps": round(enc_bytes * args.steps / wall / 1e9, 2),
+        "blocks_per_s": round(n_blocks * args.steps / wall, 1),
+        "per_shape": per_shape,
+        "roofline": {
+            "kernel": "gemm_tiles_kernel",
+            "bound": "mfma",
+            "achieved": round(flops * args.steps / dev_s / 1e12, 2),
+            "peak": MFMA_F16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(flops * args.steps / dev_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 5),
+            "traffic": None,
+            "avg_launch_us": round(dev_s * 1e6 / (args.steps * n_launch), 2),
+            "launches_per_step": n_launch,
+            "algorithmic_flops_per_launch": round(flops / n_launch, 1),
+        },
+    }
+    rt.close()
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -91,6 +187,10 @@ def main():
     ap.add_argument("--layers", type=int, default=36)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--workload", choices=["gemv", "gemm"], default="gemv",
+                    help="gemv: the headline batch-1 projection pass (default); gemm: the batched "
+                         "matrix-core path at Qwen3-8B shapes")
+    ap.add_argument("--M", type=int, default=256, help="activation rows of the gemm workload")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy three times: the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
@@ -109,6 +209,8 @@ def main():
         log("bench.py needs a GPU (there is no CPU fallback for the product path)")
         sys.exit(1)
     dev = torch.device("cuda", 0)
+    if args.workload == "gemm":
+        return bench_gemm(args, torch, llvq_amd, synth, dev)
     layers = build_layers(args.layers, args.seed)
     acts_np = {d: synth.make_activation(d, args.seed)[0] for d in (2560, 4096, 9728)}
     acts = {d: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16).to(dev) for d, a in acts_np.items()}

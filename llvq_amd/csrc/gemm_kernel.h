@@ -15,10 +15,12 @@
 //   P1  classify and bin the blocks (odd / even / generic queues);
 //   P2  unrank; every block writes its 24 weights, already multiplied by
 //       centroid[gain] / sqrt(16 shell), as binary16 into the W slice in LDS;
-//   P3  16 wavefronts run v_mfma_f32_16x16x32_f16 over the slice: A fragments
-//       from LDS, B fragments (activations) straight from global memory / L2;
-//       the wavefront grid is 2 row groups x 8 column groups and accumulators
-//       (<= 32 registers) stay live across slices.
+//   P3  16 wavefronts run v_mfma_f32_32x32x16_f16 over the slice: A fragments
+//       from LDS, B fragments (activations) straight from global memory / L2,
+//       fetched one batch ahead.  Up to 256 activation rows the wavefront grid
+//       is 2 row tiles x 8 column tiles of 32; beyond, every wavefront takes
+//       both row tiles of one of 16 column tiles.  Accumulators (16 or 32
+//       registers) stay live across slices.
 // Epilogue: row scale and the f32 tail columns in f32, then the store.  When a
 // matrix has too few bands to occupy the chip its block range is split over
 // several units; each writes its partial sums to a workspace and the unit that
@@ -29,13 +31,16 @@
 namespace llvq {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kGemmRows = 64;                 // weight rows of a band
-constexpr int kGemmKb = 20;                   // blocks per row and K-slice: 480 columns = 15 MFMA k-steps
-constexpr int kGemmTile = kGemmRows * kGemmKb;  // 1280 blocks per K-slice
+#ifndef LLVQ_GEMM_KB
+#define LLVQ_GEMM_KB 20
+#endif
+constexpr int kGemmKb = LLVQ_GEMM_KB;         // blocks per row and K-slice (20: 480 columns = 15 K-steps of 32)
+constexpr int kGemmTile = kGemmRows * kGemmKb;  // blocks per K-slice
 constexpr int kGemmP1Blocks = (kGemmTile + kWgThreads - 1) / kWgThreads;
-constexpr int kGemmRowChunks = 9;             // 16-byte units holding one row's <= 120 code bytes at any even alignment
+constexpr int kGemmRowChunks = (kGemmKb * 6 + 14 + 15) / 16;  // 16-byte units holding one row's code bytes at any even alignment
 constexpr int kGemmRowBytes = kGemmRowChunks * 16;
 constexpr int kGemmWStride = kGemmKb * 24 + 8;  // binary16 elements per W row in LDS; the pad spreads rows over banks
 constexpr int kGemmMaxM = 512;                // activation rows per launch (32 column tiles of 16)
@@ -87,8 +92,17 @@ __device__ __forceinline__ void store_y<__half>(void* y, size_t at, float v) {
   reinterpret_cast<__half*>(y)[at] = __float2half_rn(v);
 }
 
-// CT = column tiles (16 activation rows each) per wavefront: M <= 128 CT.
-template <int CT, typename OutT>
+// RT = 32-row tiles per wavefront: 1 for M <= 256 (grid 2 x 8), 2 for M <= 512 (grid 1 x 16).
+#ifdef LLVQ_PHASE_TIMING
+#define LLVQ_GSTAMP(k)                                                                                  \
+  do {                                                                                                  \
+    if (threadIdx.x == 0 && unit == blockIdx.x && si == 0) g_phase_stamps[blockIdx.x * 8 + (k)] = wall_clock64(); \
+  } while (0)
+#else
+#define LLVQ_GSTAMP(k) do {} while (0)
+#endif
+
+template <int RT, typename OutT>
 __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
   const DecodeTables T = stage_tables(smem, a.tables);
@@ -100,14 +114,11 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t nb = a.nblocks;
   const uint32_t n_units = a.n_bands * a.S;
-  // stale W contents are multiplied by zero activations in a slice's padding
-  // columns, so they must be finite from the start
-  for (uint32_t i = tid; i < (uint32_t)(kGemmRows * kGemmWStride / 8); i += kWgThreads)
-    reinterpret_cast<uint4*>(W)[i] = make_uint4(0, 0, 0, 0);
 
-  // wavefront grid of the MFMA phase
-  const uint32_t rg = wave & 1u, cg = wave >> 1;  // row group (32 rows), column group
-  const uint32_t l16 = lane & 15u, lq = lane >> 4;
+  // wavefront grid of the MFMA phase: first 32-row tile and 32-column tile of this wavefront
+  const uint32_t rt0 = RT == 2 ? 0u : (wave & 1u), ctile = RT == 2 ? wave : (wave >> 1);
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  const uint32_t my_m = ctile * 32u + l32;  // the activation row this lane feeds and receives
 
   // code bytes of (unit, slice) -> one register per lane
   auto prefetch = [&](uint32_t r0, uint32_t rows, uint32_t k0, uint32_t kb, uint4& pre) {
@@ -120,27 +131,38 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     }
   };
 
+#ifdef LLVQ_PHASE_TIMING
+  if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 7] = wall_clock64();
+#endif
   for (uint32_t unit = blockIdx.x; unit < n_units; unit += gridDim.x) {
     const uint32_t band = unit / a.S, split = unit - band * a.S;
     const uint32_t r0 = band * kGemmRows, rows = min((uint32_t)kGemmRows, a.d_out - r0);
     const uint32_t kb_lo = min(nb, split * a.bps), kb_hi = min(nb, kb_lo + a.bps);
-    float4_t acc[2][CT];
+    float16_t acc[RT];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < 16; ++j) acc[rt][j] = 0.f;
 
     uint4 pre = make_uint4(0, 0, 0, 0);
-    prefetch(r0, rows, kb_lo, min((uint32_t)kGemmKb, kb_hi - kb_lo), pre);
-    for (uint32_t k0 = kb_lo; k0 < kb_hi; k0 += kGemmKb) {
+    // Units walk their slices from different starting points (a fixed function of
+    // the band), so that the CUs do not all pull the same activation columns
+    // through the same L2 channels at the same time.
+    const uint32_t n_slices = (kb_hi - kb_lo + kGemmKb - 1) / kGemmKb;
+    uint32_t sj = n_slices ? (band * 5u) % n_slices : 0u;
+    if (n_slices) prefetch(r0, rows, kb_lo + sj * kGemmKb, min((uint32_t)kGemmKb, kb_hi - (kb_lo + sj * kGemmKb)), pre);
+    for (uint32_t si = 0; si < n_slices; ++si) {
+      const uint32_t k0 = kb_lo + sj * kGemmKb;
       const uint32_t kb = min((uint32_t)kGemmKb, kb_hi - k0);
+      sj = sj + 1 == n_slices ? 0u : sj + 1;
       const uint32_t nblk = rows * kb;
       const uint32_t inv_kb = (65536u + kb - 1u) / kb;  // floor(f / kb) = (f * inv_kb) >> 16 for f < 1536, kb <= 24
       // P0
       if (tid < 4) ctrl[tid] = 0;
       if (tid < (uint32_t)(kGemmRows * kGemmRowChunks)) reinterpret_cast<uint4*>(raw)[tid] = pre;
       __syncthreads();
-      if (k0 + kGemmKb < kb_hi) prefetch(r0, rows, k0 + kGemmKb, min((uint32_t)kGemmKb, kb_hi - k0 - kGemmKb), pre);
+      LLVQ_GSTAMP(0);
+      if (si + 1 < n_slices) prefetch(r0, rows, kb_lo + sj * kGemmKb, min((uint32_t)kGemmKb, kb_hi - (kb_lo + sj * kGemmKb)), pre);
 
       auto record_at = [&](uint32_t row, uint32_t b) -> uint64_t {
         const uint32_t off = ((((r0 + row) * nb + k0) & 7u) * 6u) & 15u;  // (6 n) mod 16 depends on n mod 8 only
@@ -215,6 +237,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         }
       }
       __syncthreads();
+      LLVQ_GSTAMP(1);
 
       // P2: unrank into the W slice
       const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
@@ -264,102 +287,171 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         }
         }
       }
+      LLVQ_GSTAMP(2);
       __syncthreads();
+      LLVQ_GSTAMP(3);
 
-      // P3: acc += W_slice (64 x 24 kb) * X^T (24 kb x M); k runs in steps of 32,
-      // the columns of a last partial step are zero on the activation side
-      if (cg * 16u < a.M) {  // column groups beyond the batch have nothing to add
-        const uint32_t kcols = kb * 24u, ksteps = (kcols + 31u) >> 5;
-        const __half* xk = a.x + (size_t)k0 * 24u;
-        constexpr int D = 8 / CT;  // k-steps whose B fragments are fetched together
-        const _Float16* arow0 = W + (size_t)(rg * 32u + l16) * kGemmWStride + lq * 8u;
-        for (uint32_t ks0 = 0; ks0 < ksteps; ks0 += D) {
-          half8_t bf[D][CT];
+      // P3: acc += W_slice (64 x 24 kb) * X^T (24 kb x M).  K runs in steps of 32
+      // (two MFMAs of 16): lane (l32, lh) holds columns [32 p + 16 lh, +16) of its
+      // row as two fragments, for W and X alike, so an activation row is read in
+      // 64-byte runs.  Columns past the slice are zeroed on both sides.
+      if (ctile * 32u < a.M) {  // column tiles beyond the batch have nothing to add
+        const uint32_t kcols = kb * 24u, psteps = (kcols + 31u) >> 5;
+        const __half* xrow = a.x + (size_t)k0 * 24u + (size_t)min(my_m, a.M - 1u) * a.ldx + lh * 16u;
+        const bool m_ok = my_m < a.M;
+        const _Float16* arow = W + (size_t)(rt0 * 32u + l32) * kGemmWStride + lh * 16u;
+        constexpr int G = 2;  // K-steps per batch of activation loads
+        const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+        half8_t cur[G][2], nxt[G][2];
+        auto fetch = [&](uint32_t p0, half8_t (&dst)[G][2]) {
 #pragma unroll
-          for (int d = 0; d < D; ++d) {
-            const uint32_t kc = (ks0 + d) * 32u + lq * 8u;
+          for (int g = 0; g < G; ++g)
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) {
-              const uint32_t m = (cg + 8u * ct) * 16u + l16;
-              half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-              if (kc < kcols && m < a.M) v = *reinterpret_cast<const half8_t*>(xk + (size_t)m * a.ldx + kc);
-              bf[d][ct] = v;
+            for (int f = 0; f < 2; ++f) {
+              const uint32_t kc = (p0 + g) * 32u + lh * 16u + f * 8u;
+              dst[g][f] = (m_ok && kc < kcols) ? *reinterpret_cast<const half8_t*>(xrow + (p0 + g) * 32u + f * 8u) : zero;
             }
-          }
+        };
+        fetch(0, cur);
+        for (uint32_t p0 = 0; p0 < psteps; p0 += G) {
+          if (p0 + G < psteps) fetch(p0 + G, nxt);
 #pragma unroll
-          for (int d = 0; d < D; ++d) {
-            if (ks0 + d < ksteps) {
-              const half8_t a0 = *reinterpret_cast<const half8_t*>(arow0 + (ks0 + d) * 32u);
-              const half8_t a1 = *reinterpret_cast<const half8_t*>(arow0 + 16 * kGemmWStride + (ks0 + d) * 32u);
+          for (int g = 0; g < G; ++g) {
+            if (p0 + g < psteps) {
 #pragma unroll
-              for (int ct = 0; ct < CT; ++ct) {
-                acc[0][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bf[d][ct], acc[0][ct], 0, 0, 0);
-                acc[1][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bf[d][ct], acc[1][ct], 0, 0, 0);
+              for (int f = 0; f < 2; ++f) {
+                const bool kin = (p0 + g) * 32u + lh * 16u + f * 8u < kcols;
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                  const half8_t av = kin ? *reinterpret_cast<const half8_t*>(arow + (size_t)rt * 32 * kGemmWStride + (p0 + g) * 32u + f * 8u) : zero;
+                  acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, cur[g][f], acc[rt], 0, 0, 0);
+                }
               }
             }
           }
+#pragma unroll
+          for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int f = 0; f < 2; ++f) cur[g][f] = nxt[g][f];
         }
       }
+      LLVQ_GSTAMP(4);
       // no barrier here: the next slice's P0/P1 touch only raw, queues and
       // counters, and its P2 starts behind two barriers every wavefront reaches
       // after leaving P3
     }
 
     // ---- epilogue ----
-    // acc[rt][ct][i] belongs to weight row r0 + rg*32 + rt*16 + lq*4 + i and activation row (cg + 8 ct)*16 + l16
+    // acc[rt][j] belongs to weight row r0 + (rt0 + rt)*32 + 8 (j/4) + 4 lh + j%4 and activation row my_m.
+    // The tail columns (f32 weights, kept out of the binary16 contraction) are
+    // staged in the W area: tl[row][t] as f32 and xt[m][t] as binary16.
     const uint32_t tw = a.tail_w;
-    const __half* xtail = a.x + (size_t)nb * 24u;
-    if (a.S == 1) {
+    float* tl = reinterpret_cast<float*>(W);
+    __half* xt = reinterpret_cast<__half*>(tl + kGemmRows * (kDim - 1));
+    static_assert((size_t)(2 * kGemmRows + kGemmMaxM) * (kDim - 1) * 2 <= (size_t)kGemmRows * kGemmWStride * 2,
+                  "tail staging fits the W area");
+    auto stage_tail = [&]() {  // call with every wavefront past its last read of W
+      for (uint32_t o = tid; o < rows * tw; o += kWgThreads) tl[o] = a.tail[(size_t)r0 * tw + o];
+      const __half* xtail = a.x + (size_t)nb * 24u;
+      for (uint32_t o = tid; o < a.M * tw; o += kWgThreads) {
+        const uint32_t m = o / tw, t = o - m * tw;
+        xt[o] = xtail[(size_t)m * a.ldx + t];
+      }
+    };
+    const bool m_ok = my_m < a.M;
+    const bool vec_ok = (a.d_out & 3u) == 0;  // four consecutive rows of one activation row store as one vector
+    bool reduce_here = false;
+    if (a.S > 1) {
+      if (m_ok) {
+        float* dst = a.ws + ((size_t)split * a.M + my_m) * a.d_out + r0;
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-          const uint32_t m = (cg + 8u * ct) * 16u + l16;
+          for (int j4 = 0; j4 < 4; ++j4) {
+            const uint32_t row = (rt0 + rt) * 32u + 8u * j4 + 4u * lh;
+            if (vec_ok && row + 3 < rows) {
+              *reinterpret_cast<float4*>(dst + row) =
+                  make_float4(acc[rt][4 * j4], acc[rt][4 * j4 + 1], acc[rt][4 * j4 + 2], acc[rt][4 * j4 + 3]);
+            } else {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const uint32_t row = rg * 32u + rt * 16u + lq * 4u + i;
-            if (row < rows && m < a.M) {
-              float v = acc[rt][ct][i] * a.rscale[r0 + row];
-              for (uint32_t t = 0; t < tw; ++t)
-                v = fmaf(a.tail[(size_t)(r0 + row) * tw + t], __half2float(xtail[(size_t)m * a.ldx + t]), v);
-              store_y<OutT>(a.y, (size_t)m * a.d_out + r0 + row, v);
+              for (int i = 0; i < 4; ++i)
+                if (row + i < rows) dst[row + i] = acc[rt][4 * j4 + i];
             }
           }
-        }
-    } else {
-#pragma unroll
-      for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-          const uint32_t m = (cg + 8u * ct) * 16u + l16;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const uint32_t row = rg * 32u + rt * 16u + lq * 4u + i;
-            if (row < rows && m < a.M) a.ws[((size_t)split * a.M + m) * a.d_out + r0 + row] = acc[rt][ct][i];
-          }
-        }
-      // the unit that arrives last at the band's counter adds the partial sums
-      __threadfence();
-      __syncthreads();
-      if (tid == 0) ctrl[0] = __hip_atomic_fetch_add(&a.counters[band], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-      __syncthreads();
-      const bool last = ctrl[0] == a.S - 1;
-      __syncthreads();  // ctrl[0] is rewritten by the next unit's first slice
-      if (last) {
-        __threadfence();
-        for (uint32_t o = tid; o < rows * a.M; o += kWgThreads) {
-          const uint32_t m = o / rows, row = o - m * rows;
-          float s = 0.f;
-          for (uint32_t sp = 0; sp < a.S; ++sp)
-            s += a.ws[((size_t)sp * a.M + m) * a.d_out + r0 + row];
-          float v = s * a.rscale[r0 + row];
-          for (uint32_t t = 0; t < tw; ++t)
-            v = fmaf(a.tail[(size_t)(r0 + row) * tw + t], __half2float(xtail[(size_t)m * a.ldx + t]), v);
-          store_y<OutT>(a.y, (size_t)m * a.d_out + r0 + row, v);
-        }
-        if (tid == 0) a.counters[band] = 0;  // ready for the next launch
       }
+      // The unit that arrives last at the band's counter adds the partial sums.
+      // One lane publishes for the workgroup: the barrier orders every lane's
+      // stores before its device-scope release, and its acquire after the
+      // counter read orders the other units' stores before this workgroup's loads.
+      __syncthreads();
+      if (tid == 0) {
+        const uint32_t seen = __hip_atomic_fetch_add(&a.counters[band], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        ctrl[0] = seen;
+      }
+      __syncthreads();
+      reduce_here = ctrl[0] == a.S - 1;
+    } else {
+      __syncthreads();  // W is about to hold the tail staging
     }
+    if (a.S == 1 || reduce_here) {
+      if (tw) stage_tail();
+      __syncthreads();
+    }
+    if (a.S == 1) {
+      if (m_ok) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int j4 = 0; j4 < 4; ++j4) {
+            const uint32_t row = (rt0 + rt) * 32u + 8u * j4 + 4u * lh;
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const uint32_t r = min(row + i, rows - 1u);
+              float ts = 0.f;
+              for (uint32_t t = 0; t < tw; ++t) ts = fmaf(tl[r * tw + t], __half2float(xt[my_m * tw + t]), ts);
+              v[i] = fmaf(acc[rt][4 * j4 + i], a.rscale[r0 + r], ts);
+            }
+            const size_t at = (size_t)my_m * a.d_out + r0 + row;
+            if (vec_ok && row + 3 < rows) {
+              if constexpr (sizeof(OutT) == 4) {
+                *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
+              } else {
+                const __half2 lo = __float22half2_rn(make_float2(v[0], v[1])), hi = __float22half2_rn(make_float2(v[2], v[3]));
+                uint2 pk;
+                pk.x = *reinterpret_cast<const uint32_t*>(&lo);
+                pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+                *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(a.y) + at) = pk;
+              }
+            } else {
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (row + i < rows) store_y<OutT>(a.y, at + i, v[i]);
+            }
+          }
+      }
+    } else if (reduce_here) {
+      for (uint32_t o = tid; o < rows * a.M; o += kWgThreads) {
+        const uint32_t m = o / rows, row = o - m * rows;
+        const float* src = a.ws + (size_t)m * a.d_out + r0 + row;
+        const size_t sstride = (size_t)a.M * a.d_out;
+        float sum = 0.f;
+        uint32_t sp = 0;
+        for (; sp + 4 <= a.S; sp += 4) {  // four loads in flight, added in split order
+          const float p0 = src[(size_t)sp * sstride], p1 = src[(size_t)(sp + 1) * sstride];
+          const float p2 = src[(size_t)(sp + 2) * sstride], p3 = src[(size_t)(sp + 3) * sstride];
+          sum = (((sum + p0) + p1) + p2) + p3;
+        }
+        for (; sp < a.S; ++sp) sum += src[(size_t)sp * sstride];
+        float ts = 0.f;
+        for (uint32_t t = 0; t < tw; ++t) ts = fmaf(tl[row * tw + t], __half2float(xt[m * tw + t]), ts);
+        store_y<OutT>(a.y, (size_t)m * a.d_out + r0 + row, fmaf(sum, a.rscale[r0 + row], ts));
+      }
+      if (tid == 0) a.counters[band] = 0;  // ready for the next launch
+    }
+#ifdef LLVQ_PHASE_TIMING
+    if (threadIdx.x == 0 && unit == blockIdx.x) g_phase_stamps[blockIdx.x * 8 + 5] = wall_clock64();
+#endif
     __syncthreads();  // W, raw and counters are reused by the next unit
   }
 }

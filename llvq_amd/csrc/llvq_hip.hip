@@ -616,10 +616,8 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<2, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<4, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<2, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<4, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   *out = rt;
   return LLVQ_OK;
 }
@@ -887,7 +885,7 @@ static void pick_gemm_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint
     const uint32_t bps = (nblocks + S - 1) / S;
     if ((uint64_t)(S - 1) * bps >= nblocks && S > 1) continue;  // an empty last split
     const uint32_t slices = (bps + kGemmKb - 1) / kGemmKb;
-    const double unit_us = slices * (1.0 + 0.008 * M) + 64.0 * bps * 0.0042 + (S > 1 ? 0.5 + 0.002 * M * S : 0.0);
+    const double unit_us = 2.0 + slices * (5.0 + 0.018 * M) + 64.0 * bps * 0.0042 + 0.015 * M + (S > 1 ? 0.5 + 0.01 * M * S : 0.0);
     const uint64_t units = (uint64_t)n_bands * S;
     const double t = (double)((units + grid - 1) / grid) * unit_us;
     if (t < best * 0.999) { best = t; best_s = S; best_bps = bps; }
@@ -939,15 +937,12 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
   const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
   const size_t lds = gemm_lds_bytes();
   const bool f32 = y_dtype == LLVQ_F32;
-  if (M <= 128) {
+  if (M <= 256) {
     if (f32) hipLaunchKernelGGL((gemm_tiles_kernel<1, float>), grid, wg, lds, rt->stream, a);
     else hipLaunchKernelGGL((gemm_tiles_kernel<1, __half>), grid, wg, lds, rt->stream, a);
-  } else if (M <= 256) {
+  } else {
     if (f32) hipLaunchKernelGGL((gemm_tiles_kernel<2, float>), grid, wg, lds, rt->stream, a);
     else hipLaunchKernelGGL((gemm_tiles_kernel<2, __half>), grid, wg, lds, rt->stream, a);
-  } else {
-    if (f32) hipLaunchKernelGGL((gemm_tiles_kernel<4, float>), grid, wg, lds, rt->stream, a);
-    else hipLaunchKernelGGL((gemm_tiles_kernel<4, __half>), grid, wg, lds, rt->stream, a);
   }
   HIP_TRY(hipGetLastError());
   return LLVQ_OK;

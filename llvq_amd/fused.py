@@ -208,6 +208,17 @@ class FusedRuntime:
         _ffi.check(_ffi.lib().llvq_hip_gemm(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
         return y
 
+    def forward_batched_into(self, proj: FusedProj, x, y):
+        """`forward_batched` into a caller-owned [M, d_out] f16/f32 tensor (no allocation per call)."""
+        torch = self._torch
+        if x.dtype != torch.float16 or not x.is_contiguous() or x.shape[1] != proj.d_in:
+            raise ValueError(f"{proj.name} expects a contiguous f16 [M, {proj.d_in}] activation")
+        if tuple(y.shape) != (x.shape[0], proj.d_out) or not y.is_contiguous():
+            raise ValueError(f"{proj.name}: output must be contiguous [M, {proj.d_out}]")
+        code = _ffi.F16 if y.dtype == torch.float16 else _ffi.F32
+        _ffi.check(_ffi.lib().llvq_hip_gemm(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
+        return y
+
     def decode_blocks(self, codes):
         """Parity probe: packed 6-byte records (uint8 tensor on the device) →
         (points int8 [n,24], gains uint8 [n], shells uint8 [n])."""
