@@ -135,6 +135,42 @@ int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, int M, 
 int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks,
                            int8_t* points_dev, uint8_t* gains_dev, uint8_t* shells_dev);
 
+/* ---- batch-1 decode loop ---------------------------------------------------
+ * Replaces Qwen3 / Block at l = 1 (llvq-llm/src/model.rs:589-623, :839-862):
+ * a Qwen3-architecture decoder whose projections are uploaded LLVQ matrices and
+ * whose other tensors are dense binary16.  Host pointers; everything is copied. */
+typedef struct llvq_decoder llvq_decoder;
+typedef struct llvq_decoder_desc {
+  uint32_t n_layers, hidden, n_heads, n_kv_heads, head_dim, intermediate, vocab;
+  uint32_t max_positions;               /* KV-cache length, <= 8192 */
+  double rope_theta, rms_eps;
+  const llvq_mat* const* projections;   /* [n_layers * 7]: q, k, v, o, gate, up, down per layer */
+  const uint16_t* input_norm;           /* [n_layers, hidden]   binary16 bit patterns */
+  const uint16_t* post_norm;            /* [n_layers, hidden] */
+  const uint16_t* q_norm;               /* [n_layers, head_dim] */
+  const uint16_t* k_norm;               /* [n_layers, head_dim] */
+  const uint16_t* final_norm;           /* [hidden] */
+  const uint16_t* embed;                /* [vocab, hidden] */
+  const uint16_t* lm_head;              /* [vocab, hidden]; NULL = tied to embed */
+} llvq_decoder_desc;
+/* Qwen3::new_with (model.rs:869): checks every projection's shape against the architecture. */
+int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* desc, llvq_decoder** out);
+void llvq_hip_decoder_destroy(llvq_decoder* dec);
+/* fresh_caches (model.rs:963): the next token is position 0 again. */
+int llvq_hip_decoder_reset(llvq_decoder* dec);
+int llvq_hip_decoder_position(const llvq_decoder* dec);
+/* hidden_cached at l = 1 followed by Head::project (model.rs:968-982, :578-587):
+ * feeds one token at the current position, advances it, and returns the
+ * logits (vocab f32 values, each already rounded to binary16 as the reference's
+ * f16 matmul leaves them) and their argmax (lowest index on ties).  Either
+ * output may be NULL.  Synchronises. */
+int llvq_hip_decoder_forward_token(llvq_decoder* dec, uint32_t token, float* logits_host, uint32_t* argmax_host);
+/* Qwen3::generate (model.rs:1041-1073): resets, feeds the prompt, then decodes
+ * greedily; out receives max_new tokens.  max_new = 0 returns at once.
+ * The loop never waits on the host between tokens.  Synchronises at the end. */
+int llvq_hip_decoder_generate(llvq_decoder* dec, const uint32_t* prompt, size_t n_prompt, size_t max_new,
+                              uint32_t* out);
+
 int llvq_hip_synchronize(llvq_rt* rt);
 const char* llvq_hip_last_error(void);
 const char* llvq_hip_version(void);

@@ -43,6 +43,17 @@ class RecordInfo(C.Structure):
     ]
 
 
+class DecoderDesc(C.Structure):
+    _fields_ = [
+        ("n_layers", C.c_uint32), ("hidden", C.c_uint32), ("n_heads", C.c_uint32), ("n_kv_heads", C.c_uint32),
+        ("head_dim", C.c_uint32), ("intermediate", C.c_uint32), ("vocab", C.c_uint32), ("max_positions", C.c_uint32),
+        ("rope_theta", C.c_double), ("rms_eps", C.c_double),
+        ("projections", C.POINTER(C.c_void_p)),
+        ("input_norm", C.c_void_p), ("post_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
+        ("final_norm", C.c_void_p), ("embed", C.c_void_p), ("lm_head", C.c_void_p),
+    ]
+
+
 def lib_path():
     return _LIB
 
@@ -86,6 +97,13 @@ def lib():
     L.llvq_hip_gemm.argtypes = [vp, vp, vp, C.c_int, vp, C.c_int]
     L.llvq_hip_decode_blocks.argtypes = [vp, vp, sz, vp, vp, vp]
     L.llvq_hip_synchronize.argtypes = [vp]
+    L.llvq_hip_decoder_create.argtypes = [vp, C.POINTER(DecoderDesc), C.POINTER(vp)]
+    L.llvq_hip_decoder_destroy.argtypes = [vp]
+    L.llvq_hip_decoder_destroy.restype = None
+    L.llvq_hip_decoder_reset.argtypes = [vp]
+    L.llvq_hip_decoder_position.argtypes = [vp]
+    L.llvq_hip_decoder_forward_token.argtypes = [vp, C.c_uint32, vp, C.POINTER(C.c_uint32)]
+    L.llvq_hip_decoder_generate.argtypes = [vp, vp, sz, sz, vp]
     L.llvq_hip_last_error.restype = C.c_char_p
     L.llvq_hip_version.restype = C.c_char_p
     _lib = L
@@ -104,4 +122,6 @@ EXPORTS = [
     "llvq_hip_matrix_free", "llvq_hip_matrix_info", "llvq_hip_matrix_name", "llvq_hip_gemv",
     "llvq_hip_gemv_group", "llvq_hip_gemm", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
     "llvq_hip_last_error", "llvq_hip_version",
+    "llvq_hip_decoder_create", "llvq_hip_decoder_destroy", "llvq_hip_decoder_reset", "llvq_hip_decoder_position",
+    "llvq_hip_decoder_forward_token", "llvq_hip_decoder_generate",
 ]

@@ -1,0 +1,283 @@
+// Batch-1 greedy decode loop of a Qwen3-architecture model whose seven
+// projections per layer are LLVQ matrices: the counterpart of
+// Block::forward_cached / Qwen3::hidden_cached / Qwen3::generate
+// (llvq-llm/src/model.rs:766-835, :968-982, :1041-1073) at l = 1.
+// Included by llvq_hip.hip after the GEMV launcher it drives.
+//
+// Everything between two projections runs in small hand-written kernels on the
+// runtime's stream; the token chosen at one step is read by the next step's
+// embedding kernel from device memory, so the host never waits inside a
+// generation.  Activations between kernels are binary16 (the run dtype of the
+// reference); every kernel computes in f32 and rounds once on output:
+//   embed -> h
+//   [per layer] add + RMSNorm -> qkv GEMV group -> per-head RMSNorm + RoPE +
+//   cache append -> attention over the cache -> o GEMV -> add + RMSNorm ->
+//   gate/up GEMV group -> SiLU(gate) * up -> down GEMV
+//   add + final RMSNorm -> f16 lm_head GEMV (logits rounded to binary16, as the
+//   reference's f16 matmul leaves them) -> argmax, lowest index on ties.
+#pragma once
+
+namespace llvq {
+
+constexpr int kNormThreads = 1024;
+
+__device__ __forceinline__ float block_sum_1024(float v, float* red) {
+  v = wave_sum(v);
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  __syncthreads();  // red may still be read from a previous call
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int w = 0; w < kNormThreads / 64; ++w) s += red[w];  // same order in every lane
+  return s;
+}
+
+// h = embed[token]
+__global__ __launch_bounds__(256) void embed_kernel(const __half* __restrict__ table, const uint32_t* __restrict__ token,
+                                                    uint32_t vocab, uint32_t hidden, __half* __restrict__ h) {
+  const uint32_t t = min(*token, vocab - 1u);
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < hidden; i += gridDim.x * blockDim.x)
+    h[i] = table[(size_t)t * hidden + i];
+}
+
+// h <- f16(h + delta) when delta is given; normed = f16(h / sqrt(mean(h^2) + eps) * w)
+// (candle_nn::RmsNorm: f32 inside, one rounding on the way out).
+__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(__half* __restrict__ h, const __half* __restrict__ delta,
+                                                                   const __half* __restrict__ w, __half* __restrict__ normed,
+                                                                   uint32_t n, float eps) {
+  __shared__ float red[kNormThreads / 64];
+  constexpr int kPer = 8;  // n <= 8192
+  float v[kPer];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    const uint32_t i = threadIdx.x + (uint32_t)k * kNormThreads;
+    v[k] = 0.f;
+    if (i < n) {
+      float x = __half2float(h[i]);
+      if (delta) {
+        x = __half2float(__float2half_rn(x + __half2float(delta[i])));  // the residual stream is binary16
+        h[i] = __float2half_rn(x);
+      }
+      v[k] = x;
+      ss += x * x;
+    }
+  }
+  const float total = block_sum_1024(ss, red);
+  const float inv = 1.0f / sqrtf(total / (float)n + eps);
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    const uint32_t i = threadIdx.x + (uint32_t)k * kNormThreads;
+    if (i < n) normed[i] = __float2half_rn(v[k] * inv * __half2float(w[i]));
+  }
+}
+
+// One wavefront per head: per-head RMSNorm of q and k (model.rs:800-808), RoPE at
+// the absolute position in the rotate-half convention (candle_nn::rotary_emb::rope:
+// out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i] sin + x[i + d/2] cos, with
+// the binary16 cos/sin tables of Rotary::new, model.rs:163-179), then k and v of
+// this position are appended to the cache.  Heads: [0, n_heads) are q, the next
+// n_kv are k, the last n_kv are v.  head_dim <= 256, even.
+__global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restrict__ q, const __half* __restrict__ k,
+                                                                 const __half* __restrict__ v,
+                                                                 const __half* __restrict__ qn, const __half* __restrict__ kn,
+                                                                 const __half* __restrict__ cos_t, const __half* __restrict__ sin_t,
+                                                                 __half* __restrict__ kcache, __half* __restrict__ vcache,
+                                                                 uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                                                 uint32_t pos, uint32_t max_pos, float eps) {
+  const uint32_t head = blockIdx.x, lane = threadIdx.x;
+  const uint32_t half_d = head_dim >> 1;
+  if (head >= n_heads + n_kv) {  // v: copy into the cache
+    const uint32_t kvh = head - n_heads - n_kv;
+    for (uint32_t i = lane; i < head_dim; i += 64)
+      vcache[((size_t)kvh * max_pos + pos) * head_dim + i] = v[(size_t)kvh * head_dim + i];
+    return;
+  }
+  const bool is_q = head < n_heads;
+  const uint32_t hh = is_q ? head : head - n_heads;
+  const __half* src = (is_q ? q : k) + (size_t)hh * head_dim;
+  const __half* w = is_q ? qn : kn;
+  float x[4];  // elements lane, lane + 64, lane + 128, lane + 192
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t i = lane + 64u * j;
+    x[j] = i < head_dim ? __half2float(src[i]) : 0.f;
+    ss += x[j] * x[j];
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)head_dim + eps);
+  __shared__ float normed[256];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t i = lane + 64u * j;
+    if (i < head_dim) normed[i] = __half2float(__float2half_rn(x[j] * inv * __half2float(w[i])));
+  }
+  __syncthreads();
+  __half* dst = is_q ? q + (size_t)hh * head_dim : kcache + ((size_t)hh * max_pos + pos) * head_dim;
+  for (uint32_t i = lane; i < half_d; i += 64) {
+    const float c = __half2float(cos_t[(size_t)pos * half_d + i]), s = __half2float(sin_t[(size_t)pos * half_d + i]);
+    const float x1 = normed[i], x2 = normed[i + half_d];
+    dst[i] = __float2half_rn(x1 * c - x2 * s);
+    dst[i + half_d] = __float2half_rn(x1 * s + x2 * c);
+  }
+}
+
+// Attention of one query position over the cache (model.rs:812-822): one
+// workgroup per query head, grouped-query sharing of the n_kv cached heads.
+// Scores, softmax and the weighted sum stay in f32; the context is rounded once.
+constexpr int kAttnThreads = 256;
+__global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half* __restrict__ q, const __half* __restrict__ kcache,
+                                                                   const __half* __restrict__ vcache, __half* __restrict__ ctx,
+                                                                   uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                                                   uint32_t T, uint32_t max_pos, float scale) {
+  extern __shared__ __align__(16) float att_smem[];
+  float* qs = att_smem;             // [head_dim]
+  float* sc = qs + head_dim;        // [T]
+  float* red = sc + T;              // [kAttnThreads / 64] + partial sums [2][head_dim]
+  const uint32_t head = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t kvh = head / (n_heads / n_kv);
+  const __half* K = kcache + (size_t)kvh * max_pos * head_dim;
+  const __half* V = vcache + (size_t)kvh * max_pos * head_dim;
+  for (uint32_t i = tid; i < head_dim; i += kAttnThreads) qs[i] = __half2float(q[(size_t)head * head_dim + i]);
+  __syncthreads();
+  // scores: four lanes per position, each a quarter of the head
+  float lmax = -INFINITY;
+  const uint32_t sub = tid & 3u, quarter = head_dim >> 2;
+  for (uint32_t j = tid >> 2; j < T; j += kAttnThreads / 4) {
+    const __half* kr = K + (size_t)j * head_dim + sub * quarter;
+    float d = 0.f;
+    for (uint32_t i = 0; i < quarter; i += 2) {
+      const __half2 kk = *reinterpret_cast<const __half2*>(kr + i);
+      d = fmaf(qs[sub * quarter + i], __low2float(kk), d);
+      d = fmaf(qs[sub * quarter + i + 1], __high2float(kk), d);
+    }
+    d += __shfl_xor(d, 1, 64);
+    d += __shfl_xor(d, 2, 64);
+    d *= scale;
+    if (sub == 0) sc[j] = d;
+    lmax = fmaxf(lmax, d);
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) lmax = fmaxf(lmax, __shfl_xor(lmax, o, 64));
+  if (lane == 0) red[wave] = lmax;
+  __syncthreads();
+  float gmax = red[0];
+  for (uint32_t w = 1; w < kAttnThreads / 64; ++w) gmax = fmaxf(gmax, red[w]);
+  __syncthreads();
+  float lsum = 0.f;
+  for (uint32_t j = tid; j < T; j += kAttnThreads) {
+    const float e = __expf(sc[j] - gmax);
+    sc[j] = e;
+    lsum += e;
+  }
+  lsum = wave_sum(lsum);
+  if (lane == 0) red[wave] = lsum;
+  __syncthreads();
+  float gsum = 0.f;
+  for (uint32_t w = 0; w < kAttnThreads / 64; ++w) gsum += red[w];
+  const float inv = 1.0f / gsum;
+  // context: lane d of each half of the workgroup walks half of the positions
+  float* part = red + kAttnThreads / 64;
+  const uint32_t hsel = tid / (kAttnThreads / 2), d0 = tid % (kAttnThreads / 2);
+  for (uint32_t d = d0; d < head_dim; d += kAttnThreads / 2) {
+    float a = 0.f;
+    for (uint32_t j = hsel; j < T; j += 2) a = fmaf(sc[j], __half2float(V[(size_t)j * head_dim + d]), a);
+    part[hsel * head_dim + d] = a;
+  }
+  __syncthreads();
+  for (uint32_t d = tid; d < head_dim; d += kAttnThreads)
+    ctx[(size_t)head * head_dim + d] = __float2half_rn((part[d] + part[head_dim + d]) * inv);
+}
+
+// act = f16(f16(silu(gate)) * up)   (model.rs:831: gu[0].apply(act).mul(gu[1]))
+__global__ __launch_bounds__(256) void silu_mul_kernel(const __half* __restrict__ gate, const __half* __restrict__ up,
+                                                       __half* __restrict__ out, uint32_t n) {
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+    const float g = __half2float(gate[i]);
+    const float s = __half2float(__float2half_rn(g / (1.0f + __expf(-g))));
+    out[i] = __float2half_rn(s * __half2float(up[i]));
+  }
+}
+
+// logits = f16(E h) for a dense binary16 head (Head::project, model.rs:578-587);
+// one wavefront per row at a time, 16-byte loads, f32 accumulate.  Every
+// wavefront also leaves its best (value, row), lowest row on ties.
+constexpr int kHeadThreads = 256;
+__global__ __launch_bounds__(kHeadThreads) void lm_head_kernel(const __half* __restrict__ E, const __half* __restrict__ h,
+                                                               uint32_t vocab, uint32_t hidden, float* __restrict__ logits,
+                                                               float* __restrict__ best_val, uint32_t* __restrict__ best_idx) {
+  extern __shared__ __align__(16) float hs[];  // [hidden]
+  for (uint32_t i = threadIdx.x; i < hidden; i += kHeadThreads) hs[i] = __half2float(h[i]);
+  __syncthreads();
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t gw = blockIdx.x * (kHeadThreads / 64) + (threadIdx.x >> 6), nw = gridDim.x * (kHeadThreads / 64);
+  const uint32_t chunks = hidden >> 3;  // 16-byte units per row
+  float bv = -INFINITY;
+  uint32_t bi = 0xFFFFFFFFu;
+  for (uint32_t r = gw; r < vocab; r += nw) {
+    const uint4* row = reinterpret_cast<const uint4*>(E + (size_t)r * hidden);
+    float a = 0.f;
+    for (uint32_t c = lane; c < chunks; c += 64) {
+      const uint4 u = row[c];
+      const uint32_t wv[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        a = fmaf(__half2float(__ushort_as_half((unsigned short)(wv[j] & 0xFFFFu))), hs[8 * c + 2 * j], a);
+        a = fmaf(__half2float(__ushort_as_half((unsigned short)(wv[j] >> 16))), hs[8 * c + 2 * j + 1], a);
+      }
+    }
+    a = wave_sum(a);
+    const float l = __half2float(__float2half_rn(a));
+    if (lane == 0) logits[r] = l;
+    if (l > bv) {  // rows ascend inside a wavefront, so '>' keeps the lowest row of a tie
+      bv = l;
+      bi = r;
+    }
+  }
+  if (lane == 0) {
+    best_val[gw] = bv;
+    best_idx[gw] = bi;
+  }
+}
+
+// token = argmax over the wavefront winners; lowest row on ties
+__global__ __launch_bounds__(1024) void argmax_final_kernel(const float* __restrict__ best_val, const uint32_t* __restrict__ best_idx,
+                                                            uint32_t n, uint32_t* __restrict__ token_out,
+                                                            uint32_t* __restrict__ history, uint32_t slot) {
+  __shared__ float sv[1024];
+  __shared__ uint32_t si[1024];
+  float bv = -INFINITY;
+  uint32_t bi = 0xFFFFFFFFu;
+  for (uint32_t i = threadIdx.x; i < n; i += 1024) {
+    const float v = best_val[i];
+    const uint32_t id = best_idx[i];
+    if (v > bv || (v == bv && id < bi)) {
+      bv = v;
+      bi = id;
+    }
+  }
+  sv[threadIdx.x] = bv;
+  si[threadIdx.x] = bi;
+  __syncthreads();
+  for (uint32_t s = 512; s >= 1; s >>= 1) {
+    if (threadIdx.x < s) {
+      const float v = sv[threadIdx.x + s];
+      const uint32_t id = si[threadIdx.x + s];
+      if (v > sv[threadIdx.x] || (v == sv[threadIdx.x] && id < si[threadIdx.x])) {
+        sv[threadIdx.x] = v;
+        si[threadIdx.x] = id;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    *token_out = si[0];
+    if (history) history[slot] = si[0];
+  }
+}
+
+__global__ void set_token_kernel(uint32_t* token, uint32_t value) { *token = value; }
+
+}  // namespace llvq

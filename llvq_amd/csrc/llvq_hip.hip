@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cmath>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -513,6 +514,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 }  // namespace llvq
 
 #include "gemm_kernel.h"
+#include "decoder.h"
 
 // =================================================================================
 // C ABI
@@ -985,6 +987,237 @@ int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks
   hipLaunchKernelGGL(decode_blocks_kernel, dim3((uint32_t)grid), dim3(256), kLdsImageBytes, rt->stream,
                      rt->tables, codes_dev, nblocks, points_dev, gains_dev, shells_dev);
   HIP_TRY(hipGetLastError());
+  return LLVQ_OK;
+}
+
+}  // extern "C"
+
+// =================================================================================
+// Batch-1 decode loop (C ABI)
+// =================================================================================
+struct llvq_decoder {
+  llvq_rt* rt = nullptr;
+  uint32_t n_layers = 0, hidden = 0, n_heads = 0, n_kv = 0, head_dim = 0, inter = 0, vocab = 0, max_pos = 0;
+  float eps = 1e-6f;
+  std::vector<const llvq_mat*> proj;  // [n_layers * 7]: q k v o gate up down
+  uint8_t* blob = nullptr;            // every dense tensor and buffer below, one allocation
+  __half *ln1 = nullptr, *ln2 = nullptr, *qn = nullptr, *kn = nullptr, *fnorm = nullptr;
+  __half *embed = nullptr, *head = nullptr, *cos_t = nullptr, *sin_t = nullptr;
+  __half *kcache = nullptr, *vcache = nullptr;  // [n_layers][n_kv][max_pos][head_dim]
+  __half *h = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *ctx = nullptr, *o = nullptr;
+  __half *gate = nullptr, *up = nullptr, *act = nullptr, *down = nullptr;
+  float* logits = nullptr;
+  float* best_val = nullptr;
+  uint32_t* best_idx = nullptr;
+  uint32_t* token = nullptr;    // the token the next step embeds
+  uint32_t* history = nullptr;  // [max_pos] tokens chosen by the head
+  uint32_t pos = 0;
+  uint32_t head_grid = 0;
+};
+
+namespace {
+
+// Enqueues one position: embeds *dec->token, runs the layers at position dec->pos,
+// and (want_logits) the head and the argmax, which overwrites *dec->token.
+int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool record) {
+  llvq_rt* rt = d->rt;
+  hipStream_t st = rt->stream;
+  if (d->pos >= d->max_pos) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder: position " + std::to_string(d->pos) + " is past max_positions");
+  hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, d->h);
+  const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
+  const uint32_t T = d->pos + 1;
+  const size_t attn_lds = ((size_t)d->head_dim * 3 + T + kAttnThreads / 64) * sizeof(float);
+  for (uint32_t L = 0; L < d->n_layers; ++L) {
+    const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
+    // the previous layer's MLP output joins the residual stream here
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, L ? d->down : (const __half*)nullptr,
+                       d->ln1 + (size_t)L * d->hidden, d->normed, d->hidden, d->eps);
+    void* qkv_out[3] = {d->q, d->k, d->v};
+    int rc = launch_group(rt, P, 3, d->normed, qkv_out, LLVQ_F16);
+    if (rc) return rc;
+    hipLaunchKernelGGL(qk_norm_rope_append_kernel, dim3(d->n_heads + 2 * d->n_kv), dim3(64), 0, st, d->q, d->k, d->v,
+                       d->qn + (size_t)L * d->head_dim, d->kn + (size_t)L * d->head_dim, d->cos_t, d->sin_t,
+                       d->kcache + L * cache_layer, d->vcache + L * cache_layer, d->n_heads, d->n_kv, d->head_dim, d->pos,
+                       d->max_pos, d->eps);
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(d->n_heads), dim3(kAttnThreads), attn_lds, st, d->q, d->kcache + L * cache_layer,
+                       d->vcache + L * cache_layer, d->ctx, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
+                       1.0f / sqrtf((float)d->head_dim));
+    void* o_out[1] = {d->o};
+    rc = launch_group(rt, P + 3, 1, d->ctx, o_out, LLVQ_F16);
+    if (rc) return rc;
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->o, d->ln2 + (size_t)L * d->hidden,
+                       d->normed, d->hidden, d->eps);
+    void* gu_out[2] = {d->gate, d->up};
+    rc = launch_group(rt, P + 4, 2, d->normed, gu_out, LLVQ_F16);
+    if (rc) return rc;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((d->inter + 255) / 256), dim3(256), 0, st, d->gate, d->up, d->act, d->inter);
+    void* d_out[1] = {d->down};
+    rc = launch_group(rt, P + 6, 1, d->act, d_out, LLVQ_F16);
+    if (rc) return rc;
+  }
+  if (want_logits) {
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->down, d->fnorm, d->normed, d->hidden, d->eps);
+    hipLaunchKernelGGL(lm_head_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head, d->normed,
+                       d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(1024), 0, st, d->best_val, d->best_idx,
+                       d->head_grid * (kHeadThreads / 64), d->token, record ? d->history : (uint32_t*)nullptr, history_slot);
+  }
+  HIP_TRY(hipGetLastError());
+  d->pos += 1;
+  return LLVQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decoder** out) {
+  if (!rt || !c || !out) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: null argument");
+  *out = nullptr;
+  if (!c->projections || !c->input_norm || !c->post_norm || !c->q_norm || !c->k_norm || !c->final_norm || !c->embed)
+    return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: a required tensor is null");
+  if (c->n_layers == 0 || c->hidden == 0 || c->hidden % 8 || c->hidden > 8192 || c->n_heads == 0 || c->n_kv_heads == 0 ||
+      c->n_heads % c->n_kv_heads || c->head_dim == 0 || c->head_dim % 8 || c->head_dim > 256 || c->intermediate == 0 ||
+      c->vocab == 0 || c->max_positions == 0 || c->max_positions > 8192)
+    return fail(LLVQ_ERR_UNSUPPORTED,
+                "decoder_create: shape outside what the kernels hold (hidden % 8 = 0 and <= 8192, head_dim % 8 = 0 and <= 256, "
+                "heads a multiple of kv heads, max_positions <= 8192)");
+  const uint32_t qd = c->n_heads * c->head_dim, kvd = c->n_kv_heads * c->head_dim;
+  static const char* kSite[7] = {"q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"};
+  const uint32_t want_out[7] = {qd, kvd, kvd, c->hidden, c->intermediate, c->intermediate, c->hidden};
+  const uint32_t want_in[7] = {c->hidden, c->hidden, c->hidden, qd, c->hidden, c->hidden, c->intermediate};
+  for (uint32_t L = 0; L < c->n_layers; ++L)
+    for (int j = 0; j < 7; ++j) {
+      const llvq_mat* m = c->projections[(size_t)L * 7 + j];
+      if (!m) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: layer " + std::to_string(L) + " " + kSite[j] + " is null");
+      if (m->d_out != want_out[j] || m->d_in != want_in[j])
+        return fail(LLVQ_ERR_INCONSISTENT, "decoder_create: layer " + std::to_string(L) + " " + kSite[j] + " is " +
+                                               std::to_string(m->d_out) + "x" + std::to_string(m->d_in) + ", the architecture needs " +
+                                               std::to_string(want_out[j]) + "x" + std::to_string(want_in[j]));
+    }
+  HIP_TRY(hipSetDevice(rt->device));
+  auto* d = new llvq_decoder();
+  d->rt = rt;
+  d->n_layers = c->n_layers; d->hidden = c->hidden; d->n_heads = c->n_heads; d->n_kv = c->n_kv_heads;
+  d->head_dim = c->head_dim; d->inter = c->intermediate; d->vocab = c->vocab; d->max_pos = c->max_positions;
+  d->eps = (float)c->rms_eps;
+  d->proj.assign(c->projections, c->projections + (size_t)c->n_layers * 7);
+  d->head_grid = 1024;
+  while (d->head_grid > 1 && (uint64_t)d->head_grid * (kHeadThreads / 64) > c->vocab) d->head_grid >>= 1;
+
+  // RoPE tables exactly as Rotary::new builds them (model.rs:163-179): f32 inverse
+  // frequencies from an f64 power, f32 angle = position * inv_freq, sin/cos narrowed to binary16.
+  const uint32_t half_d = c->head_dim / 2;
+  std::vector<__half> cos_h((size_t)c->max_positions * half_d), sin_h(cos_h.size());
+  for (uint32_t i = 0; i < half_d; ++i) {
+    const float inv = 1.0f / (float)std::pow(c->rope_theta, (double)(2 * i) / (double)c->head_dim);
+    for (uint32_t p = 0; p < c->max_positions; ++p) {
+      const float ang = (float)p * inv;
+      cos_h[(size_t)p * half_d + i] = __float2half_rn(std::cos(ang));
+      sin_h[(size_t)p * half_d + i] = __float2half_rn(std::sin(ang));
+    }
+  }
+
+  // one allocation, 256-byte aligned pieces
+  size_t total = 0;
+  auto take = [&](size_t bytes) { const size_t at = total; total += (bytes + 255) & ~(size_t)255; return at; };
+  const size_t hb = sizeof(__half);
+  const size_t o_ln1 = take((size_t)c->n_layers * c->hidden * hb), o_ln2 = take((size_t)c->n_layers * c->hidden * hb);
+  const size_t o_qn = take((size_t)c->n_layers * c->head_dim * hb), o_kn = take((size_t)c->n_layers * c->head_dim * hb);
+  const size_t o_fn = take((size_t)c->hidden * hb);
+  const size_t o_emb = take((size_t)c->vocab * c->hidden * hb);
+  const size_t o_head = c->lm_head ? take((size_t)c->vocab * c->hidden * hb) : o_emb;
+  const size_t o_cos = take(cos_h.size() * hb), o_sin = take(sin_h.size() * hb);
+  const size_t cache_bytes = (size_t)c->n_layers * c->n_kv_heads * c->max_positions * c->head_dim * hb;
+  const size_t o_kc = take(cache_bytes), o_vc = take(cache_bytes);
+  const size_t o_h = take(c->hidden * hb), o_nm = take(c->hidden * hb), o_q = take(qd * hb), o_k = take(kvd * hb), o_v = take(kvd * hb);
+  const size_t o_ctx = take(qd * hb), o_o = take(c->hidden * hb), o_g = take(c->intermediate * hb), o_u = take(c->intermediate * hb);
+  const size_t o_act = take(c->intermediate * hb), o_dn = take(c->hidden * hb);
+  const size_t o_log = take((size_t)c->vocab * sizeof(float));
+  const size_t n_best = (size_t)d->head_grid * (kHeadThreads / 64);
+  const size_t o_bv = take(n_best * sizeof(float)), o_bi = take(n_best * sizeof(uint32_t));
+  const size_t o_tok = take(sizeof(uint32_t)), o_hist = take((size_t)c->max_positions * sizeof(uint32_t));
+  hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->blob), total);
+  if (e != hipSuccess) { delete d; return hip_fail(e, "hipMalloc(decoder)"); }
+  auto put = [&](size_t at, const void* src, size_t bytes) { return hipMemcpy(d->blob + at, src, bytes, hipMemcpyHostToDevice); };
+  e = hipMemset(d->blob, 0, total);
+  if (e == hipSuccess) e = put(o_ln1, c->input_norm, (size_t)c->n_layers * c->hidden * hb);
+  if (e == hipSuccess) e = put(o_ln2, c->post_norm, (size_t)c->n_layers * c->hidden * hb);
+  if (e == hipSuccess) e = put(o_qn, c->q_norm, (size_t)c->n_layers * c->head_dim * hb);
+  if (e == hipSuccess) e = put(o_kn, c->k_norm, (size_t)c->n_layers * c->head_dim * hb);
+  if (e == hipSuccess) e = put(o_fn, c->final_norm, (size_t)c->hidden * hb);
+  if (e == hipSuccess) e = put(o_emb, c->embed, (size_t)c->vocab * c->hidden * hb);
+  if (e == hipSuccess && c->lm_head) e = put(o_head, c->lm_head, (size_t)c->vocab * c->hidden * hb);
+  if (e == hipSuccess) e = put(o_cos, cos_h.data(), cos_h.size() * hb);
+  if (e == hipSuccess) e = put(o_sin, sin_h.data(), sin_h.size() * hb);
+  if (e != hipSuccess) { (void)hipFree(d->blob); delete d; return hip_fail(e, "decoder upload"); }
+  auto H = [&](size_t at) { return reinterpret_cast<__half*>(d->blob + at); };
+  d->ln1 = H(o_ln1); d->ln2 = H(o_ln2); d->qn = H(o_qn); d->kn = H(o_kn); d->fnorm = H(o_fn);
+  d->embed = H(o_emb); d->head = H(o_head); d->cos_t = H(o_cos); d->sin_t = H(o_sin);
+  d->kcache = H(o_kc); d->vcache = H(o_vc);
+  d->h = H(o_h); d->normed = H(o_nm); d->q = H(o_q); d->k = H(o_k); d->v = H(o_v); d->ctx = H(o_ctx); d->o = H(o_o);
+  d->gate = H(o_g); d->up = H(o_u); d->act = H(o_act); d->down = H(o_dn);
+  d->logits = reinterpret_cast<float*>(d->blob + o_log);
+  d->best_val = reinterpret_cast<float*>(d->blob + o_bv);
+  d->best_idx = reinterpret_cast<uint32_t*>(d->blob + o_bi);
+  d->token = reinterpret_cast<uint32_t*>(d->blob + o_tok);
+  d->history = reinterpret_cast<uint32_t*>(d->blob + o_hist);
+  // attention over a long cache needs more than the default 64 KB of dynamic LDS
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(attn_decode_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  *out = d;
+  return LLVQ_OK;
+}
+
+void llvq_hip_decoder_destroy(llvq_decoder* d) {
+  if (!d) return;
+  (void)hipSetDevice(d->rt->device);
+  (void)hipStreamSynchronize(d->rt->stream);
+  (void)hipFree(d->blob);
+  delete d;
+}
+
+int llvq_hip_decoder_reset(llvq_decoder* d) {
+  if (!d) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_reset: null decoder");
+  d->pos = 0;  // the cache is overwritten position by position; nothing else carries state
+  return LLVQ_OK;
+}
+
+int llvq_hip_decoder_position(const llvq_decoder* d) { return d ? (int)d->pos : -1; }
+
+int llvq_hip_decoder_forward_token(llvq_decoder* d, uint32_t token, float* logits_host, uint32_t* argmax_host) {
+  if (!d) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_forward_token: null decoder");
+  if (token >= d->vocab) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_forward_token: token " + std::to_string(token) + " is outside the vocabulary");
+  HIP_TRY(hipSetDevice(d->rt->device));
+  hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(1), 0, d->rt->stream, d->token, token);
+  const int rc = decoder_step(d, true, 0, false);
+  if (rc) return rc;
+  if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, d->logits, (size_t)d->vocab * sizeof(float), hipMemcpyDeviceToHost, d->rt->stream));
+  if (argmax_host) HIP_TRY(hipMemcpyAsync(argmax_host, d->token, sizeof(uint32_t), hipMemcpyDeviceToHost, d->rt->stream));
+  HIP_TRY(hipStreamSynchronize(d->rt->stream));
+  return LLVQ_OK;
+}
+
+int llvq_hip_decoder_generate(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out) {
+  if (!d || (n_prompt && !prompt) || (max_new && !out)) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate: null argument");
+  if (max_new == 0) return LLVQ_OK;  // model.rs:1052-1054
+  if (n_prompt == 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate: empty prompt");
+  if (n_prompt + max_new - 1 > d->max_pos)
+    return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate: " + std::to_string(n_prompt + max_new - 1) + " positions exceed max_positions " + std::to_string(d->max_pos));
+  for (size_t i = 0; i < n_prompt; ++i)
+    if (prompt[i] >= d->vocab) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate: prompt token outside the vocabulary");
+  HIP_TRY(hipSetDevice(d->rt->device));
+  d->pos = 0;
+  for (size_t i = 0; i < n_prompt; ++i) {
+    hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(1), 0, d->rt->stream, d->token, prompt[i]);
+    const int rc = decoder_step(d, i + 1 == n_prompt, 0, true);
+    if (rc) return rc;
+  }
+  for (size_t t = 1; t < max_new; ++t) {
+    const int rc = decoder_step(d, true, (uint32_t)t, true);
+    if (rc) return rc;
+  }
+  HIP_TRY(hipMemcpyAsync(out, d->history, max_new * sizeof(uint32_t), hipMemcpyDeviceToHost, d->rt->stream));
+  HIP_TRY(hipStreamSynchronize(d->rt->stream));
   return LLVQ_OK;
 }
 

@@ -1,0 +1,152 @@
+"""Host mirror of the reference's model runner at batch 1
+(llvq-llm/src/model.rs: Qwen3::new_with :869, hidden_cached :968, generate :1041)
+over the HIP library's decode loop.  No computation happens here: the class
+assembles the descriptor and calls the C ABI."""
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _ffi, synth
+from .fused import FusedRuntime
+
+SITES = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
+         "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj")
+
+
+@dataclass
+class Qwen3Config:
+    """The fields of the reference's Config that the forward pass reads."""
+    num_hidden_layers: int
+    hidden_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    intermediate_size: int
+    vocab_size: int
+    rope_theta: float = 1e6
+    rms_norm_eps: float = 1e-6
+    max_positions: int = 1024
+    tie_word_embeddings: bool = True
+
+    def shapes(self):
+        """(site, d_out, d_in) of the seven projections of one layer."""
+        qd, kvd = self.num_attention_heads * self.head_dim, self.num_key_value_heads * self.head_dim
+        h, i = self.hidden_size, self.intermediate_size
+        return [(SITES[0], qd, h), (SITES[1], kvd, h), (SITES[2], kvd, h), (SITES[3], h, qd),
+                (SITES[4], i, h), (SITES[5], i, h), (SITES[6], h, i)]
+
+
+QWEN3_4B = Qwen3Config(36, 2560, 32, 8, 128, 9728, 151936, max_positions=768)
+
+
+@dataclass
+class DecoderWeights:
+    """Everything a decoder holds besides its LLVQ projections, as binary16 arrays."""
+    input_norm: np.ndarray   # [n_layers, hidden]
+    post_norm: np.ndarray    # [n_layers, hidden]
+    q_norm: np.ndarray       # [n_layers, head_dim]
+    k_norm: np.ndarray       # [n_layers, head_dim]
+    final_norm: np.ndarray   # [hidden]
+    embed: np.ndarray        # [vocab, hidden]
+    lm_head: np.ndarray = None  # [vocab, hidden] or None (tied)
+
+
+def synthetic_weights(cfg: Qwen3Config, seed: int = 0) -> DecoderWeights:
+    """Random-init dense tensors: norm gains 1 + 0.1 N(0,1), embedding N(0,1), head 0.05 N(0,1)."""
+    rng = np.random.default_rng(seed)
+    L, h, d = cfg.num_hidden_layers, cfg.hidden_size, cfg.head_dim
+
+    def gains(*shape):
+        return (1.0 + 0.1 * rng.standard_normal(shape, dtype=np.float32)).astype(np.float16)
+
+    embed = rng.standard_normal((cfg.vocab_size, h), dtype=np.float32).astype(np.float16)
+    head = None
+    if not cfg.tie_word_embeddings:
+        head = (0.05 * rng.standard_normal((cfg.vocab_size, h), dtype=np.float32)).astype(np.float16)
+    return DecoderWeights(gains(L, h), gains(L, h), gains(L, d), gains(L, d), gains(h), embed, head)
+
+
+def synthetic_projections(cfg: Qwen3Config, seed: int = 0):
+    """Random LLVQ codes for every projection, drawn as the single-matrix benchmark draws them."""
+    return [[synth.make_matrix(f"model.layers.{layer}.{site}.weight", do, di, seed) for site, do, di in cfg.shapes()]
+            for layer in range(cfg.num_hidden_layers)]
+
+
+class Decoder:
+    """A Qwen3-architecture model on one GPU: projections uploaded through `rt`,
+    the rest copied at construction."""
+
+    def __init__(self, rt: FusedRuntime, cfg: Qwen3Config, projections, weights: DecoderWeights):
+        self.rt, self.cfg = rt, cfg
+        self.handle = None
+        self._owned = []
+        projs = []
+        for layer in projections:
+            if len(layer) != 7:
+                raise ValueError("a layer has seven projections: q, k, v, o, gate, up, down")
+            for m in layer:
+                if hasattr(m, "handle"):
+                    projs.append(m)
+                else:
+                    p = rt.upload(m)
+                    self._owned.append(p)
+                    projs.append(p)
+        self._projs = projs
+        arr = (C.c_void_p * len(projs))(*[p.handle for p in projs])
+
+        def f16(a, shape):
+            a = np.ascontiguousarray(a, dtype=np.float16)
+            if a.shape != tuple(shape):
+                raise ValueError(f"expected shape {tuple(shape)}, got {a.shape}")
+            return a
+
+        L, h, d = cfg.num_hidden_layers, cfg.hidden_size, cfg.head_dim
+        keep = [f16(weights.input_norm, (L, h)), f16(weights.post_norm, (L, h)), f16(weights.q_norm, (L, d)),
+                f16(weights.k_norm, (L, d)), f16(weights.final_norm, (h,)), f16(weights.embed, (cfg.vocab_size, h))]
+        head = f16(weights.lm_head, (cfg.vocab_size, h)) if weights.lm_head is not None else None
+        desc = _ffi.DecoderDesc(
+            L, h, cfg.num_attention_heads, cfg.num_key_value_heads, d, cfg.intermediate_size, cfg.vocab_size,
+            cfg.max_positions, float(cfg.rope_theta), float(cfg.rms_norm_eps),
+            C.cast(arr, C.POINTER(C.c_void_p)),
+            keep[0].ctypes.data, keep[1].ctypes.data, keep[2].ctypes.data, keep[3].ctypes.data, keep[4].ctypes.data,
+            keep[5].ctypes.data, head.ctypes.data if head is not None else None)
+        out = C.c_void_p()
+        _ffi.check(_ffi.lib().llvq_hip_decoder_create(rt.handle, C.byref(desc), C.byref(out)))
+        self.handle = out
+
+    def reset(self):
+        _ffi.check(_ffi.lib().llvq_hip_decoder_reset(self.handle))
+
+    @property
+    def position(self):
+        return _ffi.lib().llvq_hip_decoder_position(self.handle)
+
+    def forward_token(self, token: int, want_logits: bool = True):
+        """One position: (logits f32 [vocab] or None, argmax)."""
+        logits = np.empty(self.cfg.vocab_size, np.float32) if want_logits else None
+        best = C.c_uint32()
+        _ffi.check(_ffi.lib().llvq_hip_decoder_forward_token(
+            self.handle, int(token), logits.ctypes.data if want_logits else None, C.byref(best)))
+        return logits, best.value
+
+    def generate(self, prompt, max_new: int) -> np.ndarray:
+        prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+        out = np.zeros(max_new, np.uint32)
+        _ffi.check(_ffi.lib().llvq_hip_decoder_generate(self.handle, prompt.ctypes.data, prompt.size, max_new,
+                                                        out.ctypes.data))
+        return out
+
+    def close(self):
+        if self.handle is not None:
+            _ffi.lib().llvq_hip_decoder_destroy(self.handle)
+            self.handle = None
+        for p in self._owned:
+            self.rt.free(p)
+        self._owned = []
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,134 @@
+"""CPU restatement of the reference's Qwen3 forward pass at batch 1, one token
+at a time with a KV cache.  TEST INFRASTRUCTURE ONLY: tests, the smoke check
+and the CPU leg of the benchmark may import this; the product never does.
+
+Follows llvq-llm/src/model.rs:
+  Rotary::new           :163-179   inverse frequencies, f32 angles, tables narrowed to the run dtype
+  Block::forward_cached :766-835   ln1 -> q/k/v -> per-head q_norm/k_norm -> RoPE at the absolute
+                                   position -> cache append -> grouped-query attention -> o_proj ->
+                                   residual -> ln2 -> gate/up -> act(gate) * up -> down_proj -> residual
+  Qwen3::hidden_cached  :968-982   embedding, blocks, final norm
+  Head::project         :578-587   h E^T at the run dtype
+  Qwen3::generate       :1041-1073 greedy loop; argmax of the logits widened to f32
+
+The projections are dense matrices here (the oracle's decode_matrix output),
+i.e. the reference's dense arm.  The run dtype is binary16: every tensor that
+crosses an operator boundary in the reference is rounded to binary16 here too,
+and each operator computes in f64 inside.
+
+PARITY UNPINNED: RMSNorm, rope, softmax and matmul are candle-nn / candle-core
+0.9 operators (Cargo.toml pins "0.9"; the crates are not vendored in the
+reference tree), restated from their published definitions.  Which of their
+internal steps round to binary16 (e.g. the score matrix before the softmax) is
+not fixed by anything the reference's own tests hold for this path, so this
+file rounds only at operator outputs that the reference materialises as tensors
+of the run dtype, except inside attention, which is kept in f64 from the scores
+to the context.
+"""
+import numpy as np
+
+
+def r16(x):
+    """Round to binary16 (nearest even) and widen again."""
+    return np.asarray(x, dtype=np.float64).astype(np.float16).astype(np.float64)
+
+
+def rope_tables(head_dim, theta, max_positions):
+    """model.rs:163-179: inv_i = 1f32 / (theta^(i/dim) as f32), i even; freqs = t * inv in f32; sin/cos -> f16."""
+    i = np.arange(0, head_dim, 2, dtype=np.float64)
+    inv = (np.float32(1.0) / np.power(float(theta), i / float(head_dim)).astype(np.float32)).astype(np.float32)
+    t = np.arange(max_positions, dtype=np.float32).reshape(-1, 1)
+    freqs = (t * inv.reshape(1, -1)).astype(np.float32)
+    return r16(np.cos(freqs)), r16(np.sin(freqs))
+
+
+def rms_norm(x, w, eps):
+    """candle_nn::RmsNorm: x / sqrt(mean(x^2) + eps) * w, one rounding on the way out."""
+    x = np.asarray(x, np.float64)
+    return r16(x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps) * w)
+
+
+def silu(x):
+    return x / (1.0 + np.exp(-x))
+
+
+class Qwen3Oracle:
+    def __init__(self, cfg, dense_projections, weights):
+        """cfg: object with the Qwen3 Config field names; dense_projections[layer][j]: [d_out, d_in]
+        arrays in the order q, k, v, o, gate, up, down; weights: binary16 arrays (input_norm,
+        post_norm, q_norm, k_norm, final_norm, embed, lm_head or None)."""
+        self.cfg = cfg
+        self.W = [[np.asarray(m, np.float64) for m in layer] for layer in dense_projections]
+        f = lambda a: np.asarray(a, np.float16).astype(np.float64)
+        self.ln1, self.ln2 = f(weights.input_norm), f(weights.post_norm)
+        self.qn, self.kn, self.fn = f(weights.q_norm), f(weights.k_norm), f(weights.final_norm)
+        self.embed = np.asarray(weights.embed, np.float16)
+        self.head = self.embed if weights.lm_head is None else np.asarray(weights.lm_head, np.float16)
+        self.cos, self.sin = rope_tables(cfg.head_dim, cfg.rope_theta, cfg.max_positions)
+        self.reset()
+
+    def reset(self):
+        L = self.cfg.num_hidden_layers
+        self.K = [[] for _ in range(L)]
+        self.V = [[] for _ in range(L)]
+        self.pos = 0
+
+    def forward_token(self, token):
+        """hidden_cached at l = 1, then the head: returns the logits (f32, binary16-valued)."""
+        c = self.cfg
+        nh, nkv, hd = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+        eps = c.rms_norm_eps
+        h = self.embed[int(token)].astype(np.float64)
+        cos, sin = self.cos[self.pos], self.sin[self.pos]
+        for L in range(c.num_hidden_layers):
+            Wq, Wk, Wv, Wo, Wg, Wu, Wd = self.W[L]
+            x = rms_norm(h, self.ln1[L], eps)
+            q = r16(Wq @ x).reshape(nh, hd)
+            k = r16(Wk @ x).reshape(nkv, hd)
+            v = r16(Wv @ x).reshape(nkv, hd)
+            q = rms_norm(q, self.qn[L], eps)
+            k = rms_norm(k, self.kn[L], eps)
+
+            def rope(t):  # rotate-half: candle_nn::rotary_emb::rope
+                t1, t2 = t[:, : hd // 2], t[:, hd // 2:]
+                return r16(np.concatenate([t1 * cos - t2 * sin, t1 * sin + t2 * cos], axis=1))
+
+            q, k = rope(q), rope(k)
+            self.K[L].append(k)
+            self.V[L].append(v)
+            Kc = np.stack(self.K[L], axis=1)  # [nkv, T, hd]
+            Vc = np.stack(self.V[L], axis=1)
+            groups = nh // nkv
+            ctx = np.empty((nh, hd))
+            for head in range(nh):  # repeat_kv: query head -> cached head head // groups
+                kv = head // groups
+                s = (Kc[kv] @ q[head]) / np.sqrt(float(hd))
+                p = np.exp(s - s.max())
+                p /= p.sum()
+                ctx[head] = p @ Vc[kv]
+            ctx = r16(ctx.reshape(-1))
+            h = r16(h + r16(Wo @ ctx))
+            x = rms_norm(h, self.ln2[L], eps)
+            g, u = r16(Wg @ x), r16(Wu @ x)
+            a = r16(r16(silu(g)) * u)
+            h = r16(h + r16(Wd @ a))
+        x = rms_norm(h, self.fn, eps)
+        self.pos += 1
+        return r16(self.head.astype(np.float64) @ x).astype(np.float32)
+
+    def generate(self, prompt, max_new):
+        """model.rs:1041-1073; also returns the logits of every decoding step."""
+        if max_new == 0:
+            return np.zeros(0, np.uint32), []
+        self.reset()
+        logits = None
+        for t in prompt:
+            logits = self.forward_token(t)
+        out, trace = [], []
+        while True:
+            trace.append(logits)
+            nxt = int(np.argmax(logits))  # first index on ties
+            out.append(nxt)
+            if len(out) == max_new:
+                return np.array(out, np.uint32), trace
+            logits = self.forward_token(nxt)
