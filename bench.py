@@ -83,6 +83,38 @@ def cpu_baseline(layer_mats, acts, threads):
     }
 
 
+def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
+    """BASELINE config 2: the whole Qwen3-4B-architecture loop (36 layers over the projections already on the
+    device, f16 embedding tied to the head, vocabulary 151936): a 512-token random prompt, then 256 greedy
+    tokens.  Decode rate = (time of prompt + 256 tokens) - (time of prompt + 1 token), over 255 steps."""
+    from llvq_amd import decoder
+
+    cfg = decoder.QWEN3_4B
+    t0 = time.time()
+    weights = decoder.synthetic_weights(cfg, seed)
+    dec = decoder.Decoder(rt, cfg, projs, weights)
+    log(f"[bench] decoder built in {time.time() - t0:.1f}s")
+    prompt = np.random.default_rng(seed).integers(0, cfg.vocab_size, size=n_prompt)
+    dec.generate(prompt[:8], 4)  # warm-up
+    t0 = time.perf_counter()
+    first = dec.generate(prompt, 1)
+    t1 = time.perf_counter()
+    toks = dec.generate(prompt, n_new)
+    t2 = time.perf_counter()
+    dec.close()
+    assert toks[0] == first[0]
+    step_s = ((t2 - t1) - (t1 - t0)) / (n_new - 1)
+    return {
+        "tokens_per_s": round(1.0 / step_s, 2),
+        "ms_per_token": round(step_s * 1e3, 4),
+        "prompt_tokens": n_prompt,
+        "new_tokens": n_new,
+        "prefill_tokens_per_s": round(n_prompt / (t1 - t0), 2),
+        "prefill": "one position at a time through the same kernels",
+        "distinct_tokens": int(np.unique(toks).size),
+    }
+
+
 QWEN3_8B_LAYER = [  # (site, d_out, d_in): hidden 4096, intermediate 12288, 32 query / 8 KV heads of 128
     ("self_attn.q_proj", 4096, 4096),
     ("self_attn.k_proj", 1024, 4096),
@@ -187,6 +219,8 @@ def main():
     ap.add_argument("--layers", type=int, default=36)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true",
+                    help="skip the greedy-decode leg (tokens/s of the full model loop) of the gemv workload")
     ap.add_argument("--workload", choices=["gemv", "gemm"], default="gemv",
                     help="gemv: the headline batch-1 projection pass (default); gemm: the batched "
                          "matrix-core path at Qwen3-8B shapes")
@@ -306,6 +340,8 @@ def main():
             "algorithmic_bytes_per_launch": round(enc_bytes / n_kernels, 1),
         },
     }
+    if not args.no_decode and args.layers == 36:
+        out["decode"] = decode_leg(rt, projs, args.seed)
     if args.copy_probe:
         src = torch.arange(1 << 26, dtype=torch.int32, device=dev)  # 256 MiB
         dst = torch.empty_like(src)

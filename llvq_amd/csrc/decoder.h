@@ -124,71 +124,121 @@ __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restr
   }
 }
 
-// Attention of one query position over the cache (model.rs:812-822): one
-// workgroup per query head, grouped-query sharing of the n_kv cached heads.
-// Scores, softmax and the weighted sum stay in f32; the context is rounded once.
+// Attention of one query position over the cache (model.rs:812-822), split over
+// the cache: workgroup (kv head, split) takes a contiguous range of positions
+// and all query heads that share the kv head (one wavefront per query head, so
+// K and V rows are fetched once per group), and leaves an unnormalised partial
+// (running max, sum of exponentials, weighted V sum).  The workgroup that
+// arrives last at the kv head's counter merges the partials in split order and
+// rounds the context once.  Scores, softmax and sums stay in f32.
 constexpr int kAttnThreads = 256;
+constexpr int kAttnSplits = 16;
+constexpr int kAttnMaxDim = 256;
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half* __restrict__ q, const __half* __restrict__ kcache,
                                                                    const __half* __restrict__ vcache, __half* __restrict__ ctx,
+                                                                   float* __restrict__ part, uint32_t* __restrict__ counters,
                                                                    uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                                                    uint32_t T, uint32_t max_pos, float scale) {
-  extern __shared__ __align__(16) float att_smem[];
-  float* qs = att_smem;             // [head_dim]
-  float* sc = qs + head_dim;        // [T]
-  float* red = sc + T;              // [kAttnThreads / 64] + partial sums [2][head_dim]
-  const uint32_t head = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const uint32_t kvh = head / (n_heads / n_kv);
+  extern __shared__ __align__(16) float att_smem[];  // [4][chunk] scores
+  __shared__ uint32_t arrived;
+  const uint32_t kvh = blockIdx.x / kAttnSplits, split = blockIdx.x % kAttnSplits;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t groups = n_heads / n_kv;
+  const uint32_t chunk = (T + kAttnSplits - 1) / kAttnSplits;
+  const uint32_t j0 = min(T, split * chunk), j1 = min(T, j0 + chunk);
   const __half* K = kcache + (size_t)kvh * max_pos * head_dim;
   const __half* V = vcache + (size_t)kvh * max_pos * head_dim;
-  for (uint32_t i = tid; i < head_dim; i += kAttnThreads) qs[i] = __half2float(q[(size_t)head * head_dim + i]);
-  __syncthreads();
-  // scores: four lanes per position, each a quarter of the head
-  float lmax = -INFINITY;
-  const uint32_t sub = tid & 3u, quarter = head_dim >> 2;
-  for (uint32_t j = tid >> 2; j < T; j += kAttnThreads / 4) {
-    const __half* kr = K + (size_t)j * head_dim + sub * quarter;
-    float d = 0.f;
-    for (uint32_t i = 0; i < quarter; i += 2) {
-      const __half2 kk = *reinterpret_cast<const __half2*>(kr + i);
-      d = fmaf(qs[sub * quarter + i], __low2float(kk), d);
-      d = fmaf(qs[sub * quarter + i + 1], __high2float(kk), d);
-    }
-    d += __shfl_xor(d, 1, 64);
-    d += __shfl_xor(d, 2, 64);
-    d *= scale;
-    if (sub == 0) sc[j] = d;
-    lmax = fmaxf(lmax, d);
-  }
+  float* sc = att_smem + (size_t)wave * chunk;
+  const uint32_t stride = head_dim + 2;  // floats per partial: max, sum, head_dim sums
+  const uint32_t sub = lane & 15u, pj = lane >> 4;  // 16 lanes x 8 dims (zero-padded) cover a position's row
+  const uint32_t dsteps = (head_dim + 127) >> 7;   // 128-dim passes over a row
+  for (uint32_t g = wave; g < groups; g += kAttnThreads / 64) {
+    const uint32_t head = kvh * groups + g;
+    float m = -INFINITY, l = 0.f;
+    // scores of this wavefront's query head over [j0, j1)
+    for (uint32_t p0 = j0; p0 < j1; p0 += 4) {
+      const uint32_t j = p0 + pj;
+      float d = 0.f;
+      for (uint32_t ds = 0; ds < dsteps; ++ds) {
+        const uint32_t i0 = ds * 128u + sub * 8u;
+        if (j < j1 && i0 < head_dim) {
+          const uint4 kk = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0);
+          const uint4 qq = *reinterpret_cast<const uint4*>(q + (size_t)head * head_dim + i0);
+          const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w}, qw[4] = {qq.x, qq.y, qq.z, qq.w};
 #pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) lmax = fmaxf(lmax, __shfl_xor(lmax, o, 64));
-  if (lane == 0) red[wave] = lmax;
-  __syncthreads();
-  float gmax = red[0];
-  for (uint32_t w = 1; w < kAttnThreads / 64; ++w) gmax = fmaxf(gmax, red[w]);
-  __syncthreads();
-  float lsum = 0.f;
-  for (uint32_t j = tid; j < T; j += kAttnThreads) {
-    const float e = __expf(sc[j] - gmax);
-    sc[j] = e;
-    lsum += e;
+          for (int t = 0; t < 4; ++t) {
+            d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] & 0xFFFFu))),
+                     __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu))), d);
+            d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] >> 16))),
+                     __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16))), d);
+          }
+        }
+      }
+      d += __shfl_xor(d, 1, 64);
+      d += __shfl_xor(d, 2, 64);
+      d += __shfl_xor(d, 4, 64);
+      d += __shfl_xor(d, 8, 64);
+      d *= scale;
+      if (j < j1) {
+        if (sub == 0) sc[j - j0] = d;
+        m = fmaxf(m, d);
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    for (uint32_t j = j0 + lane; j < j1; j += 64) {
+      const float e = __expf(sc[j - j0] - m);
+      sc[j - j0] = e;
+      l += e;
+    }
+    l = wave_sum(l);
+    __threadfence_block();
+    // weighted V sum: lane owns dims 2 lane, 2 lane + 1 of each 128-dim pass
+    float* dst = part + ((size_t)head * kAttnSplits + split) * stride;
+    for (uint32_t ds = 0; ds < dsteps; ++ds) {
+      const uint32_t i0 = ds * 128u + lane * 2u;
+      float a0 = 0.f, a1 = 0.f;
+      if (i0 < head_dim)
+        for (uint32_t j = j0; j < j1; ++j) {
+          const __half2 vv = *reinterpret_cast<const __half2*>(V + (size_t)j * head_dim + i0);
+          const float p = sc[j - j0];
+          a0 = fmaf(p, __low2float(vv), a0);
+          a1 = fmaf(p, __high2float(vv), a1);
+        }
+      if (i0 < head_dim) {
+        dst[2 + i0] = a0;
+        dst[2 + i0 + 1] = a1;
+      }
+    }
+    if (lane == 0) {
+      dst[0] = m;  // -inf for an empty range
+      dst[1] = l;
+    }
+    __builtin_amdgcn_wave_barrier();  // sc is reused by this wavefront's next query head
   }
-  lsum = wave_sum(lsum);
-  if (lane == 0) red[wave] = lsum;
+  // publish, and let the last workgroup of this kv head merge (one lane's
+  // device-scope release / acquire stands for the workgroup, ordered by the barriers)
   __syncthreads();
-  float gsum = 0.f;
-  for (uint32_t w = 0; w < kAttnThreads / 64; ++w) gsum += red[w];
-  const float inv = 1.0f / gsum;
-  // context: lane d of each half of the workgroup walks half of the positions
-  float* part = red + kAttnThreads / 64;
-  const uint32_t hsel = tid / (kAttnThreads / 2), d0 = tid % (kAttnThreads / 2);
-  for (uint32_t d = d0; d < head_dim; d += kAttnThreads / 2) {
-    float a = 0.f;
-    for (uint32_t j = hsel; j < T; j += 2) a = fmaf(sc[j], __half2float(V[(size_t)j * head_dim + d]), a);
-    part[hsel * head_dim + d] = a;
+  if (tid == 0) arrived = __hip_atomic_fetch_add(&counters[kvh], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (arrived != kAttnSplits - 1) return;
+  for (uint32_t o = tid; o < groups * head_dim; o += kAttnThreads) {
+    const uint32_t g = o / head_dim, i = o - g * head_dim;
+    const uint32_t head = kvh * groups + g;
+    const float* src = part + (size_t)head * kAttnSplits * stride;
+    float M = -INFINITY;
+    for (uint32_t s = 0; s < kAttnSplits; ++s) M = fmaxf(M, src[(size_t)s * stride]);
+    float L = 0.f, A = 0.f;
+    for (uint32_t s = 0; s < kAttnSplits; ++s) {
+      const float w = __expf(src[(size_t)s * stride] - M);  // 0 for an empty range
+      L = fmaf(src[(size_t)s * stride + 1], w, L);
+      A = fmaf(src[(size_t)s * stride + 2 + i], w, A);
+    }
+    ctx[(size_t)head * head_dim + i] = __float2half_rn(A / L);
   }
-  __syncthreads();
-  for (uint32_t d = tid; d < head_dim; d += kAttnThreads)
-    ctx[(size_t)head * head_dim + d] = __float2half_rn((part[d] + part[head_dim + d]) * inv);
+  if (tid == 0) counters[kvh] = 0;  // ready for the next launch
 }
 
 // act = f16(f16(silu(gate)) * up)   (model.rs:831: gu[0].apply(act).mul(gu[1]))

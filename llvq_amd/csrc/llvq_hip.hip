@@ -1011,6 +1011,8 @@ struct llvq_decoder {
   uint32_t* best_idx = nullptr;
   uint32_t* token = nullptr;    // the token the next step embeds
   uint32_t* history = nullptr;  // [max_pos] tokens chosen by the head
+  float* attn_part = nullptr;   // [n_heads][kAttnSplits][head_dim + 2] partial attention sums
+  uint32_t* attn_counters = nullptr;  // [n_kv], zero between launches
   uint32_t pos = 0;
   uint32_t head_grid = 0;
 };
@@ -1026,7 +1028,7 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, d->h);
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
   const uint32_t T = d->pos + 1;
-  const size_t attn_lds = ((size_t)d->head_dim * 3 + T + kAttnThreads / 64) * sizeof(float);
+  const size_t attn_lds = (size_t)(kAttnThreads / 64) * ((T + kAttnSplits - 1) / kAttnSplits) * sizeof(float);
   for (uint32_t L = 0; L < d->n_layers; ++L) {
     const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
     // the previous layer's MLP output joins the residual stream here
@@ -1039,9 +1041,9 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
                        d->qn + (size_t)L * d->head_dim, d->kn + (size_t)L * d->head_dim, d->cos_t, d->sin_t,
                        d->kcache + L * cache_layer, d->vcache + L * cache_layer, d->n_heads, d->n_kv, d->head_dim, d->pos,
                        d->max_pos, d->eps);
-    hipLaunchKernelGGL(attn_decode_kernel, dim3(d->n_heads), dim3(kAttnThreads), attn_lds, st, d->q, d->kcache + L * cache_layer,
-                       d->vcache + L * cache_layer, d->ctx, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
-                       1.0f / sqrtf((float)d->head_dim));
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(d->n_kv * kAttnSplits), dim3(kAttnThreads), attn_lds, st, d->q,
+                       d->kcache + L * cache_layer, d->vcache + L * cache_layer, d->ctx, d->attn_part, d->attn_counters,
+                       d->n_heads, d->n_kv, d->head_dim, T, d->max_pos, 1.0f / sqrtf((float)d->head_dim));
     void* o_out[1] = {d->o};
     rc = launch_group(rt, P + 3, 1, d->ctx, o_out, LLVQ_F16);
     if (rc) return rc;
@@ -1137,6 +1139,7 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   const size_t n_best = (size_t)d->head_grid * (kHeadThreads / 64);
   const size_t o_bv = take(n_best * sizeof(float)), o_bi = take(n_best * sizeof(uint32_t));
   const size_t o_tok = take(sizeof(uint32_t)), o_hist = take((size_t)c->max_positions * sizeof(uint32_t));
+  const size_t o_ap = take((size_t)c->n_heads * kAttnSplits * (c->head_dim + 2) * sizeof(float)), o_ac = take((size_t)c->n_kv_heads * sizeof(uint32_t));
   hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->blob), total);
   if (e != hipSuccess) { delete d; return hip_fail(e, "hipMalloc(decoder)"); }
   auto put = [&](size_t at, const void* src, size_t bytes) { return hipMemcpy(d->blob + at, src, bytes, hipMemcpyHostToDevice); };
@@ -1162,8 +1165,8 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   d->best_idx = reinterpret_cast<uint32_t*>(d->blob + o_bi);
   d->token = reinterpret_cast<uint32_t*>(d->blob + o_tok);
   d->history = reinterpret_cast<uint32_t*>(d->blob + o_hist);
-  // attention over a long cache needs more than the default 64 KB of dynamic LDS
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(attn_decode_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  d->attn_part = reinterpret_cast<float*>(d->blob + o_ap);
+  d->attn_counters = reinterpret_cast<uint32_t*>(d->blob + o_ac);
   *out = d;
   return LLVQ_OK;
 }

@@ -37,7 +37,7 @@ class Qwen3Config:
                 (SITES[4], i, h), (SITES[5], i, h), (SITES[6], h, i)]
 
 
-QWEN3_4B = Qwen3Config(36, 2560, 32, 8, 128, 9728, 151936, max_positions=768)
+QWEN3_4B = Qwen3Config(36, 2560, 32, 8, 128, 9728, 151936, max_positions=768, tie_word_embeddings=False)
 
 
 @dataclass
