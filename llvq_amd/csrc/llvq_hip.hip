@@ -12,6 +12,7 @@
 #include <cmath>
 #include <cstring>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "../../include/llvq_hip.h"
@@ -139,9 +140,22 @@ struct MatArg {
   uint32_t tile_begin;  // first tile of this matrix in the launch
 };
 
+// What a launch may do to produce its activation before the product.
+enum : uint32_t {
+  kPrologueNone = 0,
+  kPrologueSiluMul = 1,    // x[i] = f16(f16(silu(x2[i])) * x[i])           (model.rs:831)
+  kPrologueAddRmsNorm = 2  // r = f16(x[i] + x2[i]) (x2 may be null: r = x[i]); resid_out = r;
+                           // x[i] = f16(r / sqrt(mean(r^2) + eps) * norm_w[i])  (model.rs:781, :827-829)
+};
+
 struct GroupArgs {
   GlobalTables tables;
   const __half* x;
+  const __half* x2;
+  const __half* norm_w;
+  __half* resid_out;  // written by workgroup 0 only; must not alias x
+  float eps;
+  uint32_t prologue;
   uint32_t nblocks, tail_w, n_mats, rows_per_tile, n_tiles;
   float inv_nblocks;  // 1 / nblocks, for the block -> column split
   MatArg m[kMaxGroup];
@@ -287,9 +301,56 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   static_assert(kRawBytes <= 2 * 16 * kWgThreads, "two 16-byte registers per lane hold a tile's code bytes");
   uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0;
   prefetch_tile(a, blockIdx.x, tid, pre0, pre1);
+  const __half* xsrc = a.x;
+  if (a.prologue != kPrologueNone) {
+    // Every workgroup derives the activation for itself (a few thousand values)
+    // instead of waiting for a kernel of its own; it is staged, as binary16, where
+    // the tile's code bytes will go.
+    __half* xs = reinterpret_cast<__half*>(raw);
+    const uint32_t d_in = nb * kDim + a.tail_w;
+    if (a.prologue == kPrologueSiluMul) {
+      for (uint32_t i = tid; i < d_in; i += kWgThreads) {
+        const float g = __half2float(a.x2[i]);
+        const float sg = __half2float(__float2half_rn(g / (1.0f + __expf(-g))));
+        xs[i] = __float2half_rn(sg * __half2float(a.x[i]));
+      }
+    } else {
+      float* red = partial;  // free until the first tile's P2
+      constexpr int kPer = (kRawBytes / 2 + kWgThreads - 1) / kWgThreads;
+      float v[kPer];
+      float ss = 0.f;
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) {
+        const uint32_t i = tid + (uint32_t)k * kWgThreads;
+        v[k] = 0.f;
+        if (i < d_in) {
+          float r = __half2float(a.x[i]);
+          if (a.x2) r = __half2float(__float2half_rn(r + __half2float(a.x2[i])));
+          if (a.resid_out && blockIdx.x == 0) a.resid_out[i] = __float2half_rn(r);
+          v[k] = r;
+          ss += r * r;
+        }
+      }
+      ss = wave_sum(ss);
+      if (lane == 0) red[wave] = ss;
+      __syncthreads();
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) total += red[w];
+      const float inv = 1.0f / sqrtf(total / (float)d_in + a.eps);
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) {
+        const uint32_t i = tid + (uint32_t)k * kWgThreads;
+        if (i < d_in) xs[i] = __float2half_rn(v[k] * inv * __half2float(a.norm_w[i]));
+      }
+    }
+    __syncthreads();
+    xsrc = xs;
+  }
   for (uint32_t col = tid; col < nb; col += kWgThreads)
-    quantize_block(a.x + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
-  if (tid < a.tail_w) xtail[tid] = __half2float(a.x[(size_t)nb * kDim + tid]);
+    quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+  if (tid < a.tail_w) xtail[tid] = __half2float(xsrc[(size_t)nb * kDim + tid]);
+  if (a.prologue != kPrologueNone) __syncthreads();  // the staging area becomes the code-byte buffer
 
 #ifdef LLVQ_PHASE_TIMING
   if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 7] = wall_clock64();
@@ -814,8 +875,16 @@ static uint32_t pick_rows_per_tile(const llvq_mat* const* mats, int n, uint32_t 
   return r < 1 ? 1 : r;
 }
 
+struct Prologue {
+  uint32_t kind = kPrologueNone;
+  const void* x2 = nullptr;
+  const void* norm_w = nullptr;
+  void* resid_out = nullptr;
+  float eps = 0.f;
+};
+
 static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, void* const* y,
-                        int y_dtype) {
+                        int y_dtype, const Prologue* pro = nullptr) {
   const llvq_mat* m0 = mats[0];
   if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv: unknown output dtype");
   const size_t lds = gemv_lds_bytes(m0->nblocks);
@@ -828,6 +897,15 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   GroupArgs a{};
   a.tables = rt->tables;
   a.x = reinterpret_cast<const __half*>(x);
+  if (pro) {
+    if ((size_t)m0->d_in * 2 > (size_t)kRawBytes)
+      return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": d_in too wide for a fused activation prologue");
+    a.prologue = pro->kind;
+    a.x2 = reinterpret_cast<const __half*>(pro->x2);
+    a.norm_w = reinterpret_cast<const __half*>(pro->norm_w);
+    a.resid_out = reinterpret_cast<__half*>(pro->resid_out);
+    a.eps = pro->eps;
+  }
   a.nblocks = m0->nblocks;
   a.tail_w = m0->tail_w;
   a.n_mats = (uint32_t)n;
@@ -1004,7 +1082,7 @@ struct llvq_decoder {
   __half *ln1 = nullptr, *ln2 = nullptr, *qn = nullptr, *kn = nullptr, *fnorm = nullptr;
   __half *embed = nullptr, *head = nullptr, *cos_t = nullptr, *sin_t = nullptr;
   __half *kcache = nullptr, *vcache = nullptr;  // [n_layers][n_kv][max_pos][head_dim]
-  __half *h = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *ctx = nullptr, *o = nullptr;
+  __half *h = nullptr, *h_alt = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *ctx = nullptr, *o = nullptr;
   __half *gate = nullptr, *up = nullptr, *act = nullptr, *down = nullptr;
   float* logits = nullptr;
   float* best_val = nullptr;
@@ -1029,14 +1107,23 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
   const uint32_t T = d->pos + 1;
   const size_t attn_lds = (size_t)(kAttnThreads / 64) * ((T + kAttnSplits - 1) / kAttnSplits) * sizeof(float);
+  // The residual stream alternates between two buffers: a projection launch whose
+  // prologue adds the previous branch reads one and (workgroup 0) writes the other.
   for (uint32_t L = 0; L < d->n_layers; ++L) {
     const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
-    // the previous layer's MLP output joins the residual stream here
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, L ? d->down : (const __half*)nullptr,
-                       d->ln1 + (size_t)L * d->hidden, d->normed, d->hidden, d->eps);
+    // the previous layer's MLP output joins the residual stream in the q/k/v launch
+    Prologue ln1;
+    ln1.kind = kPrologueAddRmsNorm;
+    ln1.norm_w = d->ln1 + (size_t)L * d->hidden;
+    ln1.eps = d->eps;
+    if (L) {
+      ln1.x2 = d->down;
+      ln1.resid_out = d->h_alt;
+    }
     void* qkv_out[3] = {d->q, d->k, d->v};
-    int rc = launch_group(rt, P, 3, d->normed, qkv_out, LLVQ_F16);
+    int rc = launch_group(rt, P, 3, d->h, qkv_out, LLVQ_F16, &ln1);
     if (rc) return rc;
+    if (L) std::swap(d->h, d->h_alt);
     hipLaunchKernelGGL(qk_norm_rope_append_kernel, dim3(d->n_heads + 2 * d->n_kv), dim3(64), 0, st, d->q, d->k, d->v,
                        d->qn + (size_t)L * d->head_dim, d->kn + (size_t)L * d->head_dim, d->cos_t, d->sin_t,
                        d->kcache + L * cache_layer, d->vcache + L * cache_layer, d->n_heads, d->n_kv, d->head_dim, d->pos,
@@ -1047,14 +1134,21 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     void* o_out[1] = {d->o};
     rc = launch_group(rt, P + 3, 1, d->ctx, o_out, LLVQ_F16);
     if (rc) return rc;
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->o, d->ln2 + (size_t)L * d->hidden,
-                       d->normed, d->hidden, d->eps);
+    Prologue ln2;
+    ln2.kind = kPrologueAddRmsNorm;
+    ln2.norm_w = d->ln2 + (size_t)L * d->hidden;
+    ln2.eps = d->eps;
+    ln2.x2 = d->o;
+    ln2.resid_out = d->h_alt;
     void* gu_out[2] = {d->gate, d->up};
-    rc = launch_group(rt, P + 4, 2, d->normed, gu_out, LLVQ_F16);
+    rc = launch_group(rt, P + 4, 2, d->h, gu_out, LLVQ_F16, &ln2);
     if (rc) return rc;
-    hipLaunchKernelGGL(silu_mul_kernel, dim3((d->inter + 255) / 256), dim3(256), 0, st, d->gate, d->up, d->act, d->inter);
+    std::swap(d->h, d->h_alt);
+    Prologue act;
+    act.kind = kPrologueSiluMul;
+    act.x2 = d->gate;
     void* d_out[1] = {d->down};
-    rc = launch_group(rt, P + 6, 1, d->act, d_out, LLVQ_F16);
+    rc = launch_group(rt, P + 6, 1, d->up, d_out, LLVQ_F16, &act);
     if (rc) return rc;
   }
   if (want_logits) {
@@ -1132,7 +1226,7 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   const size_t o_cos = take(cos_h.size() * hb), o_sin = take(sin_h.size() * hb);
   const size_t cache_bytes = (size_t)c->n_layers * c->n_kv_heads * c->max_positions * c->head_dim * hb;
   const size_t o_kc = take(cache_bytes), o_vc = take(cache_bytes);
-  const size_t o_h = take(c->hidden * hb), o_nm = take(c->hidden * hb), o_q = take(qd * hb), o_k = take(kvd * hb), o_v = take(kvd * hb);
+  const size_t o_h = take(c->hidden * hb), o_h2 = take(c->hidden * hb), o_nm = take(c->hidden * hb), o_q = take(qd * hb), o_k = take(kvd * hb), o_v = take(kvd * hb);
   const size_t o_ctx = take(qd * hb), o_o = take(c->hidden * hb), o_g = take(c->intermediate * hb), o_u = take(c->intermediate * hb);
   const size_t o_act = take(c->intermediate * hb), o_dn = take(c->hidden * hb);
   const size_t o_log = take((size_t)c->vocab * sizeof(float));
@@ -1158,7 +1252,7 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   d->ln1 = H(o_ln1); d->ln2 = H(o_ln2); d->qn = H(o_qn); d->kn = H(o_kn); d->fnorm = H(o_fn);
   d->embed = H(o_emb); d->head = H(o_head); d->cos_t = H(o_cos); d->sin_t = H(o_sin);
   d->kcache = H(o_kc); d->vcache = H(o_vc);
-  d->h = H(o_h); d->normed = H(o_nm); d->q = H(o_q); d->k = H(o_k); d->v = H(o_v); d->ctx = H(o_ctx); d->o = H(o_o);
+  d->h = H(o_h); d->h_alt = H(o_h2); d->normed = H(o_nm); d->q = H(o_q); d->k = H(o_k); d->v = H(o_v); d->ctx = H(o_ctx); d->o = H(o_o);
   d->gate = H(o_g); d->up = H(o_u); d->act = H(o_act); d->down = H(o_dn);
   d->logits = reinterpret_cast<float*>(d->blob + o_log);
   d->best_val = reinterpret_cast<float*>(d->blob + o_bv);

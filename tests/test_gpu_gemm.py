@@ -1,10 +1,12 @@
 """Parity of the batched matrix-core path (llvq_hip_gemm, M >= 2) against the
 CPU oracle: Y = X W^T with W the oracle's decoded matrix, in f64.
 
-Bar: |y - y_ref| / sum|w_i x_i| < 1e-3 and plain relative error < 1e-3 where
-|y_ref| is not tiny.  Weights enter the matrix cores as binary16 (one rounding
-of value * centroid / sqrt(16 shell)), accumulation is f32; row scale and tail
-columns are applied in f32.
+Bar: |y - y_ref| / sum|w_i x_i| < 1e-3.  Weights enter the matrix cores as
+binary16 (one rounding of value * centroid / sqrt(16 shell), 2^-11 relative per
+weight), accumulation is f32; row scale and tail columns are applied in f32.
+That rounding is of the order of 1e-4 of sum|w_i x_i|, so the plain relative
+error of an output is below 1e-3 only where the sum does not cancel
+(|y_ref| >= 0.2 sum|w_i x_i|); both are asserted.
 """
 import numpy as np
 import pytest
@@ -33,10 +35,10 @@ def _check(Y, Y_ref, A_ref, tol=TOL):
     Y = Y.astype(np.float64)
     e = np.abs(Y - Y_ref) / np.maximum(A_ref, 1e-30)
     assert e.max() < tol, f"max |dy|/sum|wx| = {e.max():.3e}"
-    big = np.abs(Y_ref) > 1e-2 * A_ref
+    big = np.abs(Y_ref) >= 0.2 * A_ref
     if big.any():
         rel = (np.abs(Y - Y_ref)[big] / np.abs(Y_ref)[big]).max()
-        assert rel < 0.1, f"max relative error {rel:.3e}"  # |y| >= 1e-2 sum|wx| turns the bound above into this one
+        assert rel < tol, f"max relative error {rel:.3e}"
     return e.max()
 
 
