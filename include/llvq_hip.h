@@ -40,7 +40,7 @@ typedef enum llvq_status {
   LLVQ_ERR_CODEBOOK_MISMATCH = 10,/* Error::CodebookMismatch */
   LLVQ_ERR_UNKNOWN_VERSION = 11,  /* Error::UnknownVersion */
   LLVQ_ERR_INVALID_ARGUMENT = 32, /* null pointer, wrong shape, unsupported dtype */
-  LLVQ_ERR_UNSUPPORTED = 33,      /* e.g. centroid count != 2, rotated matrix */
+  LLVQ_ERR_UNSUPPORTED = 33,      /* e.g. centroid count != 2, rotation with an odd factor above 32 */
   LLVQ_ERR_DEVICE = 34            /* a HIP call failed; message carries hipGetErrorString */
 } llvq_status;
 
@@ -64,7 +64,7 @@ typedef struct llvq_matrix_desc {
   const uint8_t* codes;      /* packed stream, >= 6 * d_out * (d_in / 24) bytes */
   size_t code_bytes;
   uint64_t rotation_seed;
-  uint32_t has_rotation;     /* rotated matrices are refused (LLVQ_ERR_UNSUPPORTED) */
+  uint32_t has_rotation;     /* stored as W Q^T: the activation is rotated by Q(d_in, rotation_seed) first */
 } llvq_matrix_desc;
 
 /* FusedRuntime::new (fused_cuda.rs:182): builds the Golay / class tables on the
@@ -115,12 +115,30 @@ int llvq_hip_matrix_info(const llvq_mat* m, uint32_t* d_out, uint32_t* d_in, uin
                          uint32_t* tail_w, uint64_t* device_bytes);
 const char* llvq_hip_matrix_name(const llvq_mat* m);
 
-/* forward_rotated (fused_cuda.rs:384) for one activation: y = W x.
+/* Proj::forward (model.rs:337-345) = rotate + forward_rotated for one activation:
+ * y = W x in the natural basis, whatever basis the matrix is stored in.
  * x: d_in binary16 values on the device; y: d_out values of y_dtype. */
 int llvq_hip_gemv(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, void* y_dev, int y_dtype);
 
+/* FusedRuntime::rotate (fused_cuda.rs:362): one binary16 activation into the
+ * basis the matrix was quantized in, x' = Q x with Q = Rotation::new(d_in, seed)
+ * (llvq-quant/src/rotation.rs:60-105), as d_in f32 values.  A natural-basis
+ * matrix widens the activation unchanged.  Odd factors of d_in above 32 are
+ * refused at upload (fused.rs:698-704). */
+int llvq_hip_rotate(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, float* xr_f32_dev);
+/* FusedRuntime::forward_rotated (fused_cuda.rs:384): y = W' xr for an activation
+ * already in the matrix's basis (llvq_hip_rotate's output). */
+int llvq_hip_gemv_rotated(llvq_rt* rt, const llvq_mat* m, const float* xr_f32_dev, void* y_dev, int y_dtype);
+/* The same rotation on the host, from the tables the kernels are handed (sign
+ * bitmap, f32 mixing block, f32 1/sqrt m) with f64 arithmetic: v <- Q v.  The
+ * check of fused.rs:1272-1331 ("the tables describe the rotation").  Needs no GPU. */
+int llvq_hip_host_rotate(uint32_t n, uint64_t seed, double* v);
+/* RotKey of a matrix (fused.rs:672-674): whether it is stored rotated, and the seed. */
+int llvq_hip_matrix_rotation(const llvq_mat* m, uint32_t* has_rotation, uint64_t* seed);
+
 /* group_forward (llvq-llm/src/model.rs:497-536) for projections that share an
- * activation (q/k/v, gate/up): one launch over the concatenated rows. */
+ * activation (q/k/v, gate/up): one launch over the concatenated rows of
+ * consecutive matrices that share a basis; the activation is rotated once per basis. */
 int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x_f16_dev,
                         void* const* y_dev, int y_dtype);
 

@@ -41,11 +41,12 @@ __global__ __launch_bounds__(256) void embed_kernel(const __half* __restrict__ t
     h[i] = table[(size_t)t * hidden + i];
 }
 
-// h <- f16(h + delta) when delta is given; normed = f16(h / sqrt(mean(h^2) + eps) * w)
+// r = f16(h + delta) when delta is given (else h), written to h_out when that is given
+// (it may be h itself); normed = f16(r / sqrt(mean(r^2) + eps) * w)
 // (candle_nn::RmsNorm: f32 inside, one rounding on the way out).
-__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(__half* __restrict__ h, const __half* __restrict__ delta,
-                                                                   const __half* __restrict__ w, __half* __restrict__ normed,
-                                                                   uint32_t n, float eps) {
+__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(const __half* h, const __half* __restrict__ delta,
+                                                                   const __half* __restrict__ w, __half* h_out,
+                                                                   __half* __restrict__ normed, uint32_t n, float eps) {
   __shared__ float red[kNormThreads / 64];
   constexpr int kPer = 8;  // n <= 8192
   float v[kPer];
@@ -56,10 +57,8 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(__half* __res
     v[k] = 0.f;
     if (i < n) {
       float x = __half2float(h[i]);
-      if (delta) {
-        x = __half2float(__float2half_rn(x + __half2float(delta[i])));  // the residual stream is binary16
-        h[i] = __float2half_rn(x);
-      }
+      if (delta) x = __half2float(__float2half_rn(x + __half2float(delta[i])));  // the residual stream is binary16
+      if (h_out) h_out[i] = __float2half_rn(x);
       v[k] = x;
       ss += x * x;
     }

@@ -19,6 +19,7 @@
 #include "artifact.hpp"
 #include "codebook.hpp"
 #include "decode_core.h"
+#include "rotation.hpp"
 
 namespace llvq {
 
@@ -151,6 +152,7 @@ enum : uint32_t {
 struct GroupArgs {
   GlobalTables tables;
   const __half* x;
+  const float* x_f32;  // when set, the activation is these f32 values (a rotated activation) and x is unused
   const __half* x2;
   const __half* norm_w;
   __half* resid_out;  // written by workgroup 0 only; must not alias x
@@ -191,8 +193,7 @@ __device__ __forceinline__ void queue_push(uint32_t* counter, uint32_t* queue, b
 }
 
 // One 24-column block of the activation -> scale and byte planes.
-__device__ __forceinline__ void quantize_block(const __half* x, uint32_t* planes, float* scale) {
-  float v[kDim];
+__device__ __forceinline__ void load_block_f16(const __half* x, float (&v)[kDim]) {
   if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
     const uint4* src = reinterpret_cast<const uint4*>(x);
 #pragma unroll
@@ -209,12 +210,31 @@ __device__ __forceinline__ void quantize_block(const __half* x, uint32_t* planes
 #pragma unroll
     for (int j = 0; j < kDim; ++j) v[j] = __half2float(x[j]);
   }
+}
+
+__device__ __forceinline__ void quantize_values(const float (&v)[kDim], uint32_t* planes, float* scale);
+
+__device__ __forceinline__ void quantize_block(const __half* x, uint32_t* planes, float* scale) {
+  float v[kDim];
+  load_block_f16(x, v);
+  quantize_values(v, planes, scale);
+}
+
+// f32 activation (a rotated one, fused_cuda.rs:384): same block-scaled fixed point
+__device__ __forceinline__ void quantize_block_f32(const float* x, uint32_t* planes, float* scale) {
+  float v[kDim];
+#pragma unroll
+  for (int j = 0; j < kDim; ++j) v[j] = x[j];
+  quantize_values(v, planes, scale);
+}
+
+__device__ __forceinline__ void quantize_values(const float (&v)[kDim], uint32_t* planes, float* scale) {
   float amax = 0.f;
 #pragma unroll
   for (int j = 0; j < kDim; ++j) amax = fmaxf(amax, fabsf(v[j]));
   bool bad = false;
 #pragma unroll
-  for (int j = 0; j < kDim; ++j) bad |= !(fabsf(v[j]) <= 65504.f);  // inf or NaN
+  for (int j = 0; j < kDim; ++j) bad |= !(fabsf(v[j]) <= 3.4028234e38f);  // inf or NaN
   int e = 0;
   (void)frexpf(amax, &e);  // amax = m 2^e, m in [0.5, 1)
   const float up = ldexpf(1.f, 22 - e);
@@ -347,9 +367,15 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     __syncthreads();
     xsrc = xs;
   }
-  for (uint32_t col = tid; col < nb; col += kWgThreads)
-    quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
-  if (tid < a.tail_w) xtail[tid] = __half2float(xsrc[(size_t)nb * kDim + tid]);
+  if (a.x_f32) {
+    for (uint32_t col = tid; col < nb; col += kWgThreads)
+      quantize_block_f32(a.x_f32 + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+    if (tid < a.tail_w) xtail[tid] = a.x_f32[(size_t)nb * kDim + tid];
+  } else {
+    for (uint32_t col = tid; col < nb; col += kWgThreads)
+      quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+    if (tid < a.tail_w) xtail[tid] = __half2float(xsrc[(size_t)nb * kDim + tid]);
+  }
   if (a.prologue != kPrologueNone) __syncthreads();  // the staging area becomes the code-byte buffer
 
 #ifdef LLVQ_PHASE_TIMING
@@ -572,6 +598,65 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   }
 }
 
+
+// ---- incoherence rotation of an activation ----------------------------------------
+// x' = Q x for Q = (S (x) I_m)(I_k (x) H_m / sqrt m) D (llvq-quant/src/rotation.rs:97-105),
+// in f32 like the reference's device rotation (llvq-cuda/kernels/llvq_rot.cuh): signs on
+// load, radix-2 Walsh-Hadamard butterflies inside each group of m, then the k x k block
+// across groups with the 1/sqrt m factor applied first.  One workgroup per activation row.
+struct RotArgs {
+  const __half* x;        // [rows, n]
+  void* out;              // [rows, n] f32 or f16
+  const uint32_t* signbits;
+  const float* small;     // k x k
+  uint32_t n, m, k;
+  float inv;
+};
+
+// the identity rotation: binary16 -> f32
+__global__ __launch_bounds__(256) void widen_kernel(const __half* __restrict__ x, float* __restrict__ out, uint32_t n) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = __half2float(x[i]);
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(1024) void rotate_kernel(RotArgs a) {
+  extern __shared__ __align__(16) float rot_s[];
+  const uint32_t tid = threadIdx.x, n = a.n, m = a.m, k = a.k;
+  const __half* x = a.x + (size_t)blockIdx.x * n;
+  for (uint32_t i = tid; i < n; i += 1024) {
+    const float v = __half2float(x[i]);
+    rot_s[i] = ((a.signbits[i >> 5] >> (i & 31u)) & 1u) ? -v : v;
+  }
+  __syncthreads();
+  for (uint32_t len = 1; len < m; len <<= 1) {  // groups are contiguous, so one pass covers all of them
+    for (uint32_t p = tid; p < (n >> 1); p += 1024) {
+      const uint32_t j = (p / len) * (len << 1) + (p % len);
+      const float u = rot_s[j], w = rot_s[j + len];
+      rot_s[j] = u + w;
+      rot_s[j + len] = u - w;
+    }
+    __syncthreads();
+  }
+  OutT* out = reinterpret_cast<OutT*>(a.out) + (size_t)blockIdx.x * n;
+  if (k == 1) {
+    for (uint32_t i = tid; i < n; i += 1024) out[i] = (OutT)(rot_s[i] * a.inv);
+    return;
+  }
+  for (uint32_t j = tid; j < m; j += 1024) {
+    float col[kRotKMax];
+#pragma unroll
+    for (uint32_t t = 0; t < kRotKMax; ++t) col[t] = t < k ? rot_s[t * m + j] * a.inv : 0.f;
+    for (uint32_t g = 0; g < k; ++g) {
+      float acc = 0.f;
+#pragma unroll
+      for (uint32_t t = 0; t < kRotKMax; ++t)
+        if (t < k) acc = fmaf(a.small[g * k + t], col[t], acc);
+      out[g * m + j] = (OutT)acc;
+    }
+  }
+}
+
 }  // namespace llvq
 
 #include "gemm_kernel.h"
@@ -588,6 +673,20 @@ struct llvq_rt {
   uint8_t* blob = nullptr;  // one device allocation holding every table
   GlobalTables tables{};
   int cu_count = 0;
+  // rotations by (width, seed) — shared by every matrix that consumes the same activation
+  // (llvq-llm/src/fused.rs:672-674) — and the scratch rotated activations land in
+  struct DevRotation {
+    uint32_t n = 0, m = 0, k = 0;
+    uint64_t seed = 0;
+    float inv = 1.f;
+    uint32_t* signbits = nullptr;
+    float* small = nullptr;
+  };
+  std::vector<DevRotation*> rotations;
+  float* rot_scratch = nullptr;   // one rotated activation, f32
+  size_t rot_scratch_elems = 0;
+  __half* rot_rows = nullptr;     // rotated batch rows, f16 (matrix-core path)
+  size_t rot_rows_elems = 0;
   // split-K state of the batched kernel: partial sums and per-band arrival counters
   float* gemm_ws = nullptr;
   size_t gemm_ws_bytes = 0;
@@ -604,6 +703,9 @@ struct llvq_mat {
   float* tail = nullptr;     // device
   uint64_t device_bytes = 0;
   uint64_t encoded_bytes = 0;
+  bool has_rotation = false;
+  uint64_t rotation_seed = 0;
+  const llvq_rt::DevRotation* rot = nullptr;  // owned by the runtime
 };
 
 static thread_local std::string g_last_error;
@@ -677,6 +779,8 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   const int max_lds = 160 * 1024;
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<2, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
@@ -691,6 +795,13 @@ void llvq_hip_runtime_destroy(llvq_rt* rt) {
   (void)hipFree(rt->blob);
   (void)hipFree(rt->gemm_ws);
   (void)hipFree(rt->gemm_counters);
+  (void)hipFree(rt->rot_scratch);
+  (void)hipFree(rt->rot_rows);
+  for (auto* r : rt->rotations) {
+    (void)hipFree(r->signbits);
+    (void)hipFree(r->small);
+    delete r;
+  }
   delete rt;
 }
 
@@ -706,10 +817,44 @@ int llvq_hip_synchronize(llvq_rt* rt) {
   return LLVQ_OK;
 }
 
+// The device tables of rotation (n, seed), built once per runtime.  Also makes
+// sure the f32 scratch holds n values.
+static int runtime_rotation(llvq_rt* rt, uint32_t n, uint64_t seed, const llvq_rt::DevRotation** out) {
+  for (auto* r : rt->rotations)
+    if (r->n == n && r->seed == seed) { *out = r; return LLVQ_OK; }
+  RotationTables t;
+  std::string err;
+  if (!build_rotation(n, seed, &t, &err)) return fail(LLVQ_ERR_UNSUPPORTED, err);
+  if ((size_t)n * sizeof(float) > 160 * 1024 - 64)
+    return fail(LLVQ_ERR_UNSUPPORTED, "width " + std::to_string(n) + " does not fit the rotation kernel's LDS");
+  auto* r = new llvq_rt::DevRotation();
+  r->n = t.n; r->m = t.m; r->k = t.k; r->seed = seed; r->inv = t.inv;
+  hipError_t e = hipMalloc(reinterpret_cast<void**>(&r->signbits), t.signbits.size() * 4);
+  if (e == hipSuccess) e = hipMemcpy(r->signbits, t.signbits.data(), t.signbits.size() * 4, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&r->small), t.small.size() * 4);
+  if (e == hipSuccess) e = hipMemcpy(r->small, t.small.data(), t.small.size() * 4, hipMemcpyHostToDevice);
+  if (e == hipSuccess && n > rt->rot_scratch_elems) {
+    (void)hipFree(rt->rot_scratch);
+    rt->rot_scratch = nullptr;
+    rt->rot_scratch_elems = 0;
+    e = hipMalloc(reinterpret_cast<void**>(&rt->rot_scratch), (size_t)n * sizeof(float));
+    if (e == hipSuccess) rt->rot_scratch_elems = n;
+  }
+  if (e != hipSuccess) {
+    (void)hipFree(r->signbits);
+    (void)hipFree(r->small);
+    delete r;
+    return hip_fail(e, "rotation tables");
+  }
+  rt->rotations.push_back(r);
+  *out = r;
+  return LLVQ_OK;
+}
+
 static int upload_impl(llvq_rt* rt, const std::string& name, uint32_t d_out, uint32_t d_in,
                        uint32_t shell_cap, uint32_t n_centroids, const double* centroids,
                        const double* row_scales, const float* tail, const uint8_t* codes,
-                       size_t code_bytes, bool has_rotation, llvq_mat** out) {
+                       size_t code_bytes, bool has_rotation, uint64_t rotation_seed, llvq_mat** out) {
   if (shell_cap > (uint32_t)kMaxShell)
     return fail(LLVQ_ERR_INCONSISTENT, name + ": shell cap " + std::to_string(shell_cap) +
                                            " exceeds the supported ball (m <= 13)");
@@ -722,8 +867,6 @@ static int upload_impl(llvq_rt* rt, const std::string& name, uint32_t d_out, uin
     return fail(LLVQ_ERR_UNSUPPORTED, name + ": shell cap " + std::to_string(shell_cap) + " packs " +
                                           std::to_string(ib + 1) +
                                           " bits per block; the kernels read 6-byte records (cap 12)");
-  if (has_rotation)
-    return fail(LLVQ_ERR_UNSUPPORTED, name + ": stored in a rotated basis; activation rotation is not built yet");
   const uint32_t nblocks = d_in / kDim, tail_w = d_in % kDim;
   const uint64_t total_blocks = (uint64_t)d_out * nblocks;
   if ((unsigned __int128)total_blocks * 48 > (unsigned __int128)code_bytes * 8)
@@ -745,7 +888,15 @@ static int upload_impl(llvq_rt* rt, const std::string& name, uint32_t d_out, uin
   }
 
   HIP_TRY(hipSetDevice(rt->device));
+  const llvq_rt::DevRotation* rot = nullptr;
+  if (has_rotation) {
+    const int rc = runtime_rotation(rt, d_in, rotation_seed, &rot);
+    if (rc) return rc;
+  }
   auto* m = new llvq_mat();
+  m->has_rotation = has_rotation;
+  m->rotation_seed = rotation_seed;
+  m->rot = rot;
   m->name = name;
   m->d_out = d_out;
   m->d_in = d_in;
@@ -785,7 +936,7 @@ int llvq_hip_matrix_upload(llvq_rt* rt, const llvq_matrix_desc* d, llvq_mat** ou
   *out = nullptr;
   return upload_impl(rt, d->name ? d->name : "", d->d_out, d->d_in, d->shell_cap, d->n_centroids,
                      d->centroids, d->row_scales, d->tail, d->codes, d->code_bytes,
-                     d->has_rotation != 0, out);
+                     d->has_rotation != 0, d->rotation_seed, out);
 }
 
 int llvq_hip_read_header(const uint8_t* buf, size_t len, size_t* pos, uint32_t* version,
@@ -832,7 +983,7 @@ int llvq_hip_matrix_from_record(llvq_rt* rt, const uint8_t* buf, size_t len, siz
   int rc = parse_matrix_record(buf, len, &p, &r, &err);
   if (rc) return fail(rc, err);
   rc = upload_impl(rt, r.name, r.d_out, r.d_in, r.shell_cap, r.n_centroids, r.centroids.data(),
-                   r.row_scales.data(), r.tail.data(), r.codes, r.code_bytes, r.has_rotation, out);
+                   r.row_scales.data(), r.tail.data(), r.codes, r.code_bytes, r.has_rotation, r.rotation_seed, out);
   if (rc == LLVQ_OK) *pos = p;
   return rc;
 }
@@ -884,7 +1035,7 @@ struct Prologue {
 };
 
 static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, void* const* y,
-                        int y_dtype, const Prologue* pro = nullptr) {
+                        int y_dtype, const Prologue* pro = nullptr, const float* x_f32 = nullptr) {
   const llvq_mat* m0 = mats[0];
   if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv: unknown output dtype");
   const size_t lds = gemv_lds_bytes(m0->nblocks);
@@ -897,6 +1048,7 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   GroupArgs a{};
   a.tables = rt->tables;
   a.x = reinterpret_cast<const __half*>(x);
+  a.x_f32 = x_f32;
   if (pro) {
     if ((size_t)m0->d_in * 2 > (size_t)kRawBytes)
       return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": d_in too wide for a fused activation prologue");
@@ -927,14 +1079,93 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   return LLVQ_OK;
 }
 
+// Enqueues x' = Q x for `rows` activation rows of width rot->n.
+static int launch_rotate(llvq_rt* rt, const llvq_rt::DevRotation* rot, const void* x_f16, uint32_t rows, void* out,
+                         bool out_f16) {
+  RotArgs a{};
+  a.x = reinterpret_cast<const __half*>(x_f16);
+  a.out = out;
+  a.signbits = rot->signbits;
+  a.small = rot->small;
+  a.n = rot->n;
+  a.m = rot->m;
+  a.k = rot->k;
+  a.inv = rot->inv;
+  const size_t lds = (size_t)rot->n * sizeof(float);
+  if (out_f16) hipLaunchKernelGGL(rotate_kernel<__half>, dim3(rows), dim3(1024), lds, rt->stream, a);
+  else hipLaunchKernelGGL(rotate_kernel<float>, dim3(rows), dim3(1024), lds, rt->stream, a);
+  HIP_TRY(hipGetLastError());
+  return LLVQ_OK;
+}
+
+static bool same_basis(const llvq_mat* a, const llvq_mat* b) {
+  return a->has_rotation == b->has_rotation && (!a->has_rotation || a->rotation_seed == b->rotation_seed);
+}
+
+// One activation through projections that share it: consecutive matrices in the
+// same basis go out as one launch (at most kMaxGroup); a rotated basis gets its
+// activation rotated once, into the runtime's scratch, before its launches.
+static int forward_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, void* const* y, int y_dtype) {
+  int i = 0;
+  while (i < n) {
+    int j = i + 1;
+    while (j < n && j - i < kMaxGroup && same_basis(mats[i], mats[j])) ++j;
+    const float* xr = nullptr;
+    if (mats[i]->has_rotation) {
+      // the scratch may still hold this very rotation if the previous run used it; rotating again is cheap and always right
+      const int rc = launch_rotate(rt, mats[i]->rot, x, 1, rt->rot_scratch, false);
+      if (rc) return rc;
+      xr = rt->rot_scratch;
+    }
+    const int rc = launch_group(rt, mats + i, j - i, x, y + i, y_dtype, nullptr, xr);
+    if (rc) return rc;
+    i = j;
+  }
+  return LLVQ_OK;
+}
+
 static int launch_gemv(llvq_rt* rt, const llvq_mat* m, const void* x, void* y, int y_dtype) {
-  return launch_group(rt, &m, 1, x, &y, y_dtype);
+  return forward_group(rt, &m, 1, x, &y, y_dtype);
 }
 
 int llvq_hip_gemv(llvq_rt* rt, const llvq_mat* m, const void* x, void* y, int y_dtype) {
   if (!rt || !m || !x || !y) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv: null argument");
   HIP_TRY(hipSetDevice(rt->device));
   return launch_gemv(rt, m, x, y, y_dtype);
+}
+
+int llvq_hip_rotate(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, float* xr_f32_dev) {
+  if (!rt || !m || !x_f16_dev || !xr_f32_dev) return fail(LLVQ_ERR_INVALID_ARGUMENT, "rotate: null argument");
+  HIP_TRY(hipSetDevice(rt->device));
+  if (m->has_rotation) return launch_rotate(rt, m->rot, x_f16_dev, 1, xr_f32_dev, false);
+  hipLaunchKernelGGL(widen_kernel, dim3((m->d_in + 255) / 256), dim3(256), 0, rt->stream,
+                     reinterpret_cast<const __half*>(x_f16_dev), xr_f32_dev, m->d_in);
+  HIP_TRY(hipGetLastError());
+  return LLVQ_OK;
+}
+
+int llvq_hip_gemv_rotated(llvq_rt* rt, const llvq_mat* m, const float* xr_f32_dev, void* y, int y_dtype) {
+  if (!rt || !m || !xr_f32_dev || !y) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv_rotated: null argument");
+  HIP_TRY(hipSetDevice(rt->device));
+  return launch_group(rt, &m, 1, nullptr, &y, y_dtype, nullptr, xr_f32_dev);
+}
+
+int llvq_hip_host_rotate(uint32_t n, uint64_t seed, double* v) {
+  if (!v) return fail(LLVQ_ERR_INVALID_ARGUMENT, "host_rotate: null vector");
+  RotationTables t;
+  std::string err;
+  if (!build_rotation(n, seed, &t, &err)) return fail(LLVQ_ERR_UNSUPPORTED, err);
+  std::vector<double> w(v, v + n);
+  host_rotate(t, &w);
+  std::memcpy(v, w.data(), (size_t)n * sizeof(double));
+  return LLVQ_OK;
+}
+
+int llvq_hip_matrix_rotation(const llvq_mat* m, uint32_t* has_rotation, uint64_t* seed) {
+  if (!m) return fail(LLVQ_ERR_INVALID_ARGUMENT, "matrix_rotation: matrix is null");
+  if (has_rotation) *has_rotation = m->has_rotation ? 1u : 0u;
+  if (seed) *seed = m->rotation_seed;
+  return LLVQ_OK;
 }
 
 int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x,
@@ -946,12 +1177,7 @@ int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
       return fail(LLVQ_ERR_INVALID_ARGUMENT, mats[i]->name + ": projections of one group must share d_in");
   }
   HIP_TRY(hipSetDevice(rt->device));
-  for (int i = 0; i < n; i += kMaxGroup) {
-    const int k = n - i < kMaxGroup ? n - i : kMaxGroup;
-    const int rc = launch_group(rt, mats + i, k, x, y + i, y_dtype);
-    if (rc) return rc;
-  }
-  return LLVQ_OK;
+  return forward_group(rt, mats, n, x, y, y_dtype);
 }
 
 // Split of a matrix's block range over work units: the count that minimises a
@@ -1037,6 +1263,26 @@ int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y,
   uint8_t* yb = reinterpret_cast<uint8_t*>(y);
   // The matrix-core kernel reads activations as 16-byte vectors; a single row,
   // or a shape that breaks that alignment, runs as GEMV launches instead.
+  if (m->has_rotation && M >= 2 && m->d_in % 8 == 0 && m->nblocks > 0) {
+    // rows are rotated (f32 inside) and narrowed to the binary16 the matrix cores take
+    const size_t need = (size_t)M * m->d_in;
+    if (need > rt->rot_rows_elems) {
+      (void)hipFree(rt->rot_rows);
+      rt->rot_rows = nullptr;
+      rt->rot_rows_elems = 0;
+      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->rot_rows), need * sizeof(__half)));
+      rt->rot_rows_elems = need;
+    }
+    const int rc = launch_rotate(rt, m->rot, x, (uint32_t)M, rt->rot_rows, true);
+    if (rc) return rc;
+    xb = reinterpret_cast<const uint8_t*>(rt->rot_rows);
+    for (int m0 = 0; m0 < M; m0 += kGemmMaxM) {
+      const uint32_t mc = (uint32_t)(M - m0 < kGemmMaxM ? M - m0 : kGemmMaxM);
+      const int rc2 = launch_gemm(rt, m, xb + (size_t)m0 * m->d_in * 2, mc, yb + (size_t)m0 * m->d_out * esz, y_dtype);
+      if (rc2) return rc2;
+    }
+    return LLVQ_OK;
+  }
   const bool mfma_ok = M >= 2 && m->d_in % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && m->nblocks > 0;
   if (!mfma_ok) {
     for (int r = 0; r < M; ++r) {
@@ -1107,6 +1353,26 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
   const uint32_t T = d->pos + 1;
   const size_t attn_lds = (size_t)(kAttnThreads / 64) * ((T + kAttnSplits - 1) / kAttnSplits) * sizeof(float);
+  // Projections in the natural basis derive their activation in the launch's
+  // prologue; a rotated basis needs the activation as a tensor first (it goes
+  // through the rotation kernel), so its prologue runs as a kernel of its own.
+  auto project = [&](const llvq_mat* const* mats, int n, const __half* x, void* const* outs, const Prologue& pro) -> int {
+    bool rotated = false;
+    for (int i = 0; i < n; ++i) rotated |= mats[i]->has_rotation;
+    if (!rotated) return launch_group(rt, mats, n, x, outs, LLVQ_F16, &pro);
+    const __half* staged = nullptr;
+    if (pro.kind == kPrologueAddRmsNorm) {
+      hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, x, reinterpret_cast<const __half*>(pro.x2),
+                         reinterpret_cast<const __half*>(pro.norm_w), reinterpret_cast<__half*>(pro.resid_out), d->normed,
+                         d->hidden, pro.eps);
+      staged = d->normed;
+    } else {
+      hipLaunchKernelGGL(silu_mul_kernel, dim3((d->inter + 255) / 256), dim3(256), 0, st, reinterpret_cast<const __half*>(pro.x2),
+                         x, d->act, d->inter);
+      staged = d->act;
+    }
+    return forward_group(rt, mats, n, staged, outs, LLVQ_F16);
+  };
   // The residual stream alternates between two buffers: a projection launch whose
   // prologue adds the previous branch reads one and (workgroup 0) writes the other.
   for (uint32_t L = 0; L < d->n_layers; ++L) {
@@ -1121,7 +1387,7 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
       ln1.resid_out = d->h_alt;
     }
     void* qkv_out[3] = {d->q, d->k, d->v};
-    int rc = launch_group(rt, P, 3, d->h, qkv_out, LLVQ_F16, &ln1);
+    int rc = project(P, 3, d->h, qkv_out, ln1);
     if (rc) return rc;
     if (L) std::swap(d->h, d->h_alt);
     hipLaunchKernelGGL(qk_norm_rope_append_kernel, dim3(d->n_heads + 2 * d->n_kv), dim3(64), 0, st, d->q, d->k, d->v,
@@ -1132,7 +1398,7 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
                        d->kcache + L * cache_layer, d->vcache + L * cache_layer, d->ctx, d->attn_part, d->attn_counters,
                        d->n_heads, d->n_kv, d->head_dim, T, d->max_pos, 1.0f / sqrtf((float)d->head_dim));
     void* o_out[1] = {d->o};
-    rc = launch_group(rt, P + 3, 1, d->ctx, o_out, LLVQ_F16);
+    rc = forward_group(rt, P + 3, 1, d->ctx, o_out, LLVQ_F16);
     if (rc) return rc;
     Prologue ln2;
     ln2.kind = kPrologueAddRmsNorm;
@@ -1141,18 +1407,18 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     ln2.x2 = d->o;
     ln2.resid_out = d->h_alt;
     void* gu_out[2] = {d->gate, d->up};
-    rc = launch_group(rt, P + 4, 2, d->h, gu_out, LLVQ_F16, &ln2);
+    rc = project(P + 4, 2, d->h, gu_out, ln2);
     if (rc) return rc;
     std::swap(d->h, d->h_alt);
     Prologue act;
     act.kind = kPrologueSiluMul;
     act.x2 = d->gate;
     void* d_out[1] = {d->down};
-    rc = launch_group(rt, P + 6, 1, d->up, d_out, LLVQ_F16, &act);
+    rc = project(P + 6, 1, d->up, d_out, act);
     if (rc) return rc;
   }
   if (want_logits) {
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->down, d->fnorm, d->normed, d->hidden, d->eps);
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->down, d->fnorm, d->h, d->normed, d->hidden, d->eps);
     hipLaunchKernelGGL(lm_head_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head, d->normed,
                        d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
     hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(1024), 0, st, d->best_val, d->best_idx,

@@ -125,30 +125,38 @@ class FusedRuntime:
             proj.handle = None
 
     # -- the operator ---------------------------------------------------------------
-    def rotate(self, proj: FusedProj, x):
-        """FusedRuntime::rotate (fused_cuda.rs:362): one activation into the basis
-        the projection was quantized in.  Natural-basis matrices pass through."""
+    def _f16(self, x, proj):
         torch = self._torch
-        d_in = x.shape[-1]
-        if d_in != proj.d_in:
-            raise ValueError(f"{proj.name} expects d_in={proj.d_in}, got {d_in}")
-        rows = x.numel() // d_in
-        if rows != 1:
-            raise ValueError(f"{proj.name}: rotation asked for {rows} vectors; the row loop belongs to the caller")
-        if proj.rotation() is not None:
-            raise ValueError(f"{proj.name}: stored in a rotated basis; activation rotation is not built yet")
+        if not x.is_cuda:
+            raise ValueError("the fused LLVQ kernel has no CPU path")
+        if x.shape[-1] != proj.d_in:
+            raise ValueError(f"{proj.name} expects d_in={proj.d_in}, got {x.shape[-1]}")
         return x.to(torch.float16).contiguous()
 
+    def rotate(self, proj: FusedProj, x):
+        """FusedRuntime::rotate (fused_cuda.rs:362): one f16 activation [.., d_in] into the
+        basis the projection was quantized in, as f32 [1, d_in].  Natural-basis matrices
+        only widen it."""
+        torch = self._torch
+        x = self._f16(x, proj)
+        rows = x.numel() // proj.d_in
+        if rows != 1:
+            raise ValueError(f"{proj.name}: rotation asked for {rows} vectors; the row loop belongs to the caller")
+        xr = torch.empty((1, proj.d_in), dtype=torch.float32, device=x.device)
+        _ffi.check(_ffi.lib().llvq_hip_rotate(self.handle, proj.handle, x.data_ptr(), xr.data_ptr()))
+        return xr
+
     def forward_rotated(self, proj: FusedProj, xr, out_dims=None, out_dtype=None):
-        """FusedRuntime::forward_rotated (fused_cuda.rs:384): y = W' xr, shaped like
-        the caller's tensor with the last dim replaced by d_out.  f16 out by default."""
+        """FusedRuntime::forward_rotated (fused_cuda.rs:384): y = W' xr for `rotate`'s f32
+        output, shaped like the caller's tensor with the last dim replaced by d_out.
+        f16 out by default."""
         torch = self._torch
         if not xr.is_cuda:
             raise ValueError("the fused LLVQ kernel has no CPU path")
         if not xr.is_contiguous():
             raise ValueError("activation is not contiguous")
-        if xr.dtype != torch.float16:
-            raise ValueError(f"{proj.name}: activation must be binary16, got {xr.dtype}")
+        if xr.dtype != torch.float32:
+            raise ValueError(f"{proj.name}: a rotated activation is f32, got {xr.dtype}")
         if xr.numel() != proj.d_in:
             raise ValueError(f"rotated activation of {xr.numel()} values for d_in={proj.d_in}")
         out_dtype = out_dtype or torch.float16
@@ -156,38 +164,43 @@ class FusedRuntime:
         dims[-1] = proj.d_out
         y = torch.empty(dims, dtype=out_dtype, device=xr.device)  # uninitialised: every row is stored
         code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
-        _ffi.check(_ffi.lib().llvq_hip_gemv(self.handle, proj.handle, xr.data_ptr(), y.data_ptr(), code))
+        _ffi.check(_ffi.lib().llvq_hip_gemv_rotated(self.handle, proj.handle, xr.data_ptr(), y.data_ptr(), code))
         return y
 
     def forward(self, proj: FusedProj, x, out_dtype=None):
-        return self.forward_rotated(proj, self.rotate(proj, x), x.shape, out_dtype)
+        """Proj::forward (model.rs:337-345): rotate + forward_rotated in one call."""
+        torch = self._torch
+        x = self._f16(x, proj)
+        if x.numel() != proj.d_in:
+            raise ValueError(f"{proj.name}: one activation of {proj.d_in} values expected, got {x.numel()}")
+        out_dtype = out_dtype or torch.float16
+        dims = list(x.shape)
+        dims[-1] = proj.d_out
+        y = torch.empty(dims, dtype=out_dtype, device=x.device)
+        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        _ffi.check(_ffi.lib().llvq_hip_gemv(self.handle, proj.handle, x.data_ptr(), y.data_ptr(), code))
+        return y
 
     def forward_group(self, projs, x, out_dtype=None):
         """group_forward (llvq-llm/src/model.rs:497-536) for projections sharing one activation."""
-        torch = self._torch
-        xr = self.rotate(projs[0], x)
-        out_dtype = out_dtype or torch.float16
-        ys = [torch.empty(list(x.shape[:-1]) + [p.d_out], dtype=out_dtype, device=xr.device) for p in projs]
-        mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
-        outs = (C.c_void_p * len(projs))(*[y.data_ptr() for y in ys])
-        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
-        _ffi.check(_ffi.lib().llvq_hip_gemv_group(self.handle, mats, len(projs), xr.data_ptr(), outs, code))
+        launch, ys = self.plan_group(projs, x, out_dtype)
+        launch()
         return ys
 
     def plan_group(self, projs, x, out_dtype=None):
-        """Pre-binds one launch: returns (launch, outputs).  `launch()` enqueues the
+        """Pre-binds one group call: returns (launch, outputs).  `launch()` enqueues the
         group's GEMV on the runtime's stream with no Python-side allocation or
         argument marshalling — what a decode loop calls once per token."""
         torch = self._torch
-        xr = self.rotate(projs[0], x)
+        x = self._f16(x, projs[0])
         out_dtype = out_dtype or torch.float16
-        ys = [torch.empty(list(x.shape[:-1]) + [p.d_out], dtype=out_dtype, device=xr.device) for p in projs]
+        ys = [torch.empty(list(x.shape[:-1]) + [p.d_out], dtype=out_dtype, device=x.device) for p in projs]
         mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
         outs = (C.c_void_p * len(projs))(*[y.data_ptr() for y in ys])
         code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
         fn = _ffi.lib().llvq_hip_gemv_group
-        rt, n, xp = self.handle, len(projs), C.c_void_p(xr.data_ptr())
-        keep = (xr, ys, mats, outs)
+        rt, n, xp = self.handle, len(projs), C.c_void_p(x.data_ptr())
+        keep = (x, ys, mats, outs)
 
         def launch(_keep=keep):
             rc = fn(rt, mats, n, xp, outs, code)

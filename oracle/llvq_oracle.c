@@ -1175,34 +1175,129 @@ void orc_reconstruct(const int32_t p[ORC_DIM], uint32_t gain, const double* cent
   }
 }
 
-int orc_decode_matrix(const orc_raw_matrix* m, float* w) { /* format.rs:385-439 */
-  if (m->has_rot) return ORC_INCONSISTENT; /* natural basis only */
-  size_t nb = m->d_in / ORC_DIM, tw = m->d_in % ORC_DIM;
-  for (size_t r = 0; r < m->d_out; r++) {
-    for (size_t b = 0; b < nb; b++) {
-      int32_t p[ORC_DIM];
-      double blk[ORC_DIM];
-      size_t k = r * nb + b;
-      if (!orc_index_decode(m->indices[k], p)) return ORC_INDEX_OUT_OF_RANGE;
-      if (m->gains[k] >= m->n_centroids) return ORC_INCONSISTENT;
-      orc_reconstruct(p, m->gains[k], m->centroids, m->row_scales[r], blk);
-      for (int j = 0; j < ORC_DIM; j++) w[r * m->d_in + b * ORC_DIM + j] = (float)blk[j];
+/* ---- rotation (llvq-quant/src/rotation.rs) ----------------------------- */
+int orc_rotation_new(size_t n, uint64_t seed, orc_rotation* r) { /* rotation.rs:60-79 */
+  memset(r, 0, sizeof *r);
+  if (n == 0) return ORC_INCONSISTENT;
+  size_t m = 1;
+  while ((n & m) == 0) m <<= 1; /* 1 << n.trailing_zeros() */
+  size_t k = n / m;
+  r->n = n;
+  r->m = m;
+  r->k = k;
+  r->signs = (double*)malloc(n * sizeof(double));
+  r->small = (double*)malloc(k * k * sizeof(double));
+  if (!r->signs || !r->small) return ORC_INCONSISTENT;
+  uint64_t st = seed;
+  for (size_t i = 0; i < n; i++) r->signs[i] = orc_splitmix_gaussian(&st) < 0.0 ? -1.0 : 1.0;
+  /* orthonormal(k, rng), rotation.rs:226-247: Gram-Schmidt on Gaussian rows */
+  double* row = (double*)malloc(k * sizeof(double));
+  for (size_t i = 0; i < k; i++) {
+    for (size_t t = 0; t < k; t++) row[t] = orc_splitmix_gaussian(&st);
+    for (size_t p = 0; p < i; p++) {
+      const double* prev = r->small + p * k;
+      double d = 0.0;
+      for (size_t t = 0; t < k; t++) d += row[t] * prev[t];
+      for (size_t t = 0; t < k; t++) row[t] -= d * prev[t];
     }
-    for (size_t t = 0; t < tw; t++) w[r * m->d_in + nb * ORC_DIM + t] = (float)m->tail[r * tw + t];
+    double nrm = 0.0;
+    for (size_t t = 0; t < k; t++) nrm += row[t] * row[t];
+    nrm = sqrt(nrm);
+    for (size_t t = 0; t < k; t++) r->small[i * k + t] = row[t] / nrm;
   }
+  free(row);
   return ORC_OK;
 }
 
-int orc_fused_product(const orc_raw_matrix* m, const double* x, double* y, double* abs_out) {
-  if (m->has_rot) return ORC_INCONSISTENT;
+void orc_rotation_free(orc_rotation* r) {
+  free(r->signs);
+  free(r->small);
+  memset(r, 0, sizeof *r);
+}
+
+static void orc_wht(double* v, size_t n) { /* rotation.rs:201-222 */
+  for (size_t len = 1; len < n; len <<= 1)
+    for (size_t i = 0; i < n; i += len << 1)
+      for (size_t j = i; j < i + len; j++) {
+        double a = v[j], b = v[j + len];
+        v[j] = a + b;
+        v[j + len] = a - b;
+      }
+  double s = 1.0 / sqrt((double)n);
+  for (size_t i = 0; i < n; i++) v[i] *= s;
+}
+
+static void orc_rot_mix(const orc_rotation* r, double* v, int transpose) { /* rotation.rs:119-143 */
+  if (r->k == 1) return;
+  double* col = (double*)malloc(r->k * sizeof(double));
+  for (size_t j = 0; j < r->m; j++) {
+    for (size_t g = 0; g < r->k; g++) col[g] = v[g * r->m + j];
+    for (size_t g = 0; g < r->k; g++) {
+      double acc = 0.0;
+      for (size_t t = 0; t < r->k; t++)
+        acc += (transpose ? r->small[t * r->k + g] : r->small[g * r->k + t]) * col[t];
+      v[g * r->m + j] = acc;
+    }
+  }
+  free(col);
+}
+
+void orc_rotation_apply(const orc_rotation* r, double* v) { /* rotation.rs:97-105 */
+  for (size_t i = 0; i < r->n; i++) v[i] *= r->signs[i];
+  for (size_t g = 0; g < r->k; g++) orc_wht(v + g * r->m, r->m);
+  orc_rot_mix(r, v, 0);
+}
+
+void orc_rotation_apply_transpose(const orc_rotation* r, double* v) { /* rotation.rs:108-117 */
+  orc_rot_mix(r, v, 1);
+  for (size_t g = 0; g < r->k; g++) orc_wht(v + g * r->m, r->m);
+  for (size_t i = 0; i < r->n; i++) v[i] *= r->signs[i];
+}
+
+int orc_decode_matrix(const orc_raw_matrix* m, float* w) { /* format.rs:416-439 */
   size_t nb = m->d_in / ORC_DIM, tw = m->d_in % ORC_DIM;
-  for (size_t r = 0; r < m->d_out; r++) {
+  orc_rotation rot;
+  memset(&rot, 0, sizeof rot);
+  if (m->has_rot && orc_rotation_new(m->d_in, m->rot_seed, &rot) != ORC_OK) return ORC_INCONSISTENT;
+  double* row = (double*)malloc(m->d_in * sizeof(double));
+  int rc = ORC_OK;
+  for (size_t r = 0; r < m->d_out && rc == ORC_OK; r++) {
+    for (size_t b = 0; b < nb; b++) {
+      int32_t p[ORC_DIM];
+      size_t k = r * nb + b;
+      if (!orc_index_decode(m->indices[k], p)) { rc = ORC_INDEX_OUT_OF_RANGE; break; }
+      if (m->gains[k] >= m->n_centroids) { rc = ORC_INCONSISTENT; break; }
+      orc_reconstruct(p, m->gains[k], m->centroids, m->row_scales[r], row + b * ORC_DIM);
+    }
+    if (rc != ORC_OK) break;
+    for (size_t t = 0; t < tw; t++) row[nb * ORC_DIM + t] = m->tail[r * tw + t];
+    if (m->has_rot) orc_rotation_apply_transpose(&rot, row); /* un-rotate in f64, then narrow */
+    for (size_t c = 0; c < m->d_in; c++) w[r * m->d_in + c] = (float)row[c];
+  }
+  free(row);
+  if (m->has_rot) orc_rotation_free(&rot);
+  return rc;
+}
+
+int orc_fused_product(const orc_raw_matrix* m, const double* x_in, double* y, double* abs_out) {
+  size_t nb = m->d_in / ORC_DIM, tw = m->d_in % ORC_DIM;
+  double* xr = (double*)malloc(m->d_in * sizeof(double));
+  memcpy(xr, x_in, m->d_in * sizeof(double));
+  if (m->has_rot) { /* fused_path_matches_dense.rs:110-115: apply, not apply_transpose */
+    orc_rotation rot;
+    if (orc_rotation_new(m->d_in, m->rot_seed, &rot) != ORC_OK) { free(xr); return ORC_INCONSISTENT; }
+    orc_rotation_apply(&rot, xr);
+    orc_rotation_free(&rot);
+  }
+  const double* x = xr;
+  int rc = ORC_OK;
+  for (size_t r = 0; r < m->d_out && rc == ORC_OK; r++) {
     double acc = 0.0, aabs = 0.0;
     for (size_t b = 0; b < nb; b++) {
       int32_t p[ORC_DIM];
       size_t k = r * nb + b;
-      if (!orc_fast_decode(m->indices[k], p)) return ORC_INDEX_OUT_OF_RANGE;
-      if (m->gains[k] >= m->n_centroids) return ORC_INCONSISTENT;
+      if (!orc_fast_decode(m->indices[k], p)) { rc = ORC_INDEX_OUT_OF_RANGE; break; }
+      if (m->gains[k] >= m->n_centroids) { rc = ORC_INCONSISTENT; break; }
       int64_t sh = orc_shell_index(p);
       if (sh > 0) {
         double kk = m->centroids[m->gains[k]] * m->row_scales[r] / sqrt((double)(16 * sh));
@@ -1221,7 +1316,8 @@ int orc_fused_product(const orc_raw_matrix* m, const double* x, double* y, doubl
     y[r] = acc;
     if (abs_out) abs_out[r] = aabs;
   }
-  return ORC_OK;
+  free(xr);
+  return rc;
 }
 
 void orc_dense_matvec(const float* w, size_t d_out, size_t d_in, const double* x, double* y) {

@@ -115,14 +115,31 @@ void orc_raw_matrix_free(orc_raw_matrix* m);
 /* format.rs:238-298.  Returns an orc_err; *out is malloc'd (orc_free). */
 int orc_write_matrix_raw(const orc_raw_matrix* m, uint8_t** out, size_t* out_len);
 
+/* ---- llvq-quant/src/rotation.rs: the incoherence rotation Q ------------- */
+/* Q = (S (x) I_m) (I_k (x) H_m / sqrt m) D, n = m k with m the power-of-two part of n:
+ * signs D from the seed's Gaussian stream (rotation.rs:66-69), one Walsh-Hadamard
+ * transform per group of m (:201-222), a k x k orthonormal S by Gram-Schmidt on
+ * Gaussian rows, applied across groups (:119-143, :226-247). */
+typedef struct {
+  size_t n, m, k;
+  double* signs; /* n, +1 / -1 */
+  double* small; /* k * k, row-major */
+} orc_rotation;
+int orc_rotation_new(size_t n, uint64_t seed, orc_rotation* r); /* rotation.rs:60-79 */
+void orc_rotation_free(orc_rotation* r);
+void orc_rotation_apply(const orc_rotation* r, double* v);           /* v <- Q v,   :97-105 */
+void orc_rotation_apply_transpose(const orc_rotation* r, double* v); /* v <- Q^T v, :108-117 */
+
 /* llvq-quant/src/quantizer.rs:354-367 */
 void orc_reconstruct(const int32_t p[ORC_DIM], uint32_t gain, const double* centroids,
                      double row_scale, double out[ORC_DIM]);
 /* format.rs:385-439: decode every index (Indexer::decode) then rebuild the
- * d_out x d_in weights in f32.  Natural basis only (has_rot must be 0). */
+ * d_out x d_in weights in f64, un-rotate every row when the record carries a
+ * rotation seed (format.rs:435-437), then narrow to f32. */
 int orc_decode_matrix(const orc_raw_matrix* m, float* w /* d_out*d_in */);
-/* llvq-artifact/tests/fused_path_matches_dense.rs:96-136 without the rotation:
- * y_r = sum_b k_b sum_j p_bj x_j + tail.x, all f64.  abs_out (may be NULL)
+/* llvq-artifact/tests/fused_path_matches_dense.rs:96-136: the activation is
+ * rotated first when the record carries a rotation seed (:110-115), then
+ * y_r = sum_b k_b sum_j p_bj xr_j + tail.xr, all f64.  abs_out (may be NULL)
  * receives sum |w_i x_i| per row, the error normaliser of
  * llvq-cuda/src/bin/matvec.rs:114-120. */
 int orc_fused_product(const orc_raw_matrix* m, const double* x, double* y, double* abs_out);

@@ -45,6 +45,42 @@ class RawMatrixC(C.Structure):
 _lib = None
 
 
+class RotationC(C.Structure):
+    _fields_ = [("n", C.c_size_t), ("m", C.c_size_t), ("k", C.c_size_t),
+                ("signs", C.POINTER(C.c_double)), ("small", C.POINTER(C.c_double))]
+
+
+class Rotation:
+    """llvq-quant/src/rotation.rs: Rotation::new(n, seed), apply, apply_transpose."""
+
+    def __init__(self, n, seed):
+        self.c = RotationC()
+        rc = lib().orc_rotation_new(int(n), int(seed), C.byref(self.c))
+        if rc:
+            raise OracleError(rc)
+        self.n, self.m, self.k = self.c.n, self.c.m, self.c.k
+        self.signs = np.ctypeslib.as_array(self.c.signs, shape=(self.n,)).copy()
+        self.small = np.ctypeslib.as_array(self.c.small, shape=(self.k, self.k)).copy()
+
+    def apply(self, v):
+        v = np.array(v, dtype=np.float64)
+        assert v.size == self.n
+        lib().orc_rotation_apply(C.byref(self.c), v.ctypes.data_as(C.POINTER(C.c_double)))
+        return v
+
+    def apply_transpose(self, v):
+        v = np.array(v, dtype=np.float64)
+        assert v.size == self.n
+        lib().orc_rotation_apply_transpose(C.byref(self.c), v.ctypes.data_as(C.POINTER(C.c_double)))
+        return v
+
+    def __del__(self):
+        try:
+            lib().orc_rotation_free(C.byref(self.c))
+        except Exception:
+            pass
+
+
 def lib():
     global _lib
     if _lib is not None:
@@ -98,6 +134,13 @@ def lib():
     L.orc_raw_matrix_free.argtypes = [C.POINTER(RawMatrixC)]
     L.orc_write_matrix_raw.argtypes = [C.POINTER(RawMatrixC), C.POINTER(u8p), C.POINTER(C.c_size_t)]
     L.orc_reconstruct.argtypes = [i32p, C.c_uint32, C.POINTER(C.c_double), C.c_double, C.POINTER(C.c_double)]
+    L.orc_rotation_new.argtypes = [C.c_size_t, C.c_uint64, C.POINTER(RotationC)]
+    L.orc_rotation_free.argtypes = [C.POINTER(RotationC)]
+    L.orc_rotation_free.restype = None
+    L.orc_rotation_apply.argtypes = [C.POINTER(RotationC), C.POINTER(C.c_double)]
+    L.orc_rotation_apply.restype = None
+    L.orc_rotation_apply_transpose.argtypes = [C.POINTER(RotationC), C.POINTER(C.c_double)]
+    L.orc_rotation_apply_transpose.restype = None
     L.orc_decode_matrix.argtypes = [C.POINTER(RawMatrixC), C.POINTER(C.c_float)]
     L.orc_fused_product.argtypes = [C.POINTER(RawMatrixC), C.POINTER(C.c_double), C.POINTER(C.c_double),
                                     C.POINTER(C.c_double)]

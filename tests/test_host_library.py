@@ -119,3 +119,30 @@ def test_synthetic_configs():
     assert 6 * o * (i // 24) + 4 * o * (i % 24) + 8 * o + 16 == 6_887_440
     x = synth.make_activation(2560, 0)
     assert x.dtype == np.float16 and x.shape == (1, 2560)
+
+
+# ---- rotation tables (fused.rs:1272-1331: "the tables describe the rotation") -------------
+def test_rotation_tables_describe_the_rotation(orc):
+    import ctypes as C
+
+    from llvq_amd import _ffi
+    from llvq_amd.synth import SplitMix64
+
+    L = _ffi.lib()
+    for n, seed in [(240, 1), (2560, 2), (9728, 3), (4096, 4), (96, 5)]:  # fused.rs:1274
+        x = SplitMix64(seed ^ 0xF00D).gaussian(n)
+        got = x.copy()
+        _ffi.check(L.llvq_hip_host_rotate(n, seed, got.ctypes.data))
+        want = orc.Rotation(n, seed).apply(x)
+        dev = np.linalg.norm(got - want) / np.linalg.norm(want)
+        assert dev < 1e-6, f"n={n}: relative deviation {dev:.3e}"  # the reference's own threshold
+        assert abs(np.linalg.norm(got) / np.linalg.norm(x) - 1) < 1e-6  # 1/sqrt m, not 1/sqrt n
+
+
+def test_rotation_with_a_wide_odd_factor_is_refused():
+    from llvq_amd import LlvqError, _ffi
+
+    v = np.zeros(33 * 8)
+    with pytest.raises(LlvqError) as e:  # k = 33 > 32 (fused.rs:698-704)
+        _ffi.check(_ffi.lib().llvq_hip_host_rotate(33 * 8, 1, v.ctypes.data))
+    assert e.value.kind == "Unsupported" and "33" in str(e.value)
