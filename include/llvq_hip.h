@@ -158,6 +158,10 @@ int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks
  * a Qwen3-architecture decoder whose projections are uploaded LLVQ matrices and
  * whose other tensors are dense binary16.  Host pointers; everything is copied. */
 typedef struct llvq_decoder llvq_decoder;
+/* KvMode (llvq-llm/src/kvq.rs:10-34): binary16 cache, or 8-bit codes per group of
+ * 64 along head_dim with binary16 scale and bias (kvq.rs:110-165), chosen from
+ * the token alone and rebuilt to the same binary16 value on every read. */
+typedef enum llvq_kv_mode { LLVQ_KV_F16 = 0, LLVQ_KV_Q8 = 1 } llvq_kv_mode;
 typedef struct llvq_decoder_desc {
   uint32_t n_layers, hidden, n_heads, n_kv_heads, head_dim, intermediate, vocab;
   uint32_t max_positions;               /* KV-cache length, <= 8192 */
@@ -170,6 +174,7 @@ typedef struct llvq_decoder_desc {
   const uint16_t* final_norm;           /* [hidden] */
   const uint16_t* embed;                /* [vocab, hidden] */
   const uint16_t* lm_head;              /* [vocab, hidden]; NULL = tied to embed */
+  uint32_t kv_mode;                     /* llvq_kv_mode; q8 needs head_dim % 64 == 0 */
 } llvq_decoder_desc;
 /* Qwen3::new_with (model.rs:869): checks every projection's shape against the architecture. */
 int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* desc, llvq_decoder** out);

@@ -51,6 +51,7 @@ class DecoderDesc(C.Structure):
         ("projections", C.POINTER(C.c_void_p)),
         ("input_norm", C.c_void_p), ("post_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
         ("final_norm", C.c_void_p), ("embed", C.c_void_p), ("lm_head", C.c_void_p),
+        ("kv_mode", C.c_uint32),
     ]
 
 

@@ -72,25 +72,79 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(const __half*
   }
 }
 
+// int8 KV cache (llvq-llm/src/kvq.rs:110-165): asymmetric 8-bit codes per group
+// of 64 along head_dim, binary16 scale and bias, chosen from the token alone:
+//   s = f16((max - min) / 255), b = f16(min), q = clamp(round((x - b) / (s > 0 ? s : 1)), 0, 255)
+// and a reader gets back f16(q s + b).  The reference keeps that reconstructed
+// value in its cache; here the codes themselves are stored (1.06 bytes per
+// value instead of 2) and the same value is rebuilt on every read.
+constexpr uint32_t kKvGroup = 64;
+struct KvQ8 {
+  uint8_t* kq;    // [n_kv][max_pos][head_dim]
+  uint8_t* vq;
+  __half* ks;     // [n_kv][max_pos][head_dim / 64] scales
+  __half* kb;     //                                biases
+  __half* vs;
+  __half* vb;
+};
+
+// One group of 64 values held one per lane -> code, scale, bias.
+__device__ __forceinline__ uint8_t kv_quantize_group(float x, __half* s_out, __half* b_out) {
+  float mn = x, mx = x;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  const __half sh = __float2half_rn(__fdiv_rn(__fsub_rn(mx, mn), 255.0f));
+  const __half bh = __float2half_rn(mn);
+  const float s = __half2float(sh), b = __half2float(bh);
+  const float safe = s > 0.f ? s : 1.0f;
+  const float q = fminf(fmaxf(roundf(__fdiv_rn(__fsub_rn(x, b), safe)), 0.f), 255.f);
+  *s_out = sh;
+  *b_out = bh;
+  return (uint8_t)q;
+}
+
+__device__ __forceinline__ float kv_dequant(uint32_t q, float s, float b) {
+  return __half2float(__float2half_rn(__fadd_rn(__fmul_rn((float)q, s), b)));
+}
+
 // One wavefront per head: per-head RMSNorm of q and k (model.rs:800-808), RoPE at
 // the absolute position in the rotate-half convention (candle_nn::rotary_emb::rope:
 // out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i] sin + x[i + d/2] cos, with
 // the binary16 cos/sin tables of Rotary::new, model.rs:163-179), then k and v of
-// this position are appended to the cache.  Heads: [0, n_heads) are q, the next
-// n_kv are k, the last n_kv are v.  head_dim <= 256, even.
+// this position are appended to the cache (binary16, or int8 codes when q8 is set).
+// Heads: [0, n_heads) are q, the next n_kv are k, the last n_kv are v.
+// head_dim <= 256, a multiple of 8 (of 64 for the int8 cache).
 __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restrict__ q, const __half* __restrict__ k,
                                                                  const __half* __restrict__ v,
                                                                  const __half* __restrict__ qn, const __half* __restrict__ kn,
                                                                  const __half* __restrict__ cos_t, const __half* __restrict__ sin_t,
                                                                  __half* __restrict__ kcache, __half* __restrict__ vcache,
+                                                                 KvQ8 q8, uint32_t use_q8,
                                                                  uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                                                  uint32_t pos, uint32_t max_pos, float eps) {
   const uint32_t head = blockIdx.x, lane = threadIdx.x;
-  const uint32_t half_d = head_dim >> 1;
-  if (head >= n_heads + n_kv) {  // v: copy into the cache
+  const uint32_t half_d = head_dim >> 1, groups = head_dim / kKvGroup;
+  __shared__ float stage[256];
+  if (head >= n_heads + n_kv) {  // v: into the cache as it is
     const uint32_t kvh = head - n_heads - n_kv;
-    for (uint32_t i = lane; i < head_dim; i += 64)
-      vcache[((size_t)kvh * max_pos + pos) * head_dim + i] = v[(size_t)kvh * head_dim + i];
+    const size_t row = (size_t)kvh * max_pos + pos;
+    if (!use_q8) {
+      for (uint32_t i = lane; i < head_dim; i += 64) vcache[row * head_dim + i] = v[(size_t)kvh * head_dim + i];
+    } else {
+      for (uint32_t g = 0; g < groups; ++g) {
+        const float x = __half2float(v[(size_t)kvh * head_dim + g * kKvGroup + lane]);
+        __half sh, bh;
+        const uint8_t code = kv_quantize_group(x, &sh, &bh);
+        q8.vq[row * head_dim + g * kKvGroup + lane] = code;
+        if (lane == 0) {
+          q8.vs[row * groups + g] = sh;
+          q8.vb[row * groups + g] = bh;
+        }
+      }
+    }
     return;
   }
   const bool is_q = head < n_heads;
@@ -107,19 +161,48 @@ __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restr
   }
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)head_dim + eps);
-  __shared__ float normed[256];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const uint32_t i = lane + 64u * j;
-    if (i < head_dim) normed[i] = __half2float(__float2half_rn(x[j] * inv * __half2float(w[i])));
+    if (i < head_dim) stage[i] = __half2float(__float2half_rn(x[j] * inv * __half2float(w[i])));
   }
   __syncthreads();
-  __half* dst = is_q ? q + (size_t)hh * head_dim : kcache + ((size_t)hh * max_pos + pos) * head_dim;
-  for (uint32_t i = lane; i < half_d; i += 64) {
-    const float c = __half2float(cos_t[(size_t)pos * half_d + i]), s = __half2float(sin_t[(size_t)pos * half_d + i]);
-    const float x1 = normed[i], x2 = normed[i + half_d];
-    dst[i] = __float2half_rn(x1 * c - x2 * s);
-    dst[i + half_d] = __float2half_rn(x1 * s + x2 * c);
+  float r1[2], r2[2];  // rotated pairs (i, i + d/2) for i = lane, lane + 64
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t i = lane + 64u * j;
+    r1[j] = r2[j] = 0.f;
+    if (i < half_d) {
+      const float c = __half2float(cos_t[(size_t)pos * half_d + i]), sn = __half2float(sin_t[(size_t)pos * half_d + i]);
+      const float x1 = stage[i], x2 = stage[i + half_d];
+      r1[j] = __half2float(__float2half_rn(x1 * c - x2 * sn));
+      r2[j] = __half2float(__float2half_rn(x1 * sn + x2 * c));
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t i = lane + 64u * j;
+    if (i < half_d) {
+      stage[i] = r1[j];
+      stage[i + half_d] = r2[j];
+    }
+  }
+  __syncthreads();
+  if (is_q || !use_q8) {
+    __half* dst = is_q ? q + (size_t)hh * head_dim : kcache + ((size_t)hh * max_pos + pos) * head_dim;
+    for (uint32_t i = lane; i < head_dim; i += 64) dst[i] = __float2half_rn(stage[i]);
+  } else {
+    const size_t row = (size_t)hh * max_pos + pos;
+    for (uint32_t g = 0; g < groups; ++g) {
+      __half sh, bh;
+      const uint8_t code = kv_quantize_group(stage[g * kKvGroup + lane], &sh, &bh);
+      q8.kq[row * head_dim + g * kKvGroup + lane] = code;
+      if (lane == 0) {
+        q8.ks[row * groups + g] = sh;
+        q8.kb[row * groups + g] = bh;
+      }
+    }
   }
 }
 
@@ -131,22 +214,30 @@ __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restr
 // arrives last at the kv head's counter merges the partials in split order and
 // rounds the context once.  Scores, softmax and sums stay in f32.
 constexpr int kAttnThreads = 256;
-constexpr int kAttnSplits = 16;
-constexpr int kAttnMaxDim = 256;
+constexpr int kAttnMaxSplits = 64;  // the cache is cut into at most this many ranges (host picks by length)
+template <bool Q8>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half* __restrict__ q, const __half* __restrict__ kcache,
-                                                                   const __half* __restrict__ vcache, __half* __restrict__ ctx,
+                                                                   const __half* __restrict__ vcache, KvQ8 q8,
+                                                                   __half* __restrict__ ctx,
                                                                    float* __restrict__ part, uint32_t* __restrict__ counters,
                                                                    uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
-                                                                   uint32_t T, uint32_t max_pos, float scale) {
+                                                                   uint32_t T, uint32_t max_pos, float scale, uint32_t n_splits) {
   extern __shared__ __align__(16) float att_smem[];  // [4][chunk] scores
   __shared__ uint32_t arrived;
-  const uint32_t kvh = blockIdx.x / kAttnSplits, split = blockIdx.x % kAttnSplits;
+  const uint32_t kvh = blockIdx.x / n_splits, split = blockIdx.x % n_splits;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t groups = n_heads / n_kv;
-  const uint32_t chunk = (T + kAttnSplits - 1) / kAttnSplits;
+  const uint32_t chunk = (T + n_splits - 1) / n_splits;
   const uint32_t j0 = min(T, split * chunk), j1 = min(T, j0 + chunk);
   const __half* K = kcache + (size_t)kvh * max_pos * head_dim;
   const __half* V = vcache + (size_t)kvh * max_pos * head_dim;
+  const uint32_t kvgroups = head_dim / kKvGroup;
+  const uint8_t* Kq = q8.kq + (size_t)kvh * max_pos * head_dim;
+  const uint8_t* Vq = q8.vq + (size_t)kvh * max_pos * head_dim;
+  const __half* Ks = q8.ks + (size_t)kvh * max_pos * kvgroups;
+  const __half* Kb = q8.kb + (size_t)kvh * max_pos * kvgroups;
+  const __half* Vs = q8.vs + (size_t)kvh * max_pos * kvgroups;
+  const __half* Vb = q8.vb + (size_t)kvh * max_pos * kvgroups;
   float* sc = att_smem + (size_t)wave * chunk;
   const uint32_t stride = head_dim + 2;  // floats per partial: max, sum, head_dim sums
   const uint32_t sub = lane & 15u, pj = lane >> 4;  // 16 lanes x 8 dims (zero-padded) cover a position's row
@@ -161,15 +252,29 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
       for (uint32_t ds = 0; ds < dsteps; ++ds) {
         const uint32_t i0 = ds * 128u + sub * 8u;
         if (j < j1 && i0 < head_dim) {
-          const uint4 kk = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0);
           const uint4 qq = *reinterpret_cast<const uint4*>(q + (size_t)head * head_dim + i0);
-          const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w}, qw[4] = {qq.x, qq.y, qq.z, qq.w};
+          const uint32_t qw[4] = {qq.x, qq.y, qq.z, qq.w};
+          if constexpr (Q8) {
+            const uint2 kc = *reinterpret_cast<const uint2*>(Kq + (size_t)j * head_dim + i0);
+            const float ksc = __half2float(Ks[(size_t)j * kvgroups + i0 / kKvGroup]);
+            const float kbi = __half2float(Kb[(size_t)j * kvgroups + i0 / kKvGroup]);
+            const uint32_t kw[2] = {kc.x, kc.y};
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] & 0xFFFFu))),
-                     __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu))), d);
-            d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] >> 16))),
-                     __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16))), d);
+            for (int t = 0; t < 4; ++t) {
+              const uint32_t c0 = (kw[t >> 1] >> (16 * (t & 1))) & 0xFFu, c1 = (kw[t >> 1] >> (16 * (t & 1) + 8)) & 0xFFu;
+              d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] & 0xFFFFu))), kv_dequant(c0, ksc, kbi), d);
+              d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] >> 16))), kv_dequant(c1, ksc, kbi), d);
+            }
+          } else {
+            const uint4 kk = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0);
+            const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] & 0xFFFFu))),
+                       __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu))), d);
+              d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] >> 16))),
+                       __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16))), d);
+            }
           }
         }
       }
@@ -195,17 +300,29 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
     l = wave_sum(l);
     __threadfence_block();
     // weighted V sum: lane owns dims 2 lane, 2 lane + 1 of each 128-dim pass
-    float* dst = part + ((size_t)head * kAttnSplits + split) * stride;
+    float* dst = part + ((size_t)head * n_splits + split) * stride;
     for (uint32_t ds = 0; ds < dsteps; ++ds) {
       const uint32_t i0 = ds * 128u + lane * 2u;
       float a0 = 0.f, a1 = 0.f;
-      if (i0 < head_dim)
-        for (uint32_t j = j0; j < j1; ++j) {
-          const __half2 vv = *reinterpret_cast<const __half2*>(V + (size_t)j * head_dim + i0);
-          const float p = sc[j - j0];
-          a0 = fmaf(p, __low2float(vv), a0);
-          a1 = fmaf(p, __high2float(vv), a1);
+      if (i0 < head_dim) {
+        if constexpr (Q8) {
+          for (uint32_t j = j0; j < j1; ++j) {
+            const uint32_t vc = *reinterpret_cast<const unsigned short*>(Vq + (size_t)j * head_dim + i0);
+            const float vsc = __half2float(Vs[(size_t)j * kvgroups + i0 / kKvGroup]);
+            const float vbi = __half2float(Vb[(size_t)j * kvgroups + i0 / kKvGroup]);
+            const float p = sc[j - j0];
+            a0 = fmaf(p, kv_dequant(vc & 0xFFu, vsc, vbi), a0);
+            a1 = fmaf(p, kv_dequant(vc >> 8, vsc, vbi), a1);
+          }
+        } else {
+          for (uint32_t j = j0; j < j1; ++j) {
+            const __half2 vv = *reinterpret_cast<const __half2*>(V + (size_t)j * head_dim + i0);
+            const float p = sc[j - j0];
+            a0 = fmaf(p, __low2float(vv), a0);
+            a1 = fmaf(p, __high2float(vv), a1);
+          }
         }
+      }
       if (i0 < head_dim) {
         dst[2 + i0] = a0;
         dst[2 + i0 + 1] = a1;
@@ -222,15 +339,15 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
   __syncthreads();
   if (tid == 0) arrived = __hip_atomic_fetch_add(&counters[kvh], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
-  if (arrived != kAttnSplits - 1) return;
+  if (arrived != n_splits - 1) return;
   for (uint32_t o = tid; o < groups * head_dim; o += kAttnThreads) {
     const uint32_t g = o / head_dim, i = o - g * head_dim;
     const uint32_t head = kvh * groups + g;
-    const float* src = part + (size_t)head * kAttnSplits * stride;
+    const float* src = part + (size_t)head * n_splits * stride;
     float M = -INFINITY;
-    for (uint32_t s = 0; s < kAttnSplits; ++s) M = fmaxf(M, src[(size_t)s * stride]);
+    for (uint32_t s = 0; s < n_splits; ++s) M = fmaxf(M, src[(size_t)s * stride]);
     float L = 0.f, A = 0.f;
-    for (uint32_t s = 0; s < kAttnSplits; ++s) {
+    for (uint32_t s = 0; s < n_splits; ++s) {
       const float w = __expf(src[(size_t)s * stride] - M);  // 0 for an empty range
       L = fmaf(src[(size_t)s * stride + 1], w, L);
       A = fmaf(src[(size_t)s * stride + 2 + i], w, A);

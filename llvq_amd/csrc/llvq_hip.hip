@@ -124,9 +124,7 @@ __global__ __launch_bounds__(256) void decode_blocks_kernel(GlobalTables g, cons
 // plane sums are combined and scaled in f32.
 constexpr int kWgThreads = LLVQ_WG_THREADS;
 constexpr int kWaves = kWgThreads / 64;
-constexpr int kTileBlocks = LLVQ_TILE_BLOCKS;
-constexpr int kP1Blocks = kTileBlocks / kWgThreads;  // blocks one lane classifies per tile
-constexpr int kRawBytes = kTileBlocks * 6 + 32;
+constexpr int kTileBlocks = LLVQ_TILE_BLOCKS;  // default tile capacity; the kernel is instantiated per capacity
 constexpr int kMaxGroup = 4;
 constexpr int kPlaneDwords = 18;  // 3 planes x 6 dwords per 24-column block
 constexpr int kGenericSlots = 64; // queue of blocks that take the generic walk
@@ -163,9 +161,10 @@ struct GroupArgs {
   MatArg m[kMaxGroup];
 };
 
-__host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks) {
-  return kLdsImageBytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + kRawBytes +
-         (size_t)kTileBlocks * 4 * 2 + kGenericSlots * 4 + 16;
+constexpr int kSmallTileBlocks = 2048;  // tile of the variant for rows too wide for the full tile's LDS
+__host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks, uint32_t tile = kTileBlocks) {
+  return kLdsImageBytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + ((size_t)tile * 6 + 32) +
+         (size_t)tile * 4 * 2 + kGenericSlots * 4 + 16;
 }
 
 template <typename OutT>
@@ -301,8 +300,12 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 #define LLVQ_STAMP(k) do {} while (0)
 #endif
 
-template <typename OutT>
+template <typename OutT, int TILE = LLVQ_TILE_BLOCKS>
 __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
+  // the tile capacity of this instantiation (these shadow the namespace-level defaults)
+  constexpr int kTileBlocks = TILE;
+  constexpr int kP1Blocks = TILE / kWgThreads;
+  constexpr int kRawBytes = TILE * 6 + 32;
   extern __shared__ __align__(16) uint8_t smem[];
   const DecodeTables T = stage_tables(smem, a.tables);
   const uint32_t nb = a.nblocks;
@@ -779,6 +782,8 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   const int max_lds = 160 * 1024;
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float, kSmallTileBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half, kSmallTileBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
@@ -1011,8 +1016,8 @@ int llvq_hip_matrix_info(const llvq_mat* m, uint32_t* d_out, uint32_t* d_in, uin
 const char* llvq_hip_matrix_name(const llvq_mat* m) { return m ? m->name.c_str() : ""; }
 
 // Rows per tile: as even a split over the CUs as the tile capacity allows.
-static uint32_t pick_rows_per_tile(const llvq_mat* const* mats, int n, uint32_t nblocks, uint32_t grid) {
-  const uint32_t cap = nblocks ? (uint32_t)kTileBlocks / nblocks : 0xFFFFFFFFu;
+static uint32_t pick_rows_per_tile(const llvq_mat* const* mats, int n, uint32_t nblocks, uint32_t grid, uint32_t tile) {
+  const uint32_t cap = nblocks ? tile / nblocks : 0xFFFFFFFFu;
   uint64_t total = 0;
   for (int i = 0; i < n; ++i) total += mats[i]->d_out;
   uint32_t r = (uint32_t)((total + grid - 1) / grid);
@@ -1038,8 +1043,11 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
                         int y_dtype, const Prologue* pro = nullptr, const float* x_f32 = nullptr) {
   const llvq_mat* m0 = mats[0];
   if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv: unknown output dtype");
-  const size_t lds = gemv_lds_bytes(m0->nblocks);
-  if (lds > 160 * 1024 || m0->nblocks > (uint32_t)kTileBlocks)
+  // the full tile where the activation planes leave room for it, else the half tile
+  uint32_t tile = kTileBlocks;
+  if (gemv_lds_bytes(m0->nblocks, tile) > 160 * 1024) tile = kSmallTileBlocks;
+  const size_t lds = gemv_lds_bytes(m0->nblocks, tile);
+  if (lds > 160 * 1024 || m0->nblocks > tile)
     return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": d_in " + std::to_string(m0->d_in) + " does not fit the LDS activation tile");
   // as many workgroups as fit a CU's 160 KB of LDS side by side
   const uint32_t per_cu = (uint32_t)((160 * 1024) / lds) < 1u ? 1u : (uint32_t)((160 * 1024) / lds);
@@ -1050,7 +1058,7 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   a.x = reinterpret_cast<const __half*>(x);
   a.x_f32 = x_f32;
   if (pro) {
-    if ((size_t)m0->d_in * 2 > (size_t)kRawBytes)
+    if ((size_t)m0->d_in * 2 > (size_t)tile * 6 + 32)
       return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": d_in too wide for a fused activation prologue");
     a.prologue = pro->kind;
     a.x2 = reinterpret_cast<const __half*>(pro->x2);
@@ -1062,7 +1070,7 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   a.tail_w = m0->tail_w;
   a.n_mats = (uint32_t)n;
   a.inv_nblocks = m0->nblocks ? 1.0f / (float)m0->nblocks : 0.f;
-  a.rows_per_tile = pick_rows_per_tile(mats, n, m0->nblocks, grid_cap);
+  a.rows_per_tile = pick_rows_per_tile(mats, n, m0->nblocks, grid_cap, tile);
   uint32_t tiles = 0;
   for (int i = 0; i < n; ++i) {
     a.m[i] = MatArg{mats[i]->codes, mats[i]->rscale, mats[i]->tail, y[i], mats[i]->g[0], mats[i]->g[1],
@@ -1071,10 +1079,17 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   }
   a.n_tiles = tiles;
   const uint32_t grid = tiles < grid_cap ? tiles : grid_cap;
-  if (y_dtype == LLVQ_F32)
-    hipLaunchKernelGGL(gemv_tiles_kernel<float>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
-  else
-    hipLaunchKernelGGL(gemv_tiles_kernel<__half>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
+  if (tile == (uint32_t)kTileBlocks) {
+    if (y_dtype == LLVQ_F32)
+      hipLaunchKernelGGL(gemv_tiles_kernel<float>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
+    else
+      hipLaunchKernelGGL(gemv_tiles_kernel<__half>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
+  } else {
+    if (y_dtype == LLVQ_F32)
+      hipLaunchKernelGGL((gemv_tiles_kernel<float, kSmallTileBlocks>), dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
+    else
+      hipLaunchKernelGGL((gemv_tiles_kernel<__half, kSmallTileBlocks>), dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
+  }
   HIP_TRY(hipGetLastError());
   return LLVQ_OK;
 }
@@ -1335,7 +1350,9 @@ struct llvq_decoder {
   uint32_t* best_idx = nullptr;
   uint32_t* token = nullptr;    // the token the next step embeds
   uint32_t* history = nullptr;  // [max_pos] tokens chosen by the head
-  float* attn_part = nullptr;   // [n_heads][kAttnSplits][head_dim + 2] partial attention sums
+  float* attn_part = nullptr;   // [n_heads][kAttnMaxSplits][head_dim + 2] partial attention sums
+  bool kv_q8 = false;           // int8 KV cache (kvq.rs) instead of binary16
+  KvQ8 q8{};                    // layer 0's arrays; a layer's are at + layer * (cache_layer or cache_layer / 64 groups)
   uint32_t* attn_counters = nullptr;  // [n_kv], zero between launches
   uint32_t pos = 0;
   uint32_t head_grid = 0;
@@ -1352,7 +1369,10 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, d->h);
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
   const uint32_t T = d->pos + 1;
-  const size_t attn_lds = (size_t)(kAttnThreads / 64) * ((T + kAttnSplits - 1) / kAttnSplits) * sizeof(float);
+  uint32_t n_splits = (T + 31) / 32;  // about 32 cached positions per workgroup, at most kAttnMaxSplits ranges
+  if (n_splits > (uint32_t)kAttnMaxSplits) n_splits = kAttnMaxSplits;
+  const size_t attn_lds = (size_t)(kAttnThreads / 64) * ((T + n_splits - 1) / n_splits) * sizeof(float);
+  const size_t group_layer = cache_layer / kKvGroup;
   // Projections in the natural basis derive their activation in the launch's
   // prologue; a rotated basis needs the activation as a tensor first (it goes
   // through the rotation kernel), so its prologue runs as a kernel of its own.
@@ -1390,13 +1410,24 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     int rc = project(P, 3, d->h, qkv_out, ln1);
     if (rc) return rc;
     if (L) std::swap(d->h, d->h_alt);
+    KvQ8 lq8 = d->q8;
+    if (d->kv_q8) {
+      lq8.kq += L * cache_layer; lq8.vq += L * cache_layer;
+      lq8.ks += L * group_layer; lq8.kb += L * group_layer; lq8.vs += L * group_layer; lq8.vb += L * group_layer;
+    }
+    __half* kc = d->kv_q8 ? nullptr : d->kcache + L * cache_layer;
+    __half* vc = d->kv_q8 ? nullptr : d->vcache + L * cache_layer;
     hipLaunchKernelGGL(qk_norm_rope_append_kernel, dim3(d->n_heads + 2 * d->n_kv), dim3(64), 0, st, d->q, d->k, d->v,
                        d->qn + (size_t)L * d->head_dim, d->kn + (size_t)L * d->head_dim, d->cos_t, d->sin_t,
-                       d->kcache + L * cache_layer, d->vcache + L * cache_layer, d->n_heads, d->n_kv, d->head_dim, d->pos,
-                       d->max_pos, d->eps);
-    hipLaunchKernelGGL(attn_decode_kernel, dim3(d->n_kv * kAttnSplits), dim3(kAttnThreads), attn_lds, st, d->q,
-                       d->kcache + L * cache_layer, d->vcache + L * cache_layer, d->ctx, d->attn_part, d->attn_counters,
-                       d->n_heads, d->n_kv, d->head_dim, T, d->max_pos, 1.0f / sqrtf((float)d->head_dim));
+                       kc, vc, lq8, d->kv_q8 ? 1u : 0u, d->n_heads, d->n_kv, d->head_dim, d->pos, d->max_pos, d->eps);
+    if (d->kv_q8)
+      hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, d->q, kc, vc, lq8,
+                         d->ctx, d->attn_part, d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
+                         1.0f / sqrtf((float)d->head_dim), n_splits);
+    else
+      hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, d->q, kc, vc, lq8,
+                         d->ctx, d->attn_part, d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
+                         1.0f / sqrtf((float)d->head_dim), n_splits);
     void* o_out[1] = {d->o};
     rc = forward_group(rt, P + 3, 1, d->ctx, o_out, LLVQ_F16);
     if (rc) return rc;
@@ -1440,10 +1471,11 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
     return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: a required tensor is null");
   if (c->n_layers == 0 || c->hidden == 0 || c->hidden % 8 || c->hidden > 8192 || c->n_heads == 0 || c->n_kv_heads == 0 ||
       c->n_heads % c->n_kv_heads || c->head_dim == 0 || c->head_dim % 8 || c->head_dim > 256 || c->intermediate == 0 ||
-      c->vocab == 0 || c->max_positions == 0 || c->max_positions > 8192)
+      c->vocab == 0 || c->max_positions == 0 || c->max_positions > 8192 ||
+      (c->kv_mode != LLVQ_KV_F16 && c->kv_mode != LLVQ_KV_Q8) || (c->kv_mode == LLVQ_KV_Q8 && c->head_dim % 64))
     return fail(LLVQ_ERR_UNSUPPORTED,
                 "decoder_create: shape outside what the kernels hold (hidden % 8 = 0 and <= 8192, head_dim % 8 = 0 and <= 256, "
-                "heads a multiple of kv heads, max_positions <= 8192)");
+                "heads a multiple of kv heads, max_positions <= 8192, kv_mode f16 or q8 with head_dim % 64 = 0)");
   const uint32_t qd = c->n_heads * c->head_dim, kvd = c->n_kv_heads * c->head_dim;
   static const char* kSite[7] = {"q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"};
   const uint32_t want_out[7] = {qd, kvd, kvd, c->hidden, c->intermediate, c->intermediate, c->hidden};
@@ -1463,6 +1495,7 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   d->n_layers = c->n_layers; d->hidden = c->hidden; d->n_heads = c->n_heads; d->n_kv = c->n_kv_heads;
   d->head_dim = c->head_dim; d->inter = c->intermediate; d->vocab = c->vocab; d->max_pos = c->max_positions;
   d->eps = (float)c->rms_eps;
+  d->kv_q8 = c->kv_mode == LLVQ_KV_Q8;
   d->proj.assign(c->projections, c->projections + (size_t)c->n_layers * 7);
   d->head_grid = 1024;
   while (d->head_grid > 1 && (uint64_t)d->head_grid * (kHeadThreads / 64) > c->vocab) d->head_grid >>= 1;
@@ -1490,8 +1523,11 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   const size_t o_emb = take((size_t)c->vocab * c->hidden * hb);
   const size_t o_head = c->lm_head ? take((size_t)c->vocab * c->hidden * hb) : o_emb;
   const size_t o_cos = take(cos_h.size() * hb), o_sin = take(sin_h.size() * hb);
-  const size_t cache_bytes = (size_t)c->n_layers * c->n_kv_heads * c->max_positions * c->head_dim * hb;
-  const size_t o_kc = take(cache_bytes), o_vc = take(cache_bytes);
+  const size_t cache_vals = (size_t)c->n_layers * c->n_kv_heads * c->max_positions * c->head_dim;
+  const bool q8 = c->kv_mode == LLVQ_KV_Q8;
+  const size_t o_kc = take(cache_vals * (q8 ? 1 : hb)), o_vc = take(cache_vals * (q8 ? 1 : hb));
+  const size_t o_ks = take(q8 ? cache_vals / kKvGroup * hb : 0), o_kb = take(q8 ? cache_vals / kKvGroup * hb : 0);
+  const size_t o_vs = take(q8 ? cache_vals / kKvGroup * hb : 0), o_vb = take(q8 ? cache_vals / kKvGroup * hb : 0);
   const size_t o_h = take(c->hidden * hb), o_h2 = take(c->hidden * hb), o_nm = take(c->hidden * hb), o_q = take(qd * hb), o_k = take(kvd * hb), o_v = take(kvd * hb);
   const size_t o_ctx = take(qd * hb), o_o = take(c->hidden * hb), o_g = take(c->intermediate * hb), o_u = take(c->intermediate * hb);
   const size_t o_act = take(c->intermediate * hb), o_dn = take(c->hidden * hb);
@@ -1499,7 +1535,7 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   const size_t n_best = (size_t)d->head_grid * (kHeadThreads / 64);
   const size_t o_bv = take(n_best * sizeof(float)), o_bi = take(n_best * sizeof(uint32_t));
   const size_t o_tok = take(sizeof(uint32_t)), o_hist = take((size_t)c->max_positions * sizeof(uint32_t));
-  const size_t o_ap = take((size_t)c->n_heads * kAttnSplits * (c->head_dim + 2) * sizeof(float)), o_ac = take((size_t)c->n_kv_heads * sizeof(uint32_t));
+  const size_t o_ap = take((size_t)c->n_heads * kAttnMaxSplits * (c->head_dim + 2) * sizeof(float)), o_ac = take((size_t)c->n_kv_heads * sizeof(uint32_t));
   hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->blob), total);
   if (e != hipSuccess) { delete d; return hip_fail(e, "hipMalloc(decoder)"); }
   auto put = [&](size_t at, const void* src, size_t bytes) { return hipMemcpy(d->blob + at, src, bytes, hipMemcpyHostToDevice); };
@@ -1518,6 +1554,10 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   d->ln1 = H(o_ln1); d->ln2 = H(o_ln2); d->qn = H(o_qn); d->kn = H(o_kn); d->fnorm = H(o_fn);
   d->embed = H(o_emb); d->head = H(o_head); d->cos_t = H(o_cos); d->sin_t = H(o_sin);
   d->kcache = H(o_kc); d->vcache = H(o_vc);
+  if (q8) {
+    d->q8.kq = d->blob + o_kc; d->q8.vq = d->blob + o_vc;
+    d->q8.ks = H(o_ks); d->q8.kb = H(o_kb); d->q8.vs = H(o_vs); d->q8.vb = H(o_vb);
+  }
   d->h = H(o_h); d->h_alt = H(o_h2); d->normed = H(o_nm); d->q = H(o_q); d->k = H(o_k); d->v = H(o_v); d->ctx = H(o_ctx); d->o = H(o_o);
   d->gate = H(o_g); d->up = H(o_u); d->act = H(o_act); d->down = H(o_dn);
   d->logits = reinterpret_cast<float*>(d->blob + o_log);

@@ -28,6 +28,7 @@ class Qwen3Config:
     rms_norm_eps: float = 1e-6
     max_positions: int = 1024
     tie_word_embeddings: bool = True
+    kv_mode: str = "f16"  # KvMode::parse (kvq.rs:38-49): "f16" or "q8"
 
     def shapes(self):
         """(site, d_out, d_in) of the seven projections of one layer."""
@@ -110,10 +111,19 @@ class Decoder:
             cfg.max_positions, float(cfg.rope_theta), float(cfg.rms_norm_eps),
             C.cast(arr, C.POINTER(C.c_void_p)),
             keep[0].ctypes.data, keep[1].ctypes.data, keep[2].ctypes.data, keep[3].ctypes.data, keep[4].ctypes.data,
-            keep[5].ctypes.data, head.ctypes.data if head is not None else None)
+            keep[5].ctypes.data, head.ctypes.data if head is not None else None, self._kv_mode(cfg.kv_mode))
         out = C.c_void_p()
         _ffi.check(_ffi.lib().llvq_hip_decoder_create(rt.handle, C.byref(desc), C.byref(out)))
         self.handle = out
+
+    @staticmethod
+    def _kv_mode(v):
+        """KvMode::parse (kvq.rs:38-49): a typo is an error, never a silent default."""
+        if v in (None, "", "f16"):
+            return 0
+        if v == "q8":
+            return 1
+        raise ValueError(f"kv_mode={v}: accepted values are 'f16' (default) and 'q8'")
 
     def reset(self):
         _ffi.check(_ffi.lib().llvq_hip_decoder_reset(self.handle))

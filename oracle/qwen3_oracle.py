@@ -48,16 +48,52 @@ def rms_norm(x, w, eps):
     return r16(x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps) * w)
 
 
+KV_GROUP = 64  # kvq.rs:36
+
+
+def kv_quantize(x):
+    """llvq-llm/src/kvq.rs:110-165 up to the codes: per group of 64 along the last axis,
+    s = f16((max - min) / 255), b = f16(min), q = clamp(round((x - b) / (s if s > 0 else 1)), 0, 255),
+    every step an f32 operation as candle runs it.  Returns (q uint8, s, b) with s, b as f32 arrays
+    holding binary16 values, shaped [..., groups, 1]."""
+    x = np.asarray(x, np.float32)
+    assert x.shape[-1] % KV_GROUP == 0, "head_dim is not a multiple of the group"
+    xg = x.reshape(x.shape[:-1] + (x.shape[-1] // KV_GROUP, KV_GROUP))
+    mn = xg.min(-1, keepdims=True)
+    mx = xg.max(-1, keepdims=True)
+    s = ((mx - mn) / np.float32(255.0)).astype(np.float16).astype(np.float32)
+    b = mn.astype(np.float16).astype(np.float32)
+    safe = np.where(s > 0, s, np.float32(1.0))
+    t = (xg - b) / safe
+    r = np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))  # f32::round: half away from zero
+    q = np.clip(r, 0, 255).astype(np.uint8)
+    return q, s, b
+
+
+def kv_dequantize(q, s, b, shape):
+    """The value a reader gets back (kvq.rs:155-164): f16(q s + b); an ungraded group (s = 0) is its bias."""
+    v = (q.astype(np.float32) * s).astype(np.float32) + b
+    return v.astype(np.float16).astype(np.float64).reshape(shape)
+
+
+def quantize_dequantize(x):
+    """kvq.rs:110: what KvCache::append stores under KvMode::Q8."""
+    q, s, b = kv_quantize(x)
+    return kv_dequantize(q, s, b, np.shape(x))
+
+
 def silu(x):
     return x / (1.0 + np.exp(-x))
 
 
 class Qwen3Oracle:
-    def __init__(self, cfg, dense_projections, weights):
+    def __init__(self, cfg, dense_projections, weights, kv_mode="f16"):
         """cfg: object with the Qwen3 Config field names; dense_projections[layer][j]: [d_out, d_in]
         arrays in the order q, k, v, o, gate, up, down; weights: binary16 arrays (input_norm,
         post_norm, q_norm, k_norm, final_norm, embed, lm_head or None)."""
         self.cfg = cfg
+        assert kv_mode in ("f16", "q8")
+        self.kv_mode = kv_mode
         self.W = [[np.asarray(m, np.float64) for m in layer] for layer in dense_projections]
         f = lambda a: np.asarray(a, np.float16).astype(np.float64)
         self.ln1, self.ln2 = f(weights.input_norm), f(weights.post_norm)
@@ -94,6 +130,8 @@ class Qwen3Oracle:
                 return r16(np.concatenate([t1 * cos - t2 * sin, t1 * sin + t2 * cos], axis=1))
 
             q, k = rope(q), rope(k)
+            if self.kv_mode == "q8":  # KvCache::append, model.rs:231-237: quantized once, on the way in
+                k, v = quantize_dequantize(k), quantize_dequantize(v)
             self.K[L].append(k)
             self.V[L].append(v)
             Kc = np.stack(self.K[L], axis=1)  # [nkv, T, hd]

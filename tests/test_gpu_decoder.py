@@ -21,23 +21,30 @@ RAGGED = decoder.Qwen3Config(num_hidden_layers=2, hidden_size=200, num_attention
                              max_positions=40, tie_word_embeddings=False)
 
 
+Q8 = decoder.Qwen3Config(num_hidden_layers=2, hidden_size=256, num_attention_heads=10, num_key_value_heads=2,
+                         head_dim=64, intermediate_size=384, vocab_size=400, rope_theta=1e6, rms_norm_eps=1e-6,
+                         max_positions=80, tie_word_embeddings=True, kv_mode="q8")  # 5 query heads per kv head, as at 14B
+
+
 def _build(gpu_rt, orc, cfg, seed):
     from oracle import qwen3_oracle
 
     raws = decoder.synthetic_projections(cfg, seed)
     weights = decoder.synthetic_weights(cfg, seed)
     dense = [[orc.read_matrix_raw(artifact.write_matrix_raw(m))[0].decode_matrix() for m in layer] for layer in raws]
-    ref = qwen3_oracle.Qwen3Oracle(cfg, dense, weights)
+    ref = qwen3_oracle.Qwen3Oracle(cfg, dense, weights, kv_mode=cfg.kv_mode)
     dec = decoder.Decoder(gpu_rt, cfg, raws, weights)
     return dec, ref
 
 
-@pytest.mark.parametrize("cfg,seed", [(SMALL, 1), (RAGGED, 2)])
-def test_teacher_forced_logits(gpu_rt, orc, cfg, seed):
+@pytest.mark.parametrize("cfg,seed,n", [(SMALL, 1, 24), (RAGGED, 2, 24), (Q8, 6, 70)])
+def test_teacher_forced_logits(gpu_rt, orc, cfg, seed, n):
+    """Q8: int8 KV cache on both sides; 70 positions also take the cache past one
+    range per workgroup (more than 32 positions) in the split attention."""
     dec, ref = _build(gpu_rt, orc, cfg, seed)
     try:
         rng = np.random.default_rng(seed)
-        tokens = rng.integers(0, cfg.vocab_size, size=24)
+        tokens = rng.integers(0, cfg.vocab_size, size=n)
         worst = 0.0
         agree = 0
         for t in tokens:
@@ -77,6 +84,21 @@ def test_greedy_tokens_match_oracle(gpu_rt, orc):
         assert np.array_equal(got, again)
     finally:
         dec.close()
+
+
+def test_kv_mode_is_parsed_strictly(gpu_rt):
+    """KvMode::parse (kvq.rs:38-49, test :240-249): a typo is an error, never a silent default."""
+    import dataclasses
+
+    from llvq_amd import LlvqError
+
+    raws = decoder.synthetic_projections(RAGGED, 1)
+    weights = decoder.synthetic_weights(RAGGED, 1)
+    for bad in ("Q8", "int8", "q4"):
+        with pytest.raises(ValueError):
+            decoder.Decoder(gpu_rt, dataclasses.replace(RAGGED, kv_mode=bad), raws, weights)
+    with pytest.raises(LlvqError):  # head_dim 32 is not a multiple of the group of 64 (kvq.rs:114-120)
+        decoder.Decoder(gpu_rt, dataclasses.replace(RAGGED, kv_mode="q8"), raws, weights)
 
 
 def test_generate_edge_cases(gpu_rt, orc):

@@ -118,6 +118,19 @@ def test_gemv_small_shapes(gpu_rt, orc, d_out, d_in):
     _check_gemv(orc, y16.astype(np.float32), raw, x)
 
 
+def test_gemv_rows_wider_than_the_full_tile(gpu_rt, orc):
+    """d_in 17408 (the 14B intermediate size: 725 blocks + 8 tail columns): the activation
+    planes leave no room for the 4096-block tile, so the half-tile variant runs."""
+    import torch
+
+    raw = synth.make_matrix("model.layers.0.mlp.down_proj.weight", 40, 17408, seed=14)
+    x = synth.make_activation(17408, seed=14)[0]
+    proj = gpu_rt.upload(raw)
+    y = gpu_rt.forward(proj, _x16(x), out_dtype=torch.float32).cpu().numpy()
+    gpu_rt.free(proj)
+    assert _check_gemv(orc, y, raw, x) < 1e-5
+
+
 def test_gemv_origin_and_shell13_blocks(gpu_rt, orc):
     """A matrix whose blocks are origins (decode to zero whatever the gain) and
     shell-13 indices above N(12)."""

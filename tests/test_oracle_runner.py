@@ -126,3 +126,65 @@ def test_generate_edges():
     out, trace = ref.generate([1, 2, 3], 5)
     assert out.size == 5 and len(trace) == 5 and ref.pos == 3 + 4
     assert all(int(np.argmax(l)) == t for l, t in zip(trace, out))
+
+
+# ---- KV-q8 (llvq-llm/src/kvq.rs tests :218-344) ---------------------------------------------
+def _cache_like(t):
+    """kvq.rs:223-237: 8 KV heads x t tokens x head_dim 128, spread growing with the head."""
+    i = np.arange(8 * t * 128)
+    head = (i // (t * 128)) % 8
+    x = (i % 977).astype(np.float32) / np.float32(977.0) - np.float32(0.5)
+    v = (1.0 + head).astype(np.float32) * x * np.sign(x) * np.float32(3.0)
+    return v.reshape(1, 8, t, 128).astype(np.float16)
+
+
+def test_kvq_prefill_and_decode_agree_bit_for_bit():  # kvq.rs:252-275
+    full = _cache_like(16)
+    both = Q.quantize_dequantize(full)
+    for t in (0, 1, 7, 15):
+        assert np.array_equal(Q.quantize_dequantize(full[:, :, t:t + 1]), both[:, :, t:t + 1])
+
+
+def test_kvq_constant_group_reconstructs_exactly():  # kvq.rs:278-312
+    v = np.where(np.arange(128) < 64, 0.375, np.arange(128) / 128.0).astype(np.float16).reshape(1, 1, 1, 128)
+    out = Q.quantize_dequantize(v)
+    assert np.array_equal(out[..., :64], v[..., :64].astype(np.float64))
+    assert out[..., 64:].max() - out[..., 64:].min() > 0.4
+
+
+def test_kvq_known_codes_and_half_step_bound():
+    """Hand-computed: the ramp i/64, i = 0..63, has min 0 and max 63/64, so s = f16(63/64/255)
+    and q_i = round((i/64)/s); the extremes land on 0 and 255 and the error is half a step."""
+    x = (np.arange(64) / 64.0).astype(np.float16).reshape(1, 64)
+    q, s, b = Q.kv_quantize(x)
+    s16 = float(np.float16(np.float32(63 / 64) / np.float32(255)))
+    assert float(s.reshape(())) == s16 and float(b.reshape(())) == 0.0
+    want = np.floor(np.arange(64) / 64.0 / s16 + 0.5)
+    assert np.array_equal(q.reshape(-1), np.clip(want, 0, 255).astype(np.uint8))
+    assert q.reshape(-1)[0] == 0 and q.reshape(-1)[-1] == 255
+    deq = Q.kv_dequantize(q, s, b, x.shape)
+    assert np.abs(deq - x.astype(np.float64)).max() <= s16 / 2 + 2 ** -11  # half a step + the binary16 rounding
+    # rounding, not truncation (kvq.rs:315-344): the mean error is centred
+    big = _cache_like(4)
+    err = Q.quantize_dequantize(big) - big.astype(np.float64)
+    assert abs(err.mean()) < 0.1 * np.abs(err).mean()
+
+
+def test_runner_q8_cache_holds_reconstructed_values():
+    ref, W, w = _model(seed=13)
+    c = SimpleNamespace(**{**CFG.__dict__, "head_dim": 64, "num_attention_heads": 2, "num_key_value_heads": 1,
+                           "hidden_size": 48})
+    qd, kvd = 128, 64
+    rng = np.random.default_rng(2)
+    shapes = [(qd, 48), (kvd, 48), (kvd, 48), (48, qd), (80, 48), (80, 48), (48, 80)]
+    Wn = [[(rng.standard_normal(s) / np.sqrt(s[1])).astype(np.float32) for s in shapes] for _ in range(2)]
+    g = lambda *s: (1 + 0.1 * rng.standard_normal(s)).astype(np.float16)
+    wn = SimpleNamespace(input_norm=g(2, 48), post_norm=g(2, 48), q_norm=g(2, 64), k_norm=g(2, 64), final_norm=g(48),
+                         embed=rng.standard_normal((61, 48)).astype(np.float16), lm_head=None)
+    a = Q.Qwen3Oracle(c, Wn, wn, kv_mode="q8")
+    b = Q.Qwen3Oracle(c, Wn, wn, kv_mode="f16")
+    la, lb = a.forward_token(3), b.forward_token(3)
+    # what the q8 cache holds is the quantize-dequantize of what the f16 cache holds (layer 0: same inputs)
+    assert np.array_equal(a.K[0][0], Q.quantize_dequantize(b.K[0][0]))
+    assert np.array_equal(a.V[0][0], Q.quantize_dequantize(b.V[0][0]))
+    assert np.abs(la - lb).max() < 0.05 * np.abs(lb).max() and not np.array_equal(la, lb)
