@@ -115,6 +115,74 @@ def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
     }
 
 
+def bench_decode14b(args, torch, llvq_amd):
+    """BASELINE config 4: Qwen3-14B-architecture decode at batch 1 with an int8 KV cache and
+    split-KV attention at a long context.  A step is one decoded token at about `--context`
+    cached positions (the decoder seeks there: cache entries hold zeros except for the tokens
+    decoded here).  All 280 LLVQ matrices (3.3 GB of codes) and the f16 embedding and head are
+    resident in HBM."""
+    from llvq_amd import decoder
+
+    cfg = decoder.QWEN3_14B
+    t0 = time.time()
+    rt = llvq_amd.FusedRuntime(device=0)
+    projs = []
+    enc_bytes = 0
+    for layer in range(cfg.num_hidden_layers):
+        raws = [llvq_amd.synth.make_matrix(f"model.layers.{layer}.{site}.weight", do, di, args.seed)
+                for site, do, di in cfg.shapes()]
+        enc_bytes += sum(m.encoded_bytes() for m in raws)
+        projs.append([rt.upload(m) for m in raws])
+        if layer % 8 == 7:
+            log(f"[bench] uploaded {layer + 1}/{cfg.num_hidden_layers} layers ({time.time() - t0:.1f}s)")
+    weights = decoder.synthetic_weights(cfg, args.seed)
+    dec = decoder.Decoder(rt, cfg, projs, weights)
+    del weights
+    log(f"[bench] decoder built in {time.time() - t0:.1f}s")
+    n_new = max(8, args.steps)
+    start = max(0, min(cfg.max_positions - n_new - args.warmup - 2, args.context - n_new))
+    results = {}
+    for name, pos in (("short", 0), ("long", start)):
+        dec.seek(pos)
+        tok = 1
+        for _ in range(max(1, args.warmup)):
+            _, tok = dec.forward_token(tok, want_logits=False)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(n_new):
+            _, tok = dec.forward_token(tok, want_logits=False)
+        dt = (time.perf_counter() - t1) / n_new
+        results[name] = dt
+        log(f"[bench] {name} context ({pos}+): {dt * 1e3:.3f} ms/token")
+    dec.close()
+    step = results["long"]
+    kv_bytes = 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * (1 + 4 / 64) * (start + n_new)
+    out = {
+        "metric": "decode_tokens_per_s",
+        "value": round(1.0 / step, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": n_new,
+        "warmup": max(1, args.warmup),
+        "ms_per_step": round(step * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"Qwen3-14B-architecture batch-1 decode (BASELINE config 4): 40 layers, 280 LLVQ matrices, "
+                               f"{enc_bytes} encoded bytes, int8 KV cache, {start + n_new} cached positions, split-KV attention, "
+                               "f16 embedding and head (vocabulary 151936); one host round trip per token",
+                   "context": start + n_new, "seed": args.seed},
+        "ms_per_token_empty_cache": round(results["short"] * 1e3, 4),
+        "attention_ms_per_token": round((results["long"] - results["short"]) * 1e3, 4),
+        "kv_cache_bytes_read_per_token": int(kv_bytes),
+        "encoded_weight_GBps": round(enc_bytes / step / 1e9, 2),
+    }
+    rt.close()
+    print(json.dumps(out), flush=True)
+
+
 QWEN3_8B_LAYER = [  # (site, d_out, d_in): hidden 4096, intermediate 12288, 32 query / 8 KV heads of 128
     ("self_attn.q_proj", 4096, 4096),
     ("self_attn.k_proj", 1024, 4096),
@@ -221,7 +289,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true",
                     help="skip the greedy-decode leg (tokens/s of the full model loop) of the gemv workload")
-    ap.add_argument("--workload", choices=["gemv", "gemm"], default="gemv",
+    ap.add_argument("--context", type=int, default=8192, help="cached positions of the decode14b workload")
+    ap.add_argument("--workload", choices=["gemv", "gemm", "decode14b"], default="gemv",
                     help="gemv: the headline batch-1 projection pass (default); gemm: the batched "
                          "matrix-core path at Qwen3-8B shapes")
     ap.add_argument("--M", type=int, default=256, help="activation rows of the gemm workload")
@@ -245,6 +314,8 @@ def main():
     dev = torch.device("cuda", 0)
     if args.workload == "gemm":
         return bench_gemm(args, torch, llvq_amd, synth, dev)
+    if args.workload == "decode14b":
+        return bench_decode14b(args, torch, llvq_amd)
     layers = build_layers(args.layers, args.seed)
     acts_np = {d: synth.make_activation(d, args.seed)[0] for d in (2560, 4096, 9728)}
     acts = {d: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16).to(dev) for d, a in acts_np.items()}

@@ -182,6 +182,12 @@ void llvq_hip_decoder_destroy(llvq_decoder* dec);
 /* fresh_caches (model.rs:963): the next token is position 0 again. */
 int llvq_hip_decoder_reset(llvq_decoder* dec);
 int llvq_hip_decoder_position(const llvq_decoder* dec);
+/* Measurement aid with no counterpart in the reference: makes `position` the next
+ * position without feeding the tokens before it, so the attention cost of a long
+ * context can be timed without a long prefill.  Cache entries that were never
+ * written hold zeros (a valid key/value), so the results are well defined but
+ * are not those of any real prompt. */
+int llvq_hip_decoder_seek(llvq_decoder* dec, uint32_t position);
 /* hidden_cached at l = 1 followed by Head::project (model.rs:968-982, :578-587):
  * feeds one token at the current position, advances it, and returns the
  * logits (vocab f32 values, each already rounded to binary16 as the reference's

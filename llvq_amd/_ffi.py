@@ -107,6 +107,7 @@ def lib():
     L.llvq_hip_decoder_destroy.restype = None
     L.llvq_hip_decoder_reset.argtypes = [vp]
     L.llvq_hip_decoder_position.argtypes = [vp]
+    L.llvq_hip_decoder_seek.argtypes = [vp, C.c_uint32]
     L.llvq_hip_decoder_forward_token.argtypes = [vp, C.c_uint32, vp, C.POINTER(C.c_uint32)]
     L.llvq_hip_decoder_generate.argtypes = [vp, vp, sz, sz, vp]
     L.llvq_hip_last_error.restype = C.c_char_p
@@ -128,6 +129,6 @@ EXPORTS = [
     "llvq_hip_gemv_group", "llvq_hip_gemm", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
     "llvq_hip_last_error", "llvq_hip_version",
     "llvq_hip_host_rotate", "llvq_hip_rotate", "llvq_hip_gemv_rotated", "llvq_hip_matrix_rotation",
-    "llvq_hip_decoder_create", "llvq_hip_decoder_destroy", "llvq_hip_decoder_reset", "llvq_hip_decoder_position",
+    "llvq_hip_decoder_create", "llvq_hip_decoder_destroy", "llvq_hip_decoder_reset", "llvq_hip_decoder_position", "llvq_hip_decoder_seek",
     "llvq_hip_decoder_forward_token", "llvq_hip_decoder_generate",
 ]

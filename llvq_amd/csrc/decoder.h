@@ -208,13 +208,17 @@ __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restr
 
 // Attention of one query position over the cache (model.rs:812-822), split over
 // the cache: workgroup (kv head, split) takes a contiguous range of positions
-// and all query heads that share the kv head (one wavefront per query head, so
-// K and V rows are fetched once per group), and leaves an unnormalised partial
-// (running max, sum of exponentials, weighted V sum).  The workgroup that
-// arrives last at the kv head's counter merges the partials in split order and
-// rounds the context once.  Scores, softmax and sums stay in f32.
+// for all query heads that share the kv head, so every K and V row is fetched
+// (and, for the int8 cache, rebuilt) once per group.  Its four wavefronts take
+// positions round-robin, four positions at a time (16 lanes x 8 dims per row);
+// the workgroup leaves an unnormalised partial per query head (running max, sum
+// of exponentials, weighted V sum), and the workgroup that arrives last at the
+// kv head's counter merges the partials in split order and rounds the context
+// once.  Scores, softmax and sums stay in f32.
 constexpr int kAttnThreads = 256;
+constexpr int kAttnWaves = kAttnThreads / 64;
 constexpr int kAttnMaxSplits = 64;  // the cache is cut into at most this many ranges (host picks by length)
+constexpr int kAttnMaxGroup = 8;    // query heads per kv head
 template <bool Q8>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half* __restrict__ q, const __half* __restrict__ kcache,
                                                                    const __half* __restrict__ vcache, KvQ8 q8,
@@ -222,13 +226,17 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
                                                                    float* __restrict__ part, uint32_t* __restrict__ counters,
                                                                    uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
                                                                    uint32_t T, uint32_t max_pos, float scale, uint32_t n_splits) {
-  extern __shared__ __align__(16) float att_smem[];  // [4][chunk] scores
+  extern __shared__ __align__(16) float att_smem[];
   __shared__ uint32_t arrived;
+  __shared__ float red[kAttnWaves][kAttnMaxGroup];
   const uint32_t kvh = blockIdx.x / n_splits, split = blockIdx.x % n_splits;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const uint32_t groups = n_heads / n_kv;
+  const uint32_t groups = n_heads / n_kv;  // <= kAttnMaxGroup (checked by the host)
   const uint32_t chunk = (T + n_splits - 1) / n_splits;
-  const uint32_t j0 = min(T, split * chunk), j1 = min(T, j0 + chunk);
+  const uint32_t j0 = min(T, split * chunk), j1 = min(T, j0 + chunk), nj = j1 - j0;
+  float* qs = att_smem;                         // [groups][head_dim]
+  float* sc = qs + groups * head_dim;           // [groups][chunk]
+  float* accs = sc + groups * chunk;            // [kAttnWaves][groups][head_dim]
   const __half* K = kcache + (size_t)kvh * max_pos * head_dim;
   const __half* V = vcache + (size_t)kvh * max_pos * head_dim;
   const uint32_t kvgroups = head_dim / kKvGroup;
@@ -238,101 +246,196 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
   const __half* Kb = q8.kb + (size_t)kvh * max_pos * kvgroups;
   const __half* Vs = q8.vs + (size_t)kvh * max_pos * kvgroups;
   const __half* Vb = q8.vb + (size_t)kvh * max_pos * kvgroups;
-  float* sc = att_smem + (size_t)wave * chunk;
   const uint32_t stride = head_dim + 2;  // floats per partial: max, sum, head_dim sums
-  const uint32_t sub = lane & 15u, pj = lane >> 4;  // 16 lanes x 8 dims (zero-padded) cover a position's row
-  const uint32_t dsteps = (head_dim + 127) >> 7;   // 128-dim passes over a row
-  for (uint32_t g = wave; g < groups; g += kAttnThreads / 64) {
-    const uint32_t head = kvh * groups + g;
-    float m = -INFINITY, l = 0.f;
-    // scores of this wavefront's query head over [j0, j1)
-    for (uint32_t p0 = j0; p0 < j1; p0 += 4) {
-      const uint32_t j = p0 + pj;
-      float d = 0.f;
-      for (uint32_t ds = 0; ds < dsteps; ++ds) {
-        const uint32_t i0 = ds * 128u + sub * 8u;
-        if (j < j1 && i0 < head_dim) {
-          const uint4 qq = *reinterpret_cast<const uint4*>(q + (size_t)head * head_dim + i0);
-          const uint32_t qw[4] = {qq.x, qq.y, qq.z, qq.w};
+
+  for (uint32_t i = tid; i < groups * head_dim; i += kAttnThreads)
+    qs[i] = __half2float(q[(size_t)kvh * groups * head_dim + i]) * scale;
+  __syncthreads();
+
+  // ---- scores ----
+  const uint32_t sub = lane & 15u, pj = lane >> 4;
+  const uint32_t dsteps = (head_dim + 127) >> 7;
+  float m[kAttnMaxGroup];
+#pragma unroll
+  for (int g = 0; g < kAttnMaxGroup; ++g) m[g] = -INFINITY;
+  constexpr int PB = 4;  // row pieces fetched together, so their latencies overlap
+  for (uint32_t pb0 = wave * 4u; pb0 < nj; pb0 += kAttnWaves * 4u * PB) {
+    for (uint32_t ds = 0; ds < dsteps; ++ds) {
+      const uint32_t i0 = ds * 128u + sub * 8u;
+      uint4 kraw[PB];
+      float ksc[PB], kbi[PB];
+#pragma unroll
+      for (int b = 0; b < PB; ++b) {
+        const uint32_t jj = pb0 + (uint32_t)b * kAttnWaves * 4u + pj, j = j0 + jj;
+        kraw[b] = make_uint4(0, 0, 0, 0);
+        ksc[b] = kbi[b] = 0.f;
+        if (jj < nj && i0 < head_dim) {
           if constexpr (Q8) {
             const uint2 kc = *reinterpret_cast<const uint2*>(Kq + (size_t)j * head_dim + i0);
-            const float ksc = __half2float(Ks[(size_t)j * kvgroups + i0 / kKvGroup]);
-            const float kbi = __half2float(Kb[(size_t)j * kvgroups + i0 / kKvGroup]);
-            const uint32_t kw[2] = {kc.x, kc.y};
+            kraw[b].x = kc.x;
+            kraw[b].y = kc.y;
+            ksc[b] = __half2float(Ks[(size_t)j * kvgroups + i0 / kKvGroup]);
+            kbi[b] = __half2float(Kb[(size_t)j * kvgroups + i0 / kKvGroup]);
+          } else {
+            kraw[b] = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0);
+          }
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < PB; ++b) {
+        const uint32_t jj = pb0 + (uint32_t)b * kAttnWaves * 4u + pj;
+        float d[kAttnMaxGroup];
+#pragma unroll
+        for (int g = 0; g < kAttnMaxGroup; ++g) d[g] = 0.f;
+        if (jj < nj && i0 < head_dim) {
+          float kf[8];
+          if constexpr (Q8) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-              const uint32_t c0 = (kw[t >> 1] >> (16 * (t & 1))) & 0xFFu, c1 = (kw[t >> 1] >> (16 * (t & 1) + 8)) & 0xFFu;
-              d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] & 0xFFFFu))), kv_dequant(c0, ksc, kbi), d);
-              d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] >> 16))), kv_dequant(c1, ksc, kbi), d);
+              kf[t] = kv_dequant((kraw[b].x >> (8 * t)) & 0xFFu, ksc[b], kbi[b]);
+              kf[4 + t] = kv_dequant((kraw[b].y >> (8 * t)) & 0xFFu, ksc[b], kbi[b]);
             }
           } else {
-            const uint4 kk = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0);
-            const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w};
+            const uint32_t kw[4] = {kraw[b].x, kraw[b].y, kraw[b].z, kraw[b].w};
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-              d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] & 0xFFFFu))),
-                       __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu))), d);
-              d = fmaf(__half2float(__ushort_as_half((unsigned short)(qw[t] >> 16))),
-                       __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16))), d);
+              kf[2 * t] = __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu)));
+              kf[2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16)));
+            }
+          }
+#pragma unroll
+          for (int g = 0; g < kAttnMaxGroup; ++g)
+            if ((uint32_t)g < groups) {
+              const float* qg = qs + g * head_dim + i0;
+#pragma unroll
+              for (int t = 0; t < 8; ++t) d[g] = fmaf(qg[t], kf[t], d[g]);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < kAttnMaxGroup; ++g)
+          if ((uint32_t)g < groups) {
+            float v = d[g];
+            v += __shfl_xor(v, 1, 64);
+            v += __shfl_xor(v, 2, 64);
+            v += __shfl_xor(v, 4, 64);
+            v += __shfl_xor(v, 8, 64);
+            // a head wider than 128 accumulates its passes in the score slot
+            if (jj < nj && sub == 0) sc[g * chunk + jj] = ds ? sc[g * chunk + jj] + v : v;
+          }
+      }
+    }
+  }
+  __syncthreads();
+  // running maxima: every lane scans the scores of its positions
+  for (uint32_t jj = tid; jj < nj; jj += kAttnThreads)
+#pragma unroll
+    for (int g = 0; g < kAttnMaxGroup; ++g)
+      if ((uint32_t)g < groups) m[g] = fmaxf(m[g], sc[g * chunk + jj]);
+#pragma unroll
+  for (int g = 0; g < kAttnMaxGroup; ++g) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) m[g] = fmaxf(m[g], __shfl_xor(m[g], o, 64));
+    if (lane == 0) red[wave][g] = m[g];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < kAttnMaxGroup; ++g) {
+    m[g] = red[0][g];
+#pragma unroll
+    for (int w = 1; w < kAttnWaves; ++w) m[g] = fmaxf(m[g], red[w][g]);
+  }
+  __syncthreads();  // red is reused for the sums
+  // ---- exponentials and their sums ----
+  float l[kAttnMaxGroup];
+#pragma unroll
+  for (int g = 0; g < kAttnMaxGroup; ++g) {
+    l[g] = 0.f;
+    if ((uint32_t)g < groups)
+      for (uint32_t jj = tid; jj < nj; jj += kAttnThreads) {
+        const float e = __expf(sc[g * chunk + jj] - m[g]);
+        sc[g * chunk + jj] = e;
+        l[g] += e;
+      }
+    l[g] = wave_sum(l[g]);
+    if (lane == 0) red[wave][g] = l[g];
+  }
+  __syncthreads();
+  // ---- weighted V sums: wavefront w takes positions w, w + 4, ...; lane owns dims 2 lane, 2 lane + 1 of each 128 ----
+  for (uint32_t ds = 0; ds < dsteps; ++ds) {
+    const uint32_t i0 = ds * 128u + lane * 2u;
+    float a0[kAttnMaxGroup], a1[kAttnMaxGroup];
+#pragma unroll
+    for (int g = 0; g < kAttnMaxGroup; ++g) a0[g] = a1[g] = 0.f;
+    if (i0 < head_dim) {
+      constexpr int VB = 8;  // V rows fetched together
+      for (uint32_t jb = wave; jb < nj; jb += kAttnWaves * VB) {
+        uint32_t vraw[VB];
+        float vsc[VB], vbi[VB];
+#pragma unroll
+        for (int b = 0; b < VB; ++b) {
+          const uint32_t jj = jb + (uint32_t)b * kAttnWaves, j = j0 + jj;
+          vraw[b] = 0;
+          vsc[b] = vbi[b] = 0.f;
+          if (jj < nj) {
+            if constexpr (Q8) {
+              vraw[b] = *reinterpret_cast<const unsigned short*>(Vq + (size_t)j * head_dim + i0);
+              vsc[b] = __half2float(Vs[(size_t)j * kvgroups + i0 / kKvGroup]);
+              vbi[b] = __half2float(Vb[(size_t)j * kvgroups + i0 / kKvGroup]);
+            } else {
+              vraw[b] = *reinterpret_cast<const uint32_t*>(V + (size_t)j * head_dim + i0);
             }
           }
         }
-      }
-      d += __shfl_xor(d, 1, 64);
-      d += __shfl_xor(d, 2, 64);
-      d += __shfl_xor(d, 4, 64);
-      d += __shfl_xor(d, 8, 64);
-      d *= scale;
-      if (j < j1) {
-        if (sub == 0) sc[j - j0] = d;
-        m = fmaxf(m, d);
-      }
-    }
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-    for (uint32_t j = j0 + lane; j < j1; j += 64) {
-      const float e = __expf(sc[j - j0] - m);
-      sc[j - j0] = e;
-      l += e;
-    }
-    l = wave_sum(l);
-    __threadfence_block();
-    // weighted V sum: lane owns dims 2 lane, 2 lane + 1 of each 128-dim pass
-    float* dst = part + ((size_t)head * n_splits + split) * stride;
-    for (uint32_t ds = 0; ds < dsteps; ++ds) {
-      const uint32_t i0 = ds * 128u + lane * 2u;
-      float a0 = 0.f, a1 = 0.f;
-      if (i0 < head_dim) {
-        if constexpr (Q8) {
-          for (uint32_t j = j0; j < j1; ++j) {
-            const uint32_t vc = *reinterpret_cast<const unsigned short*>(Vq + (size_t)j * head_dim + i0);
-            const float vsc = __half2float(Vs[(size_t)j * kvgroups + i0 / kKvGroup]);
-            const float vbi = __half2float(Vb[(size_t)j * kvgroups + i0 / kKvGroup]);
-            const float p = sc[j - j0];
-            a0 = fmaf(p, kv_dequant(vc & 0xFFu, vsc, vbi), a0);
-            a1 = fmaf(p, kv_dequant(vc >> 8, vsc, vbi), a1);
-          }
-        } else {
-          for (uint32_t j = j0; j < j1; ++j) {
-            const __half2 vv = *reinterpret_cast<const __half2*>(V + (size_t)j * head_dim + i0);
-            const float p = sc[j - j0];
-            a0 = fmaf(p, __low2float(vv), a0);
-            a1 = fmaf(p, __high2float(vv), a1);
+        for (int b = 0; b < VB; ++b) {
+          const uint32_t jj = jb + (uint32_t)b * kAttnWaves;
+          if (jj < nj) {
+            float v0, v1;
+            if constexpr (Q8) {
+              v0 = kv_dequant(vraw[b] & 0xFFu, vsc[b], vbi[b]);
+              v1 = kv_dequant(vraw[b] >> 8, vsc[b], vbi[b]);
+            } else {
+              v0 = __half2float(__ushort_as_half((unsigned short)(vraw[b] & 0xFFFFu)));
+              v1 = __half2float(__ushort_as_half((unsigned short)(vraw[b] >> 16)));
+            }
+#pragma unroll
+            for (int g = 0; g < kAttnMaxGroup; ++g)
+              if ((uint32_t)g < groups) {
+                const float p = sc[g * chunk + jj];
+                a0[g] = fmaf(p, v0, a0[g]);
+                a1[g] = fmaf(p, v1, a1[g]);
+              }
           }
         }
       }
-      if (i0 < head_dim) {
-        dst[2 + i0] = a0;
-        dst[2 + i0 + 1] = a1;
-      }
+#pragma unroll
+      for (int g = 0; g < kAttnMaxGroup; ++g)
+        if ((uint32_t)g < groups) {
+          accs[((size_t)wave * groups + g) * head_dim + i0] = a0[g];
+          accs[((size_t)wave * groups + g) * head_dim + i0 + 1] = a1[g];
+        }
     }
-    if (lane == 0) {
-      dst[0] = m;  // -inf for an empty range
-      dst[1] = l;
-    }
-    __builtin_amdgcn_wave_barrier();  // sc is reused by this wavefront's next query head
+  }
+  __syncthreads();
+  // ---- this workgroup's partial: wavefront sums added in wavefront order ----
+  for (uint32_t o = tid; o < groups * head_dim; o += kAttnThreads) {
+    const uint32_t g = o / head_dim, i = o - g * head_dim;
+    float a = 0.f;
+#pragma unroll
+    for (int w = 0; w < kAttnWaves; ++w) a += accs[((size_t)w * groups + g) * head_dim + i];
+    part[((size_t)(kvh * groups + g) * n_splits + split) * stride + 2 + i] = a;
+  }
+  if (tid < groups) {
+    float ls = 0.f;
+#pragma unroll
+    for (int w = 0; w < kAttnWaves; ++w) ls += red[w][tid];
+    float* dst = part + ((size_t)(kvh * groups + tid) * n_splits + split) * stride;
+    float mg = -INFINITY;  // m[] is register-indexed by a constant only: pick by comparison
+#pragma unroll
+    for (int g = 0; g < kAttnMaxGroup; ++g)
+      if ((uint32_t)g == tid) mg = m[g];
+    dst[0] = mg;  // -inf for an empty range
+    dst[1] = ls;
   }
   // publish, and let the last workgroup of this kv head merge (one lane's
   // device-scope release / acquire stands for the workgroup, ordered by the barriers)
@@ -340,19 +443,50 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
   if (tid == 0) arrived = __hip_atomic_fetch_add(&counters[kvh], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   if (arrived != n_splits - 1) return;
+  // Merge.  The (max, sum) pairs of every (head, split) are fetched in one pass
+  // and turned into weights in LDS; the weighted sums then read the partial
+  // vectors with many loads in flight (they come from the other XCDs' writes,
+  // i.e. from memory, so latency is what matters here).
+  float* wts = att_smem;                     // [groups][n_splits] weights (the staging of this launch is dead)
+  float* Ls = wts + groups * n_splits;       // [groups]
+  for (uint32_t o = tid; o < groups * n_splits; o += kAttnThreads) {
+    const uint32_t g = o / n_splits, sp = o - g * n_splits;
+    wts[o] = part[((size_t)(kvh * groups + g) * n_splits + sp) * stride];  // the split's running max
+  }
+  __syncthreads();
+  if (tid < groups) {
+    float M = -INFINITY;
+    for (uint32_t sp = 0; sp < n_splits; ++sp) M = fmaxf(M, wts[tid * n_splits + sp]);
+    Ls[tid] = M;
+  }
+  __syncthreads();
+  for (uint32_t o = tid; o < groups * n_splits; o += kAttnThreads) {
+    const uint32_t g = o / n_splits;
+    wts[o] = __expf(wts[o] - Ls[g]);  // 0 for an empty range
+  }
+  __syncthreads();
+  if (tid < groups) {
+    float L = 0.f;
+    for (uint32_t sp = 0; sp < n_splits; ++sp)
+      L = fmaf(part[((size_t)(kvh * groups + tid) * n_splits + sp) * stride + 1], wts[tid * n_splits + sp], L);
+    Ls[tid] = L;
+  }
+  __syncthreads();
   for (uint32_t o = tid; o < groups * head_dim; o += kAttnThreads) {
     const uint32_t g = o / head_dim, i = o - g * head_dim;
     const uint32_t head = kvh * groups + g;
-    const float* src = part + (size_t)head * n_splits * stride;
-    float M = -INFINITY;
-    for (uint32_t s = 0; s < n_splits; ++s) M = fmaxf(M, src[(size_t)s * stride]);
-    float L = 0.f, A = 0.f;
-    for (uint32_t s = 0; s < n_splits; ++s) {
-      const float w = __expf(src[(size_t)s * stride] - M);  // 0 for an empty range
-      L = fmaf(src[(size_t)s * stride + 1], w, L);
-      A = fmaf(src[(size_t)s * stride + 2 + i], w, A);
+    const float* src = part + (size_t)head * n_splits * stride + 2 + i;
+    float A = 0.f;
+    uint32_t sp = 0;
+    for (; sp + 8 <= n_splits; sp += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(sp + u) * stride];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) A = fmaf(v[u], wts[g * n_splits + sp + u], A);  // split order
     }
-    ctx[(size_t)head * head_dim + i] = __float2half_rn(A / L);
+    for (; sp < n_splits; ++sp) A = fmaf(src[(size_t)sp * stride], wts[g * n_splits + sp], A);
+    ctx[(size_t)head * head_dim + i] = __float2half_rn(A / Ls[g]);
   }
   if (tid == 0) counters[kvh] = 0;  // ready for the next launch
 }

@@ -1031,6 +1031,14 @@ static uint32_t pick_rows_per_tile(const llvq_mat* const* mats, int n, uint32_t 
   return r < 1 ? 1 : r;
 }
 
+// Whether a launch over rows of this width can stage a derived activation where
+// its tile's code bytes go.
+static bool prologue_fits(const llvq_mat* m0) {
+  uint32_t tile = kTileBlocks;
+  if (gemv_lds_bytes(m0->nblocks, tile) > 160 * 1024) tile = kSmallTileBlocks;
+  return (size_t)m0->d_in * 2 <= (size_t)tile * 6 + 32;
+}
+
 struct Prologue {
   uint32_t kind = kPrologueNone;
   const void* x2 = nullptr;
@@ -1371,15 +1379,19 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   const uint32_t T = d->pos + 1;
   uint32_t n_splits = (T + 31) / 32;  // about 32 cached positions per workgroup, at most kAttnMaxSplits ranges
   if (n_splits > (uint32_t)kAttnMaxSplits) n_splits = kAttnMaxSplits;
-  const size_t attn_lds = (size_t)(kAttnThreads / 64) * ((T + n_splits - 1) / n_splits) * sizeof(float);
+  const uint32_t groups_per_kv = d->n_heads / d->n_kv;
+  size_t attn_lds = ((size_t)groups_per_kv * d->head_dim * (1 + kAttnWaves) + (size_t)groups_per_kv * ((T + n_splits - 1) / n_splits)) * sizeof(float);
+  const size_t merge_lds = (size_t)groups_per_kv * (n_splits + 1) * sizeof(float);  // the merge reuses the staging area
+  if (attn_lds < merge_lds) attn_lds = merge_lds;
   const size_t group_layer = cache_layer / kKvGroup;
   // Projections in the natural basis derive their activation in the launch's
   // prologue; a rotated basis needs the activation as a tensor first (it goes
-  // through the rotation kernel), so its prologue runs as a kernel of its own.
+  // through the rotation kernel), and so do rows too wide for the staging area:
+  // their prologue runs as a kernel of its own.
   auto project = [&](const llvq_mat* const* mats, int n, const __half* x, void* const* outs, const Prologue& pro) -> int {
     bool rotated = false;
     for (int i = 0; i < n; ++i) rotated |= mats[i]->has_rotation;
-    if (!rotated) return launch_group(rt, mats, n, x, outs, LLVQ_F16, &pro);
+    if (!rotated && prologue_fits(mats[0])) return launch_group(rt, mats, n, x, outs, LLVQ_F16, &pro);
     const __half* staged = nullptr;
     if (pro.kind == kPrologueAddRmsNorm) {
       hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, x, reinterpret_cast<const __half*>(pro.x2),
@@ -1470,12 +1482,12 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   if (!c->projections || !c->input_norm || !c->post_norm || !c->q_norm || !c->k_norm || !c->final_norm || !c->embed)
     return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: a required tensor is null");
   if (c->n_layers == 0 || c->hidden == 0 || c->hidden % 8 || c->hidden > 8192 || c->n_heads == 0 || c->n_kv_heads == 0 ||
-      c->n_heads % c->n_kv_heads || c->head_dim == 0 || c->head_dim % 8 || c->head_dim > 256 || c->intermediate == 0 ||
+      c->n_heads % c->n_kv_heads || c->n_heads / c->n_kv_heads > (uint32_t)kAttnMaxGroup || c->head_dim == 0 || c->head_dim % 8 || c->head_dim > 256 || c->intermediate == 0 ||
       c->vocab == 0 || c->max_positions == 0 || c->max_positions > 8192 ||
       (c->kv_mode != LLVQ_KV_F16 && c->kv_mode != LLVQ_KV_Q8) || (c->kv_mode == LLVQ_KV_Q8 && c->head_dim % 64))
     return fail(LLVQ_ERR_UNSUPPORTED,
                 "decoder_create: shape outside what the kernels hold (hidden % 8 = 0 and <= 8192, head_dim % 8 = 0 and <= 256, "
-                "heads a multiple of kv heads, max_positions <= 8192, kv_mode f16 or q8 with head_dim % 64 = 0)");
+                "heads a multiple of kv heads and at most 8 per kv head, max_positions <= 8192, kv_mode f16 or q8 with head_dim % 64 = 0)");
   const uint32_t qd = c->n_heads * c->head_dim, kvd = c->n_kv_heads * c->head_dim;
   static const char* kSite[7] = {"q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"};
   const uint32_t want_out[7] = {qd, kvd, kvd, c->hidden, c->intermediate, c->intermediate, c->hidden};
@@ -1586,6 +1598,13 @@ int llvq_hip_decoder_reset(llvq_decoder* d) {
 }
 
 int llvq_hip_decoder_position(const llvq_decoder* d) { return d ? (int)d->pos : -1; }
+
+int llvq_hip_decoder_seek(llvq_decoder* d, uint32_t position) {
+  if (!d) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_seek: null decoder");
+  if (position >= d->max_pos) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_seek: position past max_positions");
+  d->pos = position;
+  return LLVQ_OK;
+}
 
 int llvq_hip_decoder_forward_token(llvq_decoder* d, uint32_t token, float* logits_host, uint32_t* argmax_host) {
   if (!d) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_forward_token: null decoder");

@@ -38,6 +38,7 @@ class Qwen3Config:
                 (SITES[4], i, h), (SITES[5], i, h), (SITES[6], h, i)]
 
 
+QWEN3_14B = Qwen3Config(40, 5120, 40, 8, 128, 17408, 151936, max_positions=8192, tie_word_embeddings=False, kv_mode="q8")
 QWEN3_4B = Qwen3Config(36, 2560, 32, 8, 128, 9728, 151936, max_positions=768, tie_word_embeddings=False)
 
 
@@ -131,6 +132,10 @@ class Decoder:
     @property
     def position(self):
         return _ffi.lib().llvq_hip_decoder_position(self.handle)
+
+    def seek(self, position: int):
+        """Measurement aid: jump to `position` without feeding the tokens before it."""
+        _ffi.check(_ffi.lib().llvq_hip_decoder_seek(self.handle, int(position)))
 
     def forward_token(self, token: int, want_logits: bool = True):
         """One position: (logits f32 [vocab] or None, argmax)."""
