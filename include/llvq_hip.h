@@ -37,6 +37,7 @@ typedef enum llvq_status {
   LLVQ_ERR_INCONSISTENT = 5,      /* Error::Inconsistent */
   LLVQ_ERR_INDEX_TOO_WIDE = 7,    /* Error::IndexTooWide */
   LLVQ_ERR_INDEX_OUT_OF_RANGE = 8,/* Error::IndexOutOfRange */
+  LLVQ_ERR_BAD_RAW_ENCODING = 9,  /* Error::BadRawEncoding { tag } */
   LLVQ_ERR_CODEBOOK_MISMATCH = 10,/* Error::CodebookMismatch */
   LLVQ_ERR_UNKNOWN_VERSION = 11,  /* Error::UnknownVersion */
   LLVQ_ERR_INVALID_ARGUMENT = 32, /* null pointer, wrong shape, unsupported dtype */
@@ -110,6 +111,28 @@ int llvq_hip_matrix_from_record(llvq_rt* rt, const uint8_t* buf, size_t len, siz
                                 llvq_mat** out);
 void llvq_hip_matrix_free(llvq_rt* rt, llvq_mat* m);
 
+/* read_raw (llvq-artifact/src/sealed.rs:277-326): one raw tensor record of the
+ * sealed sections that follow the matrices (embedding, norms), as byte ranges
+ * of buf; *pos is advanced past it.  version is the file's (records below v3
+ * carry no tag and are binary16).  Needs no GPU. */
+typedef struct llvq_raw_info {
+  char name[256];            /* truncated to 255 bytes, NUL-terminated */
+  uint32_t rank;
+  uint64_t dims[8];          /* the first 8 */
+  uint32_t tag;              /* 0: binary16; 1: int4 / int8 codes + binary16 scale and bias per group */
+  uint32_t bits, group;      /* quant only */
+  uint64_t count;            /* binary16: values; quant: groups */
+  size_t data_off, data_len; /* values, or packed codes */
+  size_t scales_off, biases_off;
+} llvq_raw_info;
+int llvq_hip_parse_raw_tensor(const uint8_t* buf, size_t len, size_t* pos, uint32_t version, llvq_raw_info* out);
+/* read_blob (sealed.rs:336-341): config.json, tokenizer.json, ... */
+typedef struct llvq_blob_info {
+  char name[256];
+  size_t data_off, data_len;
+} llvq_blob_info;
+int llvq_hip_parse_blob(const uint8_t* buf, size_t len, size_t* pos, llvq_blob_info* out);
+
 /* Shape and accounting of an uploaded matrix (FusedMatrix fields, fused.rs:566-588). */
 int llvq_hip_matrix_info(const llvq_mat* m, uint32_t* d_out, uint32_t* d_in, uint32_t* nblocks,
                          uint32_t* tail_w, uint64_t* device_bytes);
@@ -162,6 +185,15 @@ typedef struct llvq_decoder llvq_decoder;
  * 64 along head_dim with binary16 scale and bias (kvq.rs:110-165), chosen from
  * the token alone and rebuilt to the same binary16 value on every read. */
 typedef enum llvq_kv_mode { LLVQ_KV_F16 = 0, LLVQ_KV_Q8 = 1 } llvq_kv_mode;
+/* An int8 tensor of the sealed sections (QuantData, sealed.rs:64-78; the q8
+ * embedding of fused_cuda.rs:408-470): one code per weight, binary16 scale and
+ * bias per group along the row, weight = scale * code + bias.  Host pointers. */
+typedef struct llvq_quant_rows {
+  const uint8_t* codes;     /* [rows, row_len]; NULL = absent */
+  const uint16_t* scales;   /* [rows, ceil(row_len / group)] */
+  const uint16_t* biases;
+  uint32_t bits, group;     /* the kernels take 8 and 64 */
+} llvq_quant_rows;
 typedef struct llvq_decoder_desc {
   uint32_t n_layers, hidden, n_heads, n_kv_heads, head_dim, intermediate, vocab;
   uint32_t max_positions;               /* KV-cache length, <= 8192 */
@@ -172,9 +204,11 @@ typedef struct llvq_decoder_desc {
   const uint16_t* q_norm;               /* [n_layers, head_dim] */
   const uint16_t* k_norm;               /* [n_layers, head_dim] */
   const uint16_t* final_norm;           /* [hidden] */
-  const uint16_t* embed;                /* [vocab, hidden] */
+  const uint16_t* embed;                /* [vocab, hidden]; NULL when embed_q8 is given */
   const uint16_t* lm_head;              /* [vocab, hidden]; NULL = tied to embed */
   uint32_t kv_mode;                     /* llvq_kv_mode; q8 needs head_dim % 64 == 0 */
+  llvq_quant_rows embed_q8;             /* int8 embedding instead of `embed` (Embed::Q8, model.rs:546-551) */
+  llvq_quant_rows lm_head_q8;           /* int8 head (Head::Q8, model.rs:569-575); absent and lm_head NULL = tied */
 } llvq_decoder_desc;
 /* Qwen3::new_with (model.rs:869): checks every projection's shape against the architecture. */
 int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* desc, llvq_decoder** out);

@@ -9,7 +9,7 @@ _LIB = os.environ.get("LLVQ_HIP_LIB") or os.path.join(_HERE, "csrc", "libllvq_hi
 
 STATUS = {
     0: "Ok", 1: "NotAnArtifact", 2: "Truncated", 3: "BadName", 5: "Inconsistent", 7: "IndexTooWide",
-    8: "IndexOutOfRange", 10: "CodebookMismatch", 11: "UnknownVersion", 32: "InvalidArgument",
+    8: "IndexOutOfRange", 9: "BadRawEncoding", 10: "CodebookMismatch", 11: "UnknownVersion", 32: "InvalidArgument",
     33: "Unsupported", 34: "Device",
 }
 F32, F16 = 0, 1
@@ -43,6 +43,23 @@ class RecordInfo(C.Structure):
     ]
 
 
+class RawInfo(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 256), ("rank", C.c_uint32), ("dims", C.c_uint64 * 8), ("tag", C.c_uint32),
+        ("bits", C.c_uint32), ("group", C.c_uint32), ("count", C.c_uint64),
+        ("data_off", C.c_size_t), ("data_len", C.c_size_t), ("scales_off", C.c_size_t), ("biases_off", C.c_size_t),
+    ]
+
+
+class BlobInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 256), ("data_off", C.c_size_t), ("data_len", C.c_size_t)]
+
+
+class QuantRows(C.Structure):
+    _fields_ = [("codes", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p), ("bits", C.c_uint32),
+                ("group", C.c_uint32)]
+
+
 class DecoderDesc(C.Structure):
     _fields_ = [
         ("n_layers", C.c_uint32), ("hidden", C.c_uint32), ("n_heads", C.c_uint32), ("n_kv_heads", C.c_uint32),
@@ -51,7 +68,7 @@ class DecoderDesc(C.Structure):
         ("projections", C.POINTER(C.c_void_p)),
         ("input_norm", C.c_void_p), ("post_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
         ("final_norm", C.c_void_p), ("embed", C.c_void_p), ("lm_head", C.c_void_p),
-        ("kv_mode", C.c_uint32),
+        ("kv_mode", C.c_uint32), ("embed_q8", QuantRows), ("lm_head_q8", QuantRows),
     ]
 
 
@@ -87,6 +104,8 @@ def lib():
     L.llvq_hip_matrix_upload.argtypes = [vp, C.POINTER(MatrixDesc), C.POINTER(vp)]
     L.llvq_hip_read_header.argtypes = [C.c_char_p, sz, C.POINTER(sz), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
     L.llvq_hip_parse_matrix_record.argtypes = [C.c_char_p, sz, C.POINTER(sz), C.POINTER(RecordInfo)]
+    L.llvq_hip_parse_raw_tensor.argtypes = [C.c_char_p, sz, C.POINTER(sz), C.c_uint32, C.POINTER(RawInfo)]
+    L.llvq_hip_parse_blob.argtypes = [C.c_char_p, sz, C.POINTER(sz), C.POINTER(BlobInfo)]
     L.llvq_hip_matrix_from_record.argtypes = [vp, C.c_char_p, sz, C.POINTER(sz), C.POINTER(vp)]
     L.llvq_hip_matrix_free.argtypes = [vp, vp]
     L.llvq_hip_matrix_free.restype = None
@@ -124,7 +143,7 @@ def check(rc):
 EXPORTS = [
     "llvq_hip_runtime_create", "llvq_hip_runtime_destroy", "llvq_hip_codebook_fingerprint",
     "llvq_hip_host_decode", "llvq_hip_matrix_upload", "llvq_hip_read_header", "llvq_hip_parse_matrix_record",
-    "llvq_hip_matrix_from_record",
+    "llvq_hip_matrix_from_record", "llvq_hip_parse_raw_tensor", "llvq_hip_parse_blob",
     "llvq_hip_matrix_free", "llvq_hip_matrix_info", "llvq_hip_matrix_name", "llvq_hip_gemv",
     "llvq_hip_gemv_group", "llvq_hip_gemm", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
     "llvq_hip_last_error", "llvq_hip_version",

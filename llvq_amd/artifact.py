@@ -50,6 +50,14 @@ class CodebookMismatch(ArtifactError):
     pass
 
 
+class BadRawEncoding(ArtifactError):
+    """Error::BadRawEncoding { tag } (error.rs:34)"""
+
+    def __init__(self, tag):
+        self.tag = tag
+        super().__init__(f"raw tensor encoding tag {tag} is unknown — file written by a newer writer, or corrupted")
+
+
 class UnknownVersion(ArtifactError):
     pass
 
@@ -230,10 +238,143 @@ def read_matrix_raw(buf, pos=0):
                      seed if flag else None), pos
 
 
-def write_file(matrices, version=4):
-    """ArtifactWriter::finish (format.rs:540-545): header, records, empty raw and blob sections."""
+# ---- sealed sections: raw tensors and blobs (llvq-artifact/src/sealed.rs) ----------------
+TAG_F16, TAG_QUANT = 0, 1
+
+
+class RawTensor:
+    """sealed.rs:80-92.  `data` is a uint16 array of binary16 bit patterns (kind "f16"),
+    or for kind "quant": `packed` uint8, `scales` / `biases` uint16, `bits` in (4, 8), `group`."""
+
+    def __init__(self, name, dims, data=None, bits=None, group=None, packed=None, scales=None, biases=None):
+        self.name, self.dims = name, [int(d) for d in dims]
+        self.kind = "f16" if data is not None else "quant"
+        self.data = None if data is None else np.ascontiguousarray(data, dtype=np.uint16)
+        self.bits, self.group = bits, group
+        self.packed = None if packed is None else np.ascontiguousarray(packed, dtype=np.uint8)
+        self.scales = None if scales is None else np.ascontiguousarray(scales, dtype=np.uint16)
+        self.biases = None if biases is None else np.ascontiguousarray(biases, dtype=np.uint16)
+
+    def __len__(self):
+        return int(np.prod(self.dims, dtype=np.int64)) if self.dims else 1
+
+    def nbytes(self):
+        """RawTensor::bytes (sealed.rs:104-111)"""
+        if self.kind == "f16":
+            return self.data.size * 2
+        return self.packed.size + (self.scales.size + self.biases.size) * 2
+
+
+class Blob:
+    def __init__(self, name, data):
+        self.name, self.data = name, bytes(data)
+
+
+def _put_str(s):
+    b = s.encode()
+    return struct.pack("<I", len(b)) + b
+
+
+def write_raw(t: RawTensor) -> bytes:
+    """sealed.rs:214-275"""
+    out = [struct.pack("<I", TAG_F16 if t.kind == "f16" else TAG_QUANT), _put_str(t.name),
+           struct.pack("<I", len(t.dims))] + [struct.pack("<Q", d) for d in t.dims]
+    n = len(t)
+    if t.kind == "f16":
+        if t.data.size != n:
+            raise Inconsistent(f"{t.name}: {t.data.size} values for dims {t.dims}")
+        out += [struct.pack("<Q", t.data.size), t.data.astype("<u2").tobytes()]
+    else:
+        row_len = max(t.dims[-1] if t.dims else 1, 1)
+        groups = (n // row_len) * ((row_len + t.group - 1) // t.group)
+        if t.bits not in (4, 8):
+            raise Inconsistent(f"{t.name}: unsupported quant width {t.bits}")
+        need = n if t.bits == 8 else (n + 1) // 2
+        if t.packed.size != need or t.scales.size != groups or t.biases.size != groups:
+            raise Inconsistent(f"{t.name}: {t.packed.size} packed bytes / {t.scales.size} scales / {t.biases.size} biases "
+                               f"for {n} values in groups of {t.group} (want {need} / {groups} / {groups})")
+        out += [struct.pack("<IIQ", t.bits, t.group, t.packed.size), t.packed.tobytes(), struct.pack("<Q", groups),
+                t.scales.astype("<u2").tobytes(), t.biases.astype("<u2").tobytes()]
+    return b"".join(out)
+
+
+def read_raw(buf, pos=0, version=4):
+    """sealed.rs:277-326 → (RawTensor, new_pos)"""
+    mv = memoryview(buf)
+    n = len(mv)
+
+    def take(k, what):
+        nonlocal pos
+        if k > n - pos:
+            raise Truncated(what)
+        at = pos
+        pos += k
+        return at
+
+    tag = TAG_F16
+    if version >= 3:
+        (tag,) = struct.unpack_from("<I", mv, take(4, "raw tensor tag"))
+    if tag not in (TAG_F16, TAG_QUANT):
+        raise BadRawEncoding(tag)
+    (nl,) = struct.unpack_from("<I", mv, take(4, "raw tensor name"))
+    at = take(nl, "raw tensor name")
+    try:
+        name = bytes(mv[at:at + nl]).decode("utf-8")
+    except UnicodeDecodeError:
+        raise BadName("raw tensor name is not valid UTF-8")
+    (rank,) = struct.unpack_from("<I", mv, take(4, "raw tensor rank"))
+    dims = [struct.unpack_from("<Q", mv, take(8, "raw tensor dims"))[0] for _ in range(rank)]
+    if tag == TAG_F16:
+        (cnt,) = struct.unpack_from("<Q", mv, take(8, "raw tensor length"))
+        if cnt > (1 << 62):
+            raise Truncated("raw tensor data")
+        at = take(2 * cnt, "raw tensor data")
+        return RawTensor(name, dims, data=np.frombuffer(mv, dtype="<u2", count=cnt, offset=at)), pos
+    bits, group = struct.unpack_from("<II", mv, take(8, "quant width"))
+    (nbytes,) = struct.unpack_from("<Q", mv, take(8, "quant packed length"))
+    at = take(nbytes, "quant packed data")
+    packed = np.frombuffer(mv, dtype=np.uint8, count=nbytes, offset=at)
+    (groups,) = struct.unpack_from("<Q", mv, take(8, "quant group count"))
+    if groups > (1 << 62):
+        raise Truncated("quant scales")
+    scales = np.frombuffer(mv, dtype="<u2", count=groups, offset=take(2 * groups, "quant scales"))
+    biases = np.frombuffer(mv, dtype="<u2", count=groups, offset=take(2 * groups, "quant biases"))
+    return RawTensor(name, dims, bits=bits & 0xFF, group=group, packed=packed, scales=scales, biases=biases), pos
+
+
+def write_blob(b: Blob) -> bytes:
+    return _put_str(b.name) + struct.pack("<Q", len(b.data)) + b.data
+
+
+def read_blob(buf, pos=0):
+    """sealed.rs:336-341 → (Blob, new_pos)"""
+    mv = memoryview(buf)
+    n = len(mv)
+    if n - pos < 4:
+        raise Truncated("blob name")
+    (nl,) = struct.unpack_from("<I", mv, pos)
+    pos += 4
+    if nl > n - pos:
+        raise Truncated("blob name")
+    try:
+        name = bytes(mv[pos:pos + nl]).decode("utf-8")
+    except UnicodeDecodeError:
+        raise BadName("blob name is not valid UTF-8")
+    pos += nl
+    if n - pos < 8:
+        raise Truncated("blob length")
+    (k,) = struct.unpack_from("<Q", mv, pos)
+    pos += 8
+    if k > n - pos:
+        raise Truncated("blob")
+    return Blob(name, mv[pos:pos + k]), pos + k
+
+
+def write_file(matrices, version=4, raws=(), blobs=()):
+    """ArtifactWriter::seal / finish (format.rs:501-545): header, matrix records, raw tensors, blobs."""
     return b"".join([write_header(version, len(matrices))] + [write_matrix_raw(m) for m in matrices]
-                    + [struct.pack("<II", 0, 0)])
+                    + [struct.pack("<I", len(raws))] + [write_raw(t) for t in raws]
+                    + [struct.pack("<I", len(blobs))] + [write_blob(b) for b in blobs])
 
 
 def read_file(buf):
@@ -243,6 +384,32 @@ def read_file(buf):
         m, pos = read_matrix_raw(buf, pos)
         out.append(m)
     return version, out
+
+
+def read_sealed(buf):
+    """The whole file: (version, matrices, raw tensors, blobs).  Files of version 1 end after the matrices."""
+    version, n, pos = read_header(buf)
+    mats = []
+    for _ in range(n):
+        m, pos = read_matrix_raw(buf, pos)
+        mats.append(m)
+    raws, blobs = [], []
+    if version >= 2:
+        if len(buf) - pos < 4:
+            raise Truncated("raw tensor count")
+        (nr,) = struct.unpack_from("<I", buf, pos)
+        pos += 4
+        for _ in range(nr):
+            t, pos = read_raw(buf, pos, version)
+            raws.append(t)
+        if len(buf) - pos < 4:
+            raise Truncated("blob count")
+        (nbl,) = struct.unpack_from("<I", buf, pos)
+        pos += 4
+        for _ in range(nbl):
+            b, pos = read_blob(buf, pos)
+            blobs.append(b)
+    return version, mats, raws, blobs
 
 
 def split_name(name):

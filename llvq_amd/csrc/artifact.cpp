@@ -161,4 +161,84 @@ int parse_matrix_record(const uint8_t* buf, size_t len, size_t* pos, RecordView*
   return LLVQ_OK;
 }
 
+namespace {
+
+int read_name(Cursor& c, const char* what, std::string* name, std::string* err) {
+  uint32_t n = 0;
+  if (!c.u32(&n)) return truncated(err, what);
+  if (c.left() < n) return truncated(err, what);
+  if (!valid_utf8(c.buf + c.pos, n)) {
+    if (err) *err = "a name is not valid UTF-8";
+    return LLVQ_ERR_BAD_NAME;
+  }
+  name->assign(reinterpret_cast<const char*>(c.buf + c.pos), n);
+  c.pos += n;
+  return LLVQ_OK;
+}
+
+}  // namespace
+
+int parse_raw_tensor(const uint8_t* buf, size_t len, size_t* pos, uint32_t version, RawTensorView* out,
+                     std::string* err) {
+  Cursor c{buf, len, *pos};
+  RawTensorView t;
+  if (version >= 3 && !c.u32(&t.tag)) return truncated(err, "raw tensor tag");
+  // refused before anything else is parsed: past an unknown tag every byte would be read against the wrong layout
+  if (t.tag != 0 && t.tag != 1) {
+    if (err) *err = "raw tensor encoding tag " + std::to_string(t.tag) + " is unknown — file written by a newer writer, or corrupted";
+    return LLVQ_ERR_BAD_RAW_ENCODING;
+  }
+  int rc = read_name(c, "raw tensor name", &t.name, err);
+  if (rc) return rc;
+  uint32_t rank = 0;
+  if (!c.u32(&rank)) return truncated(err, "raw tensor rank");
+  if ((uint64_t)rank * 8 > c.left()) return truncated(err, "raw tensor dims");
+  t.dims.resize(rank);
+  for (uint32_t i = 0; i < rank; ++i)
+    if (!c.u64(&t.dims[i])) return truncated(err, "raw tensor dims");
+  if (t.tag == 0) {
+    if (!c.u64(&t.count)) return truncated(err, "raw tensor length");
+    if (t.count > c.left() / 2) return truncated(err, "raw tensor data");  // also a count whose byte size overflows
+    t.data_off = c.pos;
+    t.data_len = (size_t)t.count * 2;
+    c.pos += t.data_len;
+  } else {
+    uint64_t nbytes = 0;
+    if (!c.u32(&t.bits)) return truncated(err, "quant width");
+    t.bits &= 0xFFu;
+    if (!c.u32(&t.group)) return truncated(err, "quant group");
+    if (!c.u64(&nbytes)) return truncated(err, "quant packed length");
+    if (nbytes > c.left()) return truncated(err, "quant packed data");
+    t.data_off = c.pos;
+    t.data_len = (size_t)nbytes;
+    c.pos += t.data_len;
+    if (!c.u64(&t.count)) return truncated(err, "quant group count");
+    if (t.count > c.left() / 2) return truncated(err, "quant scales");
+    t.scales_off = c.pos;
+    c.pos += (size_t)t.count * 2;
+    if (t.count > c.left() / 2) return truncated(err, "quant biases");
+    t.biases_off = c.pos;
+    c.pos += (size_t)t.count * 2;
+  }
+  *out = std::move(t);
+  *pos = c.pos;
+  return LLVQ_OK;
+}
+
+int parse_blob(const uint8_t* buf, size_t len, size_t* pos, BlobView* out, std::string* err) {
+  Cursor c{buf, len, *pos};
+  BlobView b;
+  int rc = read_name(c, "blob name", &b.name, err);
+  if (rc) return rc;
+  uint64_t n = 0;
+  if (!c.u64(&n)) return truncated(err, "blob length");
+  if (n > c.left()) return truncated(err, "blob");
+  b.data_off = c.pos;
+  b.data_len = (size_t)n;
+  c.pos += b.data_len;
+  *out = std::move(b);
+  *pos = c.pos;
+  return LLVQ_OK;
+}
+
 }  // namespace llvq

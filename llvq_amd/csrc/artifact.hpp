@@ -28,4 +28,24 @@ int parse_header(const uint8_t* buf, size_t len, size_t* pos, uint32_t* version,
 int parse_matrix_record(const uint8_t* buf, size_t len, size_t* pos, RecordView* out,
                         std::string* err);
 
+// A raw tensor record (llvq-artifact/src/sealed.rs:80-92, :277-326) as byte
+// ranges of the caller's buffer; nothing is copied.
+struct RawTensorView {
+  std::string name;
+  std::vector<uint64_t> dims;
+  uint32_t tag = 0;        // 0: binary16 values; 1: int4 / int8 codes with binary16 scale and bias per group
+  uint32_t bits = 0, group = 0;
+  size_t data_off = 0, data_len = 0;      // f16: values (2 bytes each); quant: packed codes
+  size_t scales_off = 0, biases_off = 0;  // quant only
+  uint64_t count = 0;                     // f16: values; quant: groups
+};
+struct BlobView {
+  std::string name;
+  size_t data_off = 0, data_len = 0;
+};
+// version < 3 records carry no tag and are binary16 (sealed.rs:278-282).
+int parse_raw_tensor(const uint8_t* buf, size_t len, size_t* pos, uint32_t version, RawTensorView* out,
+                     std::string* err);
+int parse_blob(const uint8_t* buf, size_t len, size_t* pos, BlobView* out, std::string* err);
+
 }  // namespace llvq

@@ -542,6 +542,70 @@ __global__ __launch_bounds__(kHeadThreads) void lm_head_kernel(const __half* __r
   }
 }
 
+// ---- int8 embedding / head (llvq-llm/kernels/emb_q8.cu) --------------------------------
+// One byte per weight, binary16 scale and bias per group of 64 along the row
+// (llvq-artifact/src/sealed.rs:64-78): weight = f32(s * q) + b.
+constexpr uint32_t kEmbedGroup = 64;
+struct QuantRows {
+  const uint8_t* q;      // [rows, d]
+  const __half* scales;  // [rows, ceil(d / 64)]
+  const __half* biases;
+};
+
+__device__ __forceinline__ float q8_weight(uint32_t q, float s, float b) {
+  return __fadd_rn(__fmul_rn(s, (float)q), b);
+}
+
+// h = f16(embedding row of *token)   (emb_q8_gather)
+__global__ __launch_bounds__(256) void embed_q8_kernel(QuantRows e, const uint32_t* __restrict__ token, uint32_t vocab,
+                                                       uint32_t hidden, __half* __restrict__ h) {
+  const uint32_t t = min(*token, vocab - 1u);
+  const uint32_t gpr = (hidden + kEmbedGroup - 1) / kEmbedGroup;
+  for (uint32_t c = blockIdx.x * blockDim.x + threadIdx.x; c < hidden; c += gridDim.x * blockDim.x) {
+    const size_t g = (size_t)t * gpr + c / kEmbedGroup;
+    h[c] = __float2half_rn(q8_weight(e.q[(size_t)t * hidden + c], __half2float(e.scales[g]), __half2float(e.biases[g])));
+  }
+}
+
+// logits = f16(E h) for the int8 head (tv_q8_h): one wavefront per row at a time,
+// 16 codes per lane and load (a 16-byte run never straddles a group of 64).
+__global__ __launch_bounds__(kHeadThreads) void lm_head_q8_kernel(QuantRows e, const __half* __restrict__ h, uint32_t vocab,
+                                                                  uint32_t hidden, float* __restrict__ logits,
+                                                                  float* __restrict__ best_val, uint32_t* __restrict__ best_idx) {
+  extern __shared__ __align__(16) float hs[];  // [hidden]
+  for (uint32_t i = threadIdx.x; i < hidden; i += kHeadThreads) hs[i] = __half2float(h[i]);
+  __syncthreads();
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t gw = blockIdx.x * (kHeadThreads / 64) + (threadIdx.x >> 6), nw = gridDim.x * (kHeadThreads / 64);
+  const uint32_t chunks = hidden >> 4, gpr = (hidden + kEmbedGroup - 1) / kEmbedGroup;
+  float bv = -INFINITY;
+  uint32_t bi = 0xFFFFFFFFu;
+  for (uint32_t r = gw; r < vocab; r += nw) {
+    const uint4* row = reinterpret_cast<const uint4*>(e.q + (size_t)r * hidden);
+    float a = 0.f;
+    for (uint32_t c = lane; c < chunks; c += 64) {
+      const uint4 u = row[c];
+      const float s = __half2float(e.scales[(size_t)r * gpr + (c >> 2)]), b = __half2float(e.biases[(size_t)r * gpr + (c >> 2)]);
+      const uint32_t wv[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) a = fmaf(q8_weight((wv[j] >> (8 * t)) & 0xFFu, s, b), hs[16 * c + 4 * j + t], a);
+    }
+    a = wave_sum(a);
+    const float l = __half2float(__float2half_rn(a));
+    if (lane == 0) logits[r] = l;
+    if (l > bv) {
+      bv = l;
+      bi = r;
+    }
+  }
+  if (lane == 0) {
+    best_val[gw] = bv;
+    best_idx[gw] = bi;
+  }
+}
+
 // token = argmax over the wavefront winners; lowest row on ties
 __global__ __launch_bounds__(1024) void argmax_final_kernel(const float* __restrict__ best_val, const uint32_t* __restrict__ best_idx,
                                                             uint32_t n, uint32_t* __restrict__ token_out,

@@ -977,6 +977,44 @@ int llvq_hip_parse_matrix_record(const uint8_t* buf, size_t len, size_t* pos, ll
   return LLVQ_OK;
 }
 
+int llvq_hip_parse_raw_tensor(const uint8_t* buf, size_t len, size_t* pos, uint32_t version, llvq_raw_info* out) {
+  if (!buf || !pos || !out || *pos > len) return fail(LLVQ_ERR_INVALID_ARGUMENT, "parse_raw_tensor: bad argument");
+  RawTensorView t;
+  std::string err;
+  size_t p = *pos;
+  const int rc = parse_raw_tensor(buf, len, &p, version, &t, &err);
+  if (rc) return fail(rc, err);
+  std::memset(out, 0, sizeof *out);
+  std::strncpy(out->name, t.name.c_str(), sizeof out->name - 1);
+  out->rank = (uint32_t)t.dims.size();
+  for (size_t i = 0; i < t.dims.size() && i < 8; ++i) out->dims[i] = t.dims[i];
+  out->tag = t.tag;
+  out->bits = t.bits;
+  out->group = t.group;
+  out->count = t.count;
+  out->data_off = t.data_off;
+  out->data_len = t.data_len;
+  out->scales_off = t.scales_off;
+  out->biases_off = t.biases_off;
+  *pos = p;
+  return LLVQ_OK;
+}
+
+int llvq_hip_parse_blob(const uint8_t* buf, size_t len, size_t* pos, llvq_blob_info* out) {
+  if (!buf || !pos || !out || *pos > len) return fail(LLVQ_ERR_INVALID_ARGUMENT, "parse_blob: bad argument");
+  BlobView b;
+  std::string err;
+  size_t p = *pos;
+  const int rc = parse_blob(buf, len, &p, &b, &err);
+  if (rc) return fail(rc, err);
+  std::memset(out, 0, sizeof *out);
+  std::strncpy(out->name, b.name.c_str(), sizeof out->name - 1);
+  out->data_off = b.data_off;
+  out->data_len = b.data_len;
+  *pos = p;
+  return LLVQ_OK;
+}
+
 int llvq_hip_matrix_from_record(llvq_rt* rt, const uint8_t* buf, size_t len, size_t* pos,
                                 llvq_mat** out) {
   if (!rt || !buf || !pos || !out || *pos > len)
@@ -1350,6 +1388,8 @@ struct llvq_decoder {
   uint8_t* blob = nullptr;            // every dense tensor and buffer below, one allocation
   __half *ln1 = nullptr, *ln2 = nullptr, *qn = nullptr, *kn = nullptr, *fnorm = nullptr;
   __half *embed = nullptr, *head = nullptr, *cos_t = nullptr, *sin_t = nullptr;
+  bool embed_q8 = false, head_q8 = false;  // int8 rows instead of binary16
+  QuantRows embed_q{}, head_q{};
   __half *kcache = nullptr, *vcache = nullptr;  // [n_layers][n_kv][max_pos][head_dim]
   __half *h = nullptr, *h_alt = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *ctx = nullptr, *o = nullptr;
   __half *gate = nullptr, *up = nullptr, *act = nullptr, *down = nullptr;
@@ -1374,7 +1414,10 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   llvq_rt* rt = d->rt;
   hipStream_t st = rt->stream;
   if (d->pos >= d->max_pos) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder: position " + std::to_string(d->pos) + " is past max_positions");
-  hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, d->h);
+  if (d->embed_q8)
+    hipLaunchKernelGGL(embed_q8_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed_q, d->token, d->vocab, d->hidden, d->h);
+  else
+    hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, d->h);
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
   const uint32_t T = d->pos + 1;
   uint32_t n_splits = (T + 31) / 32;  // about 32 cached positions per workgroup, at most kAttnMaxSplits ranges
@@ -1462,8 +1505,12 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   }
   if (want_logits) {
     hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->down, d->fnorm, d->h, d->normed, d->hidden, d->eps);
-    hipLaunchKernelGGL(lm_head_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head, d->normed,
-                       d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
+    if (d->head_q8)
+      hipLaunchKernelGGL(lm_head_q8_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head_q, d->normed,
+                         d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
+    else
+      hipLaunchKernelGGL(lm_head_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head, d->normed,
+                         d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
     hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(1024), 0, st, d->best_val, d->best_idx,
                        d->head_grid * (kHeadThreads / 64), d->token, record ? d->history : (uint32_t*)nullptr, history_slot);
   }
@@ -1479,8 +1526,17 @@ extern "C" {
 int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decoder** out) {
   if (!rt || !c || !out) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: null argument");
   *out = nullptr;
-  if (!c->projections || !c->input_norm || !c->post_norm || !c->q_norm || !c->k_norm || !c->final_norm || !c->embed)
+  if (!c->projections || !c->input_norm || !c->post_norm || !c->q_norm || !c->k_norm || !c->final_norm ||
+      (!c->embed && !c->embed_q8.codes))
     return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: a required tensor is null");
+  for (const llvq_quant_rows* qr : {&c->embed_q8, &c->lm_head_q8})
+    if (qr->codes) {
+      if (!qr->scales || !qr->biases) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: an int8 tensor without scales or biases");
+      // what the kernels compile in (fused_cuda.rs:418-447): 8 bits, groups of 64, whole 16-byte runs per row
+      if (qr->bits != 8 || qr->group != kEmbedGroup || c->hidden % 16)
+        return fail(LLVQ_ERR_UNSUPPORTED, "decoder_create: int" + std::to_string(qr->bits) + " g" + std::to_string(qr->group) +
+                                              " — the kernels hard-code int8 g64 and hidden % 16 = 0");
+    }
   if (c->n_layers == 0 || c->hidden == 0 || c->hidden % 8 || c->hidden > 8192 || c->n_heads == 0 || c->n_kv_heads == 0 ||
       c->n_heads % c->n_kv_heads || c->n_heads / c->n_kv_heads > (uint32_t)kAttnMaxGroup || c->head_dim == 0 || c->head_dim % 8 || c->head_dim > 256 || c->intermediate == 0 ||
       c->vocab == 0 || c->max_positions == 0 || c->max_positions > 8192 ||
@@ -1532,8 +1588,14 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   const size_t o_ln1 = take((size_t)c->n_layers * c->hidden * hb), o_ln2 = take((size_t)c->n_layers * c->hidden * hb);
   const size_t o_qn = take((size_t)c->n_layers * c->head_dim * hb), o_kn = take((size_t)c->n_layers * c->head_dim * hb);
   const size_t o_fn = take((size_t)c->hidden * hb);
-  const size_t o_emb = take((size_t)c->vocab * c->hidden * hb);
-  const size_t o_head = c->lm_head ? take((size_t)c->vocab * c->hidden * hb) : o_emb;
+  const size_t vh = (size_t)c->vocab * c->hidden, vg = (size_t)c->vocab * ((c->hidden + kEmbedGroup - 1) / kEmbedGroup);
+  const bool eq8 = c->embed_q8.codes != nullptr;
+  // the head: its own int8 or binary16 tensor, else tied to the embedding in whichever encoding that is
+  const bool hq8 = c->lm_head_q8.codes != nullptr || (!c->lm_head && eq8);
+  const bool head_own = c->lm_head_q8.codes != nullptr || c->lm_head != nullptr;
+  const size_t o_emb = take(eq8 ? vh : vh * hb), o_emb_s = take(eq8 ? vg * hb : 0), o_emb_b = take(eq8 ? vg * hb : 0);
+  const size_t o_head = head_own ? take(hq8 ? vh : vh * hb) : o_emb;
+  const size_t o_head_s = head_own ? take(hq8 ? vg * hb : 0) : o_emb_s, o_head_b = head_own ? take(hq8 ? vg * hb : 0) : o_emb_b;
   const size_t o_cos = take(cos_h.size() * hb), o_sin = take(sin_h.size() * hb);
   const size_t cache_vals = (size_t)c->n_layers * c->n_kv_heads * c->max_positions * c->head_dim;
   const bool q8 = c->kv_mode == LLVQ_KV_Q8;
@@ -1557,14 +1619,24 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   if (e == hipSuccess) e = put(o_qn, c->q_norm, (size_t)c->n_layers * c->head_dim * hb);
   if (e == hipSuccess) e = put(o_kn, c->k_norm, (size_t)c->n_layers * c->head_dim * hb);
   if (e == hipSuccess) e = put(o_fn, c->final_norm, (size_t)c->hidden * hb);
-  if (e == hipSuccess) e = put(o_emb, c->embed, (size_t)c->vocab * c->hidden * hb);
-  if (e == hipSuccess && c->lm_head) e = put(o_head, c->lm_head, (size_t)c->vocab * c->hidden * hb);
+  if (e == hipSuccess && !eq8) e = put(o_emb, c->embed, vh * hb);
+  if (e == hipSuccess && eq8) e = put(o_emb, c->embed_q8.codes, vh);
+  if (e == hipSuccess && eq8) e = put(o_emb_s, c->embed_q8.scales, vg * hb);
+  if (e == hipSuccess && eq8) e = put(o_emb_b, c->embed_q8.biases, vg * hb);
+  if (e == hipSuccess && head_own && !hq8) e = put(o_head, c->lm_head, vh * hb);
+  if (e == hipSuccess && head_own && hq8) e = put(o_head, c->lm_head_q8.codes, vh);
+  if (e == hipSuccess && head_own && hq8) e = put(o_head_s, c->lm_head_q8.scales, vg * hb);
+  if (e == hipSuccess && head_own && hq8) e = put(o_head_b, c->lm_head_q8.biases, vg * hb);
   if (e == hipSuccess) e = put(o_cos, cos_h.data(), cos_h.size() * hb);
   if (e == hipSuccess) e = put(o_sin, sin_h.data(), sin_h.size() * hb);
   if (e != hipSuccess) { (void)hipFree(d->blob); delete d; return hip_fail(e, "decoder upload"); }
   auto H = [&](size_t at) { return reinterpret_cast<__half*>(d->blob + at); };
   d->ln1 = H(o_ln1); d->ln2 = H(o_ln2); d->qn = H(o_qn); d->kn = H(o_kn); d->fnorm = H(o_fn);
   d->embed = H(o_emb); d->head = H(o_head); d->cos_t = H(o_cos); d->sin_t = H(o_sin);
+  d->embed_q8 = eq8;
+  d->head_q8 = hq8;
+  d->embed_q = QuantRows{d->blob + o_emb, H(o_emb_s), H(o_emb_b)};
+  d->head_q = QuantRows{d->blob + o_head, H(o_head_s), H(o_head_b)};
   d->kcache = H(o_kc); d->vcache = H(o_vc);
   if (q8) {
     d->q8.kq = d->blob + o_kc; d->q8.vq = d->blob + o_vc;

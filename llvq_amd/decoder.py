@@ -3,11 +3,12 @@
 over the HIP library's decode loop.  No computation happens here: the class
 assembles the descriptor and calls the C ABI."""
 import ctypes as C
+import json
 from dataclasses import dataclass
 
 import numpy as np
 
-from . import _ffi, synth
+from . import _ffi, artifact, synth
 from .fused import FusedRuntime
 
 SITES = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
@@ -50,8 +51,8 @@ class DecoderWeights:
     q_norm: np.ndarray       # [n_layers, head_dim]
     k_norm: np.ndarray       # [n_layers, head_dim]
     final_norm: np.ndarray   # [hidden]
-    embed: np.ndarray        # [vocab, hidden]
-    lm_head: np.ndarray = None  # [vocab, hidden] or None (tied)
+    embed: object            # [vocab, hidden] binary16 array, or an int8 g64 artifact.RawTensor
+    lm_head: object = None   # the same, or None (tied to the embedding)
 
 
 def synthetic_weights(cfg: Qwen3Config, seed: int = 0) -> DecoderWeights:
@@ -105,17 +106,79 @@ class Decoder:
 
         L, h, d = cfg.num_hidden_layers, cfg.hidden_size, cfg.head_dim
         keep = [f16(weights.input_norm, (L, h)), f16(weights.post_norm, (L, h)), f16(weights.q_norm, (L, d)),
-                f16(weights.k_norm, (L, d)), f16(weights.final_norm, (h,)), f16(weights.embed, (cfg.vocab_size, h))]
-        head = f16(weights.lm_head, (cfg.vocab_size, h)) if weights.lm_head is not None else None
+                f16(weights.k_norm, (L, d)), f16(weights.final_norm, (h,))]
+
+        def table(t, what):
+            """A [vocab, hidden] table: (binary16 pointer or None, QuantRows, arrays to keep alive)."""
+            if t is None:
+                return None, _ffi.QuantRows(), ()
+            if isinstance(t, artifact.RawTensor) and t.kind == "quant":
+                if t.dims != [cfg.vocab_size, h]:
+                    raise ValueError(f"{what}: dims {t.dims}, expected [{cfg.vocab_size}, {h}]")
+                alive = (np.ascontiguousarray(t.packed), np.ascontiguousarray(t.scales), np.ascontiguousarray(t.biases))
+                return None, _ffi.QuantRows(alive[0].ctypes.data, alive[1].ctypes.data, alive[2].ctypes.data,
+                                            int(t.bits), int(t.group)), alive
+            if isinstance(t, artifact.RawTensor):
+                t = t.data.view(np.float16).reshape(t.dims)
+            a = f16(t, (cfg.vocab_size, h))
+            return a.ctypes.data, _ffi.QuantRows(), (a,)
+
+        e_ptr, e_q, e_alive = table(weights.embed, "embedding")
+        h_ptr, h_q, h_alive = table(weights.lm_head, "lm_head")
         desc = _ffi.DecoderDesc(
             L, h, cfg.num_attention_heads, cfg.num_key_value_heads, d, cfg.intermediate_size, cfg.vocab_size,
             cfg.max_positions, float(cfg.rope_theta), float(cfg.rms_norm_eps),
             C.cast(arr, C.POINTER(C.c_void_p)),
             keep[0].ctypes.data, keep[1].ctypes.data, keep[2].ctypes.data, keep[3].ctypes.data, keep[4].ctypes.data,
-            keep[5].ctypes.data, head.ctypes.data if head is not None else None, self._kv_mode(cfg.kv_mode))
+            e_ptr, h_ptr, self._kv_mode(cfg.kv_mode), e_q, h_q)
+        self._alive = (keep, e_alive, h_alive)
         out = C.c_void_p()
         _ffi.check(_ffi.lib().llvq_hip_decoder_create(rt.handle, C.byref(desc), C.byref(out)))
         self.handle = out
+
+    @classmethod
+    def from_model(cls, rt: FusedRuntime, model, max_positions=None, kv_mode="f16"):
+        """Qwen3::new_with over a loaded sealed artifact (fused_cuda.rs:1226-1300 + model.rs:869):
+        the architecture comes from the file's config.json, the projections from its matrix
+        records (by `model.layers.{i}.{site}.weight`), norms and embedding from its raw tensors."""
+        c = json.loads(model.config_json.decode("utf-8"))
+        heads = c["num_attention_heads"]
+        cfg = Qwen3Config(
+            num_hidden_layers=c["num_hidden_layers"], hidden_size=c["hidden_size"], num_attention_heads=heads,
+            num_key_value_heads=c.get("num_key_value_heads", heads), head_dim=c.get("head_dim", c["hidden_size"] // heads),
+            intermediate_size=c["intermediate_size"], vocab_size=c["vocab_size"], rope_theta=c.get("rope_theta", 1e6),
+            rms_norm_eps=c.get("rms_norm_eps", 1e-6),
+            max_positions=int(max_positions or min(c.get("max_position_embeddings", 8192), 8192)),
+            tie_word_embeddings=bool(c.get("tie_word_embeddings", False)), kv_mode=kv_mode)
+        sites = {}
+        for fm in model.matrices:
+            layer, site = artifact.split_name(fm.name)
+            sites[(layer, site)] = fm
+        projections = []
+        for layer in range(cfg.num_hidden_layers):
+            row = []
+            for site in SITES:
+                if (layer, site) not in sites:
+                    raise ValueError(f"the file carries no model.layers.{layer}.{site}.weight")
+                row.append(sites[(layer, site)].raw)
+            projections.append(row)
+
+        def halves(name, shape):
+            t = model.tensor(name)
+            if t.kind != "f16":
+                raise ValueError(f"{name}: stored quantized, a norm is carried as binary16")
+            return t.data.view(np.float16).reshape(shape)
+
+        L, h, d = cfg.num_hidden_layers, cfg.hidden_size, cfg.head_dim
+        stack = lambda fmt, n: np.stack([halves(fmt.format(i), (n,)) for i in range(L)])
+        head = None
+        if not cfg.tie_word_embeddings:  # fused.rs:252-285: an untied model must carry its own head
+            head = model.tensor("lm_head.weight")
+        weights = DecoderWeights(
+            stack("model.layers.{}.input_layernorm.weight", h), stack("model.layers.{}.post_attention_layernorm.weight", h),
+            stack("model.layers.{}.self_attn.q_norm.weight", d), stack("model.layers.{}.self_attn.k_norm.weight", d),
+            halves("model.norm.weight", (h,)), model.tensor("model.embed_tokens.weight"), head)
+        return cls(rt, cfg, projections, weights)
 
     @staticmethod
     def _kv_mode(v):

@@ -11,7 +11,7 @@ import ctypes as C
 import numpy as np
 
 from . import _ffi
-from .artifact import RawMatrix, read_header, read_matrix_raw
+from .artifact import RawMatrix, read_header, read_matrix_raw, read_sealed
 
 
 class FusedMatrix:
@@ -33,26 +33,55 @@ class FusedMatrix:
         self.bytes = raw.codes.size + 4 * raw.tail.size + 4 * raw.d_out + 8
 
 
+EMBED_NAME = "model.embed_tokens.weight"  # fused.rs:204
+HEAD_NAME = "lm_head.weight"              # fused.rs:209
+
+
 class FusedModel:
-    def __init__(self, matrices):
+    """Everything a runtime needs, still on the host (fused.rs:723-752): the
+    projections, the carried raw tensors in the file's own encoding (f16 bits, or
+    int8 g64 for an embedding), config.json and tokenizer.json."""
+
+    def __init__(self, matrices, raw=(), config_json=b"", tokenizer_json=b""):
         self.matrices = list(matrices)
+        self.raw = list(raw)
+        self.config_json, self.tokenizer_json = bytes(config_json), bytes(tokenizer_json)
         self.runtime_bytes = sum(m.bytes for m in self.matrices)
+        self.quantized_weights = sum(m.d_out * m.d_in for m in self.matrices)
+        self.carried_weights = sum(len(t) for t in self.raw)
+
+    def tensor(self, name):
+        for t in self.raw:
+            if t.name == name:
+                return t
+        raise KeyError(f"the file carries no {name}")
 
 
 def load(path: str) -> FusedModel:
-    """fused::load (fused.rs:1147): header, then every matrix record, host only."""
+    """fused::load (fused.rs:1147): header, every matrix record, the raw tensors and
+    the blobs; host only.  A projections-only file (format v1) is refused, as is a
+    file without config.json or tokenizer.json (fused.rs:1151-1158, :1249-1254)."""
     with open(path, "rb") as f:
         buf = f.read()
-    return load_bytes(buf)
+    return load_bytes(buf, path)
 
 
-def load_bytes(buf) -> FusedModel:
-    _version, n, pos = read_header(buf)
-    mats = []
-    for _ in range(n):
-        raw, pos = read_matrix_raw(buf, pos)
-        mats.append(FusedMatrix(raw))
-    return FusedModel(mats)
+def load_bytes(buf, path="<bytes>", projections_only=False) -> FusedModel:
+    if projections_only:
+        _version, n, pos = read_header(buf)
+        mats = []
+        for _ in range(n):
+            raw, pos = read_matrix_raw(buf, pos)
+            mats.append(FusedMatrix(raw))
+        return FusedModel(mats)
+    version, mats, raws, blobs = read_sealed(buf)
+    if version < 2:
+        raise ValueError(f"{path} is a projections-only artifact (format v{version}); it cannot run on its own")
+    by_name = {b.name: b.data for b in blobs}
+    for need in ("config.json", "tokenizer.json"):
+        if need not in by_name:
+            raise ValueError(f"{path} carries no {need}")
+    return FusedModel([FusedMatrix(m) for m in mats], raws, by_name["config.json"], by_name["tokenizer.json"])
 
 
 class FusedProj:

@@ -98,8 +98,20 @@ class Qwen3Oracle:
         f = lambda a: np.asarray(a, np.float16).astype(np.float64)
         self.ln1, self.ln2 = f(weights.input_norm), f(weights.post_norm)
         self.qn, self.kn, self.fn = f(weights.q_norm), f(weights.k_norm), f(weights.final_norm)
-        self.embed = np.asarray(weights.embed, np.float16)
-        self.head = self.embed if weights.lm_head is None else np.asarray(weights.lm_head, np.float16)
+        # A table is a binary16 array, or (packed, scales, biases) of an int8 g64 tensor
+        # (sealed.rs:64-78): rows f16(s q + b) on the way in (emb_q8.cu emb_q8_gather),
+        # f32 weights s q + b on the way out (tv_q8_h).
+        def table(t):
+            if isinstance(t, tuple):
+                from . import sealed_oracle
+                W = sealed_oracle.q8_rows_f32(np.asarray(t[0], np.uint8), np.asarray(t[1], np.uint16),
+                                              np.asarray(t[2], np.uint16), cfg.hidden_size)
+                return W.astype(np.float16), W.astype(np.float64)
+            a = np.asarray(t, np.float16)
+            return a, a.astype(np.float64)
+
+        self.embed, embed_w = table(weights.embed)
+        self.head = embed_w if weights.lm_head is None else table(weights.lm_head)[1]
         self.cos, self.sin = rope_tables(cfg.head_dim, cfg.rope_theta, cfg.max_positions)
         self.reset()
 
@@ -152,7 +164,7 @@ class Qwen3Oracle:
             h = r16(h + r16(Wd @ a))
         x = rms_norm(h, self.fn, eps)
         self.pos += 1
-        return r16(self.head.astype(np.float64) @ x).astype(np.float32)
+        return r16(self.head @ x).astype(np.float32)
 
     def generate(self, prompt, max_new):
         """model.rs:1041-1073; also returns the logits of every decoding step."""

@@ -146,3 +146,63 @@ def test_rotation_with_a_wide_odd_factor_is_refused():
     with pytest.raises(LlvqError) as e:  # k = 33 > 32 (fused.rs:698-704)
         _ffi.check(_ffi.lib().llvq_hip_host_rotate(33 * 8, 1, v.ctypes.data))
     assert e.value.kind == "Unsupported" and "33" in str(e.value)
+
+
+# ---- sealed sections through the library's own reader (sealed.rs:277-341) ----------------
+def _parse_raw(buf, pos=0, version=3):
+    info = _ffi.RawInfo()
+    p = C.c_size_t(pos)
+    _ffi.check(_ffi.lib().llvq_hip_parse_raw_tensor(bytes(buf), len(buf), C.byref(p), version, C.byref(info)))
+    return info, p.value
+
+
+def test_library_reads_raw_tensors_and_blobs():
+    q = artifact.RawTensor("model.embed_tokens.weight", [2, 5], bits=4, group=2, packed=[0x10, 0x32, 0x54, 0x76, 0x98],
+                           scales=[0x3C00] * 6, biases=[0x0000, 0x3C00, 0x4000, 0x4200, 0x4400, 0x4500])  # raw_tensors.rs:66-78
+    f = artifact.RawTensor("model.norm.weight", [2, 3], data=[0x3C00, 0xC000, 0x0001, 0x7BFF, 0x0000, 0x8000])
+    buf = artifact.write_raw(f) + artifact.write_raw(q) + artifact.write_blob(artifact.Blob("config.json", b"{}"))
+    a, pos = _parse_raw(buf)
+    assert a.name == b"model.norm.weight" and a.tag == 0 and a.rank == 2 and list(a.dims[:2]) == [2, 3] and a.count == 6
+    assert np.frombuffer(buf, "<u2", 6, a.data_off).tolist() == f.data.tolist() and a.data_len == 12
+    b, pos = _parse_raw(buf, pos)
+    assert b.name == b"model.embed_tokens.weight" and (b.tag, b.bits, b.group, b.count) == (1, 4, 2, 6)
+    assert buf[b.data_off:b.data_off + b.data_len] == bytes(q.packed)
+    assert np.frombuffer(buf, "<u2", 6, b.biases_off).tolist() == q.biases.tolist()
+    assert np.frombuffer(buf, "<u2", 6, b.scales_off).tolist() == q.scales.tolist()
+    blob = _ffi.BlobInfo()
+    p = C.c_size_t(pos)
+    _ffi.check(_ffi.lib().llvq_hip_parse_blob(buf, len(buf), C.byref(p), C.byref(blob)))
+    assert blob.name == b"config.json" and buf[blob.data_off:blob.data_off + blob.data_len] == b"{}" and p.value == len(buf)
+    # legacy record: no tag below version 3 (raw_tensors.rs:129-144)
+    legacy = struct.pack("<I", 1) + b"w" + struct.pack("<I", 1) + struct.pack("<Q", 3) + struct.pack("<Q", 3) + struct.pack(
+        "<3H", 0x3C00, 0xC000, 0x7BFF)
+    c, pos = _parse_raw(legacy, 0, 2)
+    assert c.name == b"w" and c.tag == 0 and c.count == 3 and pos == len(legacy)
+
+
+def test_library_refuses_hostile_sealed_sections():
+    from llvq_amd import LlvqError
+
+    with pytest.raises(LlvqError) as e:  # hostile_files.rs:172-181
+        _parse_raw(struct.pack("<I", 99) + bytes(32))
+    assert e.value.kind == "BadRawEncoding" and "encoding tag 99" in str(e.value)
+    lying = struct.pack("<I", 0) + struct.pack("<I", 1) + b"t" + struct.pack("<I", 1) + struct.pack("<Q", 4) + struct.pack(
+        "<Q", 2 ** 64 - 1)
+    with pytest.raises(LlvqError) as e:  # hostile_files.rs:184-200
+        _parse_raw(lying)
+    assert e.value.kind == "Truncated" and "raw tensor data" in str(e.value)
+    blob = struct.pack("<I", 1) + b"b" + struct.pack("<Q", 2 ** 64 - 1)
+    info = _ffi.BlobInfo()
+    p = C.c_size_t(0)
+    with pytest.raises(LlvqError) as e:  # hostile_files.rs:203-213
+        _ffi.check(_ffi.lib().llvq_hip_parse_blob(blob, len(blob), C.byref(p), C.byref(info)))
+    assert e.value.kind == "Truncated" and str(e.value).endswith("mid-blob")
+    with pytest.raises(LlvqError) as e:
+        _parse_raw(struct.pack("<I", 0) + struct.pack("<I", 2) + b"\xff\xfe" + bytes(16))
+    assert e.value.kind == "BadName"
+    # every prefix of an honest record is a truncation, never a crash
+    honest = artifact.write_raw(artifact.RawTensor("t", [3], data=[1, 2, 3]))
+    for cut in range(len(honest)):
+        with pytest.raises(LlvqError) as e:
+            _parse_raw(honest[:cut])
+        assert e.value.kind == "Truncated"
