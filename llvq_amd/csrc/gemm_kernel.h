@@ -169,73 +169,15 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         return read_record(raw, row * kGemmRowBytes + off + 6u * b);
       };
 
-      // P1: classify and bin
-      {
-        uint32_t entry[kGemmP1Blocks], ci[kGemmP1Blocks], kbits[kGemmP1Blocks], kmax = 0;
-        uint64_t zi[kGemmP1Blocks];
-#pragma unroll
-        for (int i = 0; i < kGemmP1Blocks; ++i) {
-          const uint32_t f = tid + (uint32_t)i * kWgThreads;
-          zi[i] = ~0ULL;
-          entry[i] = 0;
-          ci[i] = 0;
-          kbits[i] = 0;
-          if (f < nblk) {
-            const uint32_t row = (f * inv_kb) >> 16, b = f - row * kb;
-            const uint64_t rec = record_at(row, b);
-            entry[i] = f | ((uint32_t)(rec & 1) << 25);
-            if ((rec >> 1) == 0) {
-              entry[i] |= 0x40000000u;  // the origin: P2 writes 24 zero weights (W may still be read by P3 now)
-            } else {
-              zi[i] = (rec >> 1) - 1;
-              const uint32_t e = T.lut[(uint32_t)(zi[i] >> kLutShift)];
-              ci[i] = e & 511u;
-              kbits[i] = 1u << ((e >> 9) & 7u);
-              kmax = max(kmax, kbits[i]);
-            }
-          }
-        }
-        uint32_t kw = 1;
-#pragma unroll
-        for (uint32_t t = 1; t <= 6; ++t) kw = __any(kmax >= (1u << t)) ? (1u << t) : kw;
-        for (uint32_t step = kw >> 1; step; step >>= 1) {
-#pragma unroll
-          for (int i = 0; i < kGemmP1Blocks; ++i)
-            if (step < kbits[i] && T.starts[ci[i] + step] <= zi[i]) ci[i] += step;
-        }
-        uint32_t path[kGemmP1Blocks], odd_rank[kGemmP1Blocks], even_rank[kGemmP1Blocks], n_o = 0, n_e = 0;
-#pragma unroll
-        for (int i = 0; i < kGemmP1Blocks; ++i) {
-          path[i] = zi[i] != ~0ULL ? ((T.fast[ci[i]].meta >> kMetaPathShift) & 3u)
-                                   : ((entry[i] & 0x40000000u) ? (uint32_t)kPathOdd : 3u);
-          entry[i] |= ci[i] << 16;
-          if (path[i] == kPathGeneric) {
-            entry[i] |= 0x80000000u;
-            const uint32_t slot = atomicAdd(&ctrl[2], 1u);
-            if (slot < (uint32_t)kGenericSlots) {
-              gqueue[slot] = entry[i];
-              path[i] = 3u;
-            }
-          }
-          const uint64_t mo = __ballot(path[i] == kPathOdd || path[i] == kPathGeneric), me = __ballot(path[i] == kPathEven);
-          odd_rank[i] = n_o + __builtin_amdgcn_mbcnt_hi((uint32_t)(mo >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mo, 0));
-          even_rank[i] = n_e + __builtin_amdgcn_mbcnt_hi((uint32_t)(me >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)me, 0));
-          n_o += (uint32_t)__popcll(mo);
-          n_e += (uint32_t)__popcll(me);
-        }
-        uint32_t base_o = 0, base_e = 0;
-        if (lane == 0) {
-          base_o = atomicAdd(&ctrl[0], n_o);
-          base_e = atomicAdd(&ctrl[1], n_e);
-        }
-        base_o = __shfl(base_o, 0, 64);
-        base_e = __shfl(base_e, 0, 64);
-#pragma unroll
-        for (int i = 0; i < kGemmP1Blocks; ++i) {
-          if (path[i] == kPathOdd || path[i] == kPathGeneric) queue[base_o + odd_rank[i]] = entry[i];
-          if (path[i] == kPathEven) queue[kGemmTile - 1 - (base_e + even_rank[i])] = entry[i];
-        }
-      }
+      // P1: classify and bin.  An origin block is queued: its 24 zero weights are
+      // written in P2, because the W slice may still be read by the previous slice's P3 now.
+      classify_and_bin<kGemmP1Blocks>(
+          T, nblk, kGemmTile, queue, gqueue, ctrl,
+          [&](uint32_t f) {
+            const uint32_t row = (f * inv_kb) >> 16;
+            return record_at(row, f - row * kb);
+          },
+          [](uint32_t) { return true; });
       __syncthreads();
       LLVQ_GSTAMP(1);
 
@@ -257,7 +199,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
         const float g = (entry >> 25) & 1u ? a.g1 : a.g0;
         _Float16* wrow = W + (size_t)row * kGemmWStride + b * 24u;
-        if (entry & 0x40000000u) {
+        if (entry & kEntryOrigin) {
           uint4* dst = reinterpret_cast<uint4*>(wrow);
           dst[0] = dst[1] = dst[2] = make_uint4(0, 0, 0, 0);
         } else if (from_odd) {

@@ -178,19 +178,6 @@ __device__ __forceinline__ void store_out<__half>(void* y, uint32_t r, float v) 
   reinterpret_cast<__half*>(y)[r] = __float2half_rn(v);
 }
 
-// queue entry: block slot in the tile (12 bits) | class (9 bits) << 16 | gain << 25 | generic-walk << 31
-__device__ __forceinline__ void queue_push(uint32_t* counter, uint32_t* queue, bool mine, uint32_t entry,
-                                           bool from_top) {
-  const uint64_t m = __ballot(mine);
-  if (m == 0) return;
-  const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
-  const int first = __ffsll((long long)m) - 1;
-  uint32_t base = 0;
-  if ((int)(threadIdx.x & 63u) == first) base = atomicAdd(counter, (uint32_t)__popcll(m));
-  base = __shfl(base, first, 64);
-  if (mine) queue[from_top ? (kTileBlocks - 1 - (base + rank)) : (base + rank)] = entry;
-}
-
 // One 24-column block of the activation -> scale and byte planes.
 __device__ __forceinline__ void load_block_f16(const __half* x, float (&v)[kDim]) {
   if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
@@ -299,6 +286,95 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 #else
 #define LLVQ_STAMP(k) do {} while (0)
 #endif
+
+// P1 of both kernels: every lane classifies up to NB blocks of the tile and
+// bins them.  `record(f)` returns the 48-bit record of tile slot f < nblk;
+// `origin(f)` is called for an origin block (index 0) and returns whether the
+// block must still be queued (flagged, with the odd-coset blocks) or is settled.
+// Queue entry: slot (12 bits) | class << 16 | gain << 25 | origin << 30 | generic walk << 31.
+// The halving searches of a lane's blocks run side by side (independent LDS
+// chains); a wavefront claims queue space with one atomic per queue.  Blocks of
+// the rare generic classes take ~2000 dependent instructions: they go to a
+// small queue that P2 hands out first; what does not fit rides in the odd queue.
+constexpr uint32_t kEntryOrigin = 0x40000000u, kEntryGeneric = 0x80000000u;
+template <int NB, typename RecordFn, typename OriginFn>
+__device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t nblk, uint32_t capacity, uint32_t* queue,
+                                                 uint32_t* gqueue, uint32_t* ctrl, RecordFn record, OriginFn origin) {
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  uint32_t entry[NB], ci[NB];
+  uint64_t zi[NB];  // zero-based index, ~0 when the lane has no block / an origin
+  bool queued_origin[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const uint32_t f = tid + (uint32_t)i * kWgThreads;
+    zi[i] = ~0ULL;
+    entry[i] = 0;
+    ci[i] = 0;
+    queued_origin[i] = false;
+    if (f < nblk) {
+      const uint64_t rec = record(f);
+      entry[i] = f | ((uint32_t)(rec & 1) << 25);
+      if ((rec >> 1) == 0) {  // the origin decodes to zero whatever the gain (index.rs:335-337)
+        queued_origin[i] = origin(f);
+        if (queued_origin[i]) entry[i] |= kEntryOrigin;
+      } else {
+        zi[i] = (rec >> 1) - 1;
+      }
+    }
+  }
+  uint32_t kbits[NB], kmax = 0;  // kbits = 2^k: how many classes the bucket's search spans
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    kbits[i] = 0;
+    if (zi[i] != ~0ULL) {
+      const uint32_t e = T.lut[(uint32_t)(zi[i] >> kLutShift)];
+      ci[i] = e & 511u;
+      kbits[i] = 1u << ((e >> 9) & 7u);
+      kmax = max(kmax, kbits[i]);
+    }
+  }
+  // the wavefront runs as many halving steps as its widest bucket needs; a
+  // lane only reads the table on the steps its own bucket needs
+  uint32_t kw = 1;
+#pragma unroll
+  for (uint32_t t = 1; t <= 6; ++t) kw = __any(kmax >= (1u << t)) ? (1u << t) : kw;
+  for (uint32_t step = kw >> 1; step; step >>= 1) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+      if (step < kbits[i] && T.starts[ci[i] + step] <= zi[i]) ci[i] += step;
+  }
+  uint32_t path[NB], odd_rank[NB], even_rank[NB], n_o = 0, n_e = 0;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    path[i] = zi[i] != ~0ULL ? ((T.fast[ci[i]].meta >> kMetaPathShift) & 3u) : (queued_origin[i] ? (uint32_t)kPathOdd : 3u);
+    entry[i] |= ci[i] << 16;
+    if (path[i] == kPathGeneric) {
+      entry[i] |= kEntryGeneric;
+      const uint32_t slot = atomicAdd(&ctrl[2], 1u);
+      if (slot < (uint32_t)kGenericSlots) {
+        gqueue[slot] = entry[i];
+        path[i] = 3u;  // placed
+      }
+    }
+    const uint64_t mo = __ballot(path[i] == kPathOdd || path[i] == kPathGeneric), me = __ballot(path[i] == kPathEven);
+    odd_rank[i] = n_o + __builtin_amdgcn_mbcnt_hi((uint32_t)(mo >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mo, 0));
+    even_rank[i] = n_e + __builtin_amdgcn_mbcnt_hi((uint32_t)(me >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)me, 0));
+    n_o += (uint32_t)__popcll(mo);
+    n_e += (uint32_t)__popcll(me);
+  }
+  uint32_t base_o = 0, base_e = 0;
+  if (lane == 0) {
+    base_o = atomicAdd(&ctrl[0], n_o);
+    base_e = atomicAdd(&ctrl[1], n_e);
+  }
+  base_o = __shfl(base_o, 0, 64);
+  base_e = __shfl(base_e, 0, 64);
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    if (path[i] == kPathOdd || path[i] == kPathGeneric) queue[base_o + odd_rank[i]] = entry[i];  // odd from the bottom
+    if (path[i] == kPathEven) queue[capacity - 1 - (base_e + even_rank[i])] = entry[i];          // even from the top
+  }
+}
 
 template <typename OutT, int TILE = LLVQ_TILE_BLOCKS>
 __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
@@ -415,85 +491,13 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     __syncthreads();
     LLVQ_STAMP(1);
 
-    // P1: classify and bin.  Each lane owns up to kP1Blocks blocks and walks their
-    // class searches side by side (independent LDS chains); a wavefront then
-    // claims queue space with one atomic per queue.
-    {
-      uint32_t entry[kP1Blocks], ci[kP1Blocks];
-      uint64_t zi[kP1Blocks];  // zero-based index, ~0 when the lane has no block / an origin
-#pragma unroll
-      for (int i = 0; i < kP1Blocks; ++i) {
-        const uint32_t f = tid + (uint32_t)i * kWgThreads;
-        zi[i] = ~0ULL;
-        entry[i] = 0;
-        ci[i] = 0;
-        if (f < nblk) {
-          const uint64_t rec = read_record(raw, off + 6 * f);
-          entry[i] = f | ((uint32_t)(rec & 1) << 25);
-          if ((rec >> 1) == 0) partial[f] = 0.f;  // the origin decodes to zero whatever the gain (index.rs:335-337)
-          else zi[i] = (rec >> 1) - 1;
-        }
-      }
-      uint32_t kbits[kP1Blocks], kmax = 0;  // kbits = 2^k: how many classes the bucket's search spans
-#pragma unroll
-      for (int i = 0; i < kP1Blocks; ++i) {
-        kbits[i] = 0;
-        if (zi[i] != ~0ULL) {
-          const uint32_t e = T.lut[(uint32_t)(zi[i] >> kLutShift)];
-          ci[i] = e & 511u;
-          kbits[i] = 1u << ((e >> 9) & 7u);
-          kmax = max(kmax, kbits[i]);
-        }
-      }
-      // the wavefront runs as many halving steps as its widest bucket needs; a
-      // lane only reads the table on the steps its own bucket needs
-      uint32_t kw = 1;
-#pragma unroll
-      for (uint32_t t = 1; t <= 6; ++t) kw = __any(kmax >= (1u << t)) ? (1u << t) : kw;
-      for (uint32_t step = kw >> 1; step; step >>= 1) {
-#pragma unroll
-        for (int i = 0; i < kP1Blocks; ++i)
-          if (step < kbits[i] && T.starts[ci[i] + step] <= zi[i]) ci[i] += step;
-      }
-      uint32_t path[kP1Blocks];
-#pragma unroll
-      for (int i = 0; i < kP1Blocks; ++i) {
-        path[i] = zi[i] != ~0ULL ? ((T.fast[ci[i]].meta >> kMetaPathShift) & 3u) : 3u;
-        entry[i] |= ci[i] << 16;
-      }
-      // Blocks of the rare generic classes take ~2000 dependent instructions: they
-      // go to a small queue that P2 hands out first; what does not fit rides in the
-      // odd queue.  Either way bit 31 marks them.
-      uint32_t odd_rank[kP1Blocks], even_rank[kP1Blocks], n_o = 0, n_e = 0;
-#pragma unroll
-      for (int i = 0; i < kP1Blocks; ++i) {
-        if (path[i] == kPathGeneric) {
-          entry[i] |= 0x80000000u;
-          const uint32_t slot = atomicAdd(&ctrl[2], 1u);
-          if (slot < (uint32_t)kGenericSlots) {
-            gqueue[slot] = entry[i];
-            path[i] = 3u;  // placed
-          }
-        }
-        const uint64_t mo = __ballot(path[i] == kPathOdd || path[i] == kPathGeneric), me = __ballot(path[i] == kPathEven);
-        odd_rank[i] = n_o + __builtin_amdgcn_mbcnt_hi((uint32_t)(mo >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mo, 0));
-        even_rank[i] = n_e + __builtin_amdgcn_mbcnt_hi((uint32_t)(me >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)me, 0));
-        n_o += (uint32_t)__popcll(mo);
-        n_e += (uint32_t)__popcll(me);
-      }
-      uint32_t base_o = 0, base_e = 0;
-      if (lane == 0) {
-        base_o = atomicAdd(&ctrl[0], n_o);
-        base_e = atomicAdd(&ctrl[1], n_e);
-      }
-      base_o = __shfl(base_o, 0, 64);
-      base_e = __shfl(base_e, 0, 64);
-#pragma unroll
-      for (int i = 0; i < kP1Blocks; ++i) {
-        if (path[i] == kPathOdd || path[i] == kPathGeneric) queue[base_o + odd_rank[i]] = entry[i];
-        if (path[i] == kPathEven) queue[kTileBlocks - 1 - (base_e + even_rank[i])] = entry[i];
-      }
-    }
+    // P1: classify and bin
+    classify_and_bin<kP1Blocks>(
+        T, nblk, kTileBlocks, queue, gqueue, ctrl, [&](uint32_t f) { return read_record(raw, off + 6 * f); },
+        [&](uint32_t f) {
+          partial[f] = 0.f;
+          return false;
+        });
     __syncthreads();
     LLVQ_STAMP(2);
     prefetch_tile(a, tile + gridDim.x, tid, pre0, pre1);
