@@ -9,7 +9,7 @@
 //
 // Work unit: a band of 64 weight rows x a range of blocks of those rows.  One
 // persistent 1024-lane workgroup per CU walks its unit in K-slices of at most
-// 20 blocks per row (480 columns, 1280 blocks):
+// 32 blocks per row (768 columns, 2048 blocks):
 //   P0  the slice's code bytes, 16-byte loads -> LDS (next slice's loads are
 //       already in flight while this one is decoded);
 //   P1  classify and bin the blocks (odd / even / generic queues);
@@ -23,9 +23,9 @@
 //       registers) stay live across slices.
 // Epilogue: row scale and the f32 tail columns in f32, then the store.  When a
 // matrix has too few bands to occupy the chip its block range is split over
-// several units; each writes its partial sums to a workspace and the unit that
-// arrives last at the band's counter adds them in a fixed order, so the result
-// does not depend on scheduling.
+// several units; each writes its partial sums to a workspace and a second,
+// chip-wide kernel (gemm_reduce_kernel) adds them in split order and applies
+// the epilogue, so the result does not depend on scheduling.
 #pragma once
 
 namespace llvq {
@@ -35,9 +35,9 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kGemmRows = 64;                 // weight rows of a band
 #ifndef LLVQ_GEMM_KB
-#define LLVQ_GEMM_KB 20
+#define LLVQ_GEMM_KB 32
 #endif
-constexpr int kGemmKb = LLVQ_GEMM_KB;         // blocks per row and K-slice (20: 480 columns = 15 K-steps of 32)
+constexpr int kGemmKb = LLVQ_GEMM_KB;         // blocks per row and K-slice (32: 768 columns = 24 K-steps of 32, 2048 blocks = two 64-block chunks per wavefront)
 constexpr int kGemmTile = kGemmRows * kGemmKb;  // blocks per K-slice
 constexpr int kGemmP1Blocks = (kGemmTile + kWgThreads - 1) / kWgThreads;
 constexpr int kGemmRowChunks = (kGemmKb * 6 + 14 + 15) / 16;  // 16-byte units holding one row's code bytes at any even alignment
@@ -55,14 +55,16 @@ struct GemmArgs {
   const float* tail;
   void* y;                // [M, d_out]
   float* ws;              // [S, M, d_out] partial sums when S > 1
-  uint32_t* counters;     // [n_bands], zero between launches
   float g0, g1;
   uint32_t M, ldx, d_out, nblocks, tail_w;
   uint32_t n_bands, S, bps;  // split count, blocks per split
 };
 
+// The batched kernel keeps the Golay words and the support-arrangement table in L2:
+// the 33 KB they would take in LDS buy a W slice of 32 blocks per row instead of 20.
+constexpr size_t kGemmImageBytes = kLdsImageBytesLean;
 constexpr size_t gemm_lds_bytes() {
-  return kLdsImageBytes + (size_t)kGemmRows * kGemmRowBytes + (size_t)kGemmTile * 4 + kGenericSlots * 4 + 16 +
+  return kGemmImageBytes + (size_t)kGemmRows * kGemmRowBytes + (size_t)kGemmTile * 4 + kGenericSlots * 4 + 16 +
          (size_t)kGemmRows * kGemmWStride * 2;
 }
 static_assert(gemm_lds_bytes() <= 160 * 1024, "GEMM workgroup state must fit one CU's LDS");
@@ -105,8 +107,8 @@ __device__ __forceinline__ void store_y<__half>(void* y, size_t at, float v) {
 template <int RT, typename OutT>
 __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
-  const DecodeTables T = stage_tables(smem, a.tables);
-  uint8_t* raw = smem + kLdsImageBytes;
+  const DecodeTables T = stage_tables<false>(smem, a.tables);
+  uint8_t* raw = smem + kGemmImageBytes;
   uint32_t* queue = reinterpret_cast<uint32_t*>(raw + kGemmRows * kGemmRowBytes);
   uint32_t* gqueue = queue + kGemmTile;
   uint32_t* ctrl = gqueue + kGenericSlots;
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       const uint32_t kb = min((uint32_t)kGemmKb, kb_hi - k0);
       sj = sj + 1 == n_slices ? 0u : sj + 1;
       const uint32_t nblk = rows * kb;
-      const uint32_t inv_kb = (65536u + kb - 1u) / kb;  // floor(f / kb) = (f * inv_kb) >> 16 for f < 1536, kb <= 24
+      const uint32_t inv_kb = (65536u + kb - 1u) / kb;  // floor(f / kb) = (f * inv_kb) >> 16 for f < 2048, kb <= 32
       // P0
       if (tid < 4) ctrl[tid] = 0;
       if (tid < (uint32_t)(kGemmRows * kGemmRowChunks)) reinterpret_cast<uint4*>(raw)[tid] = pre;
@@ -302,7 +304,6 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     };
     const bool m_ok = my_m < a.M;
     const bool vec_ok = (a.d_out & 3u) == 0;  // four consecutive rows of one activation row store as one vector
-    bool reduce_here = false;
     if (a.S > 1) {
       if (m_ok) {
         float* dst = a.ws + ((size_t)split * a.M + my_m) * a.d_out + r0;
@@ -321,25 +322,13 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
             }
           }
       }
-      // The unit that arrives last at the band's counter adds the partial sums.
-      // One lane publishes for the workgroup: the barrier orders every lane's
-      // stores before its device-scope release, and its acquire after the
-      // counter read orders the other units' stores before this workgroup's loads.
-      __syncthreads();
-      if (tid == 0) {
-        const uint32_t seen = __hip_atomic_fetch_add(&a.counters[band], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        ctrl[0] = seen;
-      }
-      __syncthreads();
-      reduce_here = ctrl[0] == a.S - 1;
+      // gemm_reduce_kernel finishes these rows
     } else {
       __syncthreads();  // W is about to hold the tail staging
     }
-    if (a.S == 1 || reduce_here) {
+    if (a.S == 1) {
       if (tw) stage_tail();
       __syncthreads();
-    }
-    if (a.S == 1) {
       if (m_ok) {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
@@ -372,29 +361,82 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
             }
           }
       }
-    } else if (reduce_here) {
-      for (uint32_t o = tid; o < rows * a.M; o += kWgThreads) {
-        const uint32_t m = o / rows, row = o - m * rows;
-        const float* src = a.ws + (size_t)m * a.d_out + r0 + row;
-        const size_t sstride = (size_t)a.M * a.d_out;
-        float sum = 0.f;
-        uint32_t sp = 0;
-        for (; sp + 4 <= a.S; sp += 4) {  // four loads in flight, added in split order
-          const float p0 = src[(size_t)sp * sstride], p1 = src[(size_t)(sp + 1) * sstride];
-          const float p2 = src[(size_t)(sp + 2) * sstride], p3 = src[(size_t)(sp + 3) * sstride];
-          sum = (((sum + p0) + p1) + p2) + p3;
-        }
-        for (; sp < a.S; ++sp) sum += src[(size_t)sp * sstride];
-        float ts = 0.f;
-        for (uint32_t t = 0; t < tw; ++t) ts = fmaf(tl[row * tw + t], __half2float(xt[m * tw + t]), ts);
-        store_y<OutT>(a.y, (size_t)m * a.d_out + r0 + row, fmaf(sum, a.rscale[r0 + row], ts));
-      }
-      if (tid == 0) a.counters[band] = 0;  // ready for the next launch
     }
 #ifdef LLVQ_PHASE_TIMING
     if (threadIdx.x == 0 && unit == blockIdx.x) g_phase_stamps[blockIdx.x * 8 + 5] = wall_clock64();
 #endif
     __syncthreads();  // W, raw and counters are reused by the next unit
+  }
+}
+
+// Second pass of a split launch: y[m][r] = (sum over splits, in split order, of the
+// partial sums) * rscale[r] + tail[r] . x_tail[m].  One lane per four consecutive
+// rows of one activation row; the partial sums are read with all their loads in
+// flight (eight splits at a time).
+struct GemmReduceArgs {
+  const float* ws;  // [S, M, d_out]
+  const __half* x;  // [M, ldx]
+  const float* rscale;
+  const float* tail;
+  void* y;
+  uint32_t M, ldx, d_out, nblocks, tail_w, S;
+};
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
+  const uint32_t quads = (a.d_out + 3u) >> 2;
+  const size_t items = (size_t)quads * a.M, sstride = (size_t)a.M * a.d_out;
+  const bool vec_ok = (a.d_out & 3u) == 0;
+  for (size_t it = (size_t)blockIdx.x * blockDim.x + threadIdx.x; it < items; it += (size_t)gridDim.x * blockDim.x) {
+    const uint32_t m = (uint32_t)(it / quads), row = (uint32_t)(it - (size_t)m * quads) * 4u;
+    const float* src = a.ws + (size_t)m * a.d_out + row;
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    if (vec_ok) {
+      for (uint32_t s0 = 0; s0 < a.S; s0 += 8) {
+        float4 p[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          p[u] = s0 + u < a.S ? *reinterpret_cast<const float4*>(src + (size_t)(s0 + u) * sstride) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < a.S) {
+            sum[0] += p[u].x;
+            sum[1] += p[u].y;
+            sum[2] += p[u].z;
+            sum[3] += p[u].w;
+          }
+      }
+    } else {
+      for (uint32_t s = 0; s < a.S; ++s)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (row + i < a.d_out) sum[i] += src[(size_t)s * sstride + i];
+    }
+    const __half* xt = a.x + (size_t)m * a.ldx + (size_t)a.nblocks * 24u;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t r = min(row + i, a.d_out - 1u);
+      float ts = 0.f;
+      for (uint32_t t = 0; t < a.tail_w; ++t) ts = fmaf(a.tail[(size_t)r * a.tail_w + t], __half2float(xt[t]), ts);
+      v[i] = fmaf(sum[i], a.rscale[r], ts);
+    }
+    const size_t at = (size_t)m * a.d_out + row;
+    if (vec_ok) {
+      if constexpr (sizeof(OutT) == 4) {
+        *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+        const __half2 lo = __float22half2_rn(make_float2(v[0], v[1])), hi = __float22half2_rn(make_float2(v[2], v[3]));
+        uint2 pk;
+        pk.x = *reinterpret_cast<const uint32_t*>(&lo);
+        pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+        *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(a.y) + at) = pk;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (row + i < a.d_out) store_y<OutT>(a.y, at + i, v[i]);
+    }
   }
 }
 

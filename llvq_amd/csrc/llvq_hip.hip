@@ -56,12 +56,19 @@ struct GlobalTables {
   const uint32_t* expand;
 };
 
+constexpr size_t kLdsImageBytesLean = offsetof(TableImage, golay);  // without the Golay words and the support-arrangement table
+static_assert(kLdsImageBytesLean % 16 == 0, "LDS part of the table image is copied in 16-byte units");
+
+// kFull: the whole image goes to LDS; otherwise its last two tables (33 KB) are
+// read through L2, for a kernel that needs the LDS for something else.
+template <bool kFull = (LLVQ_LDS_GOLAY != 0)>
 __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const GlobalTables& g) {
   const uint4* src = reinterpret_cast<const uint4*>(g.image);
   uint4* dst = reinterpret_cast<uint4*>(smem);
-  for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) dst[i] = src[i];
+  constexpr size_t kBytes = kFull ? sizeof(TableImage) : kLdsImageBytesLean;
+  for (uint32_t i = threadIdx.x; i < kBytes / 16; i += blockDim.x) dst[i] = src[i];
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
-  const TableImage* far = LLVQ_LDS_GOLAY ? s : g.image;
+  const TableImage* far = kFull ? s : g.image;
   return DecodeTables{far->golay, g.cls, s->fast, s->starts, s->lut, s->rcp, far->on_lut, g.off_lut, g.expand, s->pdep4, s->step};
 }
 
@@ -694,11 +701,9 @@ struct llvq_rt {
   size_t rot_scratch_elems = 0;
   __half* rot_rows = nullptr;     // rotated batch rows, f16 (matrix-core path)
   size_t rot_rows_elems = 0;
-  // split-K state of the batched kernel: partial sums and per-band arrival counters
+  // split-K workspace of the batched kernel: partial sums [S, M, d_out]
   float* gemm_ws = nullptr;
   size_t gemm_ws_bytes = 0;
-  uint32_t* gemm_counters = nullptr;
-  size_t gemm_counter_slots = 0;
 };
 
 struct llvq_mat {
@@ -803,7 +808,6 @@ void llvq_hip_runtime_destroy(llvq_rt* rt) {
   (void)hipSetDevice(rt->device);
   (void)hipFree(rt->blob);
   (void)hipFree(rt->gemm_ws);
-  (void)hipFree(rt->gemm_counters);
   (void)hipFree(rt->rot_scratch);
   (void)hipFree(rt->rot_rows);
   for (auto* r : rt->rotations) {
@@ -1256,9 +1260,11 @@ static void pick_gemm_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint
     const uint32_t bps = (nblocks + S - 1) / S;
     if ((uint64_t)(S - 1) * bps >= nblocks && S > 1) continue;  // an empty last split
     const uint32_t slices = (bps + kGemmKb - 1) / kGemmKb;
-    const double unit_us = 2.0 + slices * (5.0 + 0.018 * M) + 64.0 * bps * 0.0042 + 0.015 * M + (S > 1 ? 0.5 + 0.01 * M * S : 0.0);
+    const double unit_us = 2.0 + slices * (5.0 + 0.018 * M) + 64.0 * bps * 0.0042 + 0.015 * M + (S > 1 ? 0.002 * M : 0.0);
     const uint64_t units = (uint64_t)n_bands * S;
-    const double t = (double)((units + grid - 1) / grid) * unit_us;
+    // a split launch pays a second, chip-wide pass over S partial sums per output
+    const double reduce_us = S > 1 ? 6.0 + (double)S * M * 64.0 * n_bands * 4.0 / 2.0e6 : 0.0;
+    const double t = (double)((units + grid - 1) / grid) * unit_us + reduce_us;
     if (t < best * 0.999) { best = t; best_s = S; best_bps = bps; }
   }
   *S_out = best_s;
@@ -1292,17 +1298,7 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
       HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_ws), need));
       rt->gemm_ws_bytes = need;
     }
-    if (a.n_bands > rt->gemm_counter_slots) {
-      (void)hipFree(rt->gemm_counters);
-      rt->gemm_counters = nullptr;
-      rt->gemm_counter_slots = 0;
-      const size_t slots = (size_t)a.n_bands + 1024;
-      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_counters), slots * sizeof(uint32_t)));
-      HIP_TRY(hipMemset(rt->gemm_counters, 0, slots * sizeof(uint32_t)));
-      rt->gemm_counter_slots = slots;
-    }
     a.ws = rt->gemm_ws;
-    a.counters = rt->gemm_counters;
   }
   const uint32_t units = a.n_bands * a.S;
   const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
@@ -1316,6 +1312,27 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
     else hipLaunchKernelGGL((gemm_tiles_kernel<2, __half>), grid, wg, lds, rt->stream, a);
   }
   HIP_TRY(hipGetLastError());
+  if (a.S > 1) {
+    GemmReduceArgs r{};
+    r.ws = a.ws;
+    r.x = a.x;
+    r.rscale = a.rscale;
+    r.tail = a.tail;
+    r.y = a.y;
+    r.M = a.M;
+    r.ldx = a.ldx;
+    r.d_out = a.d_out;
+    r.nblocks = a.nblocks;
+    r.tail_w = a.tail_w;
+    r.S = a.S;
+    const size_t items = (size_t)((m->d_out + 3) / 4) * M;
+    size_t rgrid = (items + 255) / 256;
+    const size_t rcap = (size_t)grid_cap * 8;
+    if (rgrid > rcap) rgrid = rcap;
+    if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3((uint32_t)rgrid), dim3(256), 0, rt->stream, r);
+    else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3((uint32_t)rgrid), dim3(256), 0, rt->stream, r);
+    HIP_TRY(hipGetLastError());
+  }
   return LLVQ_OK;
 }
 
