@@ -225,7 +225,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
                                                                    __half* __restrict__ ctx,
                                                                    float* __restrict__ part, uint32_t* __restrict__ counters,
                                                                    uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
-                                                                   uint32_t T, uint32_t max_pos, float scale, uint32_t n_splits) {
+                                                                   uint32_t T, uint32_t max_pos, float scale, uint32_t n_splits,
+                                                                   uint32_t merge_inline) {
   extern __shared__ __align__(16) float att_smem[];
   __shared__ uint32_t arrived;
   __shared__ float red[kAttnWaves][kAttnMaxGroup];
@@ -437,6 +438,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
     dst[0] = mg;  // -inf for an empty range
     dst[1] = ls;
   }
+  if (!merge_inline) return;  // attn_merge_kernel finishes (long caches: many partials, merged chip-wide)
   // publish, and let the last workgroup of this kv head merge (one lane's
   // device-scope release / acquire stands for the workgroup, ordered by the barriers)
   __syncthreads();
@@ -489,6 +491,44 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
     ctx[(size_t)head * head_dim + i] = __float2half_rn(A / Ls[g]);
   }
   if (tid == 0) counters[kvh] = 0;  // ready for the next launch
+}
+
+// Merge of the attention partials as a kernel of its own: one workgroup per query
+// head, one lane per output dimension, the partial vectors read eight splits at a
+// time.  Same arithmetic and order as the in-kernel merge.
+__global__ __launch_bounds__(128) void attn_merge_kernel(const float* __restrict__ part, __half* __restrict__ ctx,
+                                                         uint32_t head_dim, uint32_t n_splits) {
+  __shared__ float wts[kAttnMaxSplits];
+  __shared__ float Lsum;
+  const uint32_t head = blockIdx.x, tid = threadIdx.x;
+  const uint32_t stride = head_dim + 2;
+  const float* src = part + (size_t)head * n_splits * stride;
+  if (tid < n_splits) wts[tid] = src[(size_t)tid * stride];
+  __syncthreads();
+  float M = -INFINITY;
+  for (uint32_t s = 0; s < n_splits; ++s) M = fmaxf(M, wts[s]);
+  __syncthreads();
+  if (tid < n_splits) wts[tid] = __expf(wts[tid] - M);
+  __syncthreads();
+  if (tid == 0) {
+    float L = 0.f;
+    for (uint32_t s = 0; s < n_splits; ++s) L = fmaf(src[(size_t)s * stride + 1], wts[s], L);
+    Lsum = L;
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < head_dim; i += 128) {
+    float A = 0.f;
+    uint32_t sp = 0;
+    for (; sp + 8 <= n_splits; sp += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(sp + u) * stride + 2 + i];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) A = fmaf(v[u], wts[sp + u], A);
+    }
+    for (; sp < n_splits; ++sp) A = fmaf(src[(size_t)sp * stride + 2 + i], wts[sp], A);
+    ctx[(size_t)head * head_dim + i] = __float2half_rn(A / Lsum);
+  }
 }
 
 // act = f16(f16(silu(gate)) * up)   (model.rs:831: gu[0].apply(act).mul(gu[1]))

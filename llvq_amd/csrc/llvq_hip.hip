@@ -1448,6 +1448,8 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   const size_t merge_lds = (size_t)groups_per_kv * (n_splits + 1) * sizeof(float);  // the merge reuses the staging area
   if (attn_lds < merge_lds) attn_lds = merge_lds;
   const size_t group_layer = cache_layer / kKvGroup;
+  // few partials: the last workgroup of a kv head merges them; many: a chip-wide merge kernel does
+  const uint32_t merge_inline = n_splits <= 16 ? 1u : 0u;
   // Projections in the natural basis derive their activation in the launch's
   // prologue; a rotated basis needs the activation as a tensor first (it goes
   // through the rotation kernel), and so do rows too wide for the staging area:
@@ -1499,11 +1501,13 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     if (d->kv_q8)
       hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, d->q, kc, vc, lq8,
                          d->ctx, d->attn_part, d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
-                         1.0f / sqrtf((float)d->head_dim), n_splits);
+                         1.0f / sqrtf((float)d->head_dim), n_splits, merge_inline);
     else
       hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, d->q, kc, vc, lq8,
                          d->ctx, d->attn_part, d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
-                         1.0f / sqrtf((float)d->head_dim), n_splits);
+                         1.0f / sqrtf((float)d->head_dim), n_splits, merge_inline);
+    if (!merge_inline)
+      hipLaunchKernelGGL(attn_merge_kernel, dim3(d->n_heads), dim3(128), 0, st, d->attn_part, d->ctx, d->head_dim, n_splits);
     void* o_out[1] = {d->o};
     rc = forward_group(rt, P + 3, 1, d->ctx, o_out, LLVQ_F16);
     if (rc) return rc;

@@ -66,6 +66,26 @@ def test_teacher_forced_logits(gpu_rt, orc, cfg, seed, n):
         dec.close()
 
 
+def test_long_cache_takes_the_merge_kernel(gpu_rt, orc):
+    """Past 512 cached positions the attention partials (more than 16 ranges) are merged
+    by a kernel of their own; the logits must keep agreeing with the oracle across the switch."""
+    import dataclasses
+
+    cfg = dataclasses.replace(Q8, num_hidden_layers=1, max_positions=560, vocab_size=200)
+    dec, ref = _build(gpu_rt, orc, cfg, 9)
+    try:
+        tokens = np.random.default_rng(9).integers(0, cfg.vocab_size, size=548)
+        worst = 0.0
+        for i, t in enumerate(tokens):
+            want = ref.forward_token(int(t))
+            got, _ = dec.forward_token(int(t), want_logits=i >= 500)
+            if i >= 500:
+                worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
+        assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
+    finally:
+        dec.close()
+
+
 def test_greedy_tokens_match_oracle(gpu_rt, orc):
     dec, ref = _build(gpu_rt, orc, SMALL, 3)
     try:
