@@ -58,6 +58,7 @@ struct GemmArgs {
   float g0, g1;
   uint32_t M, ldx, d_out, nblocks, tail_w;
   uint32_t n_bands, S, bps;  // split count, blocks per split
+  uint32_t ct_shift;         // log2 of the column tiles the wavefronts spread over (0..4)
 };
 
 // The batched kernel keeps the Golay words and the support-arrangement table in L2:
@@ -94,7 +95,10 @@ __device__ __forceinline__ void store_y<__half>(void* y, size_t at, float v) {
   reinterpret_cast<__half*>(y)[at] = __float2half_rn(v);
 }
 
-// RT = 32-row tiles per wavefront: 1 for M <= 256 (grid 2 x 8), 2 for M <= 512 (grid 1 x 16).
+// Wavefront grid of the MFMA phase: every wavefront owns both 32-row tiles of the band
+// and one 32-column tile of the batch.  A batch of fewer than sixteen column tiles
+// leaves wavefronts over; they take the same tiles on interleaved K-steps (kpart) and
+// the unit's epilogue adds their sums in kpart order.
 #ifdef LLVQ_PHASE_TIMING
 #define LLVQ_GSTAMP(k)                                                                                  \
   do {                                                                                                  \
@@ -104,7 +108,7 @@ __device__ __forceinline__ void store_y<__half>(void* y, size_t at, float v) {
 #define LLVQ_GSTAMP(k) do {} while (0)
 #endif
 
-template <int RT, typename OutT>
+template <typename OutT>
 __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
   const DecodeTables T = stage_tables<false>(smem, a.tables);
@@ -117,10 +121,16 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   const uint32_t nb = a.nblocks;
   const uint32_t n_units = a.n_bands * a.S;
 
-  // wavefront grid of the MFMA phase: first 32-row tile and 32-column tile of this wavefront
-  const uint32_t rt0 = RT == 2 ? 0u : (wave & 1u), ctile = RT == 2 ? wave : (wave >> 1);
+  // 32-row and 32-column tiles per wavefront.  Two column tiles would halve the operand
+  // traffic per MFMA, but 64 accumulator registers beside the decode phases' state spill
+  // (measured: 124 instead of 196 TFLOP/s at M = 512).
+  constexpr int RT = 2, CT = 1;
+  const uint32_t ctn = 1u << a.ct_shift, kparts = 16u >> a.ct_shift;
+  const uint32_t ctile = wave & (ctn - 1u), kpart = wave >> a.ct_shift;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
-  const uint32_t my_m = ctile * 32u + l32;  // the activation row this lane feeds and receives
+  uint32_t my_m[CT];  // the activation rows this lane feeds and receives
+#pragma unroll
+  for (int c = 0; c < CT; ++c) my_m[c] = (ctile * CT + c) * 32u + l32;
 
   // code bytes of (unit, slice) -> one register per lane
   auto prefetch = [&](uint32_t r0, uint32_t rows, uint32_t k0, uint32_t kb, uint4& pre) {
@@ -140,11 +150,13 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     const uint32_t band = unit / a.S, split = unit - band * a.S;
     const uint32_t r0 = band * kGemmRows, rows = min((uint32_t)kGemmRows, a.d_out - r0);
     const uint32_t kb_lo = min(nb, split * a.bps), kb_hi = min(nb, kb_lo + a.bps);
-    float16_t acc[RT];
+    float16_t acc[RT][CT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int j = 0; j < 16; ++j) acc[rt][j] = 0.f;
+      for (int c = 0; c < CT; ++c)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[rt][c][j] = 0.f;
 
     uint4 pre = make_uint4(0, 0, 0, 0);
     // Units walk their slices from different starting points (a fixed function of
@@ -239,36 +251,47 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       // (two MFMAs of 16): lane (l32, lh) holds columns [32 p + 16 lh, +16) of its
       // row as two fragments, for W and X alike, so an activation row is read in
       // 64-byte runs.  Columns past the slice are zeroed on both sides.
-      if (ctile * 32u < a.M) {  // column tiles beyond the batch have nothing to add
+      if (ctile * CT * 32u < a.M) {  // column tiles beyond the batch have nothing to add
         const uint32_t kcols = kb * 24u, psteps = (kcols + 31u) >> 5;
-        const __half* xrow = a.x + (size_t)k0 * 24u + (size_t)min(my_m, a.M - 1u) * a.ldx + lh * 16u;
-        const bool m_ok = my_m < a.M;
-        const _Float16* arow = W + (size_t)(rt0 * 32u + l32) * kGemmWStride + lh * 16u;
-        constexpr int G = 2;  // K-steps per batch of activation loads
+        const __half* xrow[CT];
+        bool m_in[CT];
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+          xrow[c] = a.x + (size_t)k0 * 24u + (size_t)min(my_m[c], a.M - 1u) * a.ldx + lh * 16u;
+          m_in[c] = my_m[c] < a.M;
+        }
+        const _Float16* arow = W + (size_t)l32 * kGemmWStride + lh * 16u;
+        constexpr int G = CT == 1 ? 2 : 1;  // K-steps per batch of activation loads
         const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-        half8_t cur[G][2], nxt[G][2];
-        auto fetch = [&](uint32_t p0, half8_t (&dst)[G][2]) {
+        half8_t cur[G][CT][2], nxt[G][CT][2];
+        auto fetch = [&](uint32_t i0, half8_t (&dst)[G][CT][2]) {  // owned K-steps i0 .. i0+G-1
 #pragma unroll
           for (int g = 0; g < G; ++g)
 #pragma unroll
-            for (int f = 0; f < 2; ++f) {
-              const uint32_t kc = (p0 + g) * 32u + lh * 16u + f * 8u;
-              dst[g][f] = (m_ok && kc < kcols) ? *reinterpret_cast<const half8_t*>(xrow + (p0 + g) * 32u + f * 8u) : zero;
-            }
-        };
-        fetch(0, cur);
-        for (uint32_t p0 = 0; p0 < psteps; p0 += G) {
-          if (p0 + G < psteps) fetch(p0 + G, nxt);
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            if (p0 + g < psteps) {
+            for (int c = 0; c < CT; ++c)
 #pragma unroll
               for (int f = 0; f < 2; ++f) {
-                const bool kin = (p0 + g) * 32u + lh * 16u + f * 8u < kcols;
+                const uint32_t p = kpart + (i0 + g) * kparts, kc = p * 32u + lh * 16u + f * 8u;
+                dst[g][c][f] = (m_in[c] && kc < kcols) ? *reinterpret_cast<const half8_t*>(xrow[c] + p * 32u + f * 8u) : zero;
+              }
+        };
+        const uint32_t n_own = kpart < psteps ? (psteps - kpart + kparts - 1u) / kparts : 0u;
+        fetch(0, cur);
+        for (uint32_t i0 = 0; i0 < n_own; i0 += G) {
+          if (i0 + G < n_own) fetch(i0 + G, nxt);
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            if (i0 + g < n_own) {
+              const uint32_t p = kpart + (i0 + g) * kparts;
+#pragma unroll
+              for (int f = 0; f < 2; ++f) {
+                const bool kin = p * 32u + lh * 16u + f * 8u < kcols;
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                  const half8_t av = kin ? *reinterpret_cast<const half8_t*>(arow + (size_t)rt * 32 * kGemmWStride + (p0 + g) * 32u + f * 8u) : zero;
-                  acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, cur[g][f], acc[rt], 0, 0, 0);
+                  const half8_t av = kin ? *reinterpret_cast<const half8_t*>(arow + (size_t)rt * 32 * kGemmWStride + p * 32u + f * 8u) : zero;
+#pragma unroll
+                  for (int c = 0; c < CT; ++c)
+                    acc[rt][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, cur[g][c][f], acc[rt][c], 0, 0, 0);
                 }
               }
             }
@@ -276,7 +299,9 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 #pragma unroll
           for (int g = 0; g < G; ++g)
 #pragma unroll
-            for (int f = 0; f < 2; ++f) cur[g][f] = nxt[g][f];
+            for (int c = 0; c < CT; ++c)
+#pragma unroll
+              for (int f = 0; f < 2; ++f) cur[g][c][f] = nxt[g][c][f];
         }
       }
       LLVQ_GSTAMP(4);
@@ -286,7 +311,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     }
 
     // ---- epilogue ----
-    // acc[rt][j] belongs to weight row r0 + (rt0 + rt)*32 + 8 (j/4) + 4 lh + j%4 and activation row my_m.
+    // acc[rt][c][j] belongs to weight row r0 + rt*32 + 8 (j/4) + 4 lh + j%4 and activation row my_m[c].
     // The tail columns (f32 weights, kept out of the binary16 contraction) are
     // staged in the W area: tl[row][t] as f32 and xt[m][t] as binary16.
     const uint32_t tw = a.tail_w;
@@ -302,64 +327,97 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         xt[o] = xtail[(size_t)m * a.ldx + t];
       }
     };
-    const bool m_ok = my_m < a.M;
     const bool vec_ok = (a.d_out & 3u) == 0;  // four consecutive rows of one activation row store as one vector
-    if (a.S > 1) {
-      if (m_ok) {
-        float* dst = a.ws + ((size_t)split * a.M + my_m) * a.d_out + r0;
+    __syncthreads();  // every wavefront is past its last read of W
+    if (kparts > 1) {
+      // sums of the K-step shares -> the kpart 0 wavefront of each column group, one
+      // 32 x 32 tile at a time through the W area: red[kpart - 1][ctile][j4][lane]
+      float4* red = reinterpret_cast<float4*>(W);
+      static_assert((size_t)15 * 4 * 64 * 16 <= (size_t)kGemmRows * kGemmWStride * 2, "K-step shares fit the W area");
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-          for (int j4 = 0; j4 < 4; ++j4) {
-            const uint32_t row = (rt0 + rt) * 32u + 8u * j4 + 4u * lh;
-            if (vec_ok && row + 3 < rows) {
-              *reinterpret_cast<float4*>(dst + row) =
-                  make_float4(acc[rt][4 * j4], acc[rt][4 * j4 + 1], acc[rt][4 * j4 + 2], acc[rt][4 * j4 + 3]);
-            } else {
+        for (int c = 0; c < CT; ++c) {
+          if (kpart > 0) {
 #pragma unroll
-              for (int i = 0; i < 4; ++i)
-                if (row + i < rows) dst[row + i] = acc[rt][4 * j4 + i];
-            }
+            for (int j4 = 0; j4 < 4; ++j4)
+              red[(((kpart - 1u) * ctn + ctile) * 4u + j4) * 64u + lane] =
+                  make_float4(acc[rt][c][4 * j4], acc[rt][c][4 * j4 + 1], acc[rt][c][4 * j4 + 2], acc[rt][c][4 * j4 + 3]);
           }
-      }
-      // gemm_reduce_kernel finishes these rows
-    } else {
-      __syncthreads();  // W is about to hold the tail staging
+          __syncthreads();
+          if (kpart == 0) {
+            for (uint32_t kp = 1; kp < kparts; ++kp)
+#pragma unroll
+              for (int j4 = 0; j4 < 4; ++j4) {
+                const float4 v = red[(((kp - 1u) * ctn + ctile) * 4u + j4) * 64u + lane];
+                acc[rt][c][4 * j4] += v.x;
+                acc[rt][c][4 * j4 + 1] += v.y;
+                acc[rt][c][4 * j4 + 2] += v.z;
+                acc[rt][c][4 * j4 + 3] += v.w;
+              }
+          }
+          __syncthreads();
+        }
     }
-    if (a.S == 1) {
+    if (a.S > 1) {
+      // gemm_reduce_kernel finishes these rows
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        if (kpart == 0 && my_m[c] < a.M) {
+          float* dst = a.ws + ((size_t)split * a.M + my_m[c]) * a.d_out + r0;
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int j4 = 0; j4 < 4; ++j4) {
+              const uint32_t row = rt * 32u + 8u * j4 + 4u * lh;
+              if (vec_ok && row + 3 < rows) {
+                *reinterpret_cast<float4*>(dst + row) =
+                    make_float4(acc[rt][c][4 * j4], acc[rt][c][4 * j4 + 1], acc[rt][c][4 * j4 + 2], acc[rt][c][4 * j4 + 3]);
+              } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                  if (row + i < rows) dst[row + i] = acc[rt][c][4 * j4 + i];
+              }
+            }
+        }
+      }
+    } else {
       if (tw) stage_tail();
       __syncthreads();
-      if (m_ok) {
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+      for (int c = 0; c < CT; ++c) {
+        if (kpart == 0 && my_m[c] < a.M) {
 #pragma unroll
-          for (int j4 = 0; j4 < 4; ++j4) {
-            const uint32_t row = (rt0 + rt) * 32u + 8u * j4 + 4u * lh;
-            float v[4];
+          for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const uint32_t r = min(row + i, rows - 1u);
-              float ts = 0.f;
-              for (uint32_t t = 0; t < tw; ++t) ts = fmaf(tl[r * tw + t], __half2float(xt[my_m * tw + t]), ts);
-              v[i] = fmaf(acc[rt][4 * j4 + i], a.rscale[r0 + r], ts);
-            }
-            const size_t at = (size_t)my_m * a.d_out + r0 + row;
-            if (vec_ok && row + 3 < rows) {
-              if constexpr (sizeof(OutT) == 4) {
-                *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
-              } else {
-                const __half2 lo = __float22half2_rn(make_float2(v[0], v[1])), hi = __float22half2_rn(make_float2(v[2], v[3]));
-                uint2 pk;
-                pk.x = *reinterpret_cast<const uint32_t*>(&lo);
-                pk.y = *reinterpret_cast<const uint32_t*>(&hi);
-                *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(a.y) + at) = pk;
+            for (int j4 = 0; j4 < 4; ++j4) {
+              const uint32_t row = rt * 32u + 8u * j4 + 4u * lh;
+              float v[4];
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const uint32_t r = min(row + i, rows - 1u);
+                float ts = 0.f;
+                for (uint32_t t = 0; t < tw; ++t) ts = fmaf(tl[r * tw + t], __half2float(xt[my_m[c] * tw + t]), ts);
+                v[i] = fmaf(acc[rt][c][4 * j4 + i], a.rscale[r0 + r], ts);
               }
-            } else {
+              const size_t at = (size_t)my_m[c] * a.d_out + r0 + row;
+              if (vec_ok && row + 3 < rows) {
+                if constexpr (sizeof(OutT) == 4) {
+                  *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                  const __half2 lo = __float22half2_rn(make_float2(v[0], v[1])), hi = __float22half2_rn(make_float2(v[2], v[3]));
+                  uint2 pk;
+                  pk.x = *reinterpret_cast<const uint32_t*>(&lo);
+                  pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+                  *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(a.y) + at) = pk;
+                }
+              } else {
 #pragma unroll
-              for (int i = 0; i < 4; ++i)
-                if (row + i < rows) store_y<OutT>(a.y, at + i, v[i]);
+                for (int i = 0; i < 4; ++i)
+                  if (row + i < rows) store_y<OutT>(a.y, at + i, v[i]);
+              }
             }
-          }
+        }
       }
     }
 #ifdef LLVQ_PHASE_TIMING

@@ -795,10 +795,8 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half, kSmallTileBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<2, float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<1, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<2, __half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   *out = rt;
   return LLVQ_OK;
 }
@@ -1256,11 +1254,15 @@ static void pick_gemm_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint
                             uint32_t* bps_out) {
   double best = 1e30;
   uint32_t best_s = 1, best_bps = nblocks ? nblocks : 1;
+  // MFMA phase of a full slice: 24 K-steps shared by the wavefronts of a column tile
+  uint32_t col_tiles = 1;
+  while (col_tiles * 32u < M && col_tiles < 16) col_tiles *= 2;
+  const double mfma_us = 0.5 + 0.75 * ((24 * col_tiles + 15) / 16);
   for (uint32_t S = 1; S <= 64 && S <= (nblocks ? nblocks : 1); ++S) {
     const uint32_t bps = (nblocks + S - 1) / S;
     if ((uint64_t)(S - 1) * bps >= nblocks && S > 1) continue;  // an empty last split
     const uint32_t slices = (bps + kGemmKb - 1) / kGemmKb;
-    const double unit_us = 2.0 + slices * (5.0 + 0.018 * M) + 64.0 * bps * 0.0042 + 0.015 * M + (S > 1 ? 0.002 * M : 0.0);
+    const double unit_us = 2.0 + slices * (4.5 + mfma_us) + 64.0 * bps * 0.0042 + 0.015 * M + (S > 1 ? 0.002 * M : 0.0);
     const uint64_t units = (uint64_t)n_bands * S;
     // a split launch pays a second, chip-wide pass over S partial sums per output
     const double reduce_us = S > 1 ? 6.0 + (double)S * M * 64.0 * n_bands * 4.0 / 2.0e6 : 0.0;
@@ -1304,13 +1306,11 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
   const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
   const size_t lds = gemm_lds_bytes();
   const bool f32 = y_dtype == LLVQ_F32;
-  if (M <= 256) {
-    if (f32) hipLaunchKernelGGL((gemm_tiles_kernel<1, float>), grid, wg, lds, rt->stream, a);
-    else hipLaunchKernelGGL((gemm_tiles_kernel<1, __half>), grid, wg, lds, rt->stream, a);
-  } else {
-    if (f32) hipLaunchKernelGGL((gemm_tiles_kernel<2, float>), grid, wg, lds, rt->stream, a);
-    else hipLaunchKernelGGL((gemm_tiles_kernel<2, __half>), grid, wg, lds, rt->stream, a);
-  }
+  // sixteen wavefronts over the batch's 32-column tiles, the count rounded up to a power of two
+  a.ct_shift = 0;
+  while ((32u << a.ct_shift) < M && a.ct_shift < 4) ++a.ct_shift;
+  if (f32) hipLaunchKernelGGL(gemm_tiles_kernel<float>, grid, wg, lds, rt->stream, a);
+  else hipLaunchKernelGGL(gemm_tiles_kernel<__half>, grid, wg, lds, rt->stream, a);
   HIP_TRY(hipGetLastError());
   if (a.S > 1) {
     GemmReduceArgs r{};
