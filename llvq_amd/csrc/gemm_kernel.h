@@ -54,7 +54,7 @@ struct GemmArgs {
   const float* rscale;
   const float* tail;
   void* y;                // [M, d_out]
-  float* ws;              // [S, M, d_out] partial sums when S > 1
+  float* ws;              // [S, n_bands, M, 64] partial sums when S > 1
   float g0, g1;
   uint32_t M, ldx, d_out, nblocks, tail_w;
   uint32_t n_bands, S, bps;  // split count, blocks per split
@@ -360,25 +360,19 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         }
     }
     if (a.S > 1) {
-      // gemm_reduce_kernel finishes these rows
+      // gemm_reduce_kernel finishes these rows.  The workspace is [split][band][m][64]:
+      // a unit's partial sums are one contiguous piece, and rows past the end of the
+      // last band are written but never read.
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
         if (kpart == 0 && my_m[c] < a.M) {
-          float* dst = a.ws + ((size_t)split * a.M + my_m[c]) * a.d_out + r0;
+          float* dst = a.ws + (((size_t)split * a.n_bands + band) * a.M + my_m[c]) * kGemmRows;
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-            for (int j4 = 0; j4 < 4; ++j4) {
-              const uint32_t row = rt * 32u + 8u * j4 + 4u * lh;
-              if (vec_ok && row + 3 < rows) {
-                *reinterpret_cast<float4*>(dst + row) =
-                    make_float4(acc[rt][c][4 * j4], acc[rt][c][4 * j4 + 1], acc[rt][c][4 * j4 + 2], acc[rt][c][4 * j4 + 3]);
-              } else {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                  if (row + i < rows) dst[row + i] = acc[rt][c][4 * j4 + i];
-              }
-            }
+            for (int j4 = 0; j4 < 4; ++j4)
+              *reinterpret_cast<float4*>(dst + rt * 32u + 8u * j4 + 4u * lh) =
+                  make_float4(acc[rt][c][4 * j4], acc[rt][c][4 * j4 + 1], acc[rt][c][4 * j4 + 2], acc[rt][c][4 * j4 + 3]);
         }
       }
     } else {
@@ -428,73 +422,81 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 }
 
 // Second pass of a split launch: y[m][r] = (sum over splits, in split order, of the
-// partial sums) * rscale[r] + tail[r] . x_tail[m].  One lane per four consecutive
-// rows of one activation row; the partial sums are read with all their loads in
-// flight (eight splits at a time).
+// partial sums) * rscale[r] + tail[r] . x_tail[m].  One workgroup per (band, 16
+// activation rows), one lane per four consecutive weight rows of one activation row;
+// the band's tail weights and the activation tails are staged in LDS once, and the
+// partial sums are read with all their loads in flight (eight splits at a time).
 struct GemmReduceArgs {
-  const float* ws;  // [S, M, d_out]
+  const float* ws;  // [S, n_bands, M, 64]
   const __half* x;  // [M, ldx]
   const float* rscale;
   const float* tail;
   void* y;
-  uint32_t M, ldx, d_out, nblocks, tail_w, S;
+  uint32_t M, ldx, d_out, nblocks, tail_w, S, n_bands;
 };
+
+constexpr int kReduceRowsM = 16;  // activation rows per workgroup
 
 template <typename OutT>
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
-  const uint32_t quads = (a.d_out + 3u) >> 2;
-  const size_t items = (size_t)quads * a.M, sstride = (size_t)a.M * a.d_out;
-  const bool vec_ok = (a.d_out & 3u) == 0;
-  for (size_t it = (size_t)blockIdx.x * blockDim.x + threadIdx.x; it < items; it += (size_t)gridDim.x * blockDim.x) {
-    const uint32_t m = (uint32_t)(it / quads), row = (uint32_t)(it - (size_t)m * quads) * 4u;
-    const float* src = a.ws + (size_t)m * a.d_out + row;
-    float sum[4] = {0.f, 0.f, 0.f, 0.f};
-    if (vec_ok) {
-      for (uint32_t s0 = 0; s0 < a.S; s0 += 8) {
-        float4 p[8];
+  __shared__ float tl[kGemmRows * kDim];            // [row][pitch], pitch odd
+  __shared__ float xt[kReduceRowsM * (kDim - 1)];   // [m][tail_w]
+  const uint32_t mchunks = (a.M + kReduceRowsM - 1) / kReduceRowsM;
+  const uint32_t band = blockIdx.x / mchunks, mc = blockIdx.x - band * mchunks;
+  const uint32_t r0 = band * kGemmRows, rows = min((uint32_t)kGemmRows, a.d_out - r0);
+  const uint32_t tw = a.tail_w, pitch = tw | 1u;
+  const uint32_t tid = threadIdx.x, quad = tid & 15u, ml = tid >> 4;
+  const uint32_t m = mc * kReduceRowsM + ml, row = quad * 4u;
+  for (uint32_t o = tid; o < rows * tw; o += 256) {
+    const uint32_t r = o / tw, t = o - r * tw;
+    tl[r * pitch + t] = a.tail[(size_t)r0 * tw + o];
+  }
+  for (uint32_t o = tid; o < kReduceRowsM * tw; o += 256) {
+    const uint32_t mm = mc * kReduceRowsM + o / tw, t = o % tw;
+    xt[o] = mm < a.M ? __half2float(a.x[(size_t)mm * a.ldx + (size_t)a.nblocks * 24u + t]) : 0.f;
+  }
+  __syncthreads();
+  if (m >= a.M || row >= rows) return;
+  const size_t sstride = (size_t)a.n_bands * a.M * kGemmRows;
+  const float* src = a.ws + ((size_t)band * a.M + m) * kGemmRows + row;
+  float sum[4] = {0.f, 0.f, 0.f, 0.f};
+  for (uint32_t s0 = 0; s0 < a.S; s0 += 8) {
+    float4 p[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          p[u] = s0 + u < a.S ? *reinterpret_cast<const float4*>(src + (size_t)(s0 + u) * sstride) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int u = 0; u < 8; ++u)
+      p[u] = s0 + u < a.S ? *reinterpret_cast<const float4*>(src + (size_t)(s0 + u) * sstride) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          if (s0 + u < a.S) {
-            sum[0] += p[u].x;
-            sum[1] += p[u].y;
-            sum[2] += p[u].z;
-            sum[3] += p[u].w;
-          }
+    for (int u = 0; u < 8; ++u)
+      if (s0 + u < a.S) {
+        sum[0] += p[u].x;
+        sum[1] += p[u].y;
+        sum[2] += p[u].z;
+        sum[3] += p[u].w;
       }
+  }
+  float v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t r = min(row + i, rows - 1u);
+    float ts = 0.f;
+    for (uint32_t t = 0; t < tw; ++t) ts = fmaf(tl[r * pitch + t], xt[ml * tw + t], ts);
+    v[i] = fmaf(sum[i], a.rscale[r0 + r], ts);
+  }
+  const size_t at = (size_t)m * a.d_out + r0 + row;
+  if ((a.d_out & 3u) == 0 && row + 3 < rows) {
+    if constexpr (sizeof(OutT) == 4) {
+      *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
     } else {
-      for (uint32_t s = 0; s < a.S; ++s)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (row + i < a.d_out) sum[i] += src[(size_t)s * sstride + i];
+      const __half2 lo = __float22half2_rn(make_float2(v[0], v[1])), hi = __float22half2_rn(make_float2(v[2], v[3]));
+      uint2 pk;
+      pk.x = *reinterpret_cast<const uint32_t*>(&lo);
+      pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+      *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(a.y) + at) = pk;
     }
-    const __half* xt = a.x + (size_t)m * a.ldx + (size_t)a.nblocks * 24u;
-    float v[4];
+  } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t r = min(row + i, a.d_out - 1u);
-      float ts = 0.f;
-      for (uint32_t t = 0; t < a.tail_w; ++t) ts = fmaf(a.tail[(size_t)r * a.tail_w + t], __half2float(xt[t]), ts);
-      v[i] = fmaf(sum[i], a.rscale[r], ts);
-    }
-    const size_t at = (size_t)m * a.d_out + row;
-    if (vec_ok) {
-      if constexpr (sizeof(OutT) == 4) {
-        *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
-      } else {
-        const __half2 lo = __float22half2_rn(make_float2(v[0], v[1])), hi = __float22half2_rn(make_float2(v[2], v[3]));
-        uint2 pk;
-        pk.x = *reinterpret_cast<const uint32_t*>(&lo);
-        pk.y = *reinterpret_cast<const uint32_t*>(&hi);
-        *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(a.y) + at) = pk;
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (row + i < a.d_out) store_y<OutT>(a.y, at + i, v[i]);
-    }
+    for (int i = 0; i < 4; ++i)
+      if (row + i < rows) store_y<OutT>(a.y, at + i, v[i]);
   }
 }
 

@@ -169,8 +169,9 @@ struct GroupArgs {
 };
 
 constexpr int kSmallTileBlocks = 2048;  // tile of the variant for rows too wide for the full tile's LDS
-__host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks, uint32_t tile = kTileBlocks) {
-  return kLdsImageBytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + ((size_t)tile * 6 + 32) +
+__host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks, uint32_t tile = kTileBlocks,
+                                                    size_t image_bytes = kLdsImageBytes) {
+  return image_bytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + ((size_t)tile * 6 + 32) +
          (size_t)tile * 4 * 2 + kGenericSlots * 4 + 16;
 }
 
@@ -383,16 +384,18 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
   }
 }
 
-template <typename OutT, int TILE = LLVQ_TILE_BLOCKS>
+// LEAN: the Golay words and the support-arrangement table stay in L2, which leaves
+// room for the full tile beside the activation planes of a very wide row.
+template <typename OutT, int TILE = LLVQ_TILE_BLOCKS, bool LEAN = false>
 __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   // the tile capacity of this instantiation (these shadow the namespace-level defaults)
   constexpr int kTileBlocks = TILE;
   constexpr int kP1Blocks = TILE / kWgThreads;
   constexpr int kRawBytes = TILE * 6 + 32;
   extern __shared__ __align__(16) uint8_t smem[];
-  const DecodeTables T = stage_tables(smem, a.tables);
+  const DecodeTables T = stage_tables<!LEAN && (LLVQ_LDS_GOLAY != 0)>(smem, a.tables);
   const uint32_t nb = a.nblocks;
-  uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + kLdsImageBytes);
+  uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + (LEAN ? kLdsImageBytesLean : kLdsImageBytes));
   float* xscale = reinterpret_cast<float*>(xplanes + (size_t)nb * kPlaneDwords);
   float* xtail = xscale + nb;
   uint8_t* raw = reinterpret_cast<uint8_t*>(xtail + 32);
@@ -793,6 +796,8 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float, kSmallTileBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half, kSmallTileBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float, kTileBlocks, true>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half, kTileBlocks, true>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
@@ -1077,10 +1082,24 @@ static uint32_t pick_rows_per_tile(const llvq_mat* const* mats, int n, uint32_t 
 
 // Whether a launch over rows of this width can stage a derived activation where
 // its tile's code bytes go.
+struct GemvShape {
+  uint32_t tile;
+  bool lean;
+  size_t lds;
+};
+
+// The kernel variant for rows of nblocks blocks: the full tile with the whole table
+// image in LDS where that fits, else the full tile with the lean image, else the half tile.
+static GemvShape pick_gemv_shape(uint32_t nblocks) {
+  GemvShape s{(uint32_t)kTileBlocks, false, gemv_lds_bytes(nblocks, kTileBlocks)};
+  if (s.lds <= 160 * 1024) return s;
+  s = GemvShape{(uint32_t)kTileBlocks, true, gemv_lds_bytes(nblocks, kTileBlocks, kLdsImageBytesLean)};
+  if (s.lds <= 160 * 1024) return s;
+  return GemvShape{(uint32_t)kSmallTileBlocks, false, gemv_lds_bytes(nblocks, kSmallTileBlocks)};
+}
+
 static bool prologue_fits(const llvq_mat* m0) {
-  uint32_t tile = kTileBlocks;
-  if (gemv_lds_bytes(m0->nblocks, tile) > 160 * 1024) tile = kSmallTileBlocks;
-  return (size_t)m0->d_in * 2 <= (size_t)tile * 6 + 32;
+  return (size_t)m0->d_in * 2 <= (size_t)pick_gemv_shape(m0->nblocks).tile * 6 + 32;
 }
 
 struct Prologue {
@@ -1095,10 +1114,9 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
                         int y_dtype, const Prologue* pro = nullptr, const float* x_f32 = nullptr) {
   const llvq_mat* m0 = mats[0];
   if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv: unknown output dtype");
-  // the full tile where the activation planes leave room for it, else the half tile
-  uint32_t tile = kTileBlocks;
-  if (gemv_lds_bytes(m0->nblocks, tile) > 160 * 1024) tile = kSmallTileBlocks;
-  const size_t lds = gemv_lds_bytes(m0->nblocks, tile);
+  const GemvShape shape = pick_gemv_shape(m0->nblocks);
+  const uint32_t tile = shape.tile;
+  const size_t lds = shape.lds;
   if (lds > 160 * 1024 || m0->nblocks > tile)
     return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": d_in " + std::to_string(m0->d_in) + " does not fit the LDS activation tile");
   // as many workgroups as fit a CU's 160 KB of LDS side by side
@@ -1131,7 +1149,12 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   }
   a.n_tiles = tiles;
   const uint32_t grid = tiles < grid_cap ? tiles : grid_cap;
-  if (tile == (uint32_t)kTileBlocks) {
+  if (shape.lean) {
+    if (y_dtype == LLVQ_F32)
+      hipLaunchKernelGGL((gemv_tiles_kernel<float, kTileBlocks, true>), dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
+    else
+      hipLaunchKernelGGL((gemv_tiles_kernel<__half, kTileBlocks, true>), dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
+  } else if (tile == (uint32_t)kTileBlocks) {
     if (y_dtype == LLVQ_F32)
       hipLaunchKernelGGL(gemv_tiles_kernel<float>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
     else
@@ -1292,7 +1315,7 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
   a.n_bands = (m->d_out + kGemmRows - 1) / kGemmRows;
   pick_gemm_split(a.n_bands, m->nblocks, M, grid_cap, &a.S, &a.bps);
   if (a.S > 1) {
-    const size_t need = (size_t)a.S * M * m->d_out * sizeof(float);
+    const size_t need = (size_t)a.S * a.n_bands * M * kGemmRows * sizeof(float);
     if (need > rt->gemm_ws_bytes) {
       (void)hipFree(rt->gemm_ws);  // waits for launches that still use it
       rt->gemm_ws = nullptr;
@@ -1325,12 +1348,10 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
     r.nblocks = a.nblocks;
     r.tail_w = a.tail_w;
     r.S = a.S;
-    const size_t items = (size_t)((m->d_out + 3) / 4) * M;
-    size_t rgrid = (items + 255) / 256;
-    const size_t rcap = (size_t)grid_cap * 8;
-    if (rgrid > rcap) rgrid = rcap;
-    if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3((uint32_t)rgrid), dim3(256), 0, rt->stream, r);
-    else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3((uint32_t)rgrid), dim3(256), 0, rt->stream, r);
+    r.n_bands = a.n_bands;
+    const uint32_t rgrid = a.n_bands * ((M + kReduceRowsM - 1) / kReduceRowsM);
+    if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3(rgrid), dim3(256), 0, rt->stream, r);
+    else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3(rgrid), dim3(256), 0, rt->stream, r);
     HIP_TRY(hipGetLastError());
   }
   return LLVQ_OK;
