@@ -48,9 +48,11 @@ def build_layers(n_layers, seed):
     return layers
 
 
-def cpu_baseline(layer_mats, acts, threads):
+def cpu_baseline(layer_mats, acts, threads, y_device=None):
     """CPU oracle on one layer (4 185 600 blocks): 2 discarded + 5 kept rounds, median
-    (protocol of llvq-cuda/src/bin/matvec.rs:64-65)."""
+    (protocol of llvq-cuda/src/bin/matvec.rs:64-65).  `y_device` holds what the kernels gave for the
+    same seven projections before anything was timed; the oracle's outputs check them
+    (llvq-cuda/src/bin/matvec.rs:114-120: no figure without a correct result)."""
     from oracle import pyoracle as orc
 
     total_bytes = sum(m.encoded_bytes() for m in layer_mats)
@@ -58,13 +60,20 @@ def cpu_baseline(layer_mats, acts, threads):
     times = []
     for rnd in range(7):
         t0 = time.perf_counter()
+        ys = []
         for m in layer_mats:
             x = acts[m.d_in]
-            orc.cpu_gemv(m.codes, m.d_out, m.d_in, m.centroids, m.row_scales, m.tail, x.view(np.uint16), threads)
+            ys.append(orc.cpu_gemv(m.codes, m.d_out, m.d_in, m.centroids, m.row_scales, m.tail, x.view(np.uint16), threads))
         dt = time.perf_counter() - t0
         if rnd >= 2:
             times.append(dt)
     med = statistics.median(times)
+    worst = None
+    if y_device is not None:
+        # binary16 outputs: half an ulp is 4.9e-4 of the value; the bar is 1e-3 of the largest output
+        worst = max(float(np.max(np.abs(yd.astype(np.float64) - yo)) / np.max(np.abs(yo))) for yd, yo in zip(y_device, ys))
+        if not worst <= 1e-3:
+            raise SystemExit(f"[bench] device outputs differ from the CPU oracle: {worst:.3e} of the largest output")
     # decode-only cost per block on one core, as llvq-bench's decfull measures it
     m = layer_mats[1]
     nb = min(m.d_out * m.nblocks, 200_000)
@@ -80,6 +89,7 @@ def cpu_baseline(layer_mats, acts, threads):
                   f"median of 5 rounds after 2 discarded [{min(times) * 1e3:.1f}-{max(times) * 1e3:.1f} ms]",
         "ms_per_layer": round(med * 1e3, 3),
         "decode_only_ns_per_block_per_core": round(ns_per_block, 1),
+        "device_vs_oracle_max_err_over_max_abs_y": worst,
     }
 
 
@@ -330,12 +340,19 @@ def main():
     n_launch = sum(len(p) for p in projs)
 
     # one pre-bound launch per activation site: q/k/v, o, gate/up, down
-    launches = []
+    launches, outputs = [], []
     for lp in projs:
         q, k, v, o, gate, up, down = lp
         for group, d in (([q, k, v], 2560), ([o], 4096), ([gate, up], 2560), ([down], 9728)):
-            launches.append(rt.plan_group(group, acts[d])[0])
+            launch, ys = rt.plan_group(group, acts[d])
+            launches.append(launch)
+            outputs.append(ys)
     n_kernels = len(launches)
+    # layer 0's results, taken before anything is timed, for the check against the CPU oracle
+    for launch in launches[:4]:
+        launch()
+    torch.cuda.synchronize()
+    y_layer0 = [y.float().cpu().numpy() for ys in outputs[:4] for y in ys]
 
     def step():
         for launch in launches:
@@ -421,7 +438,7 @@ def main():
         torch.cuda.synchronize()
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
-        out["cpu_baseline"] = cpu_baseline(layers[0], acts_np, threads)
+        out["cpu_baseline"] = cpu_baseline(layers[0], acts_np, threads, y_layer0)
     rt.close()
     print(json.dumps(out), flush=True)
 
