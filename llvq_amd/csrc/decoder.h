@@ -110,47 +110,21 @@ __device__ __forceinline__ float kv_dequant(uint32_t q, float s, float b) {
   return __half2float(__float2half_rn(__fadd_rn(__fmul_rn((float)q, s), b)));
 }
 
-// One wavefront per head: per-head RMSNorm of q and k (model.rs:800-808), RoPE at
+// One wavefront: per-head RMSNorm of a q or k head (model.rs:800-808), then RoPE at
 // the absolute position in the rotate-half convention (candle_nn::rotary_emb::rope:
 // out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i] sin + x[i + d/2] cos, with
-// the binary16 cos/sin tables of Rotary::new, model.rs:163-179), then k and v of
-// this position are appended to the cache (binary16, or int8 codes when q8 is set).
-// Heads: [0, n_heads) are q, the next n_kv are k, the last n_kv are v.
-// head_dim <= 256, a multiple of 8 (of 64 for the int8 cache).
-__global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restrict__ q, const __half* __restrict__ k,
-                                                                 const __half* __restrict__ v,
-                                                                 const __half* __restrict__ qn, const __half* __restrict__ kn,
-                                                                 const __half* __restrict__ cos_t, const __half* __restrict__ sin_t,
-                                                                 __half* __restrict__ kcache, __half* __restrict__ vcache,
-                                                                 KvQ8 q8, uint32_t use_q8,
-                                                                 uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
-                                                                 uint32_t pos, uint32_t max_pos, float eps) {
-  const uint32_t head = blockIdx.x, lane = threadIdx.x;
-  const uint32_t half_d = head_dim >> 1, groups = head_dim / kKvGroup;
-  __shared__ float stage[256];
-  if (head >= n_heads + n_kv) {  // v: into the cache as it is
-    const uint32_t kvh = head - n_heads - n_kv;
-    const size_t row = (size_t)kvh * max_pos + pos;
-    if (!use_q8) {
-      for (uint32_t i = lane; i < head_dim; i += 64) vcache[row * head_dim + i] = v[(size_t)kvh * head_dim + i];
-    } else {
-      for (uint32_t g = 0; g < groups; ++g) {
-        const float x = __half2float(v[(size_t)kvh * head_dim + g * kKvGroup + lane]);
-        __half sh, bh;
-        const uint8_t code = kv_quantize_group(x, &sh, &bh);
-        q8.vq[row * head_dim + g * kKvGroup + lane] = code;
-        if (lane == 0) {
-          q8.vs[row * groups + g] = sh;
-          q8.vb[row * groups + g] = bh;
-        }
-      }
-    }
-    return;
-  }
-  const bool is_q = head < n_heads;
-  const uint32_t hh = is_q ? head : head - n_heads;
-  const __half* src = (is_q ? q : k) + (size_t)hh * head_dim;
-  const __half* w = is_q ? qn : kn;
+// the binary16 cos/sin tables of Rotary::new, model.rs:163-179).  Each step rounds to
+// binary16 as the reference's tensors do; the results are left, widened, in
+// stage[0, head_dim) — an LDS area of this wavefront alone.  head_dim <= 256.
+__device__ __forceinline__ void wave_lds_sync() {
+  // LDS operations of one wavefront execute in order; only the compiler must not move them
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+__device__ __forceinline__ void norm_rope_wave(const __half* __restrict__ src, const __half* __restrict__ w,
+                                               const __half* __restrict__ cos_t, const __half* __restrict__ sin_t,
+                                               uint32_t pos, uint32_t head_dim, float eps, float* stage, uint32_t lane) {
+  const uint32_t half_d = head_dim >> 1;
   float x[4];  // elements lane, lane + 64, lane + 128, lane + 192
   float ss = 0.f;
 #pragma unroll
@@ -166,7 +140,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restr
     const uint32_t i = lane + 64u * j;
     if (i < head_dim) stage[i] = __half2float(__float2half_rn(x[j] * inv * __half2float(w[i])));
   }
-  __syncthreads();
+  wave_lds_sync();
   float r1[2], r2[2];  // rotated pairs (i, i + d/2) for i = lane, lane + 64
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -179,7 +153,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restr
       r2[j] = __half2float(__float2half_rn(x1 * sn + x2 * c));
     }
   }
-  __syncthreads();
+  wave_lds_sync();
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const uint32_t i = lane + 64u * j;
@@ -188,23 +162,26 @@ __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(__half* __restr
       stage[i + half_d] = r2[j];
     }
   }
-  __syncthreads();
-  if (is_q || !use_q8) {
-    __half* dst = is_q ? q + (size_t)hh * head_dim : kcache + ((size_t)hh * max_pos + pos) * head_dim;
-    for (uint32_t i = lane; i < head_dim; i += 64) dst[i] = __float2half_rn(stage[i]);
-  } else {
-    const size_t row = (size_t)hh * max_pos + pos;
-    for (uint32_t g = 0; g < groups; ++g) {
-      __half sh, bh;
-      const uint8_t code = kv_quantize_group(stage[g * kKvGroup + lane], &sh, &bh);
-      q8.kq[row * head_dim + g * kKvGroup + lane] = code;
-      if (lane == 0) {
-        q8.ks[row * groups + g] = sh;
-        q8.kb[row * groups + g] = bh;
-      }
-    }
-  }
+  wave_lds_sync();
 }
+
+// What the attention launch is handed about the position being decoded: the raw
+// q / k / v rows the projections left, the layer's q and k norm weights and the
+// rotary tables.  The launch norms and rotates its own query heads, and the one
+// workgroup whose range ends at the new position does the same for k, appends
+// k and v to the cache and uses them from LDS.
+struct AttnNew {
+  const __half* q_raw;  // [n_heads, head_dim]
+  const __half* k_raw;  // [n_kv, head_dim]
+  const __half* v_raw;  // [n_kv, head_dim]
+  const __half* qn;     // [head_dim]
+  const __half* kn;     // [head_dim]
+  const __half* cos_t;  // [max_pos, head_dim / 2]
+  const __half* sin_t;
+  __half* kcache;       // this layer's binary16 cache (null with the int8 cache)
+  __half* vcache;
+  float eps;
+};
 
 // Attention of one query position over the cache (model.rs:812-822), split over
 // the cache: workgroup (kv head, split) takes a contiguous range of positions
@@ -220,7 +197,7 @@ constexpr int kAttnWaves = kAttnThreads / 64;
 constexpr int kAttnMaxSplits = 64;  // the cache is cut into at most this many ranges (host picks by length)
 constexpr int kAttnMaxGroup = 8;    // query heads per kv head
 template <bool Q8>
-__global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half* __restrict__ q, const __half* __restrict__ kcache,
+__global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, const __half* __restrict__ kcache,
                                                                    const __half* __restrict__ vcache, KvQ8 q8,
                                                                    __half* __restrict__ ctx,
                                                                    float* __restrict__ part, uint32_t* __restrict__ counters,
@@ -230,6 +207,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
   extern __shared__ __align__(16) float att_smem[];
   __shared__ uint32_t arrived;
   __shared__ float red[kAttnWaves][kAttnMaxGroup];
+  __shared__ float stage[kAttnWaves][256];  // one head per wavefront while it is normed and rotated
+  __shared__ float knew[256], vnew[256];    // the new position's k and v as the cache returns them
   const uint32_t kvh = blockIdx.x / n_splits, split = blockIdx.x % n_splits;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t groups = n_heads / n_kv;  // <= kAttnMaxGroup (checked by the host)
@@ -249,8 +228,62 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
   const __half* Vb = q8.vb + (size_t)kvh * max_pos * kvgroups;
   const uint32_t stride = head_dim + 2;  // floats per partial: max, sum, head_dim sums
 
-  for (uint32_t i = tid; i < groups * head_dim; i += kAttnThreads)
-    qs[i] = __half2float(q[(size_t)kvh * groups * head_dim + i]) * scale;
+  // the query heads of this kv head: norm, rotate, scale
+  const uint32_t pos = T - 1;  // the position being decoded
+  for (uint32_t g = wave; g < groups; g += kAttnWaves) {
+    norm_rope_wave(nw.q_raw + (size_t)(kvh * groups + g) * head_dim, nw.qn, nw.cos_t, nw.sin_t, pos, head_dim, nw.eps,
+                   stage[wave], lane);
+    for (uint32_t i = lane; i < head_dim; i += 64) qs[g * head_dim + i] = stage[wave][i] * scale;
+    wave_lds_sync();  // stage is rewritten by this wavefront's next head
+  }
+  // The range that ends at the new position owns its k and v: they go to the
+  // cache for later positions, and to LDS, in the form the cache gives back,
+  // for this one (nothing else reads that cache row during this launch).
+  const bool has_new = nj > 0 && j1 == T;
+  const uint32_t newj = has_new ? pos : 0xFFFFFFFFu;
+  if (has_new && wave == 0) {
+    norm_rope_wave(nw.k_raw + (size_t)kvh * head_dim, nw.kn, nw.cos_t, nw.sin_t, pos, head_dim, nw.eps, stage[0], lane);
+    const size_t row = (size_t)kvh * max_pos + pos;
+    if constexpr (Q8) {
+      for (uint32_t g = 0; g < kvgroups; ++g) {
+        __half sh, bh;
+        const uint8_t code = kv_quantize_group(stage[0][g * kKvGroup + lane], &sh, &bh);
+        q8.kq[row * head_dim + g * kKvGroup + lane] = code;
+        if (lane == 0) {
+          q8.ks[row * kvgroups + g] = sh;
+          q8.kb[row * kvgroups + g] = bh;
+        }
+        knew[g * kKvGroup + lane] = kv_dequant(code, __half2float(sh), __half2float(bh));
+      }
+    } else {
+      for (uint32_t i = lane; i < head_dim; i += 64) {
+        nw.kcache[row * head_dim + i] = __float2half_rn(stage[0][i]);
+        knew[i] = stage[0][i];
+      }
+    }
+  }
+  if (has_new && wave == 1) {
+    const size_t row = (size_t)kvh * max_pos + pos;
+    if constexpr (Q8) {
+      for (uint32_t g = 0; g < kvgroups; ++g) {
+        const float x = __half2float(nw.v_raw[(size_t)kvh * head_dim + g * kKvGroup + lane]);
+        __half sh, bh;
+        const uint8_t code = kv_quantize_group(x, &sh, &bh);
+        q8.vq[row * head_dim + g * kKvGroup + lane] = code;
+        if (lane == 0) {
+          q8.vs[row * kvgroups + g] = sh;
+          q8.vb[row * kvgroups + g] = bh;
+        }
+        vnew[g * kKvGroup + lane] = kv_dequant(code, __half2float(sh), __half2float(bh));
+      }
+    } else {
+      for (uint32_t i = lane; i < head_dim; i += 64) {
+        const __half x = nw.v_raw[(size_t)kvh * head_dim + i];
+        nw.vcache[row * head_dim + i] = x;
+        vnew[i] = __half2float(x);
+      }
+    }
+  }
   __syncthreads();
 
   // ---- scores ----
@@ -270,7 +303,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
         const uint32_t jj = pb0 + (uint32_t)b * kAttnWaves * 4u + pj, j = j0 + jj;
         kraw[b] = make_uint4(0, 0, 0, 0);
         ksc[b] = kbi[b] = 0.f;
-        if (jj < nj && i0 < head_dim) {
+        if (jj < nj && i0 < head_dim && j != newj) {
           if constexpr (Q8) {
             const uint2 kc = *reinterpret_cast<const uint2*>(Kq + (size_t)j * head_dim + i0);
             kraw[b].x = kc.x;
@@ -290,7 +323,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
         for (int g = 0; g < kAttnMaxGroup; ++g) d[g] = 0.f;
         if (jj < nj && i0 < head_dim) {
           float kf[8];
-          if constexpr (Q8) {
+          if (j0 + jj == newj) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) kf[t] = knew[i0 + t];
+          } else if constexpr (Q8) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
               kf[t] = kv_dequant((kraw[b].x >> (8 * t)) & 0xFFu, ksc[b], kbi[b]);
@@ -377,7 +413,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
           const uint32_t jj = jb + (uint32_t)b * kAttnWaves, j = j0 + jj;
           vraw[b] = 0;
           vsc[b] = vbi[b] = 0.f;
-          if (jj < nj) {
+          if (jj < nj && j != newj) {
             if constexpr (Q8) {
               vraw[b] = *reinterpret_cast<const unsigned short*>(Vq + (size_t)j * head_dim + i0);
               vsc[b] = __half2float(Vs[(size_t)j * kvgroups + i0 / kKvGroup]);
@@ -392,7 +428,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(const __half*
           const uint32_t jj = jb + (uint32_t)b * kAttnWaves;
           if (jj < nj) {
             float v0, v1;
-            if constexpr (Q8) {
+            if (j0 + jj == newj) {
+              v0 = vnew[i0];
+              v1 = vnew[i0 + 1];
+            } else if constexpr (Q8) {
               v0 = kv_dequant(vraw[b] & 0xFFu, vsc[b], vbi[b]);
               v1 = kv_dequant(vraw[b] >> 8, vsc[b], vbi[b]);
             } else {

@@ -1516,15 +1516,24 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     }
     __half* kc = d->kv_q8 ? nullptr : d->kcache + L * cache_layer;
     __half* vc = d->kv_q8 ? nullptr : d->vcache + L * cache_layer;
-    hipLaunchKernelGGL(qk_norm_rope_append_kernel, dim3(d->n_heads + 2 * d->n_kv), dim3(64), 0, st, d->q, d->k, d->v,
-                       d->qn + (size_t)L * d->head_dim, d->kn + (size_t)L * d->head_dim, d->cos_t, d->sin_t,
-                       kc, vc, lq8, d->kv_q8 ? 1u : 0u, d->n_heads, d->n_kv, d->head_dim, d->pos, d->max_pos, d->eps);
+    // q/k norm, rope and the cache append of this position ride in the attention launch
+    AttnNew nw{};
+    nw.q_raw = d->q;
+    nw.k_raw = d->k;
+    nw.v_raw = d->v;
+    nw.qn = d->qn + (size_t)L * d->head_dim;
+    nw.kn = d->kn + (size_t)L * d->head_dim;
+    nw.cos_t = d->cos_t;
+    nw.sin_t = d->sin_t;
+    nw.kcache = kc;
+    nw.vcache = vc;
+    nw.eps = d->eps;
     if (d->kv_q8)
-      hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, d->q, kc, vc, lq8,
+      hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, nw, kc, vc, lq8,
                          d->ctx, d->attn_part, d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
                          1.0f / sqrtf((float)d->head_dim), n_splits, merge_inline);
     else
-      hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, d->q, kc, vc, lq8,
+      hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, nw, kc, vc, lq8,
                          d->ctx, d->attn_part, d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
                          1.0f / sqrtf((float)d->head_dim), n_splits, merge_inline);
     if (!merge_inline)
