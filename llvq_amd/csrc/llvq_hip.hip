@@ -165,8 +165,124 @@ struct GroupArgs {
   uint32_t prologue;
   uint32_t nblocks, tail_w, n_mats, rows_per_tile, n_tiles;
   float inv_nblocks;  // 1 / nblocks, for the block -> column split
+  // the basis of these matrices, when they are stored rotated and the launch rotates its
+  // own activation (rot_m = 0: no rotation; see rotate_lds)
+  const uint32_t* rot_signbits;
+  const float* rot_small;
+  float rot_inv;
+  uint32_t rot_m, rot_k;
   MatArg m[kMaxGroup];
 };
+
+
+// x <- (S (x) I_m)(I_k (x) H_m / sqrt m) x in place on n = k m f32 values in LDS whose
+// signs D are already applied (llvq-quant/src/rotation.rs:97-105; f32 like the reference's
+// device rotation, llvq-cuda/kernels/llvq_rot.cuh).  `small` is the k x k block in device
+// memory.  Every thread of a 1024-thread workgroup calls it; the values are final after
+// the caller's next barrier.
+//  * Walsh-Hadamard levels: for m >= 512 a wavefront takes a run of 512 values, eight per
+//    lane, and does nine levels without a barrier (three in registers, six by lane
+//    exchange); the levels above 512, and every level of a narrower m, are radix-2
+//    passes over LDS (groups are contiguous, so one pass covers all of them).
+//  * the k x k block across groups, with the 1/sqrt m factor applied first, is a small
+//    dense product S (k x k) . C (k x m): a wavefront takes 32 columns of C at a time and
+//    runs it as f32 matrix-core steps of depth 2 (S padded with zeros to 32 x 32); it reads
+//    its columns whole before it writes them, and no other wavefront touches them.
+typedef float rot_acc_t __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ void rotate_lds(float* v, uint32_t n, uint32_t m, uint32_t k, float inv,
+                                           const float* __restrict__ small) {
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  const uint32_t steps = (k + 1u) >> 1;  // depth-2 steps that cover k
+  // S[l32][2 s + lh], requested before the butterflies so that the loads are back by the time they are used
+  float s_frag[kRotKMax / 2];
+#pragma unroll
+  for (uint32_t s = 0; s < kRotKMax / 2; ++s) {
+    const uint32_t t = 2u * s + lh;
+    s_frag[s] = (k > 1 && m >= 32 && l32 < k && t < k) ? small[l32 * k + t] : 0.f;
+  }
+  uint32_t len0 = 1;
+  if (m >= 512) {
+    for (uint32_t c = wave; c < (n >> 9); c += 16) {
+      float4* src = reinterpret_cast<float4*>(v + (c << 9) + lane * 8u);
+      const float4 lo = src[0], hi = src[1];
+      float r[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+      for (int l = 1; l < 8; l <<= 1)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (!(i & l)) {
+            const float u = r[i], w = r[i | l];
+            r[i] = u + w;
+            r[i | l] = u - w;
+          }
+#pragma unroll
+      for (int l = 1; l < 64; l <<= 1) {
+        const bool upper = (lane & (uint32_t)l) != 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float other = __shfl_xor(r[i], l, 64);
+          r[i] = upper ? other - r[i] : r[i] + other;
+        }
+      }
+      src[0] = make_float4(r[0], r[1], r[2], r[3]);
+      src[1] = make_float4(r[4], r[5], r[6], r[7]);
+    }
+    len0 = 512;
+  }
+  __syncthreads();
+  for (uint32_t len = len0; len < m; len <<= 1) {
+    for (uint32_t p = tid; p < (n >> 1); p += 1024) {
+      const uint32_t j = (p / len) * (len << 1) + (p % len);
+      const float u = v[j], w = v[j + len];
+      v[j] = u + w;
+      v[j + len] = u - w;
+    }
+    __syncthreads();
+  }
+  if (k == 1) {
+    for (uint32_t i = tid; i < n; i += 1024) v[i] = v[i] * inv;
+    return;
+  }
+  if (m >= 32) {
+    for (uint32_t tile = wave; tile < (m >> 5); tile += 16) {
+      const uint32_t j = (tile << 5) + l32;
+      float c_frag[kRotKMax / 2];
+#pragma unroll
+      for (uint32_t s = 0; s < kRotKMax / 2; ++s) {
+        const uint32_t t = 2u * s + lh;
+        const float x = v[(t < k ? t * m : 0u) + j];  // always a valid address, so the reads go out together
+        c_frag[s] = t < k ? x * inv : 0.f;
+      }
+      rot_acc_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (uint32_t s = 0; s < kRotKMax / 2; ++s)
+        if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(s_frag[s], c_frag[s], acc, 0, 0, 0);
+      // acc[r] is row 8 (r / 4) + 4 lh + r % 4 of column j
+#pragma unroll
+      for (uint32_t r = 0; r < 16; ++r) {
+        const uint32_t g = 8u * (r >> 2) + 4u * lh + (r & 3u);
+        if (g < k) v[g * m + j] = acc[r];
+      }
+    }
+    return;
+  }
+  // narrow groups (m < 32): one thread per column
+  for (uint32_t j = tid; j < m; j += 1024) {
+    float col[kRotKMax];
+#pragma unroll
+    for (uint32_t t = 0; t < kRotKMax; ++t) col[t] = t < k ? v[t * m + j] * inv : 0.f;
+    for (uint32_t g = 0; g < k; ++g) {
+      float acc = 0.f;
+#pragma unroll
+      for (uint32_t t = 0; t < kRotKMax; ++t)
+        if (t < k) acc = fmaf(small[g * k + t], col[t], acc);
+      v[g * m + j] = acc;
+    }
+  }
+}
 
 constexpr int kSmallTileBlocks = 2048;  // tile of the variant for rows too wide for the full tile's LDS
 __host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks, uint32_t tile = kTileBlocks,
@@ -411,20 +527,28 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0;
   prefetch_tile(a, blockIdx.x, tid, pre0, pre1);
   const __half* xsrc = a.x;
+  // A launch over matrices stored in a rotated basis rotates its activation itself: the
+  // values go, signs applied, as f32 to the area the first tile's code bytes, queues and
+  // partial sums will use (free until then), are rotated there and quantised from there.
+  const bool rotated = a.rot_m != 0;
+  float* xf = reinterpret_cast<float*>(raw);
+  const uint32_t d_in = nb * kDim + a.tail_w;
+  auto signed_f32 = [&](uint32_t i, float v) { return ((a.rot_signbits[i >> 5] >> (i & 31u)) & 1u) ? -v : v; };
   if (a.prologue != kPrologueNone) {
     // Every workgroup derives the activation for itself (a few thousand values)
     // instead of waiting for a kernel of its own; it is staged, as binary16, where
     // the tile's code bytes will go.
     __half* xs = reinterpret_cast<__half*>(raw);
-    const uint32_t d_in = nb * kDim + a.tail_w;
     if (a.prologue == kPrologueSiluMul) {
       for (uint32_t i = tid; i < d_in; i += kWgThreads) {
         const float g = __half2float(a.x2[i]);
         const float sg = __half2float(__float2half_rn(g / (1.0f + __expf(-g))));
-        xs[i] = __float2half_rn(sg * __half2float(a.x[i]));
+        const __half h = __float2half_rn(sg * __half2float(a.x[i]));
+        if (rotated) xf[i] = signed_f32(i, __half2float(h));
+        else xs[i] = h;
       }
     } else {
-      float* red = partial;  // free until the first tile's P2
+      float* red = partial + kTileBlocks - kWaves;  // the end of the partial sums: beyond the f32 staging of a rotated launch
       constexpr int kPer = (kRawBytes / 2 + kWgThreads - 1) / kWgThreads;
       float v[kPer];
       float ss = 0.f;
@@ -450,13 +574,40 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 #pragma unroll
       for (int k = 0; k < kPer; ++k) {
         const uint32_t i = tid + (uint32_t)k * kWgThreads;
-        if (i < d_in) xs[i] = __float2half_rn(v[k] * inv * __half2float(a.norm_w[i]));
+        if (i < d_in) {
+          const __half h = __float2half_rn(v[k] * inv * __half2float(a.norm_w[i]));
+          if (rotated) xf[i] = signed_f32(i, __half2float(h));
+          else xs[i] = h;
+        }
       }
     }
     __syncthreads();
     xsrc = xs;
+  } else if (rotated) {
+    // eight values per lane and pass; a width that is not a multiple of eight ends one value at a time
+    const uint32_t n8 = d_in & ~7u;
+    for (uint32_t i = tid * 8u; i < n8; i += kWgThreads * 8u) {
+      const uint4 h = *reinterpret_cast<const uint4*>(a.x + i);
+      const uint32_t sg = a.rot_signbits[i >> 5] >> (i & 31u);
+      const uint32_t w[4] = {h.x, h.y, h.z, h.w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float lo = __half2float(__ushort_as_half((unsigned short)(w[q] & 0xFFFFu)));
+        const float hi = __half2float(__ushort_as_half((unsigned short)(w[q] >> 16)));
+        xf[i + 2 * q] = ((sg >> (2 * q)) & 1u) ? -lo : lo;
+        xf[i + 2 * q + 1] = ((sg >> (2 * q + 1)) & 1u) ? -hi : hi;
+      }
+    }
+    for (uint32_t i = n8 + tid; i < d_in; i += kWgThreads) xf[i] = signed_f32(i, __half2float(a.x[i]));
+    __syncthreads();
   }
-  if (a.x_f32) {
+  if (rotated) {
+    rotate_lds(xf, d_in, a.rot_m, a.rot_k, a.rot_inv, a.rot_small);
+    __syncthreads();
+    for (uint32_t col = tid; col < nb; col += kWgThreads)
+      quantize_block_f32(xf + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+    if (tid < a.tail_w) xtail[tid] = xf[(size_t)nb * kDim + tid];
+  } else if (a.x_f32) {
     for (uint32_t col = tid; col < nb; col += kWgThreads)
       quantize_block_f32(a.x_f32 + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     if (tid < a.tail_w) xtail[tid] = a.x_f32[(size_t)nb * kDim + tid];
@@ -465,7 +616,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     if (tid < a.tail_w) xtail[tid] = __half2float(xsrc[(size_t)nb * kDim + tid]);
   }
-  if (a.prologue != kPrologueNone) __syncthreads();  // the staging area becomes the code-byte buffer
+  if (a.prologue != kPrologueNone || rotated) __syncthreads();  // the staging area becomes the code-byte buffer
 
 #ifdef LLVQ_PHASE_TIMING
   if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 7] = wall_clock64();
@@ -646,32 +797,10 @@ __global__ __launch_bounds__(1024) void rotate_kernel(RotArgs a) {
     rot_s[i] = ((a.signbits[i >> 5] >> (i & 31u)) & 1u) ? -v : v;
   }
   __syncthreads();
-  for (uint32_t len = 1; len < m; len <<= 1) {  // groups are contiguous, so one pass covers all of them
-    for (uint32_t p = tid; p < (n >> 1); p += 1024) {
-      const uint32_t j = (p / len) * (len << 1) + (p % len);
-      const float u = rot_s[j], w = rot_s[j + len];
-      rot_s[j] = u + w;
-      rot_s[j + len] = u - w;
-    }
-    __syncthreads();
-  }
+  rotate_lds(rot_s, n, m, k, a.inv, a.small);
+  __syncthreads();
   OutT* out = reinterpret_cast<OutT*>(a.out) + (size_t)blockIdx.x * n;
-  if (k == 1) {
-    for (uint32_t i = tid; i < n; i += 1024) out[i] = (OutT)(rot_s[i] * a.inv);
-    return;
-  }
-  for (uint32_t j = tid; j < m; j += 1024) {
-    float col[kRotKMax];
-#pragma unroll
-    for (uint32_t t = 0; t < kRotKMax; ++t) col[t] = t < k ? rot_s[t * m + j] * a.inv : 0.f;
-    for (uint32_t g = 0; g < k; ++g) {
-      float acc = 0.f;
-#pragma unroll
-      for (uint32_t t = 0; t < kRotKMax; ++t)
-        if (t < k) acc = fmaf(a.small[g * k + t], col[t], acc);
-      out[g * m + j] = (OutT)acc;
-    }
-  }
+  for (uint32_t i = tid; i < n; i += 1024) out[i] = (OutT)rot_s[i];
 }
 
 }  // namespace llvq
@@ -1102,6 +1231,13 @@ static bool prologue_fits(const llvq_mat* m0) {
   return (size_t)m0->d_in * 2 <= (size_t)pick_gemv_shape(m0->nblocks).tile * 6 + 32;
 }
 
+// Whether a launch over rows of this width can rotate its own activation: the f32
+// values take the place of the first tile's code bytes, queue and partial sums.
+static bool rotation_fits(const llvq_mat* m0) {
+  const size_t tile = pick_gemv_shape(m0->nblocks).tile;
+  return (size_t)m0->d_in * 4 + 64 <= tile * 6 + 32 + tile * 8;
+}
+
 struct Prologue {
   uint32_t kind = kPrologueNone;
   const void* x2 = nullptr;
@@ -1111,7 +1247,8 @@ struct Prologue {
 };
 
 static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, void* const* y,
-                        int y_dtype, const Prologue* pro = nullptr, const float* x_f32 = nullptr) {
+                        int y_dtype, const Prologue* pro = nullptr, const float* x_f32 = nullptr,
+                        const llvq_rt::DevRotation* rot = nullptr) {
   const llvq_mat* m0 = mats[0];
   if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemv: unknown output dtype");
   const GemvShape shape = pick_gemv_shape(m0->nblocks);
@@ -1135,6 +1272,15 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
     a.norm_w = reinterpret_cast<const __half*>(pro->norm_w);
     a.resid_out = reinterpret_cast<__half*>(pro->resid_out);
     a.eps = pro->eps;
+  }
+  if (rot) {
+    if (!rotation_fits(m0) || rot->n != m0->d_in)
+      return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": d_in too wide for a rotation inside the launch");
+    a.rot_signbits = rot->signbits;
+    a.rot_small = rot->small;
+    a.rot_inv = rot->inv;
+    a.rot_m = rot->m;
+    a.rot_k = rot->k;
   }
   a.nblocks = m0->nblocks;
   a.tail_w = m0->tail_w;
@@ -1193,21 +1339,31 @@ static bool same_basis(const llvq_mat* a, const llvq_mat* b) {
 }
 
 // One activation through projections that share it: consecutive matrices in the
-// same basis go out as one launch (at most kMaxGroup); a rotated basis gets its
-// activation rotated once, into the runtime's scratch, before its launches.
-static int forward_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, void* const* y, int y_dtype) {
+// same basis go out as one launch (at most kMaxGroup).  A launch in a rotated basis
+// rotates the activation itself (`pro`, when given, derives it first); rows too wide
+// for that get it rotated once, into the runtime's scratch, by a kernel of its own
+// (never together with `pro`: the caller stages the activation first then).
+static int forward_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, void* const* y, int y_dtype,
+                         const Prologue* pro = nullptr) {
   int i = 0;
   while (i < n) {
     int j = i + 1;
     while (j < n && j - i < kMaxGroup && same_basis(mats[i], mats[j])) ++j;
     const float* xr = nullptr;
+    if (mats[i]->has_rotation && rotation_fits(mats[i])) {
+      const int rc = launch_group(rt, mats + i, j - i, x, y + i, y_dtype, pro, nullptr, mats[i]->rot);
+      if (rc) return rc;
+      i = j;
+      continue;
+    }
+    if (pro && mats[i]->has_rotation) return fail(LLVQ_ERR_UNSUPPORTED, mats[i]->name + ": prologue with a rotation outside the launch");
     if (mats[i]->has_rotation) {
       // the scratch may still hold this very rotation if the previous run used it; rotating again is cheap and always right
       const int rc = launch_rotate(rt, mats[i]->rot, x, 1, rt->rot_scratch, false);
       if (rc) return rc;
       xr = rt->rot_scratch;
     }
-    const int rc = launch_group(rt, mats + i, j - i, x, y + i, y_dtype, nullptr, xr);
+    const int rc = launch_group(rt, mats + i, j - i, x, y + i, y_dtype, pro, xr);
     if (rc) return rc;
     i = j;
   }
@@ -1476,9 +1632,10 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   // through the rotation kernel), and so do rows too wide for the staging area:
   // their prologue runs as a kernel of its own.
   auto project = [&](const llvq_mat* const* mats, int n, const __half* x, void* const* outs, const Prologue& pro) -> int {
-    bool rotated = false;
-    for (int i = 0; i < n; ++i) rotated |= mats[i]->has_rotation;
-    if (!rotated && prologue_fits(mats[0])) return launch_group(rt, mats, n, x, outs, LLVQ_F16, &pro);
+    // every launch of the group can derive (and, in a rotated basis, rotate) the activation itself
+    bool fused = prologue_fits(mats[0]);
+    for (int i = 0; i < n; ++i) fused &= !mats[i]->has_rotation || rotation_fits(mats[i]);
+    if (fused) return forward_group(rt, mats, n, x, outs, LLVQ_F16, &pro);
     const __half* staged = nullptr;
     if (pro.kind == kPrologueAddRmsNorm) {
       hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, x, reinterpret_cast<const __half*>(pro.x2),

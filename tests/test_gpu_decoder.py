@@ -26,10 +26,18 @@ Q8 = decoder.Qwen3Config(num_hidden_layers=2, hidden_size=256, num_attention_hea
                          max_positions=80, tie_word_embeddings=True, kv_mode="q8")  # 5 query heads per kv head, as at 14B
 
 
-def _build(gpu_rt, orc, cfg, seed):
+def _build(gpu_rt, orc, cfg, seed, rotate=False):
     from oracle import qwen3_oracle
 
     raws = decoder.synthetic_projections(cfg, seed)
+    if rotate:
+        # stored as W Q^T (format.rs:435-437): q/k/v share a basis, gate/up another, o and down have their own;
+        # layer 1 keeps k and v in the natural basis, so one group call spans two bases
+        for li, layer in enumerate(raws):
+            for m, s in zip(layer, (11, 11, 11, 12, 13, 13, 14)):
+                m.rotation_seed = 100 * li + s
+            if li == 1:
+                layer[1].rotation_seed = layer[2].rotation_seed = None
     weights = decoder.synthetic_weights(cfg, seed)
     dense = [[orc.read_matrix_raw(artifact.write_matrix_raw(m))[0].decode_matrix() for m in layer] for layer in raws]
     ref = qwen3_oracle.Qwen3Oracle(cfg, dense, weights, kv_mode=cfg.kv_mode)
@@ -62,6 +70,23 @@ def test_teacher_forced_logits(gpu_rt, orc, cfg, seed, n):
         assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
         assert agree >= len(tokens) - 2
         assert dec.position == len(tokens)
+    finally:
+        dec.close()
+
+
+def test_rotated_projections_in_the_loop(gpu_rt, orc):
+    """Every projection stored in a rotated basis, as published artifacts are: the loop
+    rotates the activation before each product (fused_cuda.rs:362-384) and must agree with
+    the oracle, whose dense weights are un-rotated at decode (format.rs:435-437)."""
+    dec, ref = _build(gpu_rt, orc, SMALL, 4, rotate=True)
+    try:
+        tokens = np.random.default_rng(4).integers(0, SMALL.vocab_size, size=20)
+        worst = 0.0
+        for t in tokens:
+            want = ref.forward_token(int(t))
+            got, _ = dec.forward_token(int(t))
+            worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
+        assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
     finally:
         dec.close()
 
