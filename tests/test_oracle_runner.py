@@ -188,3 +188,48 @@ def test_runner_q8_cache_holds_reconstructed_values():
     assert np.array_equal(a.K[0][0], Q.quantize_dequantize(b.K[0][0]))
     assert np.array_equal(a.V[0][0], Q.quantize_dequantize(b.V[0][0]))
     assert np.abs(la - lb).max() < 0.05 * np.abs(lb).max() and not np.array_equal(la, lb)
+
+
+# ---- the reference's own golden for the runner (llvq-llm/tests/kv_cache.rs) -------------------
+def _tiny_reference_model(swap_kv=False):
+    """kv_cache.rs:31-52 (config) and :69-112 (weights): SplitMix64(0xA4_C0DE) Gaussians x 0.3 narrowed to
+    f32, drawn in the order embed, then per layer q, k, v, o, gate, up, down; every norm weight is one;
+    the head is tied; the model runs in f32 on the CPU."""
+    from llvq_amd import synth
+
+    cfg = SimpleNamespace(vocab_size=128, hidden_size=32, intermediate_size=64, num_hidden_layers=2,
+                          num_attention_heads=4, num_key_value_heads=2, head_dim=8, rope_theta=10_000.0,
+                          rms_norm_eps=1e-6, max_positions=64)
+    rng = synth.SplitMix64(0xA4C0DE)
+
+    def put(r, c):
+        return (rng.gaussian(r * c) * 0.3).astype(np.float32).reshape(r, c)
+
+    h, i, nh, nkv, hd = 32, 64, 4, 2, 8
+    embed = put(cfg.vocab_size, h)
+    layers = []
+    for _ in range(cfg.num_hidden_layers):
+        q = put(nh * hd, h)
+        first, second = put(nkv * hd, h), put(nkv * hd, h)
+        k, v = (second, first) if swap_kv else (first, second)
+        layers.append([q, k, v, put(h, nh * hd), put(i, h), put(i, h), put(h, i)])
+    ones = np.ones
+    w = SimpleNamespace(input_norm=ones((2, h), np.float32), post_norm=ones((2, h), np.float32),
+                        q_norm=ones((2, hd), np.float32), k_norm=ones((2, hd), np.float32),
+                        final_norm=ones(h, np.float32), embed=embed, lm_head=None)
+    return Q.Qwen3Oracle(cfg, layers, w, run_dtype="f32")
+
+
+def test_reference_golden_tokens_of_the_tiny_model():
+    """kv_cache.rs:140-153: prompt [3,1,4,1,5,9,2,6] -> [107,90,2,35,35,35,35,35], and exchanging
+    k_proj and v_proj moves the sequence (:156-164).  Pins the runner's structure — projection
+    order, per-head norms, the rotate-half RoPE at absolute positions, grouped-query attention over
+    the cache, residuals, the tied head, first-index argmax — on values the reference holds.  The
+    reference computes in f32 with candle's summation order and this runner in f64 between
+    roundings, so a near-tie could legitimately differ; none does on this sequence."""
+    golden = [107, 90, 2, 35, 35, 35, 35, 35]
+    prompt = [3, 1, 4, 1, 5, 9, 2, 6]
+    got, trace = _tiny_reference_model().generate(prompt, len(golden))
+    assert got.tolist() == golden, (got.tolist(), [float(np.sort(t)[-1] - np.sort(t)[-2]) for t in trace])
+    swapped, _ = _tiny_reference_model(swap_kv=True).generate(prompt, len(golden))
+    assert swapped.tolist() != golden
