@@ -102,7 +102,7 @@ def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
     cfg = decoder.QWEN3_4B
     t0 = time.time()
     weights = decoder.synthetic_weights(cfg, seed)
-    dec = decoder.Decoder(rt, cfg, projs, weights)
+    dec = decoder.Decoder(rt, cfg, projs, weights, prefill_rows=n_prompt)
     log(f"[bench] decoder built in {time.time() - t0:.1f}s")
     prompt = np.random.default_rng(seed).integers(0, cfg.vocab_size, size=n_prompt)
     dec.generate(prompt[:8], 4)  # warm-up
@@ -111,6 +111,11 @@ def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
     t1 = time.perf_counter()
     toks = dec.generate(prompt, n_new)
     t2 = time.perf_counter()
+    # the same prompt through the batched product (matrix cores, all positions of the prompt at once)
+    dec.generate(prompt, 1, batched_prefill=True)
+    t3 = time.perf_counter()
+    batched_first = dec.generate(prompt, 1, batched_prefill=True)
+    t4 = time.perf_counter()
     dec.close()
     assert toks[0] == first[0]
     step_s = ((t2 - t1) - (t1 - t0)) / (n_new - 1)
@@ -121,6 +126,8 @@ def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
         "new_tokens": n_new,
         "prefill_tokens_per_s": round(n_prompt / (t1 - t0), 2),
         "prefill": "one position at a time through the same kernels",
+        "batched_prefill_tokens_per_s": round(n_prompt / (t4 - t3), 1),
+        "batched_prefill_first_token_agrees": bool(batched_first[0] == first[0]),
         "distinct_tokens": int(np.unique(toks).size),
     }
 

@@ -209,6 +209,8 @@ typedef struct llvq_decoder_desc {
   uint32_t kv_mode;                     /* llvq_kv_mode; q8 needs head_dim % 64 == 0 */
   llvq_quant_rows embed_q8;             /* int8 embedding instead of `embed` (Embed::Q8, model.rs:546-551) */
   llvq_quant_rows lm_head_q8;           /* int8 head (Head::Q8, model.rs:569-575); absent and lm_head NULL = tied */
+  uint32_t prefill_rows;                /* positions llvq_hip_decoder_prefill takes per pass (buffers for that many
+                                           rows are allocated); 0 = the batched prompt path is not used */
 } llvq_decoder_desc;
 /* Qwen3::new_with (model.rs:869): checks every projection's shape against the architecture. */
 int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* desc, llvq_decoder** out);
@@ -233,6 +235,20 @@ int llvq_hip_decoder_forward_token(llvq_decoder* dec, uint32_t token, float* log
  * The loop never waits on the host between tokens.  Synchronises at the end. */
 int llvq_hip_decoder_generate(llvq_decoder* dec, const uint32_t* prompt, size_t n_prompt, size_t max_new,
                               uint32_t* out);
+
+/* The l > 1 arm of hidden_cached (model.rs:968-982, row loop of :521-529) with the rows of a
+ * pass going through the batched product (llvq_hip_gemm) instead of one product per row:
+ * feeds n tokens at the positions that follow the current one, prefill_rows at a time,
+ * advances the position by n and returns the last token's logits and argmax as
+ * llvq_hip_decoder_forward_token does (either may be NULL).  The weights of these products
+ * are rounded to binary16 once (see llvq_hip_gemm), so logits differ from the
+ * token-by-token path by a few 1e-3 of the largest one; the KV cache it leaves is read by
+ * the token-by-token calls that follow.  head_dim <= 128.  Synchronises. */
+int llvq_hip_decoder_prefill(llvq_decoder* dec, const uint32_t* tokens, size_t n, float* logits_host,
+                             uint32_t* argmax_host);
+/* llvq_hip_decoder_generate with the prompt taken through llvq_hip_decoder_prefill. */
+int llvq_hip_decoder_generate_prefilled(llvq_decoder* dec, const uint32_t* prompt, size_t n_prompt, size_t max_new,
+                                        uint32_t* out);
 
 int llvq_hip_synchronize(llvq_rt* rt);
 const char* llvq_hip_last_error(void);

@@ -69,6 +69,7 @@ class DecoderDesc(C.Structure):
         ("input_norm", C.c_void_p), ("post_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
         ("final_norm", C.c_void_p), ("embed", C.c_void_p), ("lm_head", C.c_void_p),
         ("kv_mode", C.c_uint32), ("embed_q8", QuantRows), ("lm_head_q8", QuantRows),
+        ("prefill_rows", C.c_uint32),
     ]
 
 
@@ -129,6 +130,8 @@ def lib():
     L.llvq_hip_decoder_seek.argtypes = [vp, C.c_uint32]
     L.llvq_hip_decoder_forward_token.argtypes = [vp, C.c_uint32, vp, C.POINTER(C.c_uint32)]
     L.llvq_hip_decoder_generate.argtypes = [vp, vp, sz, sz, vp]
+    L.llvq_hip_decoder_generate_prefilled.argtypes = [vp, vp, sz, sz, vp]
+    L.llvq_hip_decoder_prefill.argtypes = [vp, vp, sz, vp, C.POINTER(C.c_uint32)]
     L.llvq_hip_last_error.restype = C.c_char_p
     L.llvq_hip_version.restype = C.c_char_p
     _lib = L
@@ -149,5 +152,6 @@ EXPORTS = [
     "llvq_hip_last_error", "llvq_hip_version",
     "llvq_hip_host_rotate", "llvq_hip_rotate", "llvq_hip_gemv_rotated", "llvq_hip_matrix_rotation",
     "llvq_hip_decoder_create", "llvq_hip_decoder_destroy", "llvq_hip_decoder_reset", "llvq_hip_decoder_position", "llvq_hip_decoder_seek",
-    "llvq_hip_decoder_forward_token", "llvq_hip_decoder_generate",
+    "llvq_hip_decoder_forward_token", "llvq_hip_decoder_generate", "llvq_hip_decoder_generate_prefilled",
+    "llvq_hip_decoder_prefill",
 ]

@@ -33,10 +33,11 @@ __device__ __forceinline__ float block_sum_1024(float v, float* red) {
   return s;
 }
 
-// h = embed[token]
+// h[row] = embed[token[row]], row = blockIdx.y
 __global__ __launch_bounds__(256) void embed_kernel(const __half* __restrict__ table, const uint32_t* __restrict__ token,
                                                     uint32_t vocab, uint32_t hidden, __half* __restrict__ h) {
-  const uint32_t t = min(*token, vocab - 1u);
+  const uint32_t t = min(token[blockIdx.y], vocab - 1u);
+  h += (size_t)blockIdx.y * hidden;
   for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < hidden; i += gridDim.x * blockDim.x)
     h[i] = table[(size_t)t * hidden + i];
 }
@@ -48,6 +49,11 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(const __half*
                                                                    const __half* __restrict__ w, __half* h_out,
                                                                    __half* __restrict__ normed, uint32_t n, float eps) {
   __shared__ float red[kNormThreads / 64];
+  // one workgroup per row of n values
+  h += (size_t)blockIdx.x * n;
+  if (delta) delta += (size_t)blockIdx.x * n;
+  if (h_out) h_out += (size_t)blockIdx.x * n;
+  normed += (size_t)blockIdx.x * n;
   constexpr int kPer = 8;  // n <= 8192
   float v[kPer];
   float ss = 0.f;
@@ -183,6 +189,164 @@ struct AttnNew {
   float eps;
 };
 
+constexpr int kAttnThreads = 256;
+constexpr int kAttnWaves = kAttnThreads / 64;
+constexpr int kAttnMaxSplits = 64;  // the cache is cut into at most this many ranges (host picks by length)
+constexpr int kAttnMaxGroup = 8;    // query heads per kv head
+
+// ---- rows of positions at once (prompt processing through the batched product) ----
+// One wavefront per (head, row): q heads are normed and rotated in place, k heads are
+// normed, rotated and appended to the cache at position pos0 + row, v heads are appended.
+// Grid (n_heads + 2 n_kv, rows).  Same arithmetic as the one-position path.
+template <bool Q8>
+__global__ __launch_bounds__(64) void norm_rope_append_rows_kernel(__half* __restrict__ q, const __half* __restrict__ k,
+                                                                   const __half* __restrict__ v, AttnNew nw, KvQ8 q8,
+                                                                   uint32_t n_heads, uint32_t n_kv, uint32_t head_dim,
+                                                                   uint32_t pos0, uint32_t max_pos) {
+  __shared__ float stage[256];
+  const uint32_t head = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
+  const uint32_t pos = pos0 + row, kvgroups = head_dim / kKvGroup;
+  if (head < n_heads) {
+    __half* qh = q + ((size_t)row * n_heads + head) * head_dim;
+    norm_rope_wave(qh, nw.qn, nw.cos_t, nw.sin_t, pos, head_dim, nw.eps, stage, lane);
+    for (uint32_t i = lane; i < head_dim; i += 64) qh[i] = __float2half_rn(stage[i]);
+    return;
+  }
+  const bool is_k = head < n_heads + n_kv;
+  const uint32_t kvh = is_k ? head - n_heads : head - n_heads - n_kv;
+  const __half* src = (is_k ? k : v) + ((size_t)row * n_kv + kvh) * head_dim;
+  if (is_k) norm_rope_wave(src, nw.kn, nw.cos_t, nw.sin_t, pos, head_dim, nw.eps, stage, lane);
+  else {
+    for (uint32_t i = lane; i < head_dim; i += 64) stage[i] = __half2float(src[i]);
+    wave_lds_sync();
+  }
+  const size_t crow = (size_t)kvh * max_pos + pos;
+  if constexpr (Q8) {
+    uint8_t* cq = is_k ? q8.kq : q8.vq;
+    __half* cs = is_k ? q8.ks : q8.vs;
+    __half* cb = is_k ? q8.kb : q8.vb;
+    for (uint32_t g = 0; g < kvgroups; ++g) {
+      __half sh, bh;
+      const uint8_t code = kv_quantize_group(stage[g * kKvGroup + lane], &sh, &bh);
+      cq[crow * head_dim + g * kKvGroup + lane] = code;
+      if (lane == 0) {
+        cs[crow * kvgroups + g] = sh;
+        cb[crow * kvgroups + g] = bh;
+      }
+    }
+  } else {
+    __half* dst = (is_k ? nw.kcache : nw.vcache) + crow * head_dim;
+    for (uint32_t i = lane; i < head_dim; i += 64) dst[i] = __float2half_rn(stage[i]);
+  }
+}
+
+// Causal attention of a row of queries over the cache (model.rs:812-822 with the mask of
+// :938-960): one wavefront per (kv head, row) serves every query head of the group; the
+// query at row r sees positions 0 .. pos0 + r.  Lane (pj, sub) = (lane / 16, lane % 16)
+// holds dims [8 sub, 8 sub + 8) of the positions j = pj (mod 4); each of the four position
+// classes keeps its own running maximum, sum and weighted V sum (f32), merged at the end.
+// head_dim <= 128, a multiple of 8.  q is already normed and rotated; ctx is rounded once.
+template <bool Q8>
+__global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict__ q, const __half* __restrict__ kcache,
+                                                       const __half* __restrict__ vcache, KvQ8 q8, __half* __restrict__ ctx,
+                                                       uint32_t n_heads, uint32_t n_kv, uint32_t head_dim, uint32_t pos0,
+                                                       uint32_t max_pos, float scale) {
+  const uint32_t kvh = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
+  const uint32_t groups = n_heads / n_kv, T = pos0 + row + 1;
+  const uint32_t sub = lane & 15u, pj = lane >> 4, i0 = sub * 8u;
+  const bool active = i0 < head_dim;
+  const uint32_t kvgroups = head_dim / kKvGroup;
+  const size_t base = (size_t)kvh * max_pos;
+  float qv[kAttnMaxGroup][8], acc[kAttnMaxGroup][8], m[kAttnMaxGroup], l[kAttnMaxGroup];
+#pragma unroll
+  for (int g = 0; g < kAttnMaxGroup; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      acc[g][t] = 0.f;
+      qv[g][t] = ((uint32_t)g < groups && active)
+                     ? __half2float(q[((size_t)row * n_heads + kvh * groups + g) * head_dim + i0 + t]) * scale
+                     : 0.f;
+    }
+  }
+  for (uint32_t j = pj; j < T; j += 4) {
+    float kf[8], vf[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) kf[t] = vf[t] = 0.f;
+    if (active) {
+      if constexpr (Q8) {
+        const uint2 kc = *reinterpret_cast<const uint2*>(q8.kq + (base + j) * head_dim + i0);
+        const uint2 vc = *reinterpret_cast<const uint2*>(q8.vq + (base + j) * head_dim + i0);
+        const size_t gi = (base + j) * kvgroups + i0 / kKvGroup;
+        const float ks = __half2float(q8.ks[gi]), kb = __half2float(q8.kb[gi]);
+        const float vs = __half2float(q8.vs[gi]), vb = __half2float(q8.vb[gi]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          kf[t] = kv_dequant((kc.x >> (8 * t)) & 0xFFu, ks, kb);
+          kf[4 + t] = kv_dequant((kc.y >> (8 * t)) & 0xFFu, ks, kb);
+          vf[t] = kv_dequant((vc.x >> (8 * t)) & 0xFFu, vs, vb);
+          vf[4 + t] = kv_dequant((vc.y >> (8 * t)) & 0xFFu, vs, vb);
+        }
+      } else {
+        const uint4 kr = *reinterpret_cast<const uint4*>(kcache + (base + j) * head_dim + i0);
+        const uint4 vr = *reinterpret_cast<const uint4*>(vcache + (base + j) * head_dim + i0);
+        const uint32_t kw[4] = {kr.x, kr.y, kr.z, kr.w}, vw[4] = {vr.x, vr.y, vr.z, vr.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          kf[2 * t] = __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu)));
+          kf[2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16)));
+          vf[2 * t] = __half2float(__ushort_as_half((unsigned short)(vw[t] & 0xFFFFu)));
+          vf[2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(vw[t] >> 16)));
+        }
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < kAttnMaxGroup; ++g)
+      if ((uint32_t)g < groups) {
+        float d = 0.f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) d = fmaf(qv[g][t], kf[t], d);
+        d += __shfl_xor(d, 1, 64);
+        d += __shfl_xor(d, 2, 64);
+        d += __shfl_xor(d, 4, 64);
+        d += __shfl_xor(d, 8, 64);
+        const float mn = fmaxf(m[g], d);
+        const float c = __expf(m[g] - mn), p = __expf(d - mn);  // c = 0 on the first position (m = -inf)
+        l[g] = fmaf(l[g], c, p);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[g][t] = fmaf(acc[g][t], c, p * vf[t]);
+        m[g] = mn;
+      }
+  }
+  // merge the four position classes (a class with no position has m = -inf and weight 0)
+#pragma unroll
+  for (int off = 16; off <= 32; off <<= 1)
+#pragma unroll
+    for (int g = 0; g < kAttnMaxGroup; ++g)
+      if ((uint32_t)g < groups) {
+        const float mo = __shfl_xor(m[g], off, 64), lo = __shfl_xor(l[g], off, 64);
+        const float mn = fmaxf(m[g], mo);
+        const float c1 = m[g] == -INFINITY ? 0.f : __expf(m[g] - mn), c2 = mo == -INFINITY ? 0.f : __expf(mo - mn);
+        l[g] = l[g] * c1 + lo * c2;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          const float ao = __shfl_xor(acc[g][t], off, 64);
+          acc[g][t] = acc[g][t] * c1 + ao * c2;
+        }
+        m[g] = mn;
+      }
+  if (pj == 0 && active)
+#pragma unroll
+    for (int g = 0; g < kAttnMaxGroup; ++g)
+      if ((uint32_t)g < groups) {
+        __half* dst = ctx + ((size_t)row * n_heads + kvh * groups + g) * head_dim + i0;
+        const float inv = 1.0f / l[g];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) dst[t] = __float2half_rn(acc[g][t] * inv);
+      }
+}
+
 // Attention of one query position over the cache (model.rs:812-822), split over
 // the cache: workgroup (kv head, split) takes a contiguous range of positions
 // for all query heads that share the kv head, so every K and V row is fetched
@@ -192,10 +356,6 @@ struct AttnNew {
 // of exponentials, weighted V sum), and the workgroup that arrives last at the
 // kv head's counter merges the partials in split order and rounds the context
 // once.  Scores, softmax and sums stay in f32.
-constexpr int kAttnThreads = 256;
-constexpr int kAttnWaves = kAttnThreads / 64;
-constexpr int kAttnMaxSplits = 64;  // the cache is cut into at most this many ranges (host picks by length)
-constexpr int kAttnMaxGroup = 8;    // query heads per kv head
 template <bool Q8>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, const __half* __restrict__ kcache,
                                                                    const __half* __restrict__ vcache, KvQ8 q8,
@@ -638,7 +798,8 @@ __device__ __forceinline__ float q8_weight(uint32_t q, float s, float b) {
 // h = f16(embedding row of *token)   (emb_q8_gather)
 __global__ __launch_bounds__(256) void embed_q8_kernel(QuantRows e, const uint32_t* __restrict__ token, uint32_t vocab,
                                                        uint32_t hidden, __half* __restrict__ h) {
-  const uint32_t t = min(*token, vocab - 1u);
+  const uint32_t t = min(token[blockIdx.y], vocab - 1u);
+  h += (size_t)blockIdx.y * hidden;
   const uint32_t gpr = (hidden + kEmbedGroup - 1) / kEmbedGroup;
   for (uint32_t c = blockIdx.x * blockDim.x + threadIdx.x; c < hidden; c += gridDim.x * blockDim.x) {
     const size_t g = (size_t)t * gpr + c / kEmbedGroup;

@@ -1602,9 +1602,28 @@ struct llvq_decoder {
   uint32_t* attn_counters = nullptr;  // [n_kv], zero between launches
   uint32_t pos = 0;
   uint32_t head_grid = 0;
+  // rows of positions at once (llvq_hip_decoder_prefill): [prefill_rows, width] buffers, one allocation
+  uint32_t prefill_rows = 0;
+  uint8_t* pblob = nullptr;
+  __half *ph = nullptr, *ph_alt = nullptr, *pnormed = nullptr, *pq = nullptr, *pk = nullptr, *pv = nullptr, *pctx = nullptr, *po = nullptr;
+  __half *pgate = nullptr, *pup = nullptr, *pact = nullptr, *pdown = nullptr;
+  uint32_t* ptokens = nullptr;
 };
 
 namespace {
+
+// The head over dec->normed and the argmax, which overwrites *dec->token (and history[slot] when recording).
+void launch_head(llvq_decoder* d, uint32_t history_slot, bool record) {
+  hipStream_t st = d->rt->stream;
+  if (d->head_q8)
+    hipLaunchKernelGGL(lm_head_q8_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head_q, d->normed,
+                       d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
+  else
+    hipLaunchKernelGGL(lm_head_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head, d->normed,
+                       d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(1024), 0, st, d->best_val, d->best_idx,
+                     d->head_grid * (kHeadThreads / 64), d->token, record ? d->history : (uint32_t*)nullptr, history_slot);
+}
 
 // Enqueues one position: embeds *dec->token, runs the layers at position dec->pos,
 // and (want_logits) the head and the argmax, which overwrites *dec->token.
@@ -1717,17 +1736,97 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   }
   if (want_logits) {
     hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->down, d->fnorm, d->h, d->normed, d->hidden, d->eps);
-    if (d->head_q8)
-      hipLaunchKernelGGL(lm_head_q8_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head_q, d->normed,
-                         d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
-    else
-      hipLaunchKernelGGL(lm_head_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head, d->normed,
-                         d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
-    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(1024), 0, st, d->best_val, d->best_idx,
-                       d->head_grid * (kHeadThreads / 64), d->token, record ? d->history : (uint32_t*)nullptr, history_slot);
+    launch_head(d, history_slot, record);
   }
   HIP_TRY(hipGetLastError());
   d->pos += 1;
+  return LLVQ_OK;
+}
+// n <= prefill_rows positions at once, starting at dec->pos: tokens from dec->ptokens.
+// With want_logits the head runs on the last row and leaves its argmax in *dec->token.
+int decoder_prefill_pass(llvq_decoder* d, uint32_t n, bool want_logits, uint32_t history_slot, bool record) {
+  llvq_rt* rt = d->rt;
+  hipStream_t st = rt->stream;
+  if (d->pos + n > d->max_pos) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_prefill: positions past max_positions");
+  const uint32_t qd = d->n_heads * d->head_dim;
+  if (d->embed_q8)
+    hipLaunchKernelGGL(embed_q8_kernel, dim3((d->hidden + 255) / 256, n), dim3(256), 0, st, d->embed_q, d->ptokens, d->vocab, d->hidden, d->ph);
+  else
+    hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256, n), dim3(256), 0, st, d->embed, d->ptokens, d->vocab, d->hidden, d->ph);
+  const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim, group_layer = cache_layer / kKvGroup;
+  const float scale = 1.0f / sqrtf((float)d->head_dim);
+  auto rows = [&](const llvq_mat* m, const __half* x, __half* y) { return llvq_hip_gemm(rt, m, x, (int)n, y, LLVQ_F16); };
+  for (uint32_t L = 0; L < d->n_layers; ++L) {
+    const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
+    // residual + previous MLP branch, then the input norm (the branch of layer 0 is absent)
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(kNormThreads), 0, st, d->ph, L ? d->pdown : (const __half*)nullptr,
+                       d->ln1 + (size_t)L * d->hidden, L ? d->ph_alt : (__half*)nullptr, d->pnormed, d->hidden, d->eps);
+    if (L) std::swap(d->ph, d->ph_alt);
+    int rc = rows(P[0], d->pnormed, d->pq);
+    if (!rc) rc = rows(P[1], d->pnormed, d->pk);
+    if (!rc) rc = rows(P[2], d->pnormed, d->pv);
+    if (rc) return rc;
+    KvQ8 lq8 = d->q8;
+    if (d->kv_q8) {
+      lq8.kq += L * cache_layer; lq8.vq += L * cache_layer;
+      lq8.ks += L * group_layer; lq8.kb += L * group_layer; lq8.vs += L * group_layer; lq8.vb += L * group_layer;
+    }
+    __half* kc = d->kv_q8 ? nullptr : d->kcache + L * cache_layer;
+    __half* vc = d->kv_q8 ? nullptr : d->vcache + L * cache_layer;
+    AttnNew nw{};
+    nw.qn = d->qn + (size_t)L * d->head_dim;
+    nw.kn = d->kn + (size_t)L * d->head_dim;
+    nw.cos_t = d->cos_t;
+    nw.sin_t = d->sin_t;
+    nw.kcache = kc;
+    nw.vcache = vc;
+    nw.eps = d->eps;
+    const dim3 hgrid(d->n_heads + 2 * d->n_kv, n), agrid(d->n_kv, n);
+    if (d->kv_q8) {
+      hipLaunchKernelGGL(norm_rope_append_rows_kernel<true>, hgrid, dim3(64), 0, st, d->pq, d->pk, d->pv, nw, lq8, d->n_heads, d->n_kv,
+                         d->head_dim, d->pos, d->max_pos);
+      hipLaunchKernelGGL(attn_rows_kernel<true>, agrid, dim3(64), 0, st, d->pq, kc, vc, lq8, d->pctx, d->n_heads, d->n_kv, d->head_dim,
+                         d->pos, d->max_pos, scale);
+    } else {
+      hipLaunchKernelGGL(norm_rope_append_rows_kernel<false>, hgrid, dim3(64), 0, st, d->pq, d->pk, d->pv, nw, lq8, d->n_heads, d->n_kv,
+                         d->head_dim, d->pos, d->max_pos);
+      hipLaunchKernelGGL(attn_rows_kernel<false>, agrid, dim3(64), 0, st, d->pq, kc, vc, lq8, d->pctx, d->n_heads, d->n_kv, d->head_dim,
+                         d->pos, d->max_pos, scale);
+    }
+    rc = rows(P[3], d->pctx, d->po);
+    if (rc) return rc;
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(kNormThreads), 0, st, d->ph, d->po, d->ln2 + (size_t)L * d->hidden, d->ph_alt,
+                       d->pnormed, d->hidden, d->eps);
+    std::swap(d->ph, d->ph_alt);
+    rc = rows(P[4], d->pnormed, d->pgate);
+    if (!rc) rc = rows(P[5], d->pnormed, d->pup);
+    if (rc) return rc;
+    const uint32_t na = n * d->inter;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((na + 255) / 256 < 4096u ? (na + 255) / 256 : 4096u), dim3(256), 0, st, d->pgate, d->pup, d->pact, na);
+    rc = rows(P[6], d->pact, d->pdown);
+    if (rc) return rc;
+  }
+  if (want_logits) {
+    const size_t last = (size_t)(n - 1) * d->hidden;
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->ph + last, d->pdown + last, d->fnorm, d->h, d->normed,
+                       d->hidden, d->eps);
+    launch_head(d, history_slot, record);
+  }
+  HIP_TRY(hipGetLastError());
+  d->pos += n;
+  (void)qd;
+  return LLVQ_OK;
+}
+
+// The prompt through decoder_prefill_pass, prefill_rows positions at a time; the head runs after the last one.
+int decoder_prefill(llvq_decoder* d, const uint32_t* tokens, size_t n, uint32_t history_slot, bool record) {
+  if (!d->prefill_rows) return fail(LLVQ_ERR_UNSUPPORTED, "decoder_prefill: the decoder was created with prefill_rows = 0");
+  for (size_t at = 0; at < n; at += d->prefill_rows) {
+    const uint32_t c = (uint32_t)(n - at < d->prefill_rows ? n - at : d->prefill_rows);
+    HIP_TRY(hipMemcpyAsync(d->ptokens, tokens + at, c * sizeof(uint32_t), hipMemcpyHostToDevice, d->rt->stream));
+    const int rc = decoder_prefill_pass(d, c, at + c == n, history_slot, record);
+    if (rc) return rc;
+  }
   return LLVQ_OK;
 }
 
@@ -1756,6 +1855,8 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
     return fail(LLVQ_ERR_UNSUPPORTED,
                 "decoder_create: shape outside what the kernels hold (hidden % 8 = 0 and <= 8192, head_dim % 8 = 0 and <= 256, "
                 "heads a multiple of kv heads and at most 8 per kv head, max_positions <= 8192, kv_mode f16 or q8 with head_dim % 64 = 0)");
+  if (c->prefill_rows && (c->head_dim > 128 || c->prefill_rows > 4096))
+    return fail(LLVQ_ERR_UNSUPPORTED, "decoder_create: the batched prompt path takes head_dim <= 128 and at most 4096 rows per pass");
   const uint32_t qd = c->n_heads * c->head_dim, kvd = c->n_kv_heads * c->head_dim;
   static const char* kSite[7] = {"q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"};
   const uint32_t want_out[7] = {qd, kvd, kvd, c->hidden, c->intermediate, c->intermediate, c->hidden};
@@ -1863,6 +1964,24 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   d->history = reinterpret_cast<uint32_t*>(d->blob + o_hist);
   d->attn_part = reinterpret_cast<float*>(d->blob + o_ap);
   d->attn_counters = reinterpret_cast<uint32_t*>(d->blob + o_ac);
+  if (c->prefill_rows) {
+    // row buffers of the batched prompt path, one allocation
+    const size_t R = c->prefill_rows;
+    size_t ptotal = 0;
+    auto ptake = [&](size_t bytes) { const size_t at = ptotal; ptotal += (bytes + 255) & ~(size_t)255; return at; };
+    const size_t p_h = ptake(R * c->hidden * hb), p_h2 = ptake(R * c->hidden * hb), p_nm = ptake(R * c->hidden * hb);
+    const size_t p_q = ptake(R * qd * hb), p_k = ptake(R * kvd * hb), p_v = ptake(R * kvd * hb), p_ctx = ptake(R * qd * hb);
+    const size_t p_o = ptake(R * c->hidden * hb), p_g = ptake(R * c->intermediate * hb), p_u = ptake(R * c->intermediate * hb);
+    const size_t p_act = ptake(R * c->intermediate * hb), p_dn = ptake(R * c->hidden * hb), p_tok = ptake(R * sizeof(uint32_t));
+    e = hipMalloc(reinterpret_cast<void**>(&d->pblob), ptotal);
+    if (e == hipSuccess) e = hipMemset(d->pblob, 0, ptotal);
+    if (e != hipSuccess) { (void)hipFree(d->pblob); (void)hipFree(d->blob); delete d; return hip_fail(e, "hipMalloc(decoder prefill rows)"); }
+    auto PH = [&](size_t at) { return reinterpret_cast<__half*>(d->pblob + at); };
+    d->prefill_rows = c->prefill_rows;
+    d->ph = PH(p_h); d->ph_alt = PH(p_h2); d->pnormed = PH(p_nm); d->pq = PH(p_q); d->pk = PH(p_k); d->pv = PH(p_v); d->pctx = PH(p_ctx);
+    d->po = PH(p_o); d->pgate = PH(p_g); d->pup = PH(p_u); d->pact = PH(p_act); d->pdown = PH(p_dn);
+    d->ptokens = reinterpret_cast<uint32_t*>(d->pblob + p_tok);
+  }
   *out = d;
   return LLVQ_OK;
 }
@@ -1871,6 +1990,7 @@ void llvq_hip_decoder_destroy(llvq_decoder* d) {
   if (!d) return;
   (void)hipSetDevice(d->rt->device);
   (void)hipStreamSynchronize(d->rt->stream);
+  (void)hipFree(d->pblob);
   (void)hipFree(d->blob);
   delete d;
 }
@@ -1903,26 +2023,54 @@ int llvq_hip_decoder_forward_token(llvq_decoder* d, uint32_t token, float* logit
   return LLVQ_OK;
 }
 
-int llvq_hip_decoder_generate(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out) {
-  if (!d || (n_prompt && !prompt) || (max_new && !out)) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate: null argument");
+static int generate_impl(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out, bool batched,
+                         const char* who) {
+  if (!d || (n_prompt && !prompt) || (max_new && !out)) return fail(LLVQ_ERR_INVALID_ARGUMENT, std::string(who) + ": null argument");
   if (max_new == 0) return LLVQ_OK;  // model.rs:1052-1054
-  if (n_prompt == 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate: empty prompt");
+  if (n_prompt == 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, std::string(who) + ": empty prompt");
   if (n_prompt + max_new - 1 > d->max_pos)
-    return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate: " + std::to_string(n_prompt + max_new - 1) + " positions exceed max_positions " + std::to_string(d->max_pos));
+    return fail(LLVQ_ERR_INVALID_ARGUMENT, std::string(who) + ": " + std::to_string(n_prompt + max_new - 1) + " positions exceed max_positions " + std::to_string(d->max_pos));
   for (size_t i = 0; i < n_prompt; ++i)
-    if (prompt[i] >= d->vocab) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate: prompt token outside the vocabulary");
+    if (prompt[i] >= d->vocab) return fail(LLVQ_ERR_INVALID_ARGUMENT, std::string(who) + ": prompt token outside the vocabulary");
   HIP_TRY(hipSetDevice(d->rt->device));
   d->pos = 0;
-  for (size_t i = 0; i < n_prompt; ++i) {
-    hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(1), 0, d->rt->stream, d->token, prompt[i]);
-    const int rc = decoder_step(d, i + 1 == n_prompt, 0, true);
+  if (batched) {
+    const int rc = decoder_prefill(d, prompt, n_prompt, 0, true);
     if (rc) return rc;
+  } else {
+    for (size_t i = 0; i < n_prompt; ++i) {
+      hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(1), 0, d->rt->stream, d->token, prompt[i]);
+      const int rc = decoder_step(d, i + 1 == n_prompt, 0, true);
+      if (rc) return rc;
+    }
   }
   for (size_t t = 1; t < max_new; ++t) {
     const int rc = decoder_step(d, true, (uint32_t)t, true);
     if (rc) return rc;
   }
   HIP_TRY(hipMemcpyAsync(out, d->history, max_new * sizeof(uint32_t), hipMemcpyDeviceToHost, d->rt->stream));
+  HIP_TRY(hipStreamSynchronize(d->rt->stream));
+  return LLVQ_OK;
+}
+
+int llvq_hip_decoder_generate(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out) {
+  return generate_impl(d, prompt, n_prompt, max_new, out, false, "decoder_generate");
+}
+
+int llvq_hip_decoder_generate_prefilled(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out) {
+  return generate_impl(d, prompt, n_prompt, max_new, out, true, "decoder_generate_prefilled");
+}
+
+int llvq_hip_decoder_prefill(llvq_decoder* d, const uint32_t* tokens, size_t n, float* logits_host, uint32_t* argmax_host) {
+  if (!d || !tokens || n == 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_prefill: null or empty argument");
+  if (d->pos + n > d->max_pos) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_prefill: positions past max_positions");
+  for (size_t i = 0; i < n; ++i)
+    if (tokens[i] >= d->vocab) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_prefill: token outside the vocabulary");
+  HIP_TRY(hipSetDevice(d->rt->device));
+  const int rc = decoder_prefill(d, tokens, n, 0, false);
+  if (rc) return rc;
+  if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, d->logits, (size_t)d->vocab * sizeof(float), hipMemcpyDeviceToHost, d->rt->stream));
+  if (argmax_host) HIP_TRY(hipMemcpyAsync(argmax_host, d->token, sizeof(uint32_t), hipMemcpyDeviceToHost, d->rt->stream));
   HIP_TRY(hipStreamSynchronize(d->rt->stream));
   return LLVQ_OK;
 }

@@ -80,7 +80,8 @@ class Decoder:
     """A Qwen3-architecture model on one GPU: projections uploaded through `rt`,
     the rest copied at construction."""
 
-    def __init__(self, rt: FusedRuntime, cfg: Qwen3Config, projections, weights: DecoderWeights):
+    def __init__(self, rt: FusedRuntime, cfg: Qwen3Config, projections, weights: DecoderWeights, prefill_rows: int = 0):
+        """prefill_rows > 0 also allocates the row buffers of the batched prompt path (`prefill`)."""
         self.rt, self.cfg = rt, cfg
         self.handle = None
         self._owned = []
@@ -130,14 +131,14 @@ class Decoder:
             cfg.max_positions, float(cfg.rope_theta), float(cfg.rms_norm_eps),
             C.cast(arr, C.POINTER(C.c_void_p)),
             keep[0].ctypes.data, keep[1].ctypes.data, keep[2].ctypes.data, keep[3].ctypes.data, keep[4].ctypes.data,
-            e_ptr, h_ptr, self._kv_mode(cfg.kv_mode), e_q, h_q)
+            e_ptr, h_ptr, self._kv_mode(cfg.kv_mode), e_q, h_q, int(prefill_rows))
         self._alive = (keep, e_alive, h_alive)
         out = C.c_void_p()
         _ffi.check(_ffi.lib().llvq_hip_decoder_create(rt.handle, C.byref(desc), C.byref(out)))
         self.handle = out
 
     @classmethod
-    def from_model(cls, rt: FusedRuntime, model, max_positions=None, kv_mode="f16"):
+    def from_model(cls, rt: FusedRuntime, model, max_positions=None, kv_mode="f16", prefill_rows: int = 0):
         """Qwen3::new_with over a loaded sealed artifact (fused_cuda.rs:1226-1300 + model.rs:869):
         the architecture comes from the file's config.json, the projections from its matrix
         records (by `model.layers.{i}.{site}.weight`), norms and embedding from its raw tensors."""
@@ -178,7 +179,7 @@ class Decoder:
             stack("model.layers.{}.input_layernorm.weight", h), stack("model.layers.{}.post_attention_layernorm.weight", h),
             stack("model.layers.{}.self_attn.q_norm.weight", d), stack("model.layers.{}.self_attn.k_norm.weight", d),
             halves("model.norm.weight", (h,)), model.tensor("model.embed_tokens.weight"), head)
-        return cls(rt, cfg, projections, weights)
+        return cls(rt, cfg, projections, weights, prefill_rows=prefill_rows)
 
     @staticmethod
     def _kv_mode(v):
@@ -208,11 +209,23 @@ class Decoder:
             self.handle, int(token), logits.ctypes.data if want_logits else None, C.byref(best)))
         return logits, best.value
 
-    def generate(self, prompt, max_new: int) -> np.ndarray:
+    def prefill(self, tokens, want_logits: bool = True):
+        """The next len(tokens) positions through the batched product, `prefill_rows` at a time:
+        (logits of the last one or None, its argmax).  The decoder must have been built with prefill_rows > 0."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
+        logits = np.empty(self.cfg.vocab_size, np.float32) if want_logits else None
+        best = C.c_uint32()
+        _ffi.check(_ffi.lib().llvq_hip_decoder_prefill(
+            self.handle, tokens.ctypes.data, tokens.size, logits.ctypes.data if want_logits else None, C.byref(best)))
+        return logits, best.value
+
+    def generate(self, prompt, max_new: int, batched_prefill: bool = False) -> np.ndarray:
+        """Greedy tokens after `prompt`.  batched_prefill takes the prompt through `prefill` (matrix cores,
+        weights rounded to binary16 once) instead of position by position."""
         prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
         out = np.zeros(max_new, np.uint32)
-        _ffi.check(_ffi.lib().llvq_hip_decoder_generate(self.handle, prompt.ctypes.data, prompt.size, max_new,
-                                                        out.ctypes.data))
+        fn = _ffi.lib().llvq_hip_decoder_generate_prefilled if batched_prefill else _ffi.lib().llvq_hip_decoder_generate
+        _ffi.check(fn(self.handle, prompt.ctypes.data, prompt.size, max_new, out.ctypes.data))
         return out
 
     def close(self):

@@ -26,7 +26,7 @@ Q8 = decoder.Qwen3Config(num_hidden_layers=2, hidden_size=256, num_attention_hea
                          max_positions=80, tie_word_embeddings=True, kv_mode="q8")  # 5 query heads per kv head, as at 14B
 
 
-def _build(gpu_rt, orc, cfg, seed, rotate=False):
+def _build(gpu_rt, orc, cfg, seed, rotate=False, prefill_rows=0):
     from oracle import qwen3_oracle
 
     raws = decoder.synthetic_projections(cfg, seed)
@@ -41,7 +41,7 @@ def _build(gpu_rt, orc, cfg, seed, rotate=False):
     weights = decoder.synthetic_weights(cfg, seed)
     dense = [[orc.read_matrix_raw(artifact.write_matrix_raw(m))[0].decode_matrix() for m in layer] for layer in raws]
     ref = qwen3_oracle.Qwen3Oracle(cfg, dense, weights, kv_mode=cfg.kv_mode)
-    dec = decoder.Decoder(gpu_rt, cfg, raws, weights)
+    dec = decoder.Decoder(gpu_rt, cfg, raws, weights, prefill_rows=prefill_rows)
     return dec, ref
 
 
@@ -87,6 +87,49 @@ def test_rotated_projections_in_the_loop(gpu_rt, orc):
             got, _ = dec.forward_token(int(t))
             worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
         assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
+    finally:
+        dec.close()
+
+
+@pytest.mark.parametrize("cfg,seed,rotate", [(SMALL, 5, False), (RAGGED, 6, False), (Q8, 7, False), (SMALL, 8, True)])
+def test_batched_prefill_then_decode(gpu_rt, orc, cfg, seed, rotate):
+    """The prompt through the batched product, 16 positions a pass (three passes, the last one short),
+    then position-by-position decoding over the cache it left: logits against the oracle fed the same
+    tokens.  The batched product rounds weights to binary16 once, which is inside the bar the
+    token-by-token path is held to."""
+    dec, ref = _build(gpu_rt, orc, cfg, seed, rotate=rotate, prefill_rows=16)
+    try:
+        tokens = np.random.default_rng(seed).integers(0, cfg.vocab_size, size=min(38, cfg.max_positions - 7))
+        for t in tokens[:-1]:
+            ref.forward_token(int(t))
+        want = ref.forward_token(int(tokens[-1]))
+        got, best = dec.prefill(tokens)
+        assert dec.position == len(tokens)
+        worst = float(np.abs(got - want).max() / np.abs(want).max())
+        assert best == int(np.argmax(got))
+        for t in np.random.default_rng(seed + 100).integers(0, cfg.vocab_size, size=6):
+            want = ref.forward_token(int(t))
+            got, _ = dec.forward_token(int(t))
+            worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
+        assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
+    finally:
+        dec.close()
+
+
+def test_generate_with_batched_prefill_matches_token_by_token(gpu_rt, orc):
+    dec, ref = _build(gpu_rt, orc, SMALL, 3, prefill_rows=32)
+    try:
+        prompt = np.random.default_rng(3).integers(0, SMALL.vocab_size, size=40)
+        a = dec.generate(prompt, 24)
+        b = dec.generate(prompt, 24, batched_prefill=True)
+        same = a == b
+        if not same.all():  # a flip needs a near-tie in the oracle's own logits at that step
+            first = int(np.argmin(same))
+            _, trace = ref.generate(prompt, first + 1)
+            l = np.sort(trace[first])[-2:]
+            assert l[1] - l[0] < 5e-2 * np.abs(trace[first]).max(), f"first divergence at step {first} without a near-tie"
+        with pytest.raises(Exception):
+            decoder.Decoder(gpu_rt, SMALL, decoder.synthetic_projections(SMALL, 3), decoder.synthetic_weights(SMALL, 3)).prefill(prompt)
     finally:
         dec.close()
 
