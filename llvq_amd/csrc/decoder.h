@@ -245,8 +245,8 @@ __global__ __launch_bounds__(64) void norm_rope_append_rows_kernel(__half* __res
 // query at row r sees positions 0 .. pos0 + r.  Lane (pj, sub) = (lane / 16, lane % 16)
 // holds dims [8 sub, 8 sub + 8) of the positions j = pj (mod 4); each of the four position
 // classes keeps its own running maximum, sum and weighted V sum (f32), merged at the end.
-// head_dim <= 128, a multiple of 8.  q is already normed and rotated; ctx is rounded once.
-template <bool Q8>
+// head_dim <= 128, a multiple of 8; G >= query heads per kv head sizes the register arrays.  q is already normed and rotated; ctx is rounded once.
+template <bool Q8, int G>
 __global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict__ q, const __half* __restrict__ kcache,
                                                        const __half* __restrict__ vcache, KvQ8 q8, __half* __restrict__ ctx,
                                                        uint32_t n_heads, uint32_t n_kv, uint32_t head_dim, uint32_t pos0,
@@ -257,9 +257,9 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict_
   const bool active = i0 < head_dim;
   const uint32_t kvgroups = head_dim / kKvGroup;
   const size_t base = (size_t)kvh * max_pos;
-  float qv[kAttnMaxGroup][8], acc[kAttnMaxGroup][8], m[kAttnMaxGroup], l[kAttnMaxGroup];
+  float qv[G][8], acc[G][8], m[G], l[G];
 #pragma unroll
-  for (int g = 0; g < kAttnMaxGroup; ++g) {
+  for (int g = 0; g < G; ++g) {
     m[g] = -INFINITY;
     l[g] = 0.f;
 #pragma unroll
@@ -270,40 +270,60 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict_
                      : 0.f;
     }
   }
-  for (uint32_t j = pj; j < T; j += 4) {
-    float kf[8], vf[8];
+  // U positions of this lane's class per pass: their rows are requested together, then used in order
+  constexpr int U = 4;
+  for (uint32_t jb = pj; jb < T; jb += 4 * U) {
+    uint4 kraw[U], vraw[U];
+    float ks[U], kb[U], vs[U], vb[U];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) kf[t] = vf[t] = 0.f;
-    if (active) {
+    for (int u = 0; u < U; ++u) {
+      const uint32_t j = jb + 4u * u;
+      kraw[u] = vraw[u] = make_uint4(0, 0, 0, 0);
+      ks[u] = kb[u] = vs[u] = vb[u] = 0.f;
+      if (active && j < T) {
+        if constexpr (Q8) {
+          const uint2 kc = *reinterpret_cast<const uint2*>(q8.kq + (base + j) * head_dim + i0);
+          const uint2 vc = *reinterpret_cast<const uint2*>(q8.vq + (base + j) * head_dim + i0);
+          const size_t gi = (base + j) * kvgroups + i0 / kKvGroup;
+          kraw[u].x = kc.x; kraw[u].y = kc.y;
+          vraw[u].x = vc.x; vraw[u].y = vc.y;
+          ks[u] = __half2float(q8.ks[gi]); kb[u] = __half2float(q8.kb[gi]);
+          vs[u] = __half2float(q8.vs[gi]); vb[u] = __half2float(q8.vb[gi]);
+        } else {
+          kraw[u] = *reinterpret_cast<const uint4*>(kcache + (base + j) * head_dim + i0);
+          vraw[u] = *reinterpret_cast<const uint4*>(vcache + (base + j) * head_dim + i0);
+        }
+      }
+    }
+    // scores of the U positions first (independent exchanges), then the running sums in order
+    float sc[U][G], vfs[U][8];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float kf[8];
       if constexpr (Q8) {
-        const uint2 kc = *reinterpret_cast<const uint2*>(q8.kq + (base + j) * head_dim + i0);
-        const uint2 vc = *reinterpret_cast<const uint2*>(q8.vq + (base + j) * head_dim + i0);
-        const size_t gi = (base + j) * kvgroups + i0 / kKvGroup;
-        const float ks = __half2float(q8.ks[gi]), kb = __half2float(q8.kb[gi]);
-        const float vs = __half2float(q8.vs[gi]), vb = __half2float(q8.vb[gi]);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          kf[t] = kv_dequant((kc.x >> (8 * t)) & 0xFFu, ks, kb);
-          kf[4 + t] = kv_dequant((kc.y >> (8 * t)) & 0xFFu, ks, kb);
-          vf[t] = kv_dequant((vc.x >> (8 * t)) & 0xFFu, vs, vb);
-          vf[4 + t] = kv_dequant((vc.y >> (8 * t)) & 0xFFu, vs, vb);
+          kf[t] = kv_dequant((kraw[u].x >> (8 * t)) & 0xFFu, ks[u], kb[u]);
+          kf[4 + t] = kv_dequant((kraw[u].y >> (8 * t)) & 0xFFu, ks[u], kb[u]);
+          vfs[u][t] = kv_dequant((vraw[u].x >> (8 * t)) & 0xFFu, vs[u], vb[u]);
+          vfs[u][4 + t] = kv_dequant((vraw[u].y >> (8 * t)) & 0xFFu, vs[u], vb[u]);
         }
       } else {
-        const uint4 kr = *reinterpret_cast<const uint4*>(kcache + (base + j) * head_dim + i0);
-        const uint4 vr = *reinterpret_cast<const uint4*>(vcache + (base + j) * head_dim + i0);
-        const uint32_t kw[4] = {kr.x, kr.y, kr.z, kr.w}, vw[4] = {vr.x, vr.y, vr.z, vr.w};
+        const uint32_t kw[4] = {kraw[u].x, kraw[u].y, kraw[u].z, kraw[u].w}, vw[4] = {vraw[u].x, vraw[u].y, vraw[u].z, vraw[u].w};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           kf[2 * t] = __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu)));
           kf[2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16)));
-          vf[2 * t] = __half2float(__ushort_as_half((unsigned short)(vw[t] & 0xFFFFu)));
-          vf[2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(vw[t] >> 16)));
+          vfs[u][2 * t] = __half2float(__ushort_as_half((unsigned short)(vw[t] & 0xFFFFu)));
+          vfs[u][2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(vw[t] >> 16)));
         }
       }
-    }
+      if (!active) {
 #pragma unroll
-    for (int g = 0; g < kAttnMaxGroup; ++g)
-      if ((uint32_t)g < groups) {
+        for (int t = 0; t < 8; ++t) kf[t] = vfs[u][t] = 0.f;
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
         float d = 0.f;
 #pragma unroll
         for (int t = 0; t < 8; ++t) d = fmaf(qv[g][t], kf[t], d);
@@ -311,19 +331,30 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict_
         d += __shfl_xor(d, 2, 64);
         d += __shfl_xor(d, 4, 64);
         d += __shfl_xor(d, 8, 64);
-        const float mn = fmaxf(m[g], d);
-        const float c = __expf(m[g] - mn), p = __expf(d - mn);  // c = 0 on the first position (m = -inf)
-        l[g] = fmaf(l[g], c, p);
+        sc[u][g] = d;
+      }
+    }
 #pragma unroll
-        for (int t = 0; t < 8; ++t) acc[g][t] = fmaf(acc[g][t], c, p * vf[t]);
-        m[g] = mn;
+    for (int u = 0; u < U; ++u)
+      if (jb + 4u * u < T) {
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+          if ((uint32_t)g < groups) {
+            const float d = sc[u][g];
+            const float mn = fmaxf(m[g], d);
+            const float c = __expf(m[g] - mn), p = __expf(d - mn);  // c = 0 on the first position (m = -inf)
+            l[g] = fmaf(l[g], c, p);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc[g][t] = fmaf(acc[g][t], c, p * vfs[u][t]);
+            m[g] = mn;
+          }
       }
   }
   // merge the four position classes (a class with no position has m = -inf and weight 0)
 #pragma unroll
   for (int off = 16; off <= 32; off <<= 1)
 #pragma unroll
-    for (int g = 0; g < kAttnMaxGroup; ++g)
+    for (int g = 0; g < G; ++g)
       if ((uint32_t)g < groups) {
         const float mo = __shfl_xor(m[g], off, 64), lo = __shfl_xor(l[g], off, 64);
         const float mn = fmaxf(m[g], mo);
@@ -338,7 +369,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict_
       }
   if (pj == 0 && active)
 #pragma unroll
-    for (int g = 0; g < kAttnMaxGroup; ++g)
+    for (int g = 0; g < G; ++g)
       if ((uint32_t)g < groups) {
         __half* dst = ctx + ((size_t)row * n_heads + kvh * groups + g) * head_dim + i0;
         const float inv = 1.0f / l[g];

@@ -1782,16 +1782,24 @@ int decoder_prefill_pass(llvq_decoder* d, uint32_t n, bool want_logits, uint32_t
     nw.vcache = vc;
     nw.eps = d->eps;
     const dim3 hgrid(d->n_heads + 2 * d->n_kv, n), agrid(d->n_kv, n);
+    auto attend = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, agrid, dim3(64), 0, st, d->pq, kc, vc, lq8, d->pctx, d->n_heads, d->n_kv, d->head_dim, d->pos, d->max_pos, scale);
+    };
+    const uint32_t grp = d->n_heads / d->n_kv;
     if (d->kv_q8) {
       hipLaunchKernelGGL(norm_rope_append_rows_kernel<true>, hgrid, dim3(64), 0, st, d->pq, d->pk, d->pv, nw, lq8, d->n_heads, d->n_kv,
                          d->head_dim, d->pos, d->max_pos);
-      hipLaunchKernelGGL(attn_rows_kernel<true>, agrid, dim3(64), 0, st, d->pq, kc, vc, lq8, d->pctx, d->n_heads, d->n_kv, d->head_dim,
-                         d->pos, d->max_pos, scale);
+      if (grp <= 2) attend(attn_rows_kernel<true, 2>);
+      else if (grp <= 4) attend(attn_rows_kernel<true, 4>);
+      else if (grp <= 5) attend(attn_rows_kernel<true, 5>);
+      else attend(attn_rows_kernel<true, kAttnMaxGroup>);
     } else {
       hipLaunchKernelGGL(norm_rope_append_rows_kernel<false>, hgrid, dim3(64), 0, st, d->pq, d->pk, d->pv, nw, lq8, d->n_heads, d->n_kv,
                          d->head_dim, d->pos, d->max_pos);
-      hipLaunchKernelGGL(attn_rows_kernel<false>, agrid, dim3(64), 0, st, d->pq, kc, vc, lq8, d->pctx, d->n_heads, d->n_kv, d->head_dim,
-                         d->pos, d->max_pos, scale);
+      if (grp <= 2) attend(attn_rows_kernel<false, 2>);
+      else if (grp <= 4) attend(attn_rows_kernel<false, 4>);
+      else if (grp <= 5) attend(attn_rows_kernel<false, 5>);
+      else attend(attn_rows_kernel<false, kAttnMaxGroup>);
     }
     rc = rows(P[3], d->pctx, d->po);
     if (rc) return rc;
