@@ -121,7 +121,7 @@ __device__ __forceinline__ float kv_dequant(uint32_t q, float s, float b) {
 // out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i] sin + x[i + d/2] cos, with
 // the binary16 cos/sin tables of Rotary::new, model.rs:163-179).  Each step rounds to
 // binary16 as the reference's tensors do; the results are left, widened, in
-// stage[0, head_dim) — an LDS area of this wavefront alone.  head_dim <= 256.
+// stage[0, head_dim) — an LDS area of this wavefront alone.  head_dim <= 256 (the callers take 128).
 __device__ __forceinline__ void wave_lds_sync() {
   // LDS operations of one wavefront execute in order; only the compiler must not move them
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -169,6 +169,19 @@ __device__ __forceinline__ void norm_rope_wave(const __half* __restrict__ src, c
     }
   }
   wave_lds_sync();
+}
+
+// Sum over each row of 16 lanes, left in all 16 (four cross-lane moves inside the row).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float row16_sum(float x) {
+  x += dpp_move<0xB1>(x);   // quad_perm [1,0,3,2]: lane ^ 1
+  x += dpp_move<0x4E>(x);   // quad_perm [2,3,0,1]: lane ^ 2
+  x += dpp_move<0x141>(x);  // row_half_mirror: the other quad of the half row
+  x += dpp_move<0x140>(x);  // row_mirror: the other half of the row
+  return x;
 }
 
 // What the attention launch is handed about the position being decoded: the raw
@@ -327,11 +340,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict_
         float d = 0.f;
 #pragma unroll
         for (int t = 0; t < 8; ++t) d = fmaf(qv[g][t], kf[t], d);
-        d += __shfl_xor(d, 1, 64);
-        d += __shfl_xor(d, 2, 64);
-        d += __shfl_xor(d, 4, 64);
-        d += __shfl_xor(d, 8, 64);
-        sc[u][g] = d;
+        sc[u][g] = row16_sum(d);
       }
     }
 #pragma unroll
@@ -381,13 +390,16 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict_
 // Attention of one query position over the cache (model.rs:812-822), split over
 // the cache: workgroup (kv head, split) takes a contiguous range of positions
 // for all query heads that share the kv head, so every K and V row is fetched
-// (and, for the int8 cache, rebuilt) once per group.  Its four wavefronts take
-// positions round-robin, four positions at a time (16 lanes x 8 dims per row);
-// the workgroup leaves an unnormalised partial per query head (running max, sum
-// of exponentials, weighted V sum), and the workgroup that arrives last at the
-// kv head's counter merges the partials in split order and rounds the context
-// once.  Scores, softmax and sums stay in f32.
-template <bool Q8>
+// (and, for the int8 cache, rebuilt) once per group.  The range is walked once:
+// sixteen position classes (four per wavefront, 16 lanes x 8 dims each) keep a
+// running maximum, a sum of exponentials and a weighted V sum per query head,
+// with the K and V rows of four positions requested together; the classes meet
+// in LDS and the workgroup leaves an unnormalised partial per query head.  The
+// workgroup that arrives last at the kv head's counter merges the partials in
+// split order and rounds the context once.  Scores, softmax and sums stay in
+// f32.  head_dim <= 128, a multiple of 8; G >= query heads per kv head sizes
+// the register arrays.
+template <bool Q8, int G>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, const __half* __restrict__ kcache,
                                                                    const __half* __restrict__ vcache, KvQ8 q8,
                                                                    __half* __restrict__ ctx,
@@ -397,7 +409,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
                                                                    uint32_t merge_inline) {
   extern __shared__ __align__(16) float att_smem[];
   __shared__ uint32_t arrived;
-  __shared__ float red[kAttnWaves][kAttnMaxGroup];
   __shared__ float stage[kAttnWaves][256];  // one head per wavefront while it is normed and rotated
   __shared__ float knew[256], vnew[256];    // the new position's k and v as the cache returns them
   const uint32_t kvh = blockIdx.x / n_splits, split = blockIdx.x % n_splits;
@@ -406,8 +417,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
   const uint32_t chunk = (T + n_splits - 1) / n_splits;
   const uint32_t j0 = min(T, split * chunk), j1 = min(T, j0 + chunk), nj = j1 - j0;
   float* qs = att_smem;                         // [groups][head_dim]
-  float* sc = qs + groups * head_dim;           // [groups][chunk]
-  float* accs = sc + groups * chunk;            // [kAttnWaves][groups][head_dim]
+  float* cls = qs + groups * head_dim;          // [16 classes][groups][head_dim + 2]: running max, sum, weighted V sums
   const __half* K = kcache + (size_t)kvh * max_pos * head_dim;
   const __half* V = vcache + (size_t)kvh * max_pos * head_dim;
   const uint32_t kvgroups = head_dim / kKvGroup;
@@ -477,196 +487,136 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
   }
   __syncthreads();
 
-  // ---- scores ----
-  const uint32_t sub = lane & 15u, pj = lane >> 4;
-  const uint32_t dsteps = (head_dim + 127) >> 7;
-  float m[kAttnMaxGroup];
+  // ---- one pass over the range: scores, running maxima and weighted V sums together ----
+  // Lane (pj, sub) = (lane / 16, lane % 16) of wavefront w holds dims [8 sub, 8 sub + 8) of the
+  // positions of class c = 4 w + pj: jj = c, c + 16, ...  Each class keeps its own running
+  // maximum, sum of exponentials and weighted V sum (f32); U rows of K and of V are requested
+  // together, their scores are formed first (independent cross-lane sums), then folded in order.
+  const uint32_t sub = lane & 15u, pj = lane >> 4, i0 = sub * 8u, c = wave * 4u + pj;
+  const bool active = i0 < head_dim;
+  float qv[G][8], acc[G][8], m[G], l[G];
 #pragma unroll
-  for (int g = 0; g < kAttnMaxGroup; ++g) m[g] = -INFINITY;
-  constexpr int PB = 4;  // row pieces fetched together, so their latencies overlap
-  for (uint32_t pb0 = wave * 4u; pb0 < nj; pb0 += kAttnWaves * 4u * PB) {
-    for (uint32_t ds = 0; ds < dsteps; ++ds) {
-      const uint32_t i0 = ds * 128u + sub * 8u;
-      uint4 kraw[PB];
-      float ksc[PB], kbi[PB];
-#pragma unroll
-      for (int b = 0; b < PB; ++b) {
-        const uint32_t jj = pb0 + (uint32_t)b * kAttnWaves * 4u + pj, j = j0 + jj;
-        kraw[b] = make_uint4(0, 0, 0, 0);
-        ksc[b] = kbi[b] = 0.f;
-        if (jj < nj && i0 < head_dim && j != newj) {
-          if constexpr (Q8) {
-            const uint2 kc = *reinterpret_cast<const uint2*>(Kq + (size_t)j * head_dim + i0);
-            kraw[b].x = kc.x;
-            kraw[b].y = kc.y;
-            ksc[b] = __half2float(Ks[(size_t)j * kvgroups + i0 / kKvGroup]);
-            kbi[b] = __half2float(Kb[(size_t)j * kvgroups + i0 / kKvGroup]);
-          } else {
-            kraw[b] = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0);
-          }
-        }
-      }
-#pragma unroll
-      for (int b = 0; b < PB; ++b) {
-        const uint32_t jj = pb0 + (uint32_t)b * kAttnWaves * 4u + pj;
-        float d[kAttnMaxGroup];
-#pragma unroll
-        for (int g = 0; g < kAttnMaxGroup; ++g) d[g] = 0.f;
-        if (jj < nj && i0 < head_dim) {
-          float kf[8];
-          if (j0 + jj == newj) {
-#pragma unroll
-            for (int t = 0; t < 8; ++t) kf[t] = knew[i0 + t];
-          } else if constexpr (Q8) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              kf[t] = kv_dequant((kraw[b].x >> (8 * t)) & 0xFFu, ksc[b], kbi[b]);
-              kf[4 + t] = kv_dequant((kraw[b].y >> (8 * t)) & 0xFFu, ksc[b], kbi[b]);
-            }
-          } else {
-            const uint32_t kw[4] = {kraw[b].x, kraw[b].y, kraw[b].z, kraw[b].w};
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              kf[2 * t] = __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu)));
-              kf[2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16)));
-            }
-          }
-#pragma unroll
-          for (int g = 0; g < kAttnMaxGroup; ++g)
-            if ((uint32_t)g < groups) {
-              const float* qg = qs + g * head_dim + i0;
-#pragma unroll
-              for (int t = 0; t < 8; ++t) d[g] = fmaf(qg[t], kf[t], d[g]);
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < kAttnMaxGroup; ++g)
-          if ((uint32_t)g < groups) {
-            float v = d[g];
-            v += __shfl_xor(v, 1, 64);
-            v += __shfl_xor(v, 2, 64);
-            v += __shfl_xor(v, 4, 64);
-            v += __shfl_xor(v, 8, 64);
-            // a head wider than 128 accumulates its passes in the score slot
-            if (jj < nj && sub == 0) sc[g * chunk + jj] = ds ? sc[g * chunk + jj] + v : v;
-          }
-      }
-    }
-  }
-  __syncthreads();
-  // running maxima: every lane scans the scores of its positions
-  for (uint32_t jj = tid; jj < nj; jj += kAttnThreads)
-#pragma unroll
-    for (int g = 0; g < kAttnMaxGroup; ++g)
-      if ((uint32_t)g < groups) m[g] = fmaxf(m[g], sc[g * chunk + jj]);
-#pragma unroll
-  for (int g = 0; g < kAttnMaxGroup; ++g) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) m[g] = fmaxf(m[g], __shfl_xor(m[g], o, 64));
-    if (lane == 0) red[wave][g] = m[g];
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < kAttnMaxGroup; ++g) {
-    m[g] = red[0][g];
-#pragma unroll
-    for (int w = 1; w < kAttnWaves; ++w) m[g] = fmaxf(m[g], red[w][g]);
-  }
-  __syncthreads();  // red is reused for the sums
-  // ---- exponentials and their sums ----
-  float l[kAttnMaxGroup];
-#pragma unroll
-  for (int g = 0; g < kAttnMaxGroup; ++g) {
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
     l[g] = 0.f;
-    if ((uint32_t)g < groups)
-      for (uint32_t jj = tid; jj < nj; jj += kAttnThreads) {
-        const float e = __expf(sc[g * chunk + jj] - m[g]);
-        sc[g * chunk + jj] = e;
-        l[g] += e;
-      }
-    l[g] = wave_sum(l[g]);
-    if (lane == 0) red[wave][g] = l[g];
-  }
-  __syncthreads();
-  // ---- weighted V sums: wavefront w takes positions w, w + 4, ...; lane owns dims 2 lane, 2 lane + 1 of each 128 ----
-  for (uint32_t ds = 0; ds < dsteps; ++ds) {
-    const uint32_t i0 = ds * 128u + lane * 2u;
-    float a0[kAttnMaxGroup], a1[kAttnMaxGroup];
 #pragma unroll
-    for (int g = 0; g < kAttnMaxGroup; ++g) a0[g] = a1[g] = 0.f;
-    if (i0 < head_dim) {
-      constexpr int VB = 8;  // V rows fetched together
-      for (uint32_t jb = wave; jb < nj; jb += kAttnWaves * VB) {
-        uint32_t vraw[VB];
-        float vsc[VB], vbi[VB];
-#pragma unroll
-        for (int b = 0; b < VB; ++b) {
-          const uint32_t jj = jb + (uint32_t)b * kAttnWaves, j = j0 + jj;
-          vraw[b] = 0;
-          vsc[b] = vbi[b] = 0.f;
-          if (jj < nj && j != newj) {
-            if constexpr (Q8) {
-              vraw[b] = *reinterpret_cast<const unsigned short*>(Vq + (size_t)j * head_dim + i0);
-              vsc[b] = __half2float(Vs[(size_t)j * kvgroups + i0 / kKvGroup]);
-              vbi[b] = __half2float(Vb[(size_t)j * kvgroups + i0 / kKvGroup]);
-            } else {
-              vraw[b] = *reinterpret_cast<const uint32_t*>(V + (size_t)j * head_dim + i0);
-            }
-          }
-        }
-#pragma unroll
-        for (int b = 0; b < VB; ++b) {
-          const uint32_t jj = jb + (uint32_t)b * kAttnWaves;
-          if (jj < nj) {
-            float v0, v1;
-            if (j0 + jj == newj) {
-              v0 = vnew[i0];
-              v1 = vnew[i0 + 1];
-            } else if constexpr (Q8) {
-              v0 = kv_dequant(vraw[b] & 0xFFu, vsc[b], vbi[b]);
-              v1 = kv_dequant(vraw[b] >> 8, vsc[b], vbi[b]);
-            } else {
-              v0 = __half2float(__ushort_as_half((unsigned short)(vraw[b] & 0xFFFFu)));
-              v1 = __half2float(__ushort_as_half((unsigned short)(vraw[b] >> 16)));
-            }
-#pragma unroll
-            for (int g = 0; g < kAttnMaxGroup; ++g)
-              if ((uint32_t)g < groups) {
-                const float p = sc[g * chunk + jj];
-                a0[g] = fmaf(p, v0, a0[g]);
-                a1[g] = fmaf(p, v1, a1[g]);
-              }
-          }
-        }
-      }
-#pragma unroll
-      for (int g = 0; g < kAttnMaxGroup; ++g)
-        if ((uint32_t)g < groups) {
-          accs[((size_t)wave * groups + g) * head_dim + i0] = a0[g];
-          accs[((size_t)wave * groups + g) * head_dim + i0 + 1] = a1[g];
-        }
+    for (int t = 0; t < 8; ++t) {
+      acc[g][t] = 0.f;
+      qv[g][t] = ((uint32_t)g < groups && active) ? qs[g * head_dim + i0 + t] : 0.f;
     }
   }
+  constexpr int U = 4;
+  for (uint32_t jb = c; jb < nj; jb += 16u * U) {
+    uint4 kraw[U], vraw[U];
+    float ksc[U], kbi[U], vsc[U], vbi[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t jj = jb + 16u * u, j = j0 + jj;
+      kraw[u] = vraw[u] = make_uint4(0, 0, 0, 0);
+      ksc[u] = kbi[u] = vsc[u] = vbi[u] = 0.f;
+      if (active && jj < nj && j != newj) {
+        if constexpr (Q8) {
+          const uint2 kc = *reinterpret_cast<const uint2*>(Kq + (size_t)j * head_dim + i0);
+          const uint2 vc = *reinterpret_cast<const uint2*>(Vq + (size_t)j * head_dim + i0);
+          const size_t gi = (size_t)j * kvgroups + i0 / kKvGroup;
+          kraw[u].x = kc.x; kraw[u].y = kc.y;
+          vraw[u].x = vc.x; vraw[u].y = vc.y;
+          ksc[u] = __half2float(Ks[gi]); kbi[u] = __half2float(Kb[gi]);
+          vsc[u] = __half2float(Vs[gi]); vbi[u] = __half2float(Vb[gi]);
+        } else {
+          kraw[u] = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0);
+          vraw[u] = *reinterpret_cast<const uint4*>(V + (size_t)j * head_dim + i0);
+        }
+      }
+    }
+    float sc[U][G], vfs[U][8];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t jj = jb + 16u * u;
+      float kf[8];
+      if (j0 + jj == newj) {  // the row appended by this launch: from LDS, as the cache returns it
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          kf[t] = active ? knew[i0 + t] : 0.f;
+          vfs[u][t] = active ? vnew[i0 + t] : 0.f;
+        }
+      } else if constexpr (Q8) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          kf[t] = kv_dequant((kraw[u].x >> (8 * t)) & 0xFFu, ksc[u], kbi[u]);
+          kf[4 + t] = kv_dequant((kraw[u].y >> (8 * t)) & 0xFFu, ksc[u], kbi[u]);
+          vfs[u][t] = kv_dequant((vraw[u].x >> (8 * t)) & 0xFFu, vsc[u], vbi[u]);
+          vfs[u][4 + t] = kv_dequant((vraw[u].y >> (8 * t)) & 0xFFu, vsc[u], vbi[u]);
+        }
+      } else {
+        const uint32_t kw[4] = {kraw[u].x, kraw[u].y, kraw[u].z, kraw[u].w}, vw[4] = {vraw[u].x, vraw[u].y, vraw[u].z, vraw[u].w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          kf[2 * t] = __half2float(__ushort_as_half((unsigned short)(kw[t] & 0xFFFFu)));
+          kf[2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(kw[t] >> 16)));
+          vfs[u][2 * t] = __half2float(__ushort_as_half((unsigned short)(vw[t] & 0xFFFFu)));
+          vfs[u][2 * t + 1] = __half2float(__ushort_as_half((unsigned short)(vw[t] >> 16)));
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float d = 0.f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) d = fmaf(qv[g][t], kf[t], d);
+        sc[u][g] = row16_sum(d);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (jb + 16u * u < nj) {
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+          if ((uint32_t)g < groups) {
+            const float d = sc[u][g];
+            const float mn = fmaxf(m[g], d);
+            const float e0 = __expf(m[g] - mn), p = __expf(d - mn);  // e0 = 0 on the first position (m = -inf)
+            l[g] = fmaf(l[g], e0, p);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc[g][t] = fmaf(acc[g][t], e0, p * vfs[u][t]);
+            m[g] = mn;
+          }
+      }
+  }
+  // the classes' results meet in LDS
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+    if ((uint32_t)g < groups) {
+      float* dst = cls + ((size_t)c * groups + g) * stride;
+      if (sub == 0) {
+        dst[0] = m[g];
+        dst[1] = l[g];
+      }
+      if (active) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) dst[2 + i0 + t] = acc[g][t];
+      }
+    }
   __syncthreads();
-  // ---- this workgroup's partial: wavefront sums added in wavefront order ----
+  // ---- this workgroup's partial: the sixteen classes merged in class order ----
   for (uint32_t o = tid; o < groups * head_dim; o += kAttnThreads) {
     const uint32_t g = o / head_dim, i = o - g * head_dim;
-    float a = 0.f;
+    float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < kAttnWaves; ++w) a += accs[((size_t)w * groups + g) * head_dim + i];
-    part[((size_t)(kvh * groups + g) * n_splits + split) * stride + 2 + i] = a;
-  }
-  if (tid < groups) {
-    float ls = 0.f;
+    for (int cc = 0; cc < 16; ++cc) M = fmaxf(M, cls[((size_t)cc * groups + g) * stride]);
+    float A = 0.f, Lsum = 0.f;
 #pragma unroll
-    for (int w = 0; w < kAttnWaves; ++w) ls += red[w][tid];
-    float* dst = part + ((size_t)(kvh * groups + tid) * n_splits + split) * stride;
-    float mg = -INFINITY;  // m[] is register-indexed by a constant only: pick by comparison
-#pragma unroll
-    for (int g = 0; g < kAttnMaxGroup; ++g)
-      if ((uint32_t)g == tid) mg = m[g];
-    dst[0] = mg;  // -inf for an empty range
-    dst[1] = ls;
+    for (int cc = 0; cc < 16; ++cc) {
+      const float* src = cls + ((size_t)cc * groups + g) * stride;
+      const float wgt = src[0] == -INFINITY ? 0.f : __expf(src[0] - M);  // a class with no position
+      A = fmaf(src[2 + i], wgt, A);
+      Lsum = fmaf(src[1], wgt, Lsum);
+    }
+    float* dst = part + ((size_t)(kvh * groups + g) * n_splits + split) * stride;
+    dst[2 + i] = A;
+    if (i == 0) {
+      dst[0] = M;  // -inf for an empty range
+      dst[1] = Lsum;
+    }
   }
   if (!merge_inline) return;  // attn_merge_kernel finishes (long caches: many partials, merged chip-wide)
   // publish, and let the last workgroup of this kv head merge (one lane's

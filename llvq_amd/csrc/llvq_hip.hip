@@ -1640,7 +1640,8 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   uint32_t n_splits = (T + 31) / 32;  // about 32 cached positions per workgroup, at most kAttnMaxSplits ranges
   if (n_splits > (uint32_t)kAttnMaxSplits) n_splits = kAttnMaxSplits;
   const uint32_t groups_per_kv = d->n_heads / d->n_kv;
-  size_t attn_lds = ((size_t)groups_per_kv * d->head_dim * (1 + kAttnWaves) + (size_t)groups_per_kv * ((T + n_splits - 1) / n_splits)) * sizeof(float);
+  // the queries and the sixteen position classes' running results
+  size_t attn_lds = ((size_t)groups_per_kv * d->head_dim + (size_t)16 * groups_per_kv * (d->head_dim + 2)) * sizeof(float);
   const size_t merge_lds = (size_t)groups_per_kv * (n_splits + 1) * sizeof(float);  // the merge reuses the staging area
   if (attn_lds < merge_lds) attn_lds = merge_lds;
   const size_t group_layer = cache_layer / kKvGroup;
@@ -1704,14 +1705,22 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     nw.kcache = kc;
     nw.vcache = vc;
     nw.eps = d->eps;
-    if (d->kv_q8)
-      hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, nw, kc, vc, lq8,
-                         d->ctx, d->attn_part, d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
-                         1.0f / sqrtf((float)d->head_dim), n_splits, merge_inline);
-    else
-      hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, nw, kc, vc, lq8,
-                         d->ctx, d->attn_part, d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos,
-                         1.0f / sqrtf((float)d->head_dim), n_splits, merge_inline);
+    auto attend = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3(d->n_kv * n_splits), dim3(kAttnThreads), attn_lds, st, nw, kc, vc, lq8, d->ctx, d->attn_part,
+                         d->attn_counters, d->n_heads, d->n_kv, d->head_dim, T, d->max_pos, 1.0f / sqrtf((float)d->head_dim), n_splits,
+                         merge_inline);
+    };
+    if (d->kv_q8) {
+      if (groups_per_kv <= 2) attend(attn_decode_kernel<true, 2>);
+      else if (groups_per_kv <= 4) attend(attn_decode_kernel<true, 4>);
+      else if (groups_per_kv <= 5) attend(attn_decode_kernel<true, 5>);
+      else attend(attn_decode_kernel<true, kAttnMaxGroup>);
+    } else {
+      if (groups_per_kv <= 2) attend(attn_decode_kernel<false, 2>);
+      else if (groups_per_kv <= 4) attend(attn_decode_kernel<false, 4>);
+      else if (groups_per_kv <= 5) attend(attn_decode_kernel<false, 5>);
+      else attend(attn_decode_kernel<false, kAttnMaxGroup>);
+    }
     if (!merge_inline)
       hipLaunchKernelGGL(attn_merge_kernel, dim3(d->n_heads), dim3(128), 0, st, d->attn_part, d->ctx, d->head_dim, n_splits);
     void* o_out[1] = {d->o};
@@ -1857,14 +1866,13 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
                                               " — the kernels hard-code int8 g64 and hidden % 16 = 0");
     }
   if (c->n_layers == 0 || c->hidden == 0 || c->hidden % 8 || c->hidden > 8192 || c->n_heads == 0 || c->n_kv_heads == 0 ||
-      c->n_heads % c->n_kv_heads || c->n_heads / c->n_kv_heads > (uint32_t)kAttnMaxGroup || c->head_dim == 0 || c->head_dim % 8 || c->head_dim > 256 || c->intermediate == 0 ||
+      c->n_heads % c->n_kv_heads || c->n_heads / c->n_kv_heads > (uint32_t)kAttnMaxGroup || c->head_dim == 0 || c->head_dim % 8 || c->head_dim > 128 || c->intermediate == 0 ||
       c->vocab == 0 || c->max_positions == 0 || c->max_positions > 8192 ||
       (c->kv_mode != LLVQ_KV_F16 && c->kv_mode != LLVQ_KV_Q8) || (c->kv_mode == LLVQ_KV_Q8 && c->head_dim % 64))
     return fail(LLVQ_ERR_UNSUPPORTED,
-                "decoder_create: shape outside what the kernels hold (hidden % 8 = 0 and <= 8192, head_dim % 8 = 0 and <= 256, "
+                "decoder_create: shape outside what the kernels hold (hidden % 8 = 0 and <= 8192, head_dim % 8 = 0 and <= 128, "
                 "heads a multiple of kv heads and at most 8 per kv head, max_positions <= 8192, kv_mode f16 or q8 with head_dim % 64 = 0)");
-  if (c->prefill_rows && (c->head_dim > 128 || c->prefill_rows > 4096))
-    return fail(LLVQ_ERR_UNSUPPORTED, "decoder_create: the batched prompt path takes head_dim <= 128 and at most 4096 rows per pass");
+  if (c->prefill_rows > 4096) return fail(LLVQ_ERR_UNSUPPORTED, "decoder_create: the batched prompt path takes at most 4096 rows per pass");
   const uint32_t qd = c->n_heads * c->head_dim, kvd = c->n_kv_heads * c->head_dim;
   static const char* kSite[7] = {"q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"};
   const uint32_t want_out[7] = {qd, kvd, kvd, c->hidden, c->intermediate, c->intermediate, c->hidden};
