@@ -171,19 +171,6 @@ __device__ __forceinline__ void norm_rope_wave(const __half* __restrict__ src, c
   wave_lds_sync();
 }
 
-// Sum over each row of 16 lanes, left in all 16 (four cross-lane moves inside the row).
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float x) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false));
-}
-__device__ __forceinline__ float row16_sum(float x) {
-  x += dpp_move<0xB1>(x);   // quad_perm [1,0,3,2]: lane ^ 1
-  x += dpp_move<0x4E>(x);   // quad_perm [2,3,0,1]: lane ^ 2
-  x += dpp_move<0x141>(x);  // row_half_mirror: the other quad of the half row
-  x += dpp_move<0x140>(x);  // row_mirror: the other half of the row
-  return x;
-}
-
 // What the attention launch is handed about the position being decoded: the raw
 // q / k / v rows the projections left, the layer's q and k norm weights and the
 // rotary tables.  The launch norms and rotates its own query heads, and the one
@@ -598,25 +585,33 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
     }
   __syncthreads();
   // ---- this workgroup's partial: the sixteen classes merged in class order ----
-  for (uint32_t o = tid; o < groups * head_dim; o += kAttnThreads) {
-    const uint32_t g = o / head_dim, i = o - g * head_dim;
+  // per query head: the maximum over the classes, then each class's weight, once, into its slot for the maximum
+  if (tid < groups) {
     float M = -INFINITY;
 #pragma unroll
-    for (int cc = 0; cc < 16; ++cc) M = fmaxf(M, cls[((size_t)cc * groups + g) * stride]);
-    float A = 0.f, Lsum = 0.f;
+    for (int cc = 0; cc < 16; ++cc) M = fmaxf(M, cls[((size_t)cc * groups + tid) * stride]);
+    float Lsum = 0.f;
+#pragma unroll
+    for (int cc = 0; cc < 16; ++cc) {
+      float* src = cls + ((size_t)cc * groups + tid) * stride;
+      const float wgt = src[0] == -INFINITY ? 0.f : __expf(src[0] - M);  // a class with no position
+      Lsum = fmaf(src[1], wgt, Lsum);
+      src[0] = wgt;
+    }
+    float* dst = part + ((size_t)(kvh * groups + tid) * n_splits + split) * stride;
+    dst[0] = M;  // -inf for an empty range
+    dst[1] = Lsum;
+  }
+  __syncthreads();
+  for (uint32_t o = tid; o < groups * head_dim; o += kAttnThreads) {
+    const uint32_t g = o / head_dim, i = o - g * head_dim;
+    float A = 0.f;
 #pragma unroll
     for (int cc = 0; cc < 16; ++cc) {
       const float* src = cls + ((size_t)cc * groups + g) * stride;
-      const float wgt = src[0] == -INFINITY ? 0.f : __expf(src[0] - M);  // a class with no position
-      A = fmaf(src[2 + i], wgt, A);
-      Lsum = fmaf(src[1], wgt, Lsum);
+      A = fmaf(src[2 + i], src[0], A);
     }
-    float* dst = part + ((size_t)(kvh * groups + g) * n_splits + split) * stride;
-    dst[2 + i] = A;
-    if (i == 0) {
-      dst[0] = M;  // -inf for an empty range
-      dst[1] = Lsum;
-    }
+    part[((size_t)(kvh * groups + g) * n_splits + split) * stride + 2 + i] = A;
   }
   if (!merge_inline) return;  // attn_merge_kernel finishes (long caches: many partials, merged chip-wide)
   // publish, and let the last workgroup of this kv head merge (one lane's

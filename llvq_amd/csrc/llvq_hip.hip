@@ -83,10 +83,24 @@ __device__ __forceinline__ uint64_t read_record(const uint8_t* buf, size_t byte)
   return ((uint64_t)__builtin_bswap32(first) << 16) | (uint64_t)(__builtin_bswap32(second) >> 16);
 }
 
+// Sum over each row of 16 lanes, left in all 16 (four cross-lane moves inside the row).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float row16_sum(float x) {
+  x += dpp_move<0xB1>(x);   // quad_perm [1,0,3,2]: lane ^ 1
+  x += dpp_move<0x4E>(x);   // quad_perm [2,3,0,1]: lane ^ 2
+  x += dpp_move<0x141>(x);  // row_half_mirror: the other quad of the half row
+  x += dpp_move<0x140>(x);  // row_mirror: the other half of the row
+  return x;
+}
+
+// Sum over the wavefront, the same value in every lane: the four rows' sums are read as scalars.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
+  v = row16_sum(v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16)) +
+         __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
 }
 
 // ---- parity probe: unrank records to points -----------------------------------
