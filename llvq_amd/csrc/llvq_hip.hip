@@ -516,7 +516,9 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
 
 // LEAN: the Golay words and the support-arrangement table stay in L2, which leaves
 // room for the full tile beside the activation planes of a very wide row.
-template <typename OutT, int TILE = LLVQ_TILE_BLOCKS, bool LEAN = false>
+// ROT: the launch can rotate its own activation (GroupArgs::rot_m); kept out of the other
+// instantiations, whose hot loop it would otherwise cost registers and a few per cent.
+template <typename OutT, int TILE = LLVQ_TILE_BLOCKS, bool LEAN = false, bool ROT = false>
 __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   // the tile capacity of this instantiation (these shadow the namespace-level defaults)
   constexpr int kTileBlocks = TILE;
@@ -544,7 +546,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   // A launch over matrices stored in a rotated basis rotates its activation itself: the
   // values go, signs applied, as f32 to the area the first tile's code bytes, queues and
   // partial sums will use (free until then), are rotated there and quantised from there.
-  const bool rotated = a.rot_m != 0;
+  const bool rotated = ROT && a.rot_m != 0;
   float* xf = reinterpret_cast<float*>(raw);
   const uint32_t d_in = nb * kDim + a.tail_w;
   auto signed_f32 = [&](uint32_t i, float v) { return ((a.rot_signbits[i >> 5] >> (i & 31u)) & 1u) ? -v : v; };
@@ -781,6 +783,27 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 }
 
 
+// The instantiations of gemv_tiles_kernel by (f32 output, tile, lean image, in-launch rotation).
+template <typename OutT, bool ROT>
+__host__ const void* gemv_kernel_of(uint32_t tile, bool lean) {
+  if (lean) return reinterpret_cast<const void*>(gemv_tiles_kernel<OutT, LLVQ_TILE_BLOCKS, true, ROT>);
+  if (tile == (uint32_t)LLVQ_TILE_BLOCKS) return reinterpret_cast<const void*>(gemv_tiles_kernel<OutT, LLVQ_TILE_BLOCKS, false, ROT>);
+  return reinterpret_cast<const void*>(gemv_tiles_kernel<OutT, kSmallTileBlocks, false, ROT>);
+}
+__host__ const void* gemv_kernel(bool f32, uint32_t tile, bool lean, bool rot) {
+  if (f32) return rot ? gemv_kernel_of<float, true>(tile, lean) : gemv_kernel_of<float, false>(tile, lean);
+  return rot ? gemv_kernel_of<__half, true>(tile, lean) : gemv_kernel_of<__half, false>(tile, lean);
+}
+template <class Fn>
+__host__ void for_each_gemv_kernel(Fn&& fn) {
+  for (int f32 = 0; f32 < 2; ++f32)
+    for (int rot = 0; rot < 2; ++rot) {
+      fn(gemv_kernel(f32, LLVQ_TILE_BLOCKS, false, rot));
+      fn(gemv_kernel(f32, kSmallTileBlocks, false, rot));
+      fn(gemv_kernel(f32, LLVQ_TILE_BLOCKS, true, rot));
+    }
+}
+
 // ---- incoherence rotation of an activation ----------------------------------------
 // x' = Q x for Q = (S (x) I_m)(I_k (x) H_m / sqrt m) D (llvq-quant/src/rotation.rs:97-105),
 // in f32 like the reference's device rotation (llvq-cuda/kernels/llvq_rot.cuh): signs on
@@ -935,12 +958,7 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   rt->tables.expand = reinterpret_cast<const uint32_t*>(rt->blob + off_exp);
   // the activation tile of a wide matrix pushes dynamic LDS past the 64 KB default
   const int max_lds = 160 * 1024;
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float, kSmallTileBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half, kSmallTileBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<float, kTileBlocks, true>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_tiles_kernel<__half, kTileBlocks, true>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  for_each_gemv_kernel([&](const void* kernel) { (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds); });
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
@@ -1309,22 +1327,9 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   }
   a.n_tiles = tiles;
   const uint32_t grid = tiles < grid_cap ? tiles : grid_cap;
-  if (shape.lean) {
-    if (y_dtype == LLVQ_F32)
-      hipLaunchKernelGGL((gemv_tiles_kernel<float, kTileBlocks, true>), dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
-    else
-      hipLaunchKernelGGL((gemv_tiles_kernel<__half, kTileBlocks, true>), dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
-  } else if (tile == (uint32_t)kTileBlocks) {
-    if (y_dtype == LLVQ_F32)
-      hipLaunchKernelGGL(gemv_tiles_kernel<float>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
-    else
-      hipLaunchKernelGGL(gemv_tiles_kernel<__half>, dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
-  } else {
-    if (y_dtype == LLVQ_F32)
-      hipLaunchKernelGGL((gemv_tiles_kernel<float, kSmallTileBlocks>), dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
-    else
-      hipLaunchKernelGGL((gemv_tiles_kernel<__half, kSmallTileBlocks>), dim3(grid), dim3(kWgThreads), lds, rt->stream, a);
-  }
+  const void* kernel = gemv_kernel(y_dtype == LLVQ_F32, tile, shape.lean, rot != nullptr);
+  void* params[] = {&a};
+  HIP_TRY(hipLaunchKernel(kernel, dim3(grid), dim3(kWgThreads), params, lds, rt->stream));
   HIP_TRY(hipGetLastError());
   return LLVQ_OK;
 }
