@@ -1656,7 +1656,8 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, d->h);
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
   const uint32_t T = d->pos + 1;
-  uint32_t n_splits = (T + 31) / 32;  // about 32 cached positions per workgroup, at most kAttnMaxSplits ranges
+  // about 64 cached positions per workgroup (one batch of four per position class), at most kAttnMaxSplits ranges
+  uint32_t n_splits = (T + 63) / 64;
   if (n_splits > (uint32_t)kAttnMaxSplits) n_splits = kAttnMaxSplits;
   const uint32_t groups_per_kv = d->n_heads / d->n_kv;
   // the queries and the sixteen position classes' running results

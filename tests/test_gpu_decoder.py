@@ -135,19 +135,19 @@ def test_generate_with_batched_prefill_matches_token_by_token(gpu_rt, orc):
 
 
 def test_long_cache_takes_the_merge_kernel(gpu_rt, orc):
-    """Past 512 cached positions the attention partials (more than 16 ranges) are merged
+    """Past 1024 cached positions the attention partials (more than 16 ranges of 64) are merged
     by a kernel of their own; the logits must keep agreeing with the oracle across the switch."""
     import dataclasses
 
-    cfg = dataclasses.replace(Q8, num_hidden_layers=1, max_positions=560, vocab_size=200)
+    cfg = dataclasses.replace(Q8, num_hidden_layers=1, max_positions=1080, vocab_size=200)
     dec, ref = _build(gpu_rt, orc, cfg, 9)
     try:
-        tokens = np.random.default_rng(9).integers(0, cfg.vocab_size, size=548)
+        tokens = np.random.default_rng(9).integers(0, cfg.vocab_size, size=1070)
         worst = 0.0
         for i, t in enumerate(tokens):
             want = ref.forward_token(int(t))
-            got, _ = dec.forward_token(int(t), want_logits=i >= 500)
-            if i >= 500:
+            got, _ = dec.forward_token(int(t), want_logits=i >= 1000)
+            if i >= 1000:
                 worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
         assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
     finally:
