@@ -316,8 +316,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
-        log("bench.py measures one GPU: this build has no multi-GPU path (rows shard trivially; see DESIGN.md). "
-            "Run with --gpus 1.")
+        log("bench.py measures one GPU: this build has no multi-GPU path (the rows of a matrix are independent, "
+            "so more GPUs would each take a share of them). Run with --gpus 1.")
         sys.exit(2)
 
     import torch
