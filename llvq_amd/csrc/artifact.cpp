@@ -126,18 +126,18 @@ int parse_matrix_record(const uint8_t* buf, size_t len, size_t* pos, RecordView*
   if ((uint64_t)r.n_centroids * 8 > c.left()) return truncated(err, "centroids");
   r.centroids_off = c.pos;
   r.centroids.resize(r.n_centroids);
-  std::memcpy(r.centroids.data(), buf + c.pos, (size_t)r.n_centroids * 8);
+  if (r.n_centroids) std::memcpy(r.centroids.data(), buf + c.pos, (size_t)r.n_centroids * 8);
   c.pos += (size_t)r.n_centroids * 8;
   if ((uint64_t)r.d_out * 8 > c.left()) return truncated(err, "row scales");
   r.row_scales_off = c.pos;
   r.row_scales.resize(r.d_out);
-  std::memcpy(r.row_scales.data(), buf + c.pos, (size_t)r.d_out * 8);
+  if (r.d_out) std::memcpy(r.row_scales.data(), buf + c.pos, (size_t)r.d_out * 8);
   c.pos += (size_t)r.d_out * 8;
   const uint64_t tail_n = (uint64_t)r.d_out * (r.d_in % kDim);
   if (tail_n * 4 > c.left()) return truncated(err, "tail");
   r.tail_off = c.pos;
   r.tail.resize((size_t)tail_n);
-  std::memcpy(r.tail.data(), buf + c.pos, (size_t)tail_n * 4);
+  if (tail_n) std::memcpy(r.tail.data(), buf + c.pos, (size_t)tail_n * 4);  // an empty vector has no address to copy to
   c.pos += (size_t)tail_n * 4;
 
   uint64_t nbytes;

@@ -1,0 +1,105 @@
+// Host-side robustness driver, built with -fsanitize=address,undefined by tests/test_host_sanitized.py:
+// every prefix of a sealed file and a few thousand corrupted copies go through the library's readers
+// (the cases of llvq-artifact/tests/hostile_files.rs, generalised: always a status, never a fault), and
+// the index decoder the kernels share with the host runs on class boundaries and random 48-bit ranks.
+// Each input lives in a heap block of exactly its size, so a read past the end is reported.
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../llvq_amd/csrc/artifact.hpp"
+#include "../llvq_amd/csrc/codebook.hpp"
+
+using namespace llvq;
+
+static uint64_t rng_state = 1;
+static uint64_t next_u64() {  // SplitMix64
+  uint64_t z = (rng_state += 0x9E3779B97F4A7C15ULL);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+  return z ^ (z >> 31);
+}
+
+// header, matrix records, raw tensors, blobs; stops at the first refusal.  Returns the records read.
+static size_t read_all(const uint8_t* buf, size_t len) {
+  size_t pos = 0, seen = 0;
+  uint32_t version = 0, n = 0;
+  std::string err;
+  if (parse_header(buf, len, &pos, &version, &n, &err)) return seen;
+  for (uint32_t i = 0; i < n; ++i) {
+    RecordView r;
+    if (parse_matrix_record(buf, len, &pos, &r, &err)) return seen;
+    if (r.codes_off + r.code_bytes > len) { std::fprintf(stderr, "record view past the buffer\n"); std::abort(); }
+    ++seen;
+  }
+  if (version < 2) return seen;
+  auto read_u32 = [&](uint32_t* v) {
+    if (pos + 4 > len) return false;
+    std::memcpy(v, buf + pos, 4);
+    pos += 4;
+    return true;
+  };
+  uint32_t n_raw = 0, n_blob = 0;
+  if (!read_u32(&n_raw)) return seen;
+  for (uint32_t i = 0; i < n_raw; ++i) {
+    RawTensorView t;
+    if (parse_raw_tensor(buf, len, &pos, version, &t, &err)) return seen;
+    if (t.data_off + t.data_len > len) { std::fprintf(stderr, "tensor view past the buffer\n"); std::abort(); }
+    ++seen;
+  }
+  if (!read_u32(&n_blob)) return seen;
+  for (uint32_t i = 0; i < n_blob; ++i) {
+    BlobView b;
+    if (parse_blob(buf, len, &pos, &b, &err)) return seen;
+    if (b.data_off + b.data_len > len) { std::fprintf(stderr, "blob view past the buffer\n"); std::abort(); }
+    ++seen;
+  }
+  return seen;
+}
+
+int main(int argc, char** argv) {
+  if (argc < 4) return 2;
+  std::FILE* f = std::fopen(argv[1], "rb");
+  if (!f) return 2;
+  std::vector<uint8_t> file;
+  uint8_t tmp[4096];
+  for (size_t k; (k = std::fread(tmp, 1, sizeof tmp, f)) > 0;) file.insert(file.end(), tmp, tmp + k);
+  std::fclose(f);
+  rng_state = std::strtoull(argv[2], nullptr, 10);
+  const size_t n_mut = std::strtoull(argv[3], nullptr, 10);
+
+  const size_t whole = read_all(file.data(), file.size());
+  size_t cases = 0;
+  // every prefix (all of the short ones, a stride through the long code streams)
+  for (size_t len = 0; len < file.size(); len += (len < 4096 || file.size() - len < 4096) ? 1 : 97) {
+    std::unique_ptr<uint8_t[]> p(new uint8_t[len ? len : 1]);
+    std::memcpy(p.get(), file.data(), len);
+    if (read_all(p.get(), len) > whole) return 3;
+    ++cases;
+  }
+  // corrupted copies: a few bytes replaced, mostly inside the headers of the records
+  for (size_t m = 0; m < n_mut; ++m) {
+    std::unique_ptr<uint8_t[]> p(new uint8_t[file.size()]);
+    std::memcpy(p.get(), file.data(), file.size());
+    const int flips = 1 + (int)(next_u64() % 4);
+    for (int k = 0; k < flips; ++k) {
+      const size_t span = (next_u64() & 1) ? std::min<size_t>(file.size(), 512) : file.size();
+      p[next_u64() % span] = (uint8_t)next_u64();
+    }
+    (void)read_all(p.get(), file.size());
+    ++cases;
+  }
+  // the index decoder: boundaries of the 48-bit field, the ends of the valid range, random ranks
+  int8_t pt[kDim];
+  int shell = 0;
+  size_t valid = 0;
+  const uint64_t edges[] = {0, 1, 2, 196560, 196561, kN13 - 1, kN13, kN13 + 1, (1ULL << 47) - 1, 1ULL << 47, (1ULL << 48) - 1, ~0ULL};
+  for (uint64_t e : edges) valid += host_decode(e, pt, &shell) ? 1 : 0;
+  for (size_t m = 0; m < 200000; ++m) valid += host_decode(next_u64() >> 16, pt, &shell) ? 1 : 0;
+  std::printf("ok: %zu records in the whole file, %zu hostile inputs, %zu decodable ranks\n", whole, cases, valid);
+  return 0;
+}
