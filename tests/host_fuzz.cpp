@@ -1,7 +1,8 @@
 // Host-side robustness driver, built with -fsanitize=address,undefined by tests/test_host_sanitized.py:
 // every prefix of a sealed file and a few thousand corrupted copies go through the library's readers
 // (the cases of llvq-artifact/tests/hostile_files.rs, generalised: always a status, never a fault), and
-// the index decoder the kernels share with the host runs on class boundaries and random 48-bit ranks.
+// the index decoder the kernels share with the host runs on class boundaries and random 48-bit ranks, and the
+// rotation tables are built and applied for served and awkward widths.
 // Each input lives in a heap block of exactly its size, so a read past the end is reported.
 #include <cstdint>
 #include <cstdio>
@@ -13,6 +14,7 @@
 
 #include "../llvq_amd/csrc/artifact.hpp"
 #include "../llvq_amd/csrc/codebook.hpp"
+#include "../llvq_amd/csrc/rotation.hpp"
 
 using namespace llvq;
 
@@ -100,6 +102,21 @@ int main(int argc, char** argv) {
   const uint64_t edges[] = {0, 1, 2, 196560, 196561, kN13 - 1, kN13, kN13 + 1, (1ULL << 47) - 1, 1ULL << 47, (1ULL << 48) - 1, ~0ULL};
   for (uint64_t e : edges) valid += host_decode(e, pt, &shell) ? 1 : 0;
   for (size_t m = 0; m < 200000; ++m) valid += host_decode(next_u64() >> 16, pt, &shell) ? 1 : 0;
-  std::printf("ok: %zu records in the whole file, %zu hostile inputs, %zu decodable ranks\n", whole, cases, valid);
+  // rotation tables of served and awkward widths (an odd factor above 32 is a refusal, not a fault)
+  size_t rotations = 0;
+  for (uint32_t n : {1u, 8u, 24u, 104u, 256u, 1000u, 2560u, 2568u, 4096u, 9728u, 17408u}) {
+    RotationTables t;
+    std::string why;
+    if (!build_rotation(n, next_u64(), &t, &why)) continue;
+    std::vector<double> v(n);
+    for (uint32_t i = 0; i < n; ++i) v[i] = (double)(int64_t)(next_u64() >> 40) / (double)(1 << 23) - 1.0;
+    double before = 0, after = 0;
+    for (double x : v) before += x * x;
+    host_rotate(t, &v);
+    for (double x : v) after += x * x;
+    if (!(after > 0.999 * before && after < 1.001 * before)) { std::fprintf(stderr, "rotation of width %u does not keep the norm\n", n); return 4; }
+    ++rotations;
+  }
+  std::printf("ok: %zu records in the whole file, %zu hostile inputs, %zu decodable ranks, %zu rotations\n", whole, cases, valid, rotations);
   return 0;
 }

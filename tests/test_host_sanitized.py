@@ -1,6 +1,6 @@
 """The library's host code under AddressSanitizer and UBSan (host only; no GPU): the file readers on
-every prefix and on corrupted copies of a sealed file, and the shared index decoder on boundaries and
-random ranks.  Reader refusals are pinned case by case elsewhere; this run is about never faulting."""
+every prefix and on corrupted copies of a sealed file, the shared index decoder on boundaries and
+random ranks, the rotation tables on served and awkward widths.  Reader refusals are pinned case by case elsewhere; this run is about never faulting."""
 import os
 import subprocess
 
@@ -17,7 +17,7 @@ def test_readers_and_decoder_under_sanitizers(tmp_path):
     exe = tmp_path / "host_fuzz"
     cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
            "-fno-omit-frame-pointer", "-o", str(exe), os.path.join(ROOT, "tests", "host_fuzz.cpp"),
-           os.path.join(CSRC, "artifact.cpp"), os.path.join(CSRC, "codebook.cpp")]
+           os.path.join(CSRC, "artifact.cpp"), os.path.join(CSRC, "codebook.cpp"), os.path.join(CSRC, "rotation.cpp")]
     built = subprocess.run(cmd, capture_output=True, text=True)
     if built.returncode != 0 and "sanitize" in built.stderr and "cannot find" in built.stderr:
         pytest.skip("the sanitizer runtimes are not installed with this g++")
