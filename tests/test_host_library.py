@@ -206,3 +206,37 @@ def test_library_refuses_hostile_sealed_sections():
         with pytest.raises(LlvqError) as e:
             _parse_raw(honest[:cut])
         assert e.value.kind == "Truncated"
+
+
+def test_header_is_plain_c_and_matches_the_python_mirror(tmp_path):
+    """include/llvq_hip.h compiles as C99 (the boundary is a C ABI, not a C++ one), a C caller links and
+    runs the host-only entry points, and the structs have the layout the ctypes mirror assumes."""
+    import subprocess
+
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include <stddef.h>
+#include <stdio.h>
+#include "llvq_hip.h"
+int main(void) {
+  signed char pt[24];
+  int shell = 0;
+  if (llvq_hip_codebook_fingerprint() != 0x338f420f11866319ULL) return 3;
+  if (llvq_hip_host_decode(1, pt, &shell) != 1 || shell != 2) return 4;
+  printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(llvq_matrix_desc), sizeof(llvq_decoder_desc), sizeof(llvq_quant_rows),
+         sizeof(llvq_raw_info), sizeof(llvq_blob_info), offsetof(llvq_decoder_desc, kv_mode), offsetof(llvq_decoder_desc, prefill_rows));
+  return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(_ffi.lib_path())
+    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(src),
+           "-o", str(exe), "-L", libdir, "-lllvq_hip", "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"]
+    built = subprocess.run(cmd, capture_output=True, text=True)
+    assert built.returncode == 0, built.stderr[-2000:]
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.returncode, run.stderr[-500:])
+    got = [int(v) for v in run.stdout.split()]
+    want = [C.sizeof(_ffi.MatrixDesc), C.sizeof(_ffi.DecoderDesc), C.sizeof(_ffi.QuantRows), C.sizeof(_ffi.RawInfo),
+            C.sizeof(_ffi.BlobInfo), _ffi.DecoderDesc.kv_mode.offset, _ffi.DecoderDesc.prefill_rows.offset]
+    assert got == want
