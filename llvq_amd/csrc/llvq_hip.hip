@@ -1533,7 +1533,9 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
 }
 
 int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y, int y_dtype) {
-  if (!rt || !m || !x || !y || M < 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: bad argument");
+  if (!rt || !m || M < 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: bad argument");
+  if (M == 0) return LLVQ_OK;  // no rows: nothing is read or written, so the pointers may be null
+  if (!x || !y) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: null activation or output");
   if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: unknown output dtype");
   HIP_TRY(hipSetDevice(rt->device));
   const size_t esz = y_dtype == LLVQ_F32 ? 4 : 2;

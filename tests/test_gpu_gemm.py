@@ -102,6 +102,33 @@ def test_gemm_origin_shell13_and_generic_blocks(gpu_rt, orc, boundary_indices):
     _check(Y, Y_ref, A_ref)
 
 
+def test_gemm_degenerate_batches(gpu_rt, orc):
+    """One row takes the GEMV; no rows is a no-op that leaves the output alone; a matrix with no whole
+    block (tail columns only) goes row by row."""
+    import torch
+
+    raw = synth.make_matrix("model.layers.0.degenerate.weight", 24, 488, seed=3)
+    X = synth.make_activation(488, seed=4, rows=3)
+    proj = gpu_rt.upload(raw)
+    tiny = synth.make_matrix("model.layers.0.tailonly.weight", 8, 16, seed=5)
+    ptiny = gpu_rt.upload(tiny)
+    try:
+        xs = torch.from_numpy(X.view(np.int16).copy()).view(torch.float16).cuda()
+        one = gpu_rt.forward_batched(proj, xs[:1], out_dtype=torch.float32).cpu().numpy()
+        three = gpu_rt.forward_batched(proj, xs, out_dtype=torch.float32).cpu().numpy()
+        assert np.abs(one[0] - three[0]).max() <= 2e-3 * np.abs(three[0]).max()  # GEMV (exact weights) vs matrix cores (binary16 weights)
+        none = gpu_rt.forward_batched(proj, xs[:0], out_dtype=torch.float32)
+        assert tuple(none.shape) == (0, 24)
+        Xt = synth.make_activation(16, seed=6, rows=5)
+        yt = gpu_rt.forward_batched(ptiny, torch.from_numpy(Xt.view(np.int16).copy()).view(torch.float16).cuda(),
+                                    out_dtype=torch.float32).cpu().numpy()
+        want = Xt.astype(np.float64) @ tiny.tail.reshape(8, 16).astype(np.float64).T
+        assert np.abs(yt - want).max() <= 1e-5 * np.abs(want).max()
+    finally:
+        gpu_rt.free(proj)
+        gpu_rt.free(ptiny)
+
+
 def test_gemm_matches_gemv_rows(gpu_rt):
     """The batched kernel against the single-row kernel of the same library."""
     import torch
