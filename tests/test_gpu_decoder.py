@@ -174,6 +174,39 @@ def test_greedy_tokens_match_oracle(gpu_rt, orc):
         dec.close()
 
 
+def test_decoder_refusals_are_errors_not_faults(gpu_rt):
+    """Positions past the cache, tokens outside the vocabulary, a prompt that cannot fit: a status and a
+    message each time (fused_cuda.rs:365-375 convention), and the decoder stays usable afterwards."""
+    from llvq_amd import LlvqError
+
+    raws = decoder.synthetic_projections(RAGGED, 1)
+    weights = decoder.synthetic_weights(RAGGED, 1)
+    dec = decoder.Decoder(gpu_rt, RAGGED, raws, weights, prefill_rows=8)
+    try:
+        with pytest.raises(LlvqError, match="vocabulary"):
+            dec.forward_token(RAGGED.vocab_size)
+        with pytest.raises(LlvqError, match="max_positions"):
+            dec.generate(np.arange(30), RAGGED.max_positions)  # 30 + 40 - 1 positions
+        with pytest.raises(LlvqError, match="empty prompt"):
+            dec.generate(np.zeros(0, np.uint32), 3)
+        assert dec.generate(np.arange(5), 0).size == 0  # model.rs:1052-1054: nothing asked, nothing done
+        with pytest.raises(LlvqError, match="max_positions"):
+            dec.prefill(np.arange(RAGGED.max_positions + 1) % RAGGED.vocab_size)
+        with pytest.raises(LlvqError, match="vocabulary"):
+            dec.prefill([1, 2, RAGGED.vocab_size])
+        # exactly to the end of the cache, then one more position is refused
+        dec.reset()
+        dec.prefill(np.arange(RAGGED.max_positions - 1) % RAGGED.vocab_size)
+        dec.forward_token(0)
+        assert dec.position == RAGGED.max_positions
+        with pytest.raises(LlvqError, match="max_positions"):
+            dec.forward_token(0)
+        out = dec.generate(np.arange(6), 4)  # still usable
+        assert out.shape == (4,)
+    finally:
+        dec.close()
+
+
 def test_kv_mode_is_parsed_strictly(gpu_rt):
     """KvMode::parse (kvq.rs:38-49, test :240-249): a typo is an error, never a silent default."""
     import dataclasses
