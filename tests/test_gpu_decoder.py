@@ -174,6 +174,35 @@ def test_greedy_tokens_match_oracle(gpu_rt, orc):
         dec.close()
 
 
+def test_full_width_layers_tokens_match_oracle(gpu_rt, orc):
+    """Six layers at the Qwen3-4B widths (hidden 2560, 32/8 heads of 128, intermediate 9728, vocabulary
+    151 936, untied f16 head): greedy tokens of the device loop, token by token and with the prompt through
+    the batched path, against the oracle runner over the same weights decoded on the CPU.  (All 36 layers,
+    run by hand the same way, give 40 identical tokens; that takes two minutes and 30 GB of host memory.)"""
+    import dataclasses
+
+    from oracle import qwen3_oracle
+
+    cfg = dataclasses.replace(decoder.QWEN3_4B, num_hidden_layers=6, max_positions=96)
+    raws = decoder.synthetic_projections(cfg, 0)
+    weights = decoder.synthetic_weights(cfg, 0)
+    dense = [[orc.read_matrix_raw(artifact.write_matrix_raw(m))[0].decode_matrix() for m in layer] for layer in raws]
+    ref = qwen3_oracle.Qwen3Oracle(cfg, dense, weights)
+    dec = decoder.Decoder(gpu_rt, cfg, raws, weights, prefill_rows=16)
+    try:
+        prompt = np.random.default_rng(0).integers(0, cfg.vocab_size, size=24)
+        want, trace = ref.generate(prompt, 24)
+        for batched in (False, True):
+            got = dec.generate(prompt, 24, batched_prefill=batched)
+            same = want == got
+            if not same.all():  # only a near-tie of the oracle's own logits may flip a token
+                first = int(np.argmin(same))
+                l = np.sort(trace[first])[-2:]
+                assert l[1] - l[0] < 1e-2 * np.abs(trace[first]).max(), (batched, first, float(l[1] - l[0]))
+    finally:
+        dec.close()
+
+
 def test_decoder_refusals_are_errors_not_faults(gpu_rt):
     """Positions past the cache, tokens outside the vocabulary, a prompt that cannot fit: a status and a
     message each time (fused_cuda.rs:365-375 convention), and the decoder stays usable afterwards."""
