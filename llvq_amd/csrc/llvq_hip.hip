@@ -683,16 +683,42 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     // counter: the generic chunk first (longest), then odd, then even.
     const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
     const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
-    for (;;) {
-      uint32_t chunk = 0;
-      if (lane == 0) chunk = atomicAdd(&ctrl[3], 1u);
-      chunk = __shfl(chunk, 0, 64);
-      if (chunk >= c_gen + c_odd + c_even) break;
+    // the ticket counter hands out the generic chunk first (longest), then odd, then even chunks
+    auto ticket = [&]() {
+      uint32_t t = 0;
+      if (lane == 0) t = atomicAdd(&ctrl[3], 1u);
+      return (uint32_t)__shfl(t, 0, 64);
+    };
+    // generic walk of one queued block (rare classes), scalar reduction against the planes
+    auto generic_block = [&](uint32_t entry) {
+      const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
+      const uint64_t rec = read_record(raw, off + 6 * f);
+      const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+      const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
+      const uint32_t col = f - row * nb;
+      const uint8_t* xb = reinterpret_cast<const uint8_t*>(xplanes + (size_t)col * kPlaneDwords);
+      const float g = (entry >> 25) & 1u ? M.g1 : M.g0;
+      const DevClass c = T.cls[ci];
+      int d0 = 0, d1 = 0, d2 = 0;
+      auto emit = [&](int p, int v) {
+        d0 += v * (int)(int8_t)xb[p];
+        d1 += v * (int)(int8_t)xb[24 + p];
+        d2 += v * (int)(int8_t)xb[48 + p];
+      };
+      if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
+      else decode_even(T, c, li, emit);
+      partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (c.inv_norm * g);
+    };
+    uint32_t chunk = ticket();
+    if (c_gen && chunk == 0) {  // kept out of the loop below: its code and registers are not the hot path's
+      if (lane < n_gen) generic_block(gqueue[lane]);
+      chunk = ticket();
+    }
+    for (; chunk < c_gen + c_odd + c_even; chunk = ticket()) {
       if (chunk < c_gen + c_odd) {
-        const bool from_gen = chunk < c_gen;
-        const uint32_t k = from_gen ? lane : (chunk - c_gen) * 64u + lane;
-        if (k < (from_gen ? n_gen : n_odd)) {
-          const uint32_t entry = from_gen ? gqueue[k] : queue[k];
+        const uint32_t k = (chunk - c_gen) * 64u + lane;
+        const uint32_t entry = k < n_odd ? queue[k] : kEntryGeneric;
+        if (!(entry >> 31)) {  // generic blocks that found the small queue full wait for the pass below
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
           const uint64_t rec = read_record(raw, off + 6 * f);
           const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
@@ -700,29 +726,15 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
           const uint32_t col = f - row * nb;
           const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
           const float g = (entry >> 25) & 1u ? M.g1 : M.g0;
-          if (entry >> 31) {  // generic walk, scalar reduction against the planes
-            const uint8_t* xb = reinterpret_cast<const uint8_t*>(xp);
-            const DevClass c = T.cls[ci];
-            int d0 = 0, d1 = 0, d2 = 0;
-            auto emit = [&](int p, int v) {
-              d0 += v * (int)(int8_t)xb[p];
-              d1 += v * (int)(int8_t)xb[24 + p];
-              d2 += v * (int)(int8_t)xb[48 + p];
-            };
-            if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
-            else decode_even(T, c, li, emit);
-            partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (c.inv_norm * g);
-          } else {
-            const FastClass fc = T.fast[ci];
-            int d0 = 0, d1 = 0, d2 = 0;
-            odd_codes(T, fc, li, [&](int q, uint32_t sel) {
-              const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
-              d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
-              d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-              d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
-            });
-            partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * g);
-          }
+          const FastClass fc = T.fast[ci];
+          int d0 = 0, d1 = 0, d2 = 0;
+          odd_codes(T, fc, li, [&](int q, uint32_t sel) {
+            const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+            d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+            d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+            d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+          });
+          partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * g);
         }
       } else {
         const uint32_t k = (chunk - c_gen - c_odd) * 64u + lane;
@@ -747,6 +759,13 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
           });
           partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
         }
+      }
+    }
+    if (ctrl[2] > (uint32_t)kGenericSlots) {
+      // more generic blocks than the small queue holds (hostile input): the rest sit flagged in the odd queue
+      for (uint32_t k = tid; k < n_odd; k += kWgThreads) {
+        const uint32_t entry = queue[k];
+        if (entry >> 31) generic_block(entry);
       }
     }
     LLVQ_STAMP(4);

@@ -153,6 +153,44 @@ def test_gemv_origin_and_shell13_blocks(gpu_rt, orc):
     _check_gemv(orc, y, raw, x)
 
 
+def test_gemv_tiles_full_of_rare_class_blocks(gpu_rt, orc):
+    """Every block from a class that takes the generic walk (odd with five magnitudes, support weight 0 or
+    24, three word kinds): 640 of them in one tile, ten times what the kernel's queue for such blocks holds,
+    so the overflow path runs too.  Uniform draws meet these classes 0.07 % of the time."""
+    import torch
+
+    ranges = []
+    for ci in range(383):
+        info = orc.class_info(ci)
+        vals, _, _ = orc.class_levels(ci)
+        if info["shell"] > 12:
+            continue
+        if info["odd"]:
+            rare = len(vals) > 4
+        else:
+            rare = not (info["w"] in (8, 12, 16) and len([v for v in vals if abs(v) % 4 == 2]) <= 2)
+        if rare:
+            ranges.append((info["lo"], info["hi"]))
+    assert len(ranges) == 30
+    d_out, nb = 16, 40
+    rng = np.random.default_rng(11)
+    pick = rng.integers(0, len(ranges), size=d_out * nb)
+    idx = np.array([1 + int(rng.integers(ranges[p][0], ranges[p][1])) for p in pick], np.uint64)  # index = 1 + zero-based rank
+    gains = rng.integers(0, 2, size=idx.size).astype(np.uint8)
+    raw = artifact.RawMatrix("model.layers.0.rare.weight", d_out, nb * 24, 12, [0.8, 1.25], np.exp(rng.normal(size=d_out)),
+                             np.zeros(0, np.float32), artifact.pack_codes(idx, gains))
+    x = synth.make_activation(nb * 24, seed=12)[0]
+    proj = gpu_rt.upload(raw)
+    try:
+        y = gpu_rt.forward(proj, _x16(x), out_dtype=torch.float32).cpu().numpy()
+        X = torch.from_numpy(np.stack([x, x]).view(np.int16).copy()).view(torch.float16).cuda()
+        Y = gpu_rt.forward_batched(proj, X, out_dtype=torch.float32).cpu().numpy()
+    finally:
+        gpu_rt.free(proj)
+    assert _check_gemv(orc, y, raw, x) < 1e-5
+    _check_gemv(orc, Y[1], raw, x)
+
+
 def test_gemv_config0_full_size(gpu_rt, orc):
     """BASELINE config 0: gate_proj 9728 x 2560, seed 0, against the oracle's f64 product."""
     import torch
