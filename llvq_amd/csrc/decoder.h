@@ -191,7 +191,7 @@ struct AttnNew {
 
 constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = kAttnThreads / 64;
-constexpr int kAttnMaxSplits = 64;  // the cache is cut into at most this many ranges (host picks by length)
+constexpr int kAttnMaxSplits = 64;  // the cache is cut into at most this many ranges (host picks by length; 128 was measured slower at 8188 positions)
 constexpr int kAttnMaxGroup = 8;    // query heads per kv head
 
 // ---- rows of positions at once (prompt processing through the batched product) ----
@@ -673,12 +673,16 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
 // time.  Same arithmetic and order as the in-kernel merge.
 __global__ __launch_bounds__(128) void attn_merge_kernel(const float* __restrict__ part, __half* __restrict__ ctx,
                                                          uint32_t head_dim, uint32_t n_splits) {
-  __shared__ float wts[kAttnMaxSplits];
+  __shared__ float wts[kAttnMaxSplits], ls[kAttnMaxSplits];
   __shared__ float Lsum;
+  static_assert(kAttnMaxSplits <= 128, "one lane per range fetches its maximum and its sum");
   const uint32_t head = blockIdx.x, tid = threadIdx.x;
   const uint32_t stride = head_dim + 2;
   const float* src = part + (size_t)head * n_splits * stride;
-  if (tid < n_splits) wts[tid] = src[(size_t)tid * stride];
+  if (tid < n_splits) {
+    wts[tid] = src[(size_t)tid * stride];
+    ls[tid] = src[(size_t)tid * stride + 1];
+  }
   __syncthreads();
   float M = -INFINITY;
   for (uint32_t s = 0; s < n_splits; ++s) M = fmaxf(M, wts[s]);
@@ -687,7 +691,7 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(const float* __restrict
   __syncthreads();
   if (tid == 0) {
     float L = 0.f;
-    for (uint32_t s = 0; s < n_splits; ++s) L = fmaf(src[(size_t)s * stride + 1], wts[s], L);
+    for (uint32_t s = 0; s < n_splits; ++s) L = fmaf(ls[s], wts[s], L);  // range order
     Lsum = L;
   }
   __syncthreads();
