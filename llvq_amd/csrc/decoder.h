@@ -131,6 +131,20 @@ __device__ __forceinline__ void norm_rope_wave(const __half* __restrict__ src, c
                                                const __half* __restrict__ cos_t, const __half* __restrict__ sin_t,
                                                uint32_t pos, uint32_t head_dim, float eps, float* stage, uint32_t lane) {
   const uint32_t half_d = head_dim >> 1;
+  if (head_dim == 128) {
+    // the served width: a lane's two elements (lane, lane + 64) are a rotation pair, so nothing
+    // crosses lanes but the sum of squares, and every load goes out before the first use
+    const float x1 = __half2float(src[lane]), x2 = __half2float(src[lane + 64]);
+    const float w1 = __half2float(w[lane]), w2 = __half2float(w[lane + 64]);
+    const float c = __half2float(cos_t[(size_t)pos * 64 + lane]), sn = __half2float(sin_t[(size_t)pos * 64 + lane]);
+    const float ss = wave_sum(x1 * x1 + x2 * x2);
+    const float inv = 1.0f / sqrtf(ss / 128.0f + eps);
+    const float n1 = __half2float(__float2half_rn(x1 * inv * w1)), n2 = __half2float(__float2half_rn(x2 * inv * w2));
+    stage[lane] = __half2float(__float2half_rn(n1 * c - n2 * sn));
+    stage[lane + 64] = __half2float(__float2half_rn(n1 * sn + n2 * c));
+    wave_lds_sync();
+    return;
+  }
   float x[4];  // elements lane, lane + 64, lane + 128, lane + 192
   float ss = 0.f;
 #pragma unroll
