@@ -95,6 +95,66 @@ __device__ __forceinline__ void store_y<__half>(void* y, size_t at, float v) {
   reinterpret_cast<__half*>(y)[at] = __float2half_rn(v);
 }
 
+// P2 of the batched kernels: the wavefronts that call this draw 64-block chunks of the
+// tile's queues (generic walks first, then odd, then even classes) from a shared
+// counter until none is left; every block's 24 weights, multiplied by
+// centroid[gain] / sqrt(16 shell) and rounded once to binary16, go to row `row`,
+// columns [24 b, 24 b + 24) of the W slice.  CAP = queue capacity, WSTRIDE = binary16
+// elements per W row; slot f of the tile is block b = f - row kb of row = f / kb.
+template <int CAP, int WSTRIDE, typename RecordAt>
+__device__ __forceinline__ void unrank_queues_to_slice(const DecodeTables& T, const uint32_t* queue, const uint32_t* gqueue,
+                                                       uint32_t* ctrl, uint32_t kb, uint32_t inv_kb, float g0, float g1,
+                                                       _Float16* W, RecordAt record_at) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
+  const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
+  for (;;) {
+    uint32_t chunk = 0;
+    if (lane == 0) chunk = atomicAdd(&ctrl[3], 1u);
+    chunk = __shfl(chunk, 0, 64);
+    if (chunk >= c_gen + c_odd + c_even) break;
+    const bool from_gen = chunk < c_gen, from_odd = chunk < c_gen + c_odd;
+    const uint32_t k = from_gen ? lane : (from_odd ? (chunk - c_gen) * 64u + lane : (chunk - c_gen - c_odd) * 64u + lane);
+    if (k < (from_gen ? n_gen : (from_odd ? n_odd : n_even))) {
+      const uint32_t entry = from_gen ? gqueue[k] : (from_odd ? queue[k] : queue[CAP - 1 - k]);
+      const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
+      const uint32_t row = (f * inv_kb) >> 16, b = f - row * kb;
+      const uint64_t rec = record_at(row, b);
+      const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+      const float g = (entry >> 25) & 1u ? g1 : g0;
+      _Float16* wrow = W + (size_t)row * WSTRIDE + b * 24u;
+      if (entry & kEntryOrigin) {
+        uint4* dst = reinterpret_cast<uint4*>(wrow);
+        dst[0] = dst[1] = dst[2] = make_uint4(0, 0, 0, 0);
+      } else if (from_odd) {
+        if (entry >> 31) {  // generic walk
+          const DevClass c = T.cls[ci];
+          const float s = c.inv_norm * g;
+          auto emit = [&](int p, int v) { wrow[p] = (_Float16)((float)v * s); };
+          if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
+          else decode_even(T, c, li, emit);
+        } else {
+          const FastClass fc = T.fast[ci];
+          const float s = fc.inv_norm * g, bias = -128.f * s;
+          odd_codes(T, fc, li, [&](int q, uint32_t sel) {
+            const uint32_t w = __builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+            *reinterpret_cast<uint2*>(wrow + 4 * q) = scaled_halves(w, s, bias);
+          });
+        }
+      } else {
+        const FastClass fc = T.fast[ci];
+        const float s = fc.inv_norm * g, bias = -128.f * s;
+        const uint32_t fv1 = fc.u0 >> 16;
+        const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
+        even_codes(T, fc, li, [&](int q, uint32_t sel, uint32_t sel2) {
+          const uint32_t w = __builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel) | __builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2);
+          *reinterpret_cast<uint2*>(wrow + 4 * q) = scaled_halves(w, s, bias);
+        });
+      }
+    }
+  }
+}
+
 // Wavefront grid of the MFMA phase: every wavefront owns both 32-row tiles of the band
 // and one 32-column tile of the batch.  A batch of fewer than sixteen column tiles
 // leaves wavefronts over; they take the same tiles on interleaved K-steps (kpart) and
@@ -196,53 +256,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       LLVQ_GSTAMP(1);
 
       // P2: unrank into the W slice
-      const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
-      const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
-      for (;;) {
-        uint32_t chunk = 0;
-        if (lane == 0) chunk = atomicAdd(&ctrl[3], 1u);
-        chunk = __shfl(chunk, 0, 64);
-        if (chunk >= c_gen + c_odd + c_even) break;
-        const bool from_gen = chunk < c_gen, from_odd = chunk < c_gen + c_odd;
-        const uint32_t k = from_gen ? lane : (from_odd ? (chunk - c_gen) * 64u + lane : (chunk - c_gen - c_odd) * 64u + lane);
-        if (k < (from_gen ? n_gen : (from_odd ? n_odd : n_even))) {
-        const uint32_t entry = from_gen ? gqueue[k] : (from_odd ? queue[k] : queue[kGemmTile - 1 - k]);
-        const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
-        const uint32_t row = (f * inv_kb) >> 16, b = f - row * kb;
-        const uint64_t rec = record_at(row, b);
-        const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
-        const float g = (entry >> 25) & 1u ? a.g1 : a.g0;
-        _Float16* wrow = W + (size_t)row * kGemmWStride + b * 24u;
-        if (entry & kEntryOrigin) {
-          uint4* dst = reinterpret_cast<uint4*>(wrow);
-          dst[0] = dst[1] = dst[2] = make_uint4(0, 0, 0, 0);
-        } else if (from_odd) {
-          if (entry >> 31) {  // generic walk
-            const DevClass c = T.cls[ci];
-            const float s = c.inv_norm * g;
-            auto emit = [&](int p, int v) { wrow[p] = (_Float16)((float)v * s); };
-            if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
-            else decode_even(T, c, li, emit);
-          } else {
-            const FastClass fc = T.fast[ci];
-            const float s = fc.inv_norm * g, bias = -128.f * s;
-            odd_codes(T, fc, li, [&](int q, uint32_t sel) {
-              const uint32_t w = __builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
-              *reinterpret_cast<uint2*>(wrow + 4 * q) = scaled_halves(w, s, bias);
-            });
-          }
-        } else {
-          const FastClass fc = T.fast[ci];
-          const float s = fc.inv_norm * g, bias = -128.f * s;
-          const uint32_t fv1 = fc.u0 >> 16;
-          const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
-          even_codes(T, fc, li, [&](int q, uint32_t sel, uint32_t sel2) {
-            const uint32_t w = __builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel) | __builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2);
-            *reinterpret_cast<uint2*>(wrow + 4 * q) = scaled_halves(w, s, bias);
-          });
-        }
-        }
-      }
+      unrank_queues_to_slice<kGemmTile, kGemmWStride>(T, queue, gqueue, ctrl, kb, inv_kb, a.g0, a.g1, W, record_at);
       LLVQ_GSTAMP(2);
       __syncthreads();
       LLVQ_GSTAMP(3);

@@ -425,8 +425,8 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 #define LLVQ_STAMP(k) do {} while (0)
 #endif
 
-// P1 of both kernels: every lane classifies up to NB blocks of the tile and
-// bins them.  `record(f)` returns the 48-bit record of tile slot f < nblk;
+// P1 of the GEMV and GEMM kernels: each of the LANES lanes taking part (the first
+// LANES of the workgroup) classifies up to NB blocks of the tile and bins them.  `record(f)` returns the 48-bit record of tile slot f < nblk;
 // `origin(f)` is called for an origin block (index 0) and returns whether the
 // block must still be queued (flagged, with the odd-coset blocks) or is settled.
 // Queue entry: slot (12 bits) | class << 16 | gain << 25 | origin << 30 | generic walk << 31.
@@ -435,7 +435,7 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 // the rare generic classes take ~2000 dependent instructions: they go to a
 // small queue that P2 hands out first; what does not fit rides in the odd queue.
 constexpr uint32_t kEntryOrigin = 0x40000000u, kEntryGeneric = 0x80000000u;
-template <int NB, typename RecordFn, typename OriginFn>
+template <int NB, int LANES = kWgThreads, typename RecordFn, typename OriginFn>
 __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t nblk, uint32_t capacity, uint32_t* queue,
                                                  uint32_t* gqueue, uint32_t* ctrl, RecordFn record, OriginFn origin) {
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -444,7 +444,7 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
   bool queued_origin[NB];
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    const uint32_t f = tid + (uint32_t)i * kWgThreads;
+    const uint32_t f = tid + (uint32_t)i * LANES;
     zi[i] = ~0ULL;
     entry[i] = 0;
     ci[i] = 0;
@@ -862,6 +862,7 @@ __global__ __launch_bounds__(1024) void rotate_kernel(RotArgs a) {
 }  // namespace llvq
 
 #include "gemm_kernel.h"
+#include "gemm_pipe_kernel.h"
 #include "decoder.h"
 
 // =================================================================================
@@ -889,9 +890,12 @@ struct llvq_rt {
   size_t rot_scratch_elems = 0;
   __half* rot_rows = nullptr;     // rotated batch rows, f16 (matrix-core path)
   size_t rot_rows_elems = 0;
-  // split-K workspace of the batched kernel: partial sums [S, M, d_out]
+  // workspace of the batched kernels: partial sums [S, n_bands, M, 64]
   float* gemm_ws = nullptr;
   size_t gemm_ws_bytes = 0;
+  // a batch's activations in K-step tiles [n_steps, m_pad, 32] (pipelined batched kernel)
+  __half* gemm_xt = nullptr;
+  size_t gemm_xt_bytes = 0;
 };
 
 struct llvq_mat {
@@ -982,6 +986,8 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_pipe_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_pipe_kernel<12>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   *out = rt;
   return LLVQ_OK;
 }
@@ -991,6 +997,7 @@ void llvq_hip_runtime_destroy(llvq_rt* rt) {
   (void)hipSetDevice(rt->device);
   (void)hipFree(rt->blob);
   (void)hipFree(rt->gemm_ws);
+  (void)hipFree(rt->gemm_xt);
   (void)hipFree(rt->rot_scratch);
   (void)hipFree(rt->rot_rows);
   for (auto* r : rt->rotations) {
@@ -1490,6 +1497,78 @@ static void pick_gemm_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint
   *bps_out = best_bps;
 }
 
+// The same choice for the pipelined kernel: a slice of 16 blocks per row costs what its
+// unranking costs (the matrix-core work of the slice before runs beside it), a unit
+// pays one more stage to drain, and every launch ends in the chip-wide sum.  Splits are
+// whole slices, so every slice starts on a 32-column K-step of the tiled activations.
+static void pick_pipe_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint32_t kparts, uint32_t grid,
+                            uint32_t* S_out, uint32_t* bps_out) {
+  double best = 1e30;
+  const uint32_t total_slices = (nblocks + kPipeKb - 1) / kPipeKb;
+  uint32_t best_s = 1, best_bps = total_slices * kPipeKb;
+  const double stage_us = 7.5;
+  for (uint32_t per = total_slices; per >= 1; --per) {  // slices per split
+    const uint32_t S = (total_slices + per - 1) / per;
+    if (S > 64) break;
+    if ((total_slices + S - 1) / S != per) continue;  // the same S with a smaller last split: already seen
+    const double unit_us = 2.0 + (per + 1) * stage_us + 0.004 * M;
+    const uint64_t units = (uint64_t)n_bands * S;
+    const double reduce_us = 6.0 + (double)S * kparts * M * 64.0 * n_bands * 4.0 / 2.0e6;
+    const double t = (double)((units + grid - 1) / grid) * unit_us + reduce_us;
+    if (t < best * 0.999) { best = t; best_s = S; best_bps = per * kPipeKb; }
+  }
+  *S_out = best_s;
+  *bps_out = best_bps;
+}
+
+static int grow_gemm_workspace(llvq_rt* rt, size_t need) {
+  if (need <= rt->gemm_ws_bytes) return LLVQ_OK;
+  (void)hipFree(rt->gemm_ws);  // waits for launches that still use it
+  rt->gemm_ws = nullptr;
+  rt->gemm_ws_bytes = 0;
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_ws), need));
+  rt->gemm_ws_bytes = need;
+  return LLVQ_OK;
+}
+
+static int launch_gemm_reduce(llvq_rt* rt, const GemmArgs& a, uint32_t n_partials, bool f32) {
+  GemmReduceArgs r{};
+  r.ws = a.ws;
+  r.x = a.x;
+  r.rscale = a.rscale;
+  r.tail = a.tail;
+  r.y = a.y;
+  r.M = a.M;
+  r.ldx = a.ldx;
+  r.d_out = a.d_out;
+  r.nblocks = a.nblocks;
+  r.tail_w = a.tail_w;
+  r.S = n_partials;
+  r.n_bands = a.n_bands;
+  const uint32_t rgrid = a.n_bands * ((a.M + kReduceRowsM - 1) / kReduceRowsM);
+  if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3(rgrid), dim3(256), 0, rt->stream, r);
+  else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3(rgrid), dim3(256), 0, rt->stream, r);
+  HIP_TRY(hipGetLastError());
+  return LLVQ_OK;
+}
+
+// Batches of at least this many activation rows take the pipelined kernel.
+static uint32_t pipe_min_rows() {
+  static const uint32_t v = [] {
+    const char* e = std::getenv("LLVQ_GEMM_PIPE_MIN_M");
+    return e ? (uint32_t)std::strtoul(e, nullptr, 10) : 2u;
+  }();
+  return v;
+}
+
+static uint32_t pipe_narrow_rows() {
+  static const uint32_t v = [] {
+    const char* e = std::getenv("LLVQ_GEMM_PIPE_NARROW_M");
+    return e ? (uint32_t)std::strtoul(e, nullptr, 10) : 256u;
+  }();
+  return v;
+}
+
 static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M, void* y, int y_dtype) {
   const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
   GemmArgs a{};
@@ -1507,47 +1586,65 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
   a.nblocks = m->nblocks;
   a.tail_w = m->tail_w;
   a.n_bands = (m->d_out + kGemmRows - 1) / kGemmRows;
+  const bool f32 = y_dtype == LLVQ_F32;
+  if (M >= pipe_min_rows()) {
+    GemmPipeArgs pa{};
+    pa.tables = rt->tables;
+    pa.codes = m->codes;
+    pa.g0 = m->g[0];
+    pa.g1 = m->g[1];
+    pa.M = M;
+    pa.m_pad = (M + kPipeColTile - 1) / kPipeColTile * kPipeColTile;
+    pa.d_out = m->d_out;
+    pa.nblocks = m->nblocks;
+    pa.n_bands = a.n_bands;
+    // the consumer wavefronts (four up to 128 activation rows, eight beyond) over the batch's
+    // 64-row tiles, the count rounded up to a power of two
+    const uint32_t consumers = M <= pipe_narrow_rows() ? 4u : 8u;
+    pa.ct_shift = 0;
+    while (((uint32_t)kPipeColTile << pa.ct_shift) < M) ++pa.ct_shift;
+    const uint32_t kparts = consumers >> pa.ct_shift;
+    pick_pipe_split(pa.n_bands, m->nblocks, M, kparts, grid_cap, &pa.S, &pa.bps);
+    int rc = grow_gemm_workspace(rt, (size_t)pa.S * kparts * pa.n_bands * M * kGemmRows * sizeof(float));
+    if (rc) return rc;
+    const uint32_t n_steps = (m->nblocks * 24u + 31u) / 32u;
+    const size_t xt_bytes = (size_t)n_steps * pa.m_pad * 64;
+    if (xt_bytes > rt->gemm_xt_bytes) {
+      (void)hipFree(rt->gemm_xt);
+      rt->gemm_xt = nullptr;
+      rt->gemm_xt_bytes = 0;
+      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_xt), xt_bytes));
+      rt->gemm_xt_bytes = xt_bytes;
+    }
+    hipLaunchKernelGGL(tile_activations_kernel, dim3((uint32_t)((xt_bytes / 16 + 255) / 256)), dim3(256), 0, rt->stream, a.x, M,
+                       a.ldx, m->nblocks * 24u, pa.m_pad, n_steps, reinterpret_cast<uint4*>(rt->gemm_xt));
+    HIP_TRY(hipGetLastError());
+    pa.xt = rt->gemm_xt;
+    pa.ws = rt->gemm_ws;
+    a.ws = rt->gemm_ws;
+    const uint32_t units = pa.n_bands * pa.S;
+    const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
+    if (consumers == 4) hipLaunchKernelGGL(gemm_pipe_kernel<12>, grid, wg, gemm_pipe_lds_bytes(), rt->stream, pa);
+    else hipLaunchKernelGGL(gemm_pipe_kernel<8>, grid, wg, gemm_pipe_lds_bytes(), rt->stream, pa);
+    HIP_TRY(hipGetLastError());
+    return launch_gemm_reduce(rt, a, pa.S * kparts, f32);
+  }
   pick_gemm_split(a.n_bands, m->nblocks, M, grid_cap, &a.S, &a.bps);
   if (a.S > 1) {
-    const size_t need = (size_t)a.S * a.n_bands * M * kGemmRows * sizeof(float);
-    if (need > rt->gemm_ws_bytes) {
-      (void)hipFree(rt->gemm_ws);  // waits for launches that still use it
-      rt->gemm_ws = nullptr;
-      rt->gemm_ws_bytes = 0;
-      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_ws), need));
-      rt->gemm_ws_bytes = need;
-    }
+    const int rc = grow_gemm_workspace(rt, (size_t)a.S * a.n_bands * M * kGemmRows * sizeof(float));
+    if (rc) return rc;
     a.ws = rt->gemm_ws;
   }
   const uint32_t units = a.n_bands * a.S;
   const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
   const size_t lds = gemm_lds_bytes();
-  const bool f32 = y_dtype == LLVQ_F32;
   // sixteen wavefronts over the batch's 32-column tiles, the count rounded up to a power of two
   a.ct_shift = 0;
   while ((32u << a.ct_shift) < M && a.ct_shift < 4) ++a.ct_shift;
   if (f32) hipLaunchKernelGGL(gemm_tiles_kernel<float>, grid, wg, lds, rt->stream, a);
   else hipLaunchKernelGGL(gemm_tiles_kernel<__half>, grid, wg, lds, rt->stream, a);
   HIP_TRY(hipGetLastError());
-  if (a.S > 1) {
-    GemmReduceArgs r{};
-    r.ws = a.ws;
-    r.x = a.x;
-    r.rscale = a.rscale;
-    r.tail = a.tail;
-    r.y = a.y;
-    r.M = a.M;
-    r.ldx = a.ldx;
-    r.d_out = a.d_out;
-    r.nblocks = a.nblocks;
-    r.tail_w = a.tail_w;
-    r.S = a.S;
-    r.n_bands = a.n_bands;
-    const uint32_t rgrid = a.n_bands * ((M + kReduceRowsM - 1) / kReduceRowsM);
-    if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3(rgrid), dim3(256), 0, rt->stream, r);
-    else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3(rgrid), dim3(256), 0, rt->stream, r);
-    HIP_TRY(hipGetLastError());
-  }
+  if (a.S > 1) return launch_gemm_reduce(rt, a, a.S, f32);
   return LLVQ_OK;
 }
 
