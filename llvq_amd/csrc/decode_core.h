@@ -137,6 +137,22 @@ LLVQ_HD uint32_t find_class(const DecodeTables& T, uint64_t i) {
 // of the packed comparison, and the next slot's value is one fused multiply-add,
 // (t + 1 - T_j) (m / c_j) + (1 - m / c_j) with m = n - 1, both factors from one
 // 16-byte table entry.
+// One slot of the walk: n slots are left, the kind's code 4 - kind is returned.
+LLVQ_HD uint32_t odd_walk_slot(const DecodeTables& T, uint32_t n, double& t1, uint32_t& tg) {
+  const uint32_t ti1 = (uint32_t)t1;                      // floor(t) + 1
+  const uint32_t ltg = (uint32_t)mad24(-(int)ti1, (int)kFieldOnes, (int)tg) & kFieldGuard;  // guard survives iff T_m > floor(t)
+  const uint32_t jj = popc32(ltg);                        // 4 - kind
+  const uint32_t sh = jj * 6u;
+  const uint32_t lo = (tg >> sh) & 31u;
+  const uint32_t hi = (((tg << 6) | n) >> sh) & 31u;
+  tg -= ltg >> 5;
+  if (n > 1u) {
+    const double* e = T.step + 2u * ((n - 1u) * 25u + (hi - lo));
+    t1 = fma64(t1 - (double)lo, e[0], e[1]);
+  }
+  return jj;
+}
+
 template <class OnCodes>
 LLVQ_HD void odd_codes(const DecodeTables& T, const FastClass& f, uint64_t li, OnCodes&& on_codes) {
   const double local = (double)li;
@@ -149,21 +165,7 @@ LLVQ_HD void odd_codes(const DecodeTables& T, const FastClass& f, uint64_t li, O
   for (int q = 0; q < 6; ++q) {
     uint32_t sel = 0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t n = (uint32_t)(kDim - 4 * q - j);
-      const uint32_t ti1 = (uint32_t)t1;                      // floor(t) + 1
-      const uint32_t ltg = (uint32_t)mad24(-(int)ti1, (int)kFieldOnes, (int)tg) & kFieldGuard;  // guard survives iff T_m > floor(t)
-      const uint32_t jj = popc32(ltg);                        // 4 - kind
-      const uint32_t sh = jj * 6u;
-      const uint32_t lo = (tg >> sh) & 31u;
-      const uint32_t hi = (((tg << 6) | n) >> sh) & 31u;
-      tg -= ltg >> 5;
-      if (n > 1u) {
-        const double* e = T.step + 2u * ((n - 1u) * 25u + (hi - lo));
-        t1 = fma64(t1 - (double)lo, e[0], e[1]);
-      }
-      sel |= jj << (8 * j);
-    }
+    for (int j = 0; j < 4; ++j) sel |= odd_walk_slot(T, (uint32_t)(kDim - 4 * q - j), t1, tg) << (8 * j);
     // table index = jj - 1 (kinds 0..3 <-> jj 4..1), bit 2 = off the codeword's support
     on_codes(q, (sel - 0x01010101u) | ((((ncw >> (4 * q)) & 15u) * kSpread2) & 0x04040404u));
   }

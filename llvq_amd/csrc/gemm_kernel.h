@@ -7,25 +7,41 @@
 // (llvq-llm/src/model.rs:521-529); this kernel decodes every block once for
 // all M rows instead.
 //
-// Work unit: a band of 64 weight rows x a range of blocks of those rows.  One
-// persistent 1024-lane workgroup per CU walks its unit in K-slices of at most
-// 32 blocks per row (768 columns, 2048 blocks):
-//   P0  the slice's code bytes, 16-byte loads -> LDS (next slice's loads are
-//       already in flight while this one is decoded);
-//   P1  classify and bin the blocks (odd / even / generic queues);
-//   P2  unrank; every block writes its 24 weights, already multiplied by
-//       centroid[gain] / sqrt(16 shell), as binary16 into the W slice in LDS;
-//   P3  16 wavefronts run v_mfma_f32_32x32x16_f16 over the slice: A fragments
-//       from LDS, B fragments (activations) straight from global memory / L2,
-//       fetched one batch ahead.  Up to 256 activation rows the wavefront grid
-//       is 2 row tiles x 8 column tiles of 32; beyond, every wavefront takes
-//       both row tiles of one of 16 column tiles.  Accumulators (16 or 32
-//       registers) stay live across slices.
-// Epilogue: row scale and the f32 tail columns in f32, then the store.  When a
-// matrix has too few bands to occupy the chip its block range is split over
-// several units; each writes its partial sums to a workspace and a second,
-// chip-wide kernel (gemm_reduce_kernel) adds them in split order and applies
-// the epilogue, so the result does not depend on scheduling.
+// Work unit: a band of 64 weight rows x a range of blocks of those rows, walked
+// in K-slices of 16 blocks per row (384 columns = 12 K-steps of 32, 1024 blocks)
+// by one persistent 1024-lane workgroup per CU.  Its 16 wavefronts split into two
+// roles, and the unranking and the contraction of consecutive slices run at the
+// same time:
+//   producers (the first 8 or 12) slice g: code bytes -> LDS (loads issued two
+//                                slices ahead), classify and bin the blocks (odd /
+//                                even / generic queues), unrank; every block writes
+//                                its 24 weights, already multiplied by
+//                                centroid[gain] / sqrt(16 shell) and rounded once to
+//                                binary16, into W[g & 1] in LDS;
+//   consumers (the other 8 or 4) v_mfma_f32_32x32x16_f16 over slice g - 1 from
+//                                W[(g - 1) & 1]: every consumer owns all 64 weight
+//                                rows x 64 activation rows (64 accumulator
+//                                registers, live across the unit's slices), A
+//                                fragments from LDS, B fragments from global
+//                                memory / L2, three K-steps in flight.
+// The unranking is integer and f64 VALU work and the contraction runs on the
+// matrix cores, so the two overlap on every SIMD.  Because the roles are separate
+// branches of one kernel, the accumulators and the decode state are never live
+// together: both fit the 128 registers a 1024-lane workgroup leaves each
+// wavefront (one wavefront doing both in turn spills beyond 32 accumulators).
+// A narrow batch leaves the matrix cores little to do, and 12 wavefronts unrank.
+//
+// A stage has two workgroup barriers (after the classification, after the
+// unranking); the consumers cross the same two while they work through their
+// K-steps, so the W buffer written in stage g is complete before it is read in
+// stage g + 1 and is not overwritten before stage g + 2.
+//
+// Every consumer writes its sums to the workspace [split x K-share][band][m][64]
+// (consumers left over by a batch of few 64-row tiles take the same tile on
+// interleaved K-steps; matrices with few bands split their block range over
+// several units so that the chip is occupied); gemm_reduce_kernel adds the
+// partial sums in that fixed order and applies row scale and the f32 tail
+// columns, so the result does not depend on scheduling.
 #pragma once
 
 namespace llvq {
@@ -33,42 +49,12 @@ namespace llvq {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int kGemmRows = 64;                 // weight rows of a band
-#ifndef LLVQ_GEMM_KB
-#define LLVQ_GEMM_KB 32
-#endif
-constexpr int kGemmKb = LLVQ_GEMM_KB;         // blocks per row and K-slice (32: 768 columns = 24 K-steps of 32, 2048 blocks = two 64-block chunks per wavefront)
-constexpr int kGemmTile = kGemmRows * kGemmKb;  // blocks per K-slice
-constexpr int kGemmP1Blocks = (kGemmTile + kWgThreads - 1) / kWgThreads;
-constexpr int kGemmRowChunks = (kGemmKb * 6 + 14 + 15) / 16;  // 16-byte units holding one row's code bytes at any even alignment
-constexpr int kGemmRowBytes = kGemmRowChunks * 16;
-constexpr int kGemmWStride = kGemmKb * 24 + 8;  // binary16 elements per W row in LDS; the pad spreads rows over banks
-constexpr int kGemmMaxM = 512;                // activation rows per launch (32 column tiles of 16)
-static_assert(kGemmRows * kGemmRowChunks <= kWgThreads, "one 16-byte load per lane covers a slice's code bytes");
-static_assert(kGemmTile <= 4096, "queue entries keep the block slot in 12 bits");
-
-struct GemmArgs {
-  GlobalTables tables;
-  const __half* x;        // [M, ldx] row-major
-  const uint8_t* codes;
-  const float* rscale;
-  const float* tail;
-  void* y;                // [M, d_out]
-  float* ws;              // [S, n_bands, M, 64] partial sums when S > 1
-  float g0, g1;
-  uint32_t M, ldx, d_out, nblocks, tail_w;
-  uint32_t n_bands, S, bps;  // split count, blocks per split
-  uint32_t ct_shift;         // log2 of the column tiles the wavefronts spread over (0..4)
-};
+constexpr int kGemmRows = 64;    // weight rows of a band
+constexpr int kGemmMaxM = 512;   // activation rows per launch (eight consumers x 64)
 
 // The batched kernel keeps the Golay words and the support-arrangement table in L2:
-// the 33 KB they would take in LDS buy a W slice of 32 blocks per row instead of 20.
+// the 33 KB they would take in LDS buy the second W buffer.
 constexpr size_t kGemmImageBytes = kLdsImageBytesLean;
-constexpr size_t gemm_lds_bytes() {
-  return kGemmImageBytes + (size_t)kGemmRows * kGemmRowBytes + (size_t)kGemmTile * 4 + kGenericSlots * 4 + 16 +
-         (size_t)kGemmRows * kGemmWStride * 2;
-}
-static_assert(gemm_lds_bytes() <= 160 * 1024, "GEMM workgroup state must fit one CU's LDS");
 
 // four packed signed bytes -> four binary16 values w * s, one rounding each
 __device__ __forceinline__ uint2 scaled_halves(uint32_t w, float s, float bias) {
@@ -95,7 +81,7 @@ __device__ __forceinline__ void store_y<__half>(void* y, size_t at, float v) {
   reinterpret_cast<__half*>(y)[at] = __float2half_rn(v);
 }
 
-// P2 of the batched kernels: the wavefronts that call this draw 64-block chunks of the
+// The producers' unranking: the wavefronts that call this draw 64-block chunks of the
 // tile's queues (generic walks first, then odd, then even classes) from a shared
 // counter until none is left; every block's 24 weights, multiplied by
 // centroid[gain] / sqrt(16 shell) and rounded once to binary16, go to row `row`,
@@ -155,283 +141,324 @@ __device__ __forceinline__ void unrank_queues_to_slice(const DecodeTables& T, co
   }
 }
 
-// Wavefront grid of the MFMA phase: every wavefront owns both 32-row tiles of the band
-// and one 32-column tile of the batch.  A batch of fewer than sixteen column tiles
-// leaves wavefronts over; they take the same tiles on interleaved K-steps (kpart) and
-// the unit's epilogue adds their sums in kpart order.
+constexpr int kGemmKb = 16;                                   // blocks per row and K-slice
+constexpr int kGemmTile = kGemmRows * kGemmKb;                // blocks per K-slice
+constexpr int kGemmMinProducers = 512;                        // lanes of the producer role, at least
+constexpr int kGemmRowChunks = (kGemmKb * 6 + 14 + 15) / 16;  // 16-byte units holding one row's code bytes at any even alignment
+constexpr int kGemmRowBytes = kGemmRowChunks * 16;
+constexpr int kGemmWStride = kGemmKb * 24 + 8;                // binary16 elements per W row in LDS
+constexpr int kGemmColTile = 64;                              // activation rows per consumer
+static_assert(kGemmRows * kGemmRowChunks <= kGemmMinProducers, "one 16-byte load per producer lane covers a slice's code bytes");
+static_assert(kGemmMaxM <= (kWgThreads - kGemmMinProducers) / 64 * kGemmColTile, "the consumers cover a launch's activation rows");
+
+constexpr size_t gemm_lds_bytes() {
+  return kGemmImageBytes + 2 * (size_t)kGemmRows * kGemmRowBytes + (size_t)kGemmTile * 4 + kGenericSlots * 4 + 32 +
+         2 * (size_t)kGemmRows * kGemmWStride * 2;
+}
+static_assert(gemm_lds_bytes() <= 160 * 1024, "GEMM workgroup state must fit one CU's LDS");
+
+__device__ __forceinline__ void wg_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// The consumers' side of a barrier.  They only read LDS and have nothing to publish, so the
+// barrier must not wait for their global loads: those stay in flight across it.
+__device__ __forceinline__ void consumer_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// The activations as the consumers read them: xt[p][m][32] holds columns [32 p, 32 p + 32)
+// of activation row m, so the 64 rows x 64 bytes a consumer needs for one K-step are one
+// contiguous 4 KB run (in x they are 64 half cache lines, 2 ldx bytes apart).  Columns from
+// `kcols` on (the tail columns, which the f32 epilogue handles) and rows from M on are
+// zero, which leaves the consumers' loads unconditional.  One lane per 16 bytes.
+__global__ __launch_bounds__(256) void tile_activations_kernel(const __half* x, uint32_t M, uint32_t ldx, uint32_t kcols,
+                                                               uint32_t m_pad, uint32_t n_steps, uint4* xt) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)n_steps * m_pad * 4) return;
+  const uint32_t c = (uint32_t)(idx & 3), m = (uint32_t)((idx >> 2) % m_pad), p = (uint32_t)((idx >> 2) / m_pad);
+  const uint32_t col = p * 32u + c * 8u;  // kcols is a multiple of 8: a 16-byte piece is all inside or all outside
+  xt[idx] = (m < M && col < kcols) ? *reinterpret_cast<const uint4*>(x + (size_t)m * ldx + col) : make_uint4(0, 0, 0, 0);
+}
+
+// Position of a role in the workgroup's sequence of (unit, slice) pairs.  Both roles
+// step through the same sequence, the consumers one stage behind.
+struct SliceWalk {
+  uint32_t unit, si, n_slices, sj;  // sj: the slice walked at step si (units start at a band-dependent offset)
+  uint32_t band, split, r0, rows, kb_lo, kb_hi;
+};
+
 #ifdef LLVQ_PHASE_TIMING
-#define LLVQ_GSTAMP(k)                                                                                  \
-  do {                                                                                                  \
-    if (threadIdx.x == 0 && unit == blockIdx.x && si == 0) g_phase_stamps[blockIdx.x * 8 + (k)] = wall_clock64(); \
+#define LLVQ_GSTAMP(base, k)                                                                                          \
+  do {                                                                                                                \
+    if (tid == ((base) ? (uint32_t)PW * 64u : 0u) && stage_no == 3) g_phase_stamps[((base) + blockIdx.x) * 8 + (k)] = wall_clock64(); \
   } while (0)
 #else
-#define LLVQ_GSTAMP(k) do {} while (0)
+#define LLVQ_GSTAMP(base, k) do {} while (0)
 #endif
 
-template <typename OutT>
+struct GemmArgs {
+  GlobalTables tables;
+  const __half* xt;       // [n_steps, m_pad, 32]: tile_activations_kernel's output
+  const uint8_t* codes;
+  float* ws;              // [S * kparts, n_bands, M, 64] partial sums
+  float g0, g1;
+  uint32_t M, m_pad, d_out, nblocks;
+  uint32_t n_bands, S, bps;  // split count, blocks per split (a multiple of the slice)
+  uint32_t ct_shift;         // log2 of the 64-row activation tiles the consumers spread over
+};
+
+// PW = producer wavefronts (8 or 12); the other 16 - PW consume.
+template <int PW>
 __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
+  constexpr int kProducers = PW * 64, kConsumers = 16 - PW;
+  constexpr int kP1Blocks = (kGemmTile + kProducers - 1) / kProducers;
+  static_assert(kProducers >= kGemmMinProducers && (kConsumers == 8 || kConsumers == 4), "roles");
   extern __shared__ __align__(16) uint8_t smem[];
   const DecodeTables T = stage_tables<false>(smem, a.tables);
-  uint8_t* raw = smem + kGemmImageBytes;
-  uint32_t* queue = reinterpret_cast<uint32_t*>(raw + kGemmRows * kGemmRowBytes);
+  uint8_t* raw0 = smem + kGemmImageBytes;
+  constexpr uint32_t kRawBuf = kGemmRows * kGemmRowBytes;
+  uint32_t* queue = reinterpret_cast<uint32_t*>(raw0 + 2 * kRawBuf);
   uint32_t* gqueue = queue + kGemmTile;
-  uint32_t* ctrl = gqueue + kGenericSlots;
-  _Float16* W = reinterpret_cast<_Float16*>(ctrl + 4);
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  uint32_t* ctrl0 = gqueue + kGenericSlots;  // two sets of four counters
+  _Float16* W0 = reinterpret_cast<_Float16*>(ctrl0 + 8);
+  constexpr uint32_t kWBuf = kGemmRows * kGemmWStride;  // elements per W buffer
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
   const uint32_t nb = a.nblocks;
   const uint32_t n_units = a.n_bands * a.S;
 
-  // 32-row and 32-column tiles per wavefront.  Two column tiles would halve the operand
-  // traffic per MFMA, but 64 accumulator registers beside the decode phases' state spill
-  // (measured: 124 instead of 196 TFLOP/s at M = 512).
-  constexpr int RT = 2, CT = 1;
-  const uint32_t ctn = 1u << a.ct_shift, kparts = 16u >> a.ct_shift;
-  const uint32_t ctile = wave & (ctn - 1u), kpart = wave >> a.ct_shift;
-  const uint32_t l32 = lane & 31u, lh = lane >> 5;
-  uint32_t my_m[CT];  // the activation rows this lane feeds and receives
-#pragma unroll
-  for (int c = 0; c < CT; ++c) my_m[c] = (ctile * CT + c) * 32u + l32;
-
-  // code bytes of (unit, slice) -> one register per lane
-  auto prefetch = [&](uint32_t r0, uint32_t rows, uint32_t k0, uint32_t kb, uint4& pre) {
-    const uint32_t row = tid / kGemmRowChunks, j = tid - row * kGemmRowChunks;
-    if (row < rows && kb) {
-      const size_t byte0 = ((size_t)(r0 + row) * nb + k0) * 6;
-      const uint32_t off = (uint32_t)(byte0 & 15);
-      const uint32_t n16 = (off + kb * 6 + 15) >> 4;
-      if (j < n16) pre = reinterpret_cast<const uint4*>(a.codes + (byte0 - off))[j];
-    }
+  auto open_unit = [&](SliceWalk& w, uint32_t unit) {
+    w.unit = unit;
+    w.si = 0;
+    if (unit >= n_units) return;
+    w.band = unit / a.S;
+    w.split = unit - w.band * a.S;
+    w.r0 = w.band * kGemmRows;
+    w.rows = min((uint32_t)kGemmRows, a.d_out - w.r0);
+    w.kb_lo = min(nb, w.split * a.bps);
+    w.kb_hi = min(nb, w.kb_lo + a.bps);
+    w.n_slices = (w.kb_hi - w.kb_lo + kGemmKb - 1) / kGemmKb;  // >= 1: the host leaves no split empty
+    w.sj = (w.band * 5u) % w.n_slices;
+  };
+  auto advance = [&](SliceWalk& w) {
+    w.sj = w.sj + 1 == w.n_slices ? 0u : w.sj + 1;
+    if (++w.si == w.n_slices) open_unit(w, w.unit + gridDim.x);
   };
 
-#ifdef LLVQ_PHASE_TIMING
-  if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 7] = wall_clock64();
-#endif
-  for (uint32_t unit = blockIdx.x; unit < n_units; unit += gridDim.x) {
-    const uint32_t band = unit / a.S, split = unit - band * a.S;
-    const uint32_t r0 = band * kGemmRows, rows = min((uint32_t)kGemmRows, a.d_out - r0);
-    const uint32_t kb_lo = min(nb, split * a.bps), kb_hi = min(nb, kb_lo + a.bps);
-    float16_t acc[RT][CT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int c = 0; c < CT; ++c)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[rt][c][j] = 0.f;
+  // Both W buffers start as zeros: a slice shorter than 16 blocks per row leaves columns the
+  // consumers still multiply (by zero activations), which must therefore be finite.
+  for (uint32_t o = tid; o < 2 * kWBuf / 8; o += kWgThreads) reinterpret_cast<uint4*>(W0)[o] = make_uint4(0, 0, 0, 0);
 
+  if (wave < (uint32_t)PW) {
+    // ---------------- producers ----------------
+    // Stage g: P1 of slice g | barrier | code bytes of slice g + 1 -> the other raw buffer, P2 of slice g | barrier.
+    auto prefetch = [&](const SliceWalk& w, uint4& pre) {
+      if (w.unit >= n_units) return;
+      const uint32_t k0 = w.kb_lo + w.sj * kGemmKb, kb = min((uint32_t)kGemmKb, w.kb_hi - k0);
+      const uint32_t row = tid / kGemmRowChunks, j = tid - row * kGemmRowChunks;
+      if (row < w.rows) {
+        const size_t byte0 = ((size_t)(w.r0 + row) * nb + k0) * 6;
+        const uint32_t off = (uint32_t)(byte0 & 15);
+        const uint32_t n16 = (off + kb * 6 + 15) >> 4;
+        if (j < n16) pre = reinterpret_cast<const uint4*>(a.codes + (byte0 - off))[j];
+      }
+    };
+    auto stage_raw = [&](uint32_t buf, const uint4& pre) {
+      if (tid < 4) ctrl0[buf * 4 + tid] = 0;
+      if (tid < (uint32_t)(kGemmRows * kGemmRowChunks)) reinterpret_cast<uint4*>(raw0 + buf * kRawBuf)[tid] = pre;
+    };
+    SliceWalk w, ahead;
+    open_unit(w, blockIdx.x);
     uint4 pre = make_uint4(0, 0, 0, 0);
-    // Units walk their slices from different starting points (a fixed function of
-    // the band), so that the CUs do not all pull the same activation columns
-    // through the same L2 channels at the same time.
-    const uint32_t n_slices = (kb_hi - kb_lo + kGemmKb - 1) / kGemmKb;
-    uint32_t sj = n_slices ? (band * 5u) % n_slices : 0u;
-    if (n_slices) prefetch(r0, rows, kb_lo + sj * kGemmKb, min((uint32_t)kGemmKb, kb_hi - (kb_lo + sj * kGemmKb)), pre);
-    for (uint32_t si = 0; si < n_slices; ++si) {
-      const uint32_t k0 = kb_lo + sj * kGemmKb;
-      const uint32_t kb = min((uint32_t)kGemmKb, kb_hi - k0);
-      sj = sj + 1 == n_slices ? 0u : sj + 1;
-      const uint32_t nblk = rows * kb;
+    prefetch(w, pre);
+    stage_raw(0, pre);
+    ahead = w;
+    advance(ahead);
+    prefetch(ahead, pre);  // slice 1, stored during stage 0
+    wg_barrier();          // slice 0's code bytes and the table image are in LDS
+    uint32_t buf = 0;
+#ifdef LLVQ_PHASE_TIMING
+    uint32_t stage_no = 0;
+#endif
+    while (w.unit < n_units) {
+#ifdef LLVQ_PHASE_TIMING
+      ++stage_no;
+#endif
+      LLVQ_GSTAMP(0, 0);
+      const uint32_t k0 = w.kb_lo + w.sj * kGemmKb;
+      const uint32_t kb = min((uint32_t)kGemmKb, w.kb_hi - k0);
+      const uint32_t r0 = w.r0, nblk = w.rows * kb;
       const uint32_t inv_kb = (65536u + kb - 1u) / kb;  // floor(f / kb) = (f * inv_kb) >> 16 for f < 2048, kb <= 32
-      // P0
-      if (tid < 4) ctrl[tid] = 0;
-      if (tid < (uint32_t)(kGemmRows * kGemmRowChunks)) reinterpret_cast<uint4*>(raw)[tid] = pre;
-      __syncthreads();
-      LLVQ_GSTAMP(0);
-      if (si + 1 < n_slices) prefetch(r0, rows, kb_lo + sj * kGemmKb, min((uint32_t)kGemmKb, kb_hi - (kb_lo + sj * kGemmKb)), pre);
-
+      const uint8_t* raw = raw0 + buf * kRawBuf;
+      uint32_t* ctrl = ctrl0 + buf * 4;
       auto record_at = [&](uint32_t row, uint32_t b) -> uint64_t {
         const uint32_t off = ((((r0 + row) * nb + k0) & 7u) * 6u) & 15u;  // (6 n) mod 16 depends on n mod 8 only
         return read_record(raw, row * kGemmRowBytes + off + 6u * b);
       };
-
-      // P1: classify and bin.  An origin block is queued: its 24 zero weights are
-      // written in P2, because the W slice may still be read by the previous slice's P3 now.
-      classify_and_bin<kGemmP1Blocks>(
+      // P1.  An origin block is queued like any other: its 24 zero weights must be written.
+      classify_and_bin<kP1Blocks, kProducers>(
           T, nblk, kGemmTile, queue, gqueue, ctrl,
           [&](uint32_t f) {
             const uint32_t row = (f * inv_kb) >> 16;
             return record_at(row, f - row * kb);
           },
           [](uint32_t) { return true; });
-      __syncthreads();
-      LLVQ_GSTAMP(1);
-
-      // P2: unrank into the W slice
-      unrank_queues_to_slice<kGemmTile, kGemmWStride>(T, queue, gqueue, ctrl, kb, inv_kb, a.g0, a.g1, W, record_at);
-      LLVQ_GSTAMP(2);
-      __syncthreads();
-      LLVQ_GSTAMP(3);
-
-      // P3: acc += W_slice (64 x 24 kb) * X^T (24 kb x M).  K runs in steps of 32
-      // (two MFMAs of 16): lane (l32, lh) holds columns [32 p + 16 lh, +16) of its
-      // row as two fragments, for W and X alike, so an activation row is read in
-      // 64-byte runs.  Columns past the slice are zeroed on both sides.
-      if (ctile * CT * 32u < a.M) {  // column tiles beyond the batch have nothing to add
-        const uint32_t kcols = kb * 24u, psteps = (kcols + 31u) >> 5;
-        const __half* xrow[CT];
-        bool m_in[CT];
-#pragma unroll
-        for (int c = 0; c < CT; ++c) {
-          xrow[c] = a.x + (size_t)k0 * 24u + (size_t)min(my_m[c], a.M - 1u) * a.ldx + lh * 16u;
-          m_in[c] = my_m[c] < a.M;
-        }
-        const _Float16* arow = W + (size_t)l32 * kGemmWStride + lh * 16u;
-        constexpr int G = CT == 1 ? 2 : 1;  // K-steps per batch of activation loads
-        const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-        half8_t cur[G][CT][2], nxt[G][CT][2];
-        auto fetch = [&](uint32_t i0, half8_t (&dst)[G][CT][2]) {  // owned K-steps i0 .. i0+G-1
-#pragma unroll
-          for (int g = 0; g < G; ++g)
-#pragma unroll
-            for (int c = 0; c < CT; ++c)
-#pragma unroll
-              for (int f = 0; f < 2; ++f) {
-                const uint32_t p = kpart + (i0 + g) * kparts, kc = p * 32u + lh * 16u + f * 8u;
-                dst[g][c][f] = (m_in[c] && kc < kcols) ? *reinterpret_cast<const half8_t*>(xrow[c] + p * 32u + f * 8u) : zero;
-              }
-        };
-        const uint32_t n_own = kpart < psteps ? (psteps - kpart + kparts - 1u) / kparts : 0u;
-        fetch(0, cur);
-        for (uint32_t i0 = 0; i0 < n_own; i0 += G) {
-          if (i0 + G < n_own) fetch(i0 + G, nxt);
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            if (i0 + g < n_own) {
-              const uint32_t p = kpart + (i0 + g) * kparts;
-#pragma unroll
-              for (int f = 0; f < 2; ++f) {
-                const bool kin = p * 32u + lh * 16u + f * 8u < kcols;
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) {
-                  const half8_t av = kin ? *reinterpret_cast<const half8_t*>(arow + (size_t)rt * 32 * kGemmWStride + p * 32u + f * 8u) : zero;
-#pragma unroll
-                  for (int c = 0; c < CT; ++c)
-                    acc[rt][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, cur[g][c][f], acc[rt][c], 0, 0, 0);
-                }
-              }
-            }
-          }
-#pragma unroll
-          for (int g = 0; g < G; ++g)
-#pragma unroll
-            for (int c = 0; c < CT; ++c)
-#pragma unroll
-              for (int f = 0; f < 2; ++f) cur[g][c][f] = nxt[g][c][f];
-        }
-      }
-      LLVQ_GSTAMP(4);
-      // no barrier here: the next slice's P0/P1 touch only raw, queues and
-      // counters, and its P2 starts behind two barriers every wavefront reaches
-      // after leaving P3
+      LLVQ_GSTAMP(0, 1);
+      wg_barrier();
+      LLVQ_GSTAMP(0, 2);
+      // the next slice's code bytes and counters: that buffer was last read in the stage before
+      if (ahead.unit < n_units) stage_raw(buf ^ 1u, pre);
+      w = ahead;
+      advance(ahead);
+      prefetch(ahead, pre);
+      // P2
+      unrank_queues_to_slice<kGemmTile, kGemmWStride>(T, queue, gqueue, ctrl, kb, inv_kb, a.g0, a.g1, W0 + buf * kWBuf, record_at);
+      LLVQ_GSTAMP(0, 3);
+      wg_barrier();
+      LLVQ_GSTAMP(0, 4);
+      buf ^= 1u;
     }
-
-    // ---- epilogue ----
-    // acc[rt][c][j] belongs to weight row r0 + rt*32 + 8 (j/4) + 4 lh + j%4 and activation row my_m[c].
-    // The tail columns (f32 weights, kept out of the binary16 contraction) are
-    // staged in the W area: tl[row][t] as f32 and xt[m][t] as binary16.
-    const uint32_t tw = a.tail_w;
-    float* tl = reinterpret_cast<float*>(W);
-    __half* xt = reinterpret_cast<__half*>(tl + kGemmRows * (kDim - 1));
-    static_assert((size_t)(2 * kGemmRows + kGemmMaxM) * (kDim - 1) * 2 <= (size_t)kGemmRows * kGemmWStride * 2,
-                  "tail staging fits the W area");
-    auto stage_tail = [&]() {  // call with every wavefront past its last read of W
-      for (uint32_t o = tid; o < rows * tw; o += kWgThreads) tl[o] = a.tail[(size_t)r0 * tw + o];
-      const __half* xtail = a.x + (size_t)nb * 24u;
-      for (uint32_t o = tid; o < a.M * tw; o += kWgThreads) {
-        const uint32_t m = o / tw, t = o - m * tw;
-        xt[o] = xtail[(size_t)m * a.ldx + t];
-      }
+    // the consumers' last stage
+    wg_barrier();
+    wg_barrier();
+  } else {
+    // ---------------- consumers ----------------
+    // Consumer c owns activation rows [64 ctile, +64) on the K-steps p = kpart (mod kparts) of
+    // every slice: 12 / kparts steps, whatever the slice's length (past a short last slice's end
+    // the activations are zero and the W buffer holds finite leftovers).  The loop is
+    // branch-free, and the B fragments of three K-steps are in flight at any time, across
+    // barriers and from one slice into the next: step i of the sequence lives in ring slot i mod 3.
+    const uint32_t c = wave - (uint32_t)PW;
+    const uint32_t ctn = 1u << a.ct_shift, kparts = (uint32_t)kConsumers >> a.ct_shift;
+    const uint32_t ctile = c & (ctn - 1u), kpart = c >> a.ct_shift;
+    const uint32_t l32 = lane & 31u, lh = lane >> 5;
+    const uint32_t m0 = ctile * kGemmColTile;
+    const bool tile_live = m0 < a.M;  // a consumer past the batch's last tile multiplies that tile again and stores nothing
+    // K-step p of the matrix: 32 binary16 values per activation row, rows 64 bytes apart.  A load
+    // address is a wavefront-uniform base (slice, K-step) plus this lane's byte offset in the step.
+    const uint32_t lane_off = (min(m0, a.m_pad - kGemmColTile) + l32) * 64u + lh * 32u;
+    const size_t step_bytes = (size_t)a.m_pad * 64u;
+    const size_t own_bytes = (size_t)kparts * step_bytes;  // between two of this consumer's K-steps
+    const uint32_t n_own = (uint32_t)(kGemmKb * 24 / 32) / kparts;  // 12, 6 or 3 K-steps
+    auto slice_base = [&](const SliceWalk& w) {  // 24 k0 / 32 K-steps precede the slice; k0 is a multiple of 4
+      return reinterpret_cast<const uint8_t*>(a.xt) + (size_t)((w.kb_lo + w.sj * kGemmKb) * 3u / 4u + kpart) * step_bytes;
     };
-    const bool vec_ok = (a.d_out & 3u) == 0;  // four consecutive rows of one activation row store as one vector
-    __syncthreads();  // every wavefront is past its last read of W
-    if (kparts > 1) {
-      // sums of the K-step shares -> the kpart 0 wavefront of each column group, one
-      // 32 x 32 tile at a time through the W area: red[kpart - 1][ctile][j4][lane]
-      float4* red = reinterpret_cast<float4*>(W);
-      static_assert((size_t)15 * 4 * 64 * 16 <= (size_t)kGemmRows * kGemmWStride * 2, "K-step shares fit the W area");
+    half8_t ring[2][2][2];
+    auto fetch = [&](const uint8_t* step, half8_t (&dst)[2][2]) {
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+      for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-        for (int c = 0; c < CT; ++c) {
-          if (kpart > 0) {
+        for (int f = 0; f < 2; ++f) dst[ct][f] = *reinterpret_cast<const half8_t*>(step + lane_off + ct * 32 * 64 + f * 16);
+    };
+
+    SliceWalk w, ahead;
+    open_unit(w, blockIdx.x);
+    ahead = w;
+    advance(ahead);
+    const uint8_t* xs = slice_base(w);
+    fetch(xs, ring[0]);
+
+    consumer_barrier();  // the table image (unused here) and slice 0's code bytes
+    // stage 0: nothing to multiply yet
+    consumer_barrier();
+    consumer_barrier();
+
+    uint32_t buf = 0;
+    float16_t acc[2][2];
+    auto clear_acc = [&]() {
 #pragma unroll
-            for (int j4 = 0; j4 < 4; ++j4)
-              red[(((kpart - 1u) * ctn + ctile) * 4u + j4) * 64u + lane] =
-                  make_float4(acc[rt][c][4 * j4], acc[rt][c][4 * j4 + 1], acc[rt][c][4 * j4 + 2], acc[rt][c][4 * j4 + 3]);
-          }
-          __syncthreads();
-          if (kpart == 0) {
-            for (uint32_t kp = 1; kp < kparts; ++kp)
+      for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-              for (int j4 = 0; j4 < 4; ++j4) {
-                const float4 v = red[(((kp - 1u) * ctn + ctile) * 4u + j4) * 64u + lane];
-                acc[rt][c][4 * j4] += v.x;
-                acc[rt][c][4 * j4 + 1] += v.y;
-                acc[rt][c][4 * j4 + 2] += v.z;
-                acc[rt][c][4 * j4 + 3] += v.w;
-              }
-          }
-          __syncthreads();
-        }
-    }
-    if (a.S > 1) {
-      // gemm_reduce_kernel finishes these rows.  The workspace is [split][band][m][64]:
-      // a unit's partial sums are one contiguous piece, and rows past the end of the
-      // last band are written but never read.
+        for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-      for (int c = 0; c < CT; ++c) {
-        if (kpart == 0 && my_m[c] < a.M) {
-          float* dst = a.ws + (((size_t)split * a.n_bands + band) * a.M + my_m[c]) * kGemmRows;
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-            for (int j4 = 0; j4 < 4; ++j4)
-              *reinterpret_cast<float4*>(dst + rt * 32u + 8u * j4 + 4u * lh) =
-                  make_float4(acc[rt][c][4 * j4], acc[rt][c][4 * j4 + 1], acc[rt][c][4 * j4 + 2], acc[rt][c][4 * j4 + 3]);
-        }
-      }
-    } else {
-      if (tw) stage_tail();
-      __syncthreads();
-#pragma unroll
-      for (int c = 0; c < CT; ++c) {
-        if (kpart == 0 && my_m[c] < a.M) {
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-            for (int j4 = 0; j4 < 4; ++j4) {
-              const uint32_t row = rt * 32u + 8u * j4 + 4u * lh;
-              float v[4];
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                const uint32_t r = min(row + i, rows - 1u);
-                float ts = 0.f;
-                for (uint32_t t = 0; t < tw; ++t) ts = fmaf(tl[r * tw + t], __half2float(xt[my_m[c] * tw + t]), ts);
-                v[i] = fmaf(acc[rt][c][4 * j4 + i], a.rscale[r0 + r], ts);
-              }
-              const size_t at = (size_t)my_m[c] * a.d_out + r0 + row;
-              if (vec_ok && row + 3 < rows) {
-                if constexpr (sizeof(OutT) == 4) {
-                  *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
-                } else {
-                  const __half2 lo = __float22half2_rn(make_float2(v[0], v[1])), hi = __float22half2_rn(make_float2(v[2], v[3]));
-                  uint2 pk;
-                  pk.x = *reinterpret_cast<const uint32_t*>(&lo);
-                  pk.y = *reinterpret_cast<const uint32_t*>(&hi);
-                  *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(a.y) + at) = pk;
-                }
-              } else {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                  if (row + i < rows) store_y<OutT>(a.y, at + i, v[i]);
-              }
-            }
-        }
-      }
-    }
+          for (int j = 0; j < 16; ++j) acc[rt][ct][j] = 0.f;
+    };
+    clear_acc();
+    const uint32_t a_lane = (l32 * kGemmWStride + lh * 16u + kpart * 32u) * 2u;  // this lane's byte offset in a W buffer
 #ifdef LLVQ_PHASE_TIMING
-    if (threadIdx.x == 0 && unit == blockIdx.x) g_phase_stamps[blockIdx.x * 8 + 5] = wall_clock64();
+    uint32_t stage_no = 1;
 #endif
-    __syncthreads();  // W, raw and counters are reused by the next unit
+    while (w.unit < n_units) {
+#ifdef LLVQ_PHASE_TIMING
+      ++stage_no;
+#endif
+      LLVQ_GSTAMP(256, 0);
+      const bool last_of_unit = w.si + 1 == w.n_slices;
+      // The loads run ahead into the unit's next slice.  At the unit's end they re-read this
+      // slice (the ring starts afresh behind the epilogue, which needs the registers).
+      const uint8_t* xs_next = last_of_unit ? xs : slice_base(ahead);
+      const uint8_t* wbuf = reinterpret_cast<const uint8_t*>(W0 + buf * kWBuf);
+      auto multiply = [&](uint32_t i, const half8_t (&b)[2][2]) {
+        const uint8_t* ap = wbuf + a_lane + i * kparts * 64u;
+#pragma unroll
+        for (int f = 0; f < 2; ++f) {
+#pragma unroll
+          for (int rt = 0; rt < 2; ++rt) {
+            const half8_t av = *reinterpret_cast<const half8_t*>(ap + rt * 32 * kGemmWStride * 2 + f * 16);
+            acc[rt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, b[0][f], acc[rt][0], 0, 0, 0);
+            acc[rt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, b[1][f], acc[rt][1], 0, 0, 0);
+          }
+        }
+      };
+      auto step_src = [&](uint32_t i) { return i < n_own ? xs + i * own_bytes : xs_next + (i - n_own) * own_bytes; };
+      // a quarter of the K-steps beside the producers' classification, the rest beside their unranking
+      const uint32_t i_a = n_own >= 12 ? 2u : 0u;
+      uint32_t i = 0;
+      for (; i + 1 < n_own; i += 2) {
+        if (i == i_a) {
+          LLVQ_GSTAMP(256, 1);
+          consumer_barrier();
+          LLVQ_GSTAMP(256, 2);
+        }
+        fetch(step_src(i + 1), ring[1]);
+        multiply(i, ring[0]);
+        fetch(step_src(i + 2), ring[0]);
+        multiply(i + 1, ring[1]);
+      }
+      if (i < n_own) {  // an odd count (three K-steps): the last one
+        fetch(step_src(i + 1), ring[1]);
+        multiply(i, ring[0]);
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int f = 0; f < 2; ++f) ring[0][ct][f] = ring[1][ct][f];
+      }
+      LLVQ_GSTAMP(256, 3);
+      consumer_barrier();
+      LLVQ_GSTAMP(256, 4);
+
+      const SliceWalk done = w;
+      w = ahead;
+      advance(ahead);
+      xs = slice_base(w);  // past the last unit: an address that is not read
+      buf ^= 1u;
+      if (last_of_unit) {
+        // the unit's sums: acc[rt][ct][j] belongs to weight row r0 + 32 rt + 8 (j / 4) + 4 lh + j % 4
+        // and activation row m0 + 32 ct + l32
+        if (tile_live) {
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct) {
+            const uint32_t my_m = m0 + 32u * ct + l32;
+            if (my_m < a.M) {
+              float* dst = a.ws + (((size_t)(done.split * kparts + kpart) * a.n_bands + done.band) * a.M + my_m) * kGemmRows;
+#pragma unroll
+              for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                for (int j4 = 0; j4 < 4; ++j4)
+                  *reinterpret_cast<float4*>(dst + rt * 32u + 8u * j4 + 4u * lh) =
+                      make_float4(acc[rt][ct][4 * j4], acc[rt][ct][4 * j4 + 1], acc[rt][ct][4 * j4 + 2], acc[rt][ct][4 * j4 + 3]);
+            }
+          }
+        }
+        clear_acc();
+        if (w.unit < n_units) fetch(xs, ring[0]);
+      }
+    }
   }
 }
 

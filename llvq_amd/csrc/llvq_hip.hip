@@ -862,7 +862,6 @@ __global__ __launch_bounds__(1024) void rotate_kernel(RotArgs a) {
 }  // namespace llvq
 
 #include "gemm_kernel.h"
-#include "gemm_pipe_kernel.h"
 #include "decoder.h"
 
 // =================================================================================
@@ -984,10 +983,8 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   for_each_gemv_kernel([&](const void* kernel) { (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds); });
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<__half>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_pipe_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_pipe_kernel<12>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiles_kernel<12>), hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
   *out = rt;
   return LLVQ_OK;
 }
@@ -1473,39 +1470,16 @@ int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
 
 // Split of a matrix's block range over work units: the count that minimises a
 // coarse time model (rounds of units over the CUs x per-unit time), so that a
-// matrix with few 64-row bands still occupies the chip.
-static void pick_gemm_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint32_t grid, uint32_t* S_out,
-                            uint32_t* bps_out) {
-  double best = 1e30;
-  uint32_t best_s = 1, best_bps = nblocks ? nblocks : 1;
-  // MFMA phase of a full slice: 24 K-steps shared by the wavefronts of a column tile
-  uint32_t col_tiles = 1;
-  while (col_tiles * 32u < M && col_tiles < 16) col_tiles *= 2;
-  const double mfma_us = 0.5 + 0.75 * ((24 * col_tiles + 15) / 16);
-  for (uint32_t S = 1; S <= 64 && S <= (nblocks ? nblocks : 1); ++S) {
-    const uint32_t bps = (nblocks + S - 1) / S;
-    if ((uint64_t)(S - 1) * bps >= nblocks && S > 1) continue;  // an empty last split
-    const uint32_t slices = (bps + kGemmKb - 1) / kGemmKb;
-    const double unit_us = 2.0 + slices * (4.5 + mfma_us) + 64.0 * bps * 0.0042 + 0.015 * M + (S > 1 ? 0.002 * M : 0.0);
-    const uint64_t units = (uint64_t)n_bands * S;
-    // a split launch pays a second, chip-wide pass over S partial sums per output
-    const double reduce_us = S > 1 ? 6.0 + (double)S * M * 64.0 * n_bands * 4.0 / 2.0e6 : 0.0;
-    const double t = (double)((units + grid - 1) / grid) * unit_us + reduce_us;
-    if (t < best * 0.999) { best = t; best_s = S; best_bps = bps; }
-  }
-  *S_out = best_s;
-  *bps_out = best_bps;
-}
-
-// The same choice for the pipelined kernel: a slice of 16 blocks per row costs what its
-// unranking costs (the matrix-core work of the slice before runs beside it), a unit
-// pays one more stage to drain, and every launch ends in the chip-wide sum.  Splits are
-// whole slices, so every slice starts on a 32-column K-step of the tiled activations.
-static void pick_pipe_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint32_t kparts, uint32_t grid,
+// matrix with few 64-row bands still occupies the chip.  A slice of 16 blocks per
+// row costs what its unranking costs (the matrix-core work of the slice before runs
+// beside it), a unit pays one more stage to drain, and every launch ends in the
+// chip-wide sum.  Splits are whole slices, so every slice starts on a 32-column
+// K-step of the tiled activations.
+static void pick_gemm_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint32_t kparts, uint32_t grid,
                             uint32_t* S_out, uint32_t* bps_out) {
   double best = 1e30;
-  const uint32_t total_slices = (nblocks + kPipeKb - 1) / kPipeKb;
-  uint32_t best_s = 1, best_bps = total_slices * kPipeKb;
+  const uint32_t total_slices = (nblocks + kGemmKb - 1) / kGemmKb;
+  uint32_t best_s = 1, best_bps = total_slices * kGemmKb;
   const double stage_us = 7.5;
   for (uint32_t per = total_slices; per >= 1; --per) {  // slices per split
     const uint32_t S = (total_slices + per - 1) / per;
@@ -1515,136 +1489,83 @@ static void pick_pipe_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint
     const uint64_t units = (uint64_t)n_bands * S;
     const double reduce_us = 6.0 + (double)S * kparts * M * 64.0 * n_bands * 4.0 / 2.0e6;
     const double t = (double)((units + grid - 1) / grid) * unit_us + reduce_us;
-    if (t < best * 0.999) { best = t; best_s = S; best_bps = per * kPipeKb; }
+    if (t < best * 0.999) { best = t; best_s = S; best_bps = per * kGemmKb; }
   }
   *S_out = best_s;
   *bps_out = best_bps;
 }
 
-static int grow_gemm_workspace(llvq_rt* rt, size_t need) {
-  if (need <= rt->gemm_ws_bytes) return LLVQ_OK;
-  (void)hipFree(rt->gemm_ws);  // waits for launches that still use it
-  rt->gemm_ws = nullptr;
-  rt->gemm_ws_bytes = 0;
-  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_ws), need));
-  rt->gemm_ws_bytes = need;
+// Grows a device buffer of the runtime to `need` bytes (contents are not kept).
+static int grow_buffer(void** buf, size_t* have, size_t need) {
+  if (need <= *have) return LLVQ_OK;
+  (void)hipFree(*buf);  // waits for launches that still use it
+  *buf = nullptr;
+  *have = 0;
+  HIP_TRY(hipMalloc(buf, need));
+  *have = need;
   return LLVQ_OK;
 }
 
-static int launch_gemm_reduce(llvq_rt* rt, const GemmArgs& a, uint32_t n_partials, bool f32) {
-  GemmReduceArgs r{};
-  r.ws = a.ws;
-  r.x = a.x;
-  r.rscale = a.rscale;
-  r.tail = a.tail;
-  r.y = a.y;
-  r.M = a.M;
-  r.ldx = a.ldx;
-  r.d_out = a.d_out;
-  r.nblocks = a.nblocks;
-  r.tail_w = a.tail_w;
-  r.S = n_partials;
-  r.n_bands = a.n_bands;
-  const uint32_t rgrid = a.n_bands * ((a.M + kReduceRowsM - 1) / kReduceRowsM);
-  if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3(rgrid), dim3(256), 0, rt->stream, r);
-  else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3(rgrid), dim3(256), 0, rt->stream, r);
-  HIP_TRY(hipGetLastError());
-  return LLVQ_OK;
-}
-
-// Batches of at least this many activation rows take the pipelined kernel.
-static uint32_t pipe_min_rows() {
-  static const uint32_t v = [] {
-    const char* e = std::getenv("LLVQ_GEMM_PIPE_MIN_M");
-    return e ? (uint32_t)std::strtoul(e, nullptr, 10) : 2u;
-  }();
-  return v;
-}
-
-static uint32_t pipe_narrow_rows() {
-  static const uint32_t v = [] {
-    const char* e = std::getenv("LLVQ_GEMM_PIPE_NARROW_M");
-    return e ? (uint32_t)std::strtoul(e, nullptr, 10) : 256u;
-  }();
-  return v;
-}
+// Batches of up to this many activation rows leave the matrix cores little to do:
+// twelve of the sixteen wavefronts unrank and four multiply (four consumers cover 256 rows).
+constexpr uint32_t kGemmNarrowRows = 256;
 
 static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M, void* y, int y_dtype) {
   const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
+  const bool f32 = y_dtype == LLVQ_F32;
   GemmArgs a{};
   a.tables = rt->tables;
-  a.x = reinterpret_cast<const __half*>(x);
   a.codes = m->codes;
-  a.rscale = m->rscale;
-  a.tail = m->tail;
-  a.y = y;
   a.g0 = m->g[0];
   a.g1 = m->g[1];
   a.M = M;
-  a.ldx = m->d_in;
+  a.m_pad = (M + kGemmColTile - 1) / kGemmColTile * kGemmColTile;
   a.d_out = m->d_out;
   a.nblocks = m->nblocks;
-  a.tail_w = m->tail_w;
   a.n_bands = (m->d_out + kGemmRows - 1) / kGemmRows;
-  const bool f32 = y_dtype == LLVQ_F32;
-  if (M >= pipe_min_rows()) {
-    GemmPipeArgs pa{};
-    pa.tables = rt->tables;
-    pa.codes = m->codes;
-    pa.g0 = m->g[0];
-    pa.g1 = m->g[1];
-    pa.M = M;
-    pa.m_pad = (M + kPipeColTile - 1) / kPipeColTile * kPipeColTile;
-    pa.d_out = m->d_out;
-    pa.nblocks = m->nblocks;
-    pa.n_bands = a.n_bands;
-    // the consumer wavefronts (four up to 128 activation rows, eight beyond) over the batch's
-    // 64-row tiles, the count rounded up to a power of two
-    const uint32_t consumers = M <= pipe_narrow_rows() ? 4u : 8u;
-    pa.ct_shift = 0;
-    while (((uint32_t)kPipeColTile << pa.ct_shift) < M) ++pa.ct_shift;
-    const uint32_t kparts = consumers >> pa.ct_shift;
-    pick_pipe_split(pa.n_bands, m->nblocks, M, kparts, grid_cap, &pa.S, &pa.bps);
-    int rc = grow_gemm_workspace(rt, (size_t)pa.S * kparts * pa.n_bands * M * kGemmRows * sizeof(float));
-    if (rc) return rc;
-    const uint32_t n_steps = (m->nblocks * 24u + 31u) / 32u;
-    const size_t xt_bytes = (size_t)n_steps * pa.m_pad * 64;
-    if (xt_bytes > rt->gemm_xt_bytes) {
-      (void)hipFree(rt->gemm_xt);
-      rt->gemm_xt = nullptr;
-      rt->gemm_xt_bytes = 0;
-      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->gemm_xt), xt_bytes));
-      rt->gemm_xt_bytes = xt_bytes;
-    }
-    hipLaunchKernelGGL(tile_activations_kernel, dim3((uint32_t)((xt_bytes / 16 + 255) / 256)), dim3(256), 0, rt->stream, a.x, M,
-                       a.ldx, m->nblocks * 24u, pa.m_pad, n_steps, reinterpret_cast<uint4*>(rt->gemm_xt));
-    HIP_TRY(hipGetLastError());
-    pa.xt = rt->gemm_xt;
-    pa.ws = rt->gemm_ws;
-    a.ws = rt->gemm_ws;
-    const uint32_t units = pa.n_bands * pa.S;
-    const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
-    if (consumers == 4) hipLaunchKernelGGL(gemm_pipe_kernel<12>, grid, wg, gemm_pipe_lds_bytes(), rt->stream, pa);
-    else hipLaunchKernelGGL(gemm_pipe_kernel<8>, grid, wg, gemm_pipe_lds_bytes(), rt->stream, pa);
-    HIP_TRY(hipGetLastError());
-    return launch_gemm_reduce(rt, a, pa.S * kparts, f32);
-  }
-  pick_gemm_split(a.n_bands, m->nblocks, M, grid_cap, &a.S, &a.bps);
-  if (a.S > 1) {
-    const int rc = grow_gemm_workspace(rt, (size_t)a.S * a.n_bands * M * kGemmRows * sizeof(float));
-    if (rc) return rc;
-    a.ws = rt->gemm_ws;
-  }
+  // the consumer wavefronts over the batch's 64-row tiles, the count rounded up to a power of two
+  const uint32_t consumers = M <= kGemmNarrowRows ? 4u : 8u;
+  a.ct_shift = 0;
+  while (((uint32_t)kGemmColTile << a.ct_shift) < M) ++a.ct_shift;
+  const uint32_t kparts = consumers >> a.ct_shift;
+  pick_gemm_split(a.n_bands, m->nblocks, M, kparts, grid_cap, &a.S, &a.bps);
+  const uint32_t n_partials = a.S * kparts;
+  int rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes,
+                       (size_t)n_partials * a.n_bands * M * kGemmRows * sizeof(float));
+  if (rc) return rc;
+  // every slice has all its twelve K-steps in the tiled copy, zeros past the matrix's last block
+  const uint32_t n_steps = (m->nblocks + kGemmKb - 1) / kGemmKb * (kGemmKb * 24 / 32);
+  const size_t xt_bytes = (size_t)n_steps * a.m_pad * 64;
+  rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_xt), &rt->gemm_xt_bytes, xt_bytes);
+  if (rc) return rc;
+  const __half* xh = reinterpret_cast<const __half*>(x);
+  hipLaunchKernelGGL(tile_activations_kernel, dim3((uint32_t)((xt_bytes / 16 + 255) / 256)), dim3(256), 0, rt->stream, xh, M,
+                     m->d_in, m->nblocks * 24u, a.m_pad, n_steps, reinterpret_cast<uint4*>(rt->gemm_xt));
+  HIP_TRY(hipGetLastError());
+  a.xt = rt->gemm_xt;
+  a.ws = rt->gemm_ws;
   const uint32_t units = a.n_bands * a.S;
   const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
-  const size_t lds = gemm_lds_bytes();
-  // sixteen wavefronts over the batch's 32-column tiles, the count rounded up to a power of two
-  a.ct_shift = 0;
-  while ((32u << a.ct_shift) < M && a.ct_shift < 4) ++a.ct_shift;
-  if (f32) hipLaunchKernelGGL(gemm_tiles_kernel<float>, grid, wg, lds, rt->stream, a);
-  else hipLaunchKernelGGL(gemm_tiles_kernel<__half>, grid, wg, lds, rt->stream, a);
+  if (consumers == 4) hipLaunchKernelGGL(gemm_tiles_kernel<12>, grid, wg, gemm_lds_bytes(), rt->stream, a);
+  else hipLaunchKernelGGL(gemm_tiles_kernel<8>, grid, wg, gemm_lds_bytes(), rt->stream, a);
   HIP_TRY(hipGetLastError());
-  if (a.S > 1) return launch_gemm_reduce(rt, a, a.S, f32);
+  GemmReduceArgs r{};
+  r.ws = a.ws;
+  r.x = xh;
+  r.rscale = m->rscale;
+  r.tail = m->tail;
+  r.y = y;
+  r.M = M;
+  r.ldx = m->d_in;
+  r.d_out = m->d_out;
+  r.nblocks = m->nblocks;
+  r.tail_w = m->tail_w;
+  r.S = n_partials;
+  r.n_bands = a.n_bands;
+  const uint32_t rgrid = a.n_bands * ((M + kReduceRowsM - 1) / kReduceRowsM);
+  if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3(rgrid), dim3(256), 0, rt->stream, r);
+  else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3(rgrid), dim3(256), 0, rt->stream, r);
+  HIP_TRY(hipGetLastError());
   return LLVQ_OK;
 }
 
