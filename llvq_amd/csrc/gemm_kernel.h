@@ -52,9 +52,10 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 constexpr int kGemmRows = 64;    // weight rows of a band
 constexpr int kGemmMaxM = 512;   // activation rows per launch (eight consumers x 64)
 
-// The batched kernel keeps the Golay words and the support-arrangement table in L2:
-// the 33 KB they would take in LDS buy the second W buffer.
-constexpr size_t kGemmImageBytes = kLdsImageBytesLean;
+// The batched kernel keeps the Golay words, the support-arrangement table and the class
+// lookup table in L2: the 37 KB they would take in LDS buy the second W buffer and the
+// buffers that let classification and unranking of consecutive slices share a stage.
+constexpr size_t kGemmImageBytes = kLdsImageBytesLeanest;
 
 // four packed signed bytes -> four binary16 values w * s, one rounding each
 __device__ __forceinline__ uint2 scaled_halves(uint32_t w, float s, float bias) {
@@ -151,8 +152,9 @@ constexpr int kGemmColTile = 64;                              // activation rows
 static_assert(kGemmRows * kGemmRowChunks <= kGemmMinProducers, "one 16-byte load per producer lane covers a slice's code bytes");
 static_assert(kGemmMaxM <= (kWgThreads - kGemmMinProducers) / 64 * kGemmColTile, "the consumers cover a launch's activation rows");
 
+// table image | code bytes of three slices | two block queues | two generic queues | three counter sets | two W buffers
 constexpr size_t gemm_lds_bytes() {
-  return kGemmImageBytes + 2 * (size_t)kGemmRows * kGemmRowBytes + (size_t)kGemmTile * 4 + kGenericSlots * 4 + 32 +
+  return kGemmImageBytes + 3 * (size_t)kGemmRows * kGemmRowBytes + 2 * (size_t)kGemmTile * 4 + 2 * kGenericSlots * 4 + 48 +
          2 * (size_t)kGemmRows * kGemmWStride * 2;
 }
 static_assert(gemm_lds_bytes() <= 160 * 1024, "GEMM workgroup state must fit one CU's LDS");
@@ -219,13 +221,13 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   constexpr int kP1Blocks = (kGemmTile + kProducers - 1) / kProducers;
   static_assert(kProducers >= kGemmMinProducers && (kConsumers == 8 || kConsumers == 4), "roles");
   extern __shared__ __align__(16) uint8_t smem[];
-  const DecodeTables T = stage_tables<false>(smem, a.tables);
+  const DecodeTables T = stage_tables<false, false>(smem, a.tables);
   uint8_t* raw0 = smem + kGemmImageBytes;
   constexpr uint32_t kRawBuf = kGemmRows * kGemmRowBytes;
-  uint32_t* queue = reinterpret_cast<uint32_t*>(raw0 + 2 * kRawBuf);
-  uint32_t* gqueue = queue + kGemmTile;
-  uint32_t* ctrl0 = gqueue + kGenericSlots;  // two sets of four counters
-  _Float16* W0 = reinterpret_cast<_Float16*>(ctrl0 + 8);
+  uint32_t* queue0 = reinterpret_cast<uint32_t*>(raw0 + 3 * kRawBuf);
+  uint32_t* gqueue0 = queue0 + 2 * kGemmTile;
+  uint32_t* ctrl0 = gqueue0 + 2 * kGenericSlots;  // three sets of four counters
+  _Float16* W0 = reinterpret_cast<_Float16*>(ctrl0 + 12);
   constexpr uint32_t kWBuf = kGemmRows * kGemmWStride;  // elements per W buffer
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -256,7 +258,11 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 
   if (wave < (uint32_t)PW) {
     // ---------------- producers ----------------
-    // Stage g: P1 of slice g | barrier | code bytes of slice g + 1 -> the other raw buffer, P2 of slice g | barrier.
+    // Stage g, one barrier at its end: code bytes of slice g + 2 -> LDS (loaded a stage earlier),
+    // loads of slice g + 3 issued, unranking of slice g, then classification of slice g + 1.
+    // A wavefront that runs out of chunks to unrank goes on to its share of the next slice's
+    // classification, whose dependent table reads then overlap the others' arithmetic.
+    // Buffers: code bytes and counters of slice s in set s mod 3, queues and W in set s mod 2.
     auto prefetch = [&](const SliceWalk& w, uint4& pre) {
       if (w.unit >= n_units) return;
       const uint32_t k0 = w.kb_lo + w.sj * kGemmKb, kb = min((uint32_t)kGemmKb, w.kb_hi - k0);
@@ -268,64 +274,85 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         if (j < n16) pre = reinterpret_cast<const uint4*>(a.codes + (byte0 - off))[j];
       }
     };
-    auto stage_raw = [&](uint32_t buf, const uint4& pre) {
-      if (tid < 4) ctrl0[buf * 4 + tid] = 0;
-      if (tid < (uint32_t)(kGemmRows * kGemmRowChunks)) reinterpret_cast<uint4*>(raw0 + buf * kRawBuf)[tid] = pre;
+    auto stage_raw = [&](uint32_t set, const uint4& pre) {
+      if (tid < 4) ctrl0[set * 4 + tid] = 0;
+      if (tid < (uint32_t)(kGemmRows * kGemmRowChunks)) reinterpret_cast<uint4*>(raw0 + set * kRawBuf)[tid] = pre;
     };
-    SliceWalk w, ahead;
-    open_unit(w, blockIdx.x);
+    struct SliceView {  // what the phases of one slice need
+      uint32_t k0, kb, r0, nblk, inv_kb, set3, set2;
+    };
+    auto view = [&](const SliceWalk& w, uint32_t s) {
+      SliceView v;
+      v.k0 = w.kb_lo + w.sj * kGemmKb;
+      v.kb = min((uint32_t)kGemmKb, w.kb_hi - v.k0);
+      v.r0 = w.r0;
+      v.nblk = w.rows * v.kb;
+      v.inv_kb = (65536u + v.kb - 1u) / v.kb;  // floor(f / kb) = (f * inv_kb) >> 16 for f < 2048, kb <= 32
+      v.set3 = s % 3u;
+      v.set2 = s & 1u;
+      return v;
+    };
+    auto classify = [&](const SliceView& v) {  // P1.  An origin block is queued like any other: its 24 zero weights must be written.
+      const uint8_t* raw = raw0 + v.set3 * kRawBuf;
+      classify_and_bin<kP1Blocks, kProducers>(
+          T, v.nblk, kGemmTile, queue0 + v.set2 * kGemmTile, gqueue0 + v.set2 * kGenericSlots, ctrl0 + v.set3 * 4,
+          [&](uint32_t f) {
+            const uint32_t row = (f * v.inv_kb) >> 16, b = f - row * v.kb;
+            const uint32_t off = ((((v.r0 + row) * nb + v.k0) & 7u) * 6u) & 15u;  // (6 n) mod 16 depends on n mod 8 only
+            return read_record(raw, row * kGemmRowBytes + off + 6u * b);
+          },
+          [](uint32_t) { return true; });
+    };
+    auto unrank = [&](const SliceView& v) {  // P2
+      const uint8_t* raw = raw0 + v.set3 * kRawBuf;
+      unrank_queues_to_slice<kGemmTile, kGemmWStride>(
+          T, queue0 + v.set2 * kGemmTile, gqueue0 + v.set2 * kGenericSlots, ctrl0 + v.set3 * 4, v.kb, v.inv_kb, a.g0, a.g1,
+          W0 + v.set2 * kWBuf, [&](uint32_t row, uint32_t b) -> uint64_t {
+            const uint32_t off = ((((v.r0 + row) * nb + v.k0) & 7u) * 6u) & 15u;
+            return read_record(raw, row * kGemmRowBytes + off + 6u * b);
+          });
+    };
+    SliceWalk w0, w1, w2, w3;  // slices g, g + 1, g + 2, g + 3
+    open_unit(w0, blockIdx.x);
+    w1 = w0;
+    advance(w1);
+    w2 = w1;
+    if (w2.unit < n_units) advance(w2);
+    w3 = w2;
+    if (w3.unit < n_units) advance(w3);
     uint4 pre = make_uint4(0, 0, 0, 0);
-    prefetch(w, pre);
+    prefetch(w0, pre);
     stage_raw(0, pre);
-    ahead = w;
-    advance(ahead);
-    prefetch(ahead, pre);  // slice 1, stored during stage 0
-    wg_barrier();          // slice 0's code bytes and the table image are in LDS
-    uint32_t buf = 0;
+    prefetch(w1, pre);
+    wg_barrier();  // slice 0's code bytes and the table image are in LDS
+    if (w1.unit < n_units) stage_raw(1, pre);
+    prefetch(w2, pre);
+    classify(view(w0, 0));
+    wg_barrier();
+    uint32_t g = 0;
 #ifdef LLVQ_PHASE_TIMING
     uint32_t stage_no = 0;
 #endif
-    while (w.unit < n_units) {
+    while (w0.unit < n_units) {
 #ifdef LLVQ_PHASE_TIMING
       ++stage_no;
 #endif
       LLVQ_GSTAMP(0, 0);
-      const uint32_t k0 = w.kb_lo + w.sj * kGemmKb;
-      const uint32_t kb = min((uint32_t)kGemmKb, w.kb_hi - k0);
-      const uint32_t r0 = w.r0, nblk = w.rows * kb;
-      const uint32_t inv_kb = (65536u + kb - 1u) / kb;  // floor(f / kb) = (f * inv_kb) >> 16 for f < 2048, kb <= 32
-      const uint8_t* raw = raw0 + buf * kRawBuf;
-      uint32_t* ctrl = ctrl0 + buf * 4;
-      auto record_at = [&](uint32_t row, uint32_t b) -> uint64_t {
-        const uint32_t off = ((((r0 + row) * nb + k0) & 7u) * 6u) & 15u;  // (6 n) mod 16 depends on n mod 8 only
-        return read_record(raw, row * kGemmRowBytes + off + 6u * b);
-      };
-      // P1.  An origin block is queued like any other: its 24 zero weights must be written.
-      classify_and_bin<kP1Blocks, kProducers>(
-          T, nblk, kGemmTile, queue, gqueue, ctrl,
-          [&](uint32_t f) {
-            const uint32_t row = (f * inv_kb) >> 16;
-            return record_at(row, f - row * kb);
-          },
-          [](uint32_t) { return true; });
+      if (w2.unit < n_units) stage_raw((g + 2u) % 3u, pre);
+      prefetch(w3, pre);
+      unrank(view(w0, g));
       LLVQ_GSTAMP(0, 1);
-      wg_barrier();
+      if (w1.unit < n_units) classify(view(w1, g + 1u));
       LLVQ_GSTAMP(0, 2);
-      // the next slice's code bytes and counters: that buffer was last read in the stage before
-      if (ahead.unit < n_units) stage_raw(buf ^ 1u, pre);
-      w = ahead;
-      advance(ahead);
-      prefetch(ahead, pre);
-      // P2
-      unrank_queues_to_slice<kGemmTile, kGemmWStride>(T, queue, gqueue, ctrl, kb, inv_kb, a.g0, a.g1, W0 + buf * kWBuf, record_at);
-      LLVQ_GSTAMP(0, 3);
       wg_barrier();
-      LLVQ_GSTAMP(0, 4);
-      buf ^= 1u;
+      LLVQ_GSTAMP(0, 3);
+      ++g;
+      w0 = w1;
+      w1 = w2;
+      w2 = w3;
+      if (w3.unit < n_units) advance(w3);
     }
-    // the consumers' last stage
-    wg_barrier();
-    wg_barrier();
+    wg_barrier();  // the consumers' last stage
   } else {
     // ---------------- consumers ----------------
     // Consumer c owns activation rows [64 ctile, +64) on the K-steps p = kpart (mod kparts) of
@@ -364,9 +391,8 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     fetch(xs, ring[0]);
 
     consumer_barrier();  // the table image (unused here) and slice 0's code bytes
-    // stage 0: nothing to multiply yet
-    consumer_barrier();
-    consumer_barrier();
+    consumer_barrier();  // slice 0 classified
+    consumer_barrier();  // stage 0: slice 0 unranked, nothing to multiply yet
 
     uint32_t buf = 0;
     float16_t acc[2][2];
@@ -406,15 +432,8 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         }
       };
       auto step_src = [&](uint32_t i) { return i < n_own ? xs + i * own_bytes : xs_next + (i - n_own) * own_bytes; };
-      // a quarter of the K-steps beside the producers' classification, the rest beside their unranking
-      const uint32_t i_a = n_own >= 12 ? 2u : 0u;
       uint32_t i = 0;
       for (; i + 1 < n_own; i += 2) {
-        if (i == i_a) {
-          LLVQ_GSTAMP(256, 1);
-          consumer_barrier();
-          LLVQ_GSTAMP(256, 2);
-        }
         fetch(step_src(i + 1), ring[1]);
         multiply(i, ring[0]);
         fetch(step_src(i + 2), ring[0]);

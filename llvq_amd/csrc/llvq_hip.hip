@@ -38,10 +38,10 @@ namespace llvq {
 struct TableImage {
   FastClass fast[kClassSlots];
   uint64_t starts[kStartsLds];
-  uint16_t lut[2048];        // a 47-bit field only reaches the lower half of the host table
   double rcp[32];
   double step[24 * 25 * 2];
   uint8_t pdep4[256];
+  uint16_t lut[2048];        // a 47-bit field only reaches the lower half of the host table
   uint32_t golay[4096];
   uint32_t on_lut[kOnLutSlots];
 };
@@ -58,18 +58,23 @@ struct GlobalTables {
 
 constexpr size_t kLdsImageBytesLean = offsetof(TableImage, golay);  // without the Golay words and the support-arrangement table
 static_assert(kLdsImageBytesLean % 16 == 0, "LDS part of the table image is copied in 16-byte units");
+constexpr size_t kLdsImageBytesLeanest = offsetof(TableImage, lut);  // without the class lookup table either
+static_assert(kLdsImageBytesLeanest % 16 == 0, "LDS part of the table image is copied in 16-byte units");
 
 // kFull: the whole image goes to LDS; otherwise its last two tables (33 KB) are
-// read through L2, for a kernel that needs the LDS for something else.
-template <bool kFull = (LLVQ_LDS_GOLAY != 0)>
+// read through L2, for a kernel that needs the LDS for something else.  kLut = false
+// leaves the 4 KB class lookup table (one read per block) in L2 as well.
+template <bool kFull = (LLVQ_LDS_GOLAY != 0), bool kLut = true>
 __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const GlobalTables& g) {
+  static_assert(kLut || !kFull, "the tables that stay in L2 are the image's last ones");
   const uint4* src = reinterpret_cast<const uint4*>(g.image);
   uint4* dst = reinterpret_cast<uint4*>(smem);
-  constexpr size_t kBytes = kFull ? sizeof(TableImage) : kLdsImageBytesLean;
+  constexpr size_t kBytes = kFull ? sizeof(TableImage) : (kLut ? kLdsImageBytesLean : kLdsImageBytesLeanest);
   for (uint32_t i = threadIdx.x; i < kBytes / 16; i += blockDim.x) dst[i] = src[i];
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
   const TableImage* far = kFull ? s : g.image;
-  return DecodeTables{far->golay, g.cls, s->fast, s->starts, s->lut, s->rcp, far->on_lut, g.off_lut, g.expand, s->pdep4, s->step};
+  return DecodeTables{far->golay, g.cls, s->fast, s->starts, kLut ? s->lut : g.image->lut, s->rcp, far->on_lut, g.off_lut,
+                      g.expand, s->pdep4, s->step};
 }
 
 // 6-byte big-endian record at a 2-byte-aligned offset of a 4-byte-aligned buffer
