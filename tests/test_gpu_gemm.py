@@ -31,28 +31,37 @@ def _reference(orc, raw, X):
     return X @ W.T, np.abs(X) @ np.abs(W).T
 
 
-def _check(Y, Y_ref, A_ref, tol=TOL):
+def _check(Y, Y_ref, A_ref, tol=TOL, out_rounding=0.0):
+    """out_rounding: half an ulp of the output type (2^-11 for binary16 outputs), which the result
+    carries on top of the 1e-3 the computation is allowed."""
     Y = Y.astype(np.float64)
     e = np.abs(Y - Y_ref) / np.maximum(A_ref, 1e-30)
     assert e.max() < tol, f"max |dy|/sum|wx| = {e.max():.3e}"
     big = np.abs(Y_ref) >= 0.2 * A_ref
     if big.any():
         rel = (np.abs(Y - Y_ref)[big] / np.abs(Y_ref)[big]).max()
-        assert rel < tol, f"max relative error {rel:.3e}"
+        assert rel < tol + out_rounding, f"max relative error {rel:.3e}"
     return e.max()
 
 
 # d_in must keep activation rows 16-byte aligned (d_in % 8 == 0) for the matrix-core path
 CASES = [
-    # d_out, d_in, M
-    (64, 480, 16),      # one band, one full K-slice, no tail
+    # d_out, d_in, M.  A K-slice is 16 blocks per row; up to 256 activation rows four wavefronts
+    # multiply (64-row tiles, the wavefronts left over share a tile's K-steps), beyond that eight.
+    (64, 480, 16),      # one band, one full and one short K-slice, no tail
     (72, 184, 16),      # ragged band (72 = 64 + 8), 7 blocks + 16 tail columns
     (8, 2560, 2),       # tiny band, smallest batch
     (128, 2568, 17),    # ragged batch, tail
     (256, 4096, 64),    # 8B hidden size: 170 blocks + 16 tail
-    (192, 976, 130),    # two column tiles per wavefront
-    (64, 1000, 256),
-    (128, 4096, 512),   # four column tiles per wavefront
+    (64, 384, 65),      # exactly one slice; two 64-row tiles, the second with one row
+    (192, 976, 130),    # three tiles on four multiplying wavefronts: one of them idles
+    (64, 416, 129),     # 17 blocks: a full slice and a slice of one block
+    (64, 1000, 256),    # the widest batch of the four-wavefront variant
+    (64, 376, 257),     # the narrowest of the eight-wavefront variant: 15 blocks, five tiles
+    (320, 800, 300),    # 33 blocks = two full slices and one block; five tiles, three wavefronts idle
+    (19000, 80, 257),   # 297 bands on 256 CUs: workgroups walk several units, short slices throughout
+    (128, 4096, 512),   # eight tiles
+    (64, 376, 511),
     (64, 488, 600),     # more rows than one launch holds
 ]
 
@@ -72,8 +81,8 @@ def test_gemm_shapes(gpu_rt, orc, d_out, d_in, M):
     finally:
         gpu_rt.free(proj)
     e = _check(Y32, Y_ref, A_ref)
-    assert e < 2e-4  # observed level of the binary16 weight rounding
-    _check(Y16.astype(np.float32), Y_ref, A_ref)
+    assert e < 3e-4  # the binary16 weight rounding: 2^-11 = 4.9e-4 bounds a single term, sums of many stay near 1e-4
+    _check(Y16.astype(np.float32), Y_ref, A_ref, out_rounding=2.0 ** -11)
     assert np.array_equal(Y32, again)  # fixed summation order, split or not
 
 
