@@ -170,6 +170,13 @@ int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
 int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, int M, void* y_dev,
                   int y_dtype);
 
+/* The same for the projections of one group (model.rs:497-536: q/k/v, gate/up share their
+ * activation rows): y_dev[i] = X W_i^T, [M, d_out_i] each.  Consecutive matrices that share a
+ * basis go through one launch (up to four at a time), so the activations are prepared once
+ * and small matrices fill the chip together with their neighbours. */
+int llvq_hip_gemm_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x_f16_dev, int M,
+                        void* const* y_dev, int y_dtype);
+
 /* Parity probe (the role of decode_probe, llvq-cuda/kernels/preflight.cu:39):
  * unrank packed 6-byte records on the device.  points: 24 int8 per block;
  * gains: one byte per block; shells (may be NULL): one byte per block. */

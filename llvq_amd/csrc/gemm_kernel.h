@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void tile_activations_kernel(const __half* x, 
 // step through the same sequence, the consumers one stage behind.
 struct SliceWalk {
   uint32_t unit, si, n_slices, sj;  // sj: the slice walked at step si (units start at a band-dependent offset)
-  uint32_t band, split, r0, rows, kb_lo, kb_hi;
+  uint32_t band, split, mat, r0, rows, kb_lo, kb_hi;  // r0: the band's first row in matrix `mat`
 };
 
 #ifdef LLVQ_PHASE_TIMING
@@ -203,14 +203,22 @@ struct SliceWalk {
 #define LLVQ_GSTAMP(base, k) do {} while (0)
 #endif
 
+// A launch covers up to four matrices that share their activations (q/k/v, gate/up): their
+// bands are numbered through, matrix i owning bands [band_begin, next band_begin).
+constexpr int kGemmMaxGroup = 4;
+struct GemmMat {
+  const uint8_t* codes;
+  float g0, g1;
+  uint32_t d_out, band_begin;
+};
 struct GemmArgs {
   GlobalTables tables;
   const __half* xt;       // [n_steps, m_pad, 32]: tile_activations_kernel's output
-  const uint8_t* codes;
   float* ws;              // [S * kparts, n_bands, M, 64] partial sums
-  float g0, g1;
-  uint32_t M, m_pad, d_out, nblocks;
-  uint32_t n_bands, S, bps;  // split count, blocks per split (a multiple of the slice)
+  GemmMat mat[kGemmMaxGroup];
+  uint32_t n_mats;
+  uint32_t M, m_pad, nblocks;
+  uint32_t n_bands, S, bps;  // bands of all matrices, split count, blocks per split (a multiple of the slice)
   uint32_t ct_shift;         // log2 of the 64-row activation tiles the consumers spread over
 };
 
@@ -240,8 +248,12 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     if (unit >= n_units) return;
     w.band = unit / a.S;
     w.split = unit - w.band * a.S;
-    w.r0 = w.band * kGemmRows;
-    w.rows = min((uint32_t)kGemmRows, a.d_out - w.r0);
+    w.mat = 0;
+#pragma unroll
+    for (uint32_t k = 1; k < (uint32_t)kGemmMaxGroup; ++k)
+      if (k < a.n_mats && w.band >= a.mat[k].band_begin) w.mat = k;
+    w.r0 = (w.band - a.mat[w.mat].band_begin) * kGemmRows;
+    w.rows = min((uint32_t)kGemmRows, a.mat[w.mat].d_out - w.r0);
     w.kb_lo = min(nb, w.split * a.bps);
     w.kb_hi = min(nb, w.kb_lo + a.bps);
     w.n_slices = (w.kb_hi - w.kb_lo + kGemmKb - 1) / kGemmKb;  // >= 1: the host leaves no split empty
@@ -271,7 +283,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         const size_t byte0 = ((size_t)(w.r0 + row) * nb + k0) * 6;
         const uint32_t off = (uint32_t)(byte0 & 15);
         const uint32_t n16 = (off + kb * 6 + 15) >> 4;
-        if (j < n16) pre = reinterpret_cast<const uint4*>(a.codes + (byte0 - off))[j];
+        if (j < n16) pre = reinterpret_cast<const uint4*>(a.mat[w.mat].codes + (byte0 - off))[j];
       }
     };
     auto stage_raw = [&](uint32_t set, const uint4& pre) {
@@ -280,6 +292,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     };
     struct SliceView {  // what the phases of one slice need
       uint32_t k0, kb, r0, nblk, inv_kb, set3, set2;
+      float g0, g1;
     };
     auto view = [&](const SliceWalk& w, uint32_t s) {
       SliceView v;
@@ -290,6 +303,8 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       v.inv_kb = (65536u + v.kb - 1u) / v.kb;  // floor(f / kb) = (f * inv_kb) >> 16 for f < 2048, kb <= 32
       v.set3 = s % 3u;
       v.set2 = s & 1u;
+      v.g0 = a.mat[w.mat].g0;
+      v.g1 = a.mat[w.mat].g1;
       return v;
     };
     auto classify = [&](const SliceView& v) {  // P1.  An origin block is queued like any other: its 24 zero weights must be written.
@@ -306,7 +321,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     auto unrank = [&](const SliceView& v) {  // P2
       const uint8_t* raw = raw0 + v.set3 * kRawBuf;
       unrank_queues_to_slice<kGemmTile, kGemmWStride>(
-          T, queue0 + v.set2 * kGemmTile, gqueue0 + v.set2 * kGenericSlots, ctrl0 + v.set3 * 4, v.kb, v.inv_kb, a.g0, a.g1,
+          T, queue0 + v.set2 * kGemmTile, gqueue0 + v.set2 * kGenericSlots, ctrl0 + v.set3 * 4, v.kb, v.inv_kb, v.g0, v.g1,
           W0 + v.set2 * kWBuf, [&](uint32_t row, uint32_t b) -> uint64_t {
             const uint32_t off = ((((v.r0 + row) * nb + v.k0) & 7u) * 6u) & 15u;
             return read_record(raw, row * kGemmRowBytes + off + 6u * b);
@@ -486,13 +501,18 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 // activation rows), one lane per four consecutive weight rows of one activation row;
 // the band's tail weights and the activation tails are staged in LDS once, and the
 // partial sums are read with all their loads in flight (eight splits at a time).
-struct GemmReduceArgs {
-  const float* ws;  // [S, n_bands, M, 64]
-  const __half* x;  // [M, ldx]
+struct GemmReduceMat {
   const float* rscale;
   const float* tail;
   void* y;
-  uint32_t M, ldx, d_out, nblocks, tail_w, S, n_bands;
+  uint32_t d_out, band_begin;
+};
+struct GemmReduceArgs {
+  const float* ws;  // [S, n_bands, M, 64]
+  const __half* x;  // [M, ldx]
+  GemmReduceMat mat[kGemmMaxGroup];
+  uint32_t n_mats;
+  uint32_t M, ldx, nblocks, tail_w, S, n_bands;
 };
 
 constexpr int kReduceRowsM = 16;  // activation rows per workgroup
@@ -503,13 +523,18 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
   __shared__ float xt[kReduceRowsM * (kDim - 1)];   // [m][tail_w]
   const uint32_t mchunks = (a.M + kReduceRowsM - 1) / kReduceRowsM;
   const uint32_t band = blockIdx.x / mchunks, mc = blockIdx.x - band * mchunks;
-  const uint32_t r0 = band * kGemmRows, rows = min((uint32_t)kGemmRows, a.d_out - r0);
+  uint32_t mi = 0;
+#pragma unroll
+  for (uint32_t k = 1; k < (uint32_t)kGemmMaxGroup; ++k)
+    if (k < a.n_mats && band >= a.mat[k].band_begin) mi = k;
+  const GemmReduceMat mt = a.mat[mi];
+  const uint32_t r0 = (band - mt.band_begin) * kGemmRows, rows = min((uint32_t)kGemmRows, mt.d_out - r0);
   const uint32_t tw = a.tail_w, pitch = tw | 1u;
   const uint32_t tid = threadIdx.x, quad = tid & 15u, ml = tid >> 4;
   const uint32_t m = mc * kReduceRowsM + ml, row = quad * 4u;
   for (uint32_t o = tid; o < rows * tw; o += 256) {
     const uint32_t r = o / tw, t = o - r * tw;
-    tl[r * pitch + t] = a.tail[(size_t)r0 * tw + o];
+    tl[r * pitch + t] = mt.tail[(size_t)r0 * tw + o];
   }
   for (uint32_t o = tid; o < kReduceRowsM * tw; o += 256) {
     const uint32_t mm = mc * kReduceRowsM + o / tw, t = o % tw;
@@ -540,23 +565,23 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
     const uint32_t r = min(row + i, rows - 1u);
     float ts = 0.f;
     for (uint32_t t = 0; t < tw; ++t) ts = fmaf(tl[r * pitch + t], xt[ml * tw + t], ts);
-    v[i] = fmaf(sum[i], a.rscale[r0 + r], ts);
+    v[i] = fmaf(sum[i], mt.rscale[r0 + r], ts);
   }
-  const size_t at = (size_t)m * a.d_out + r0 + row;
-  if ((a.d_out & 3u) == 0 && row + 3 < rows) {
+  const size_t at = (size_t)m * mt.d_out + r0 + row;
+  if ((mt.d_out & 3u) == 0 && row + 3 < rows) {
     if constexpr (sizeof(OutT) == 4) {
-      *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
+      *reinterpret_cast<float4*>(reinterpret_cast<float*>(mt.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
     } else {
       const __half2 lo = __float22half2_rn(make_float2(v[0], v[1])), hi = __float22half2_rn(make_float2(v[2], v[3]));
       uint2 pk;
       pk.x = *reinterpret_cast<const uint32_t*>(&lo);
       pk.y = *reinterpret_cast<const uint32_t*>(&hi);
-      *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(a.y) + at) = pk;
+      *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(mt.y) + at) = pk;
     }
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (row + i < rows) store_y<OutT>(a.y, at + i, v[i]);
+      if (row + i < rows) store_y<OutT>(mt.y, at + i, v[i]);
   }
 }
 

@@ -893,7 +893,7 @@ struct llvq_rt {
   float* rot_scratch = nullptr;   // one rotated activation, f32
   size_t rot_scratch_elems = 0;
   __half* rot_rows = nullptr;     // rotated batch rows, f16 (matrix-core path)
-  size_t rot_rows_elems = 0;
+  size_t rot_rows_bytes = 0;
   // workspace of the batched kernels: partial sums [S, n_bands, M, 64]
   float* gemm_ws = nullptr;
   size_t gemm_ws_bytes = 0;
@@ -1515,37 +1515,43 @@ static int grow_buffer(void** buf, size_t* have, size_t need) {
 // twelve of the sixteen wavefronts unrank and four multiply (four consumers cover 256 rows).
 constexpr uint32_t kGemmNarrowRows = 256;
 
-static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M, void* y, int y_dtype) {
+// One launch over n <= kGemmMaxGroup matrices of equal d_in that take the same activations
+// (already in the matrices' basis), M <= kGemmMaxM rows.
+static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, uint32_t M, void* const* y,
+                       int y_dtype) {
   const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
   const bool f32 = y_dtype == LLVQ_F32;
+  const llvq_mat* m0 = mats[0];
+  const __half* xh = reinterpret_cast<const __half*>(x);
   GemmArgs a{};
+  GemmReduceArgs r{};
   a.tables = rt->tables;
-  a.codes = m->codes;
-  a.g0 = m->g[0];
-  a.g1 = m->g[1];
+  a.n_mats = r.n_mats = (uint32_t)n;
+  for (int i = 0; i < n; ++i) {
+    a.mat[i] = GemmMat{mats[i]->codes, mats[i]->g[0], mats[i]->g[1], mats[i]->d_out, a.n_bands};
+    r.mat[i] = GemmReduceMat{mats[i]->rscale, mats[i]->tail, y[i], mats[i]->d_out, a.n_bands};
+    a.n_bands += (mats[i]->d_out + kGemmRows - 1) / kGemmRows;
+  }
   a.M = M;
   a.m_pad = (M + kGemmColTile - 1) / kGemmColTile * kGemmColTile;
-  a.d_out = m->d_out;
-  a.nblocks = m->nblocks;
-  a.n_bands = (m->d_out + kGemmRows - 1) / kGemmRows;
+  a.nblocks = m0->nblocks;
   // the consumer wavefronts over the batch's 64-row tiles, the count rounded up to a power of two
   const uint32_t consumers = M <= kGemmNarrowRows ? 4u : 8u;
   a.ct_shift = 0;
   while (((uint32_t)kGemmColTile << a.ct_shift) < M) ++a.ct_shift;
   const uint32_t kparts = consumers >> a.ct_shift;
-  pick_gemm_split(a.n_bands, m->nblocks, M, kparts, grid_cap, &a.S, &a.bps);
+  pick_gemm_split(a.n_bands, m0->nblocks, M, kparts, grid_cap, &a.S, &a.bps);
   const uint32_t n_partials = a.S * kparts;
   int rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes,
                        (size_t)n_partials * a.n_bands * M * kGemmRows * sizeof(float));
   if (rc) return rc;
   // every slice has all its twelve K-steps in the tiled copy, zeros past the matrix's last block
-  const uint32_t n_steps = (m->nblocks + kGemmKb - 1) / kGemmKb * (kGemmKb * 24 / 32);
+  const uint32_t n_steps = (m0->nblocks + kGemmKb - 1) / kGemmKb * (kGemmKb * 24 / 32);
   const size_t xt_bytes = (size_t)n_steps * a.m_pad * 64;
   rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_xt), &rt->gemm_xt_bytes, xt_bytes);
   if (rc) return rc;
-  const __half* xh = reinterpret_cast<const __half*>(x);
   hipLaunchKernelGGL(tile_activations_kernel, dim3((uint32_t)((xt_bytes / 16 + 255) / 256)), dim3(256), 0, rt->stream, xh, M,
-                     m->d_in, m->nblocks * 24u, a.m_pad, n_steps, reinterpret_cast<uint4*>(rt->gemm_xt));
+                     m0->d_in, m0->nblocks * 24u, a.m_pad, n_steps, reinterpret_cast<uint4*>(rt->gemm_xt));
   HIP_TRY(hipGetLastError());
   a.xt = rt->gemm_xt;
   a.ws = rt->gemm_ws;
@@ -1554,17 +1560,12 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
   if (consumers == 4) hipLaunchKernelGGL(gemm_tiles_kernel<12>, grid, wg, gemm_lds_bytes(), rt->stream, a);
   else hipLaunchKernelGGL(gemm_tiles_kernel<8>, grid, wg, gemm_lds_bytes(), rt->stream, a);
   HIP_TRY(hipGetLastError());
-  GemmReduceArgs r{};
   r.ws = a.ws;
   r.x = xh;
-  r.rscale = m->rscale;
-  r.tail = m->tail;
-  r.y = y;
   r.M = M;
-  r.ldx = m->d_in;
-  r.d_out = m->d_out;
-  r.nblocks = m->nblocks;
-  r.tail_w = m->tail_w;
+  r.ldx = m0->d_in;
+  r.nblocks = m0->nblocks;
+  r.tail_w = m0->tail_w;
   r.S = n_partials;
   r.n_bands = a.n_bands;
   const uint32_t rgrid = a.n_bands * ((M + kReduceRowsM - 1) / kReduceRowsM);
@@ -1574,51 +1575,71 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, uint32_t M
   return LLVQ_OK;
 }
 
+// Matrices [0, n) of one group: same d_in, same basis.  The matrix-core kernel reads activations as
+// 16-byte vectors; a single row, or a shape that breaks that alignment, runs as GEMV launches instead.
+static int gemm_same_basis(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, int M, void* const* y, int y_dtype) {
+  const llvq_mat* m0 = mats[0];
+  const size_t esz = y_dtype == LLVQ_F32 ? 4 : 2;
+  const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
+  const bool mfma_ok = M >= 2 && m0->d_in % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && m0->nblocks > 0;
+  if (!mfma_ok) {
+    for (int i = 0; i < n; ++i)
+      for (int r = 0; r < M; ++r) {
+        const int rc = launch_gemv(rt, mats[i], xb + (size_t)r * m0->d_in * 2, reinterpret_cast<uint8_t*>(y[i]) + (size_t)r * mats[i]->d_out * esz, y_dtype);
+        if (rc) return rc;
+      }
+    return LLVQ_OK;
+  }
+  if (m0->has_rotation) {
+    // rows are rotated (f32 inside) and narrowed to the binary16 the matrix cores take
+    const int rc0 = grow_buffer(reinterpret_cast<void**>(&rt->rot_rows), &rt->rot_rows_bytes, (size_t)M * m0->d_in * sizeof(__half));
+    if (rc0) return rc0;
+    const int rc = launch_rotate(rt, m0->rot, x, (uint32_t)M, rt->rot_rows, true);
+    if (rc) return rc;
+    xb = reinterpret_cast<const uint8_t*>(rt->rot_rows);
+  }
+  for (int m_lo = 0; m_lo < M; m_lo += kGemmMaxM) {
+    const uint32_t mc = (uint32_t)(M - m_lo < kGemmMaxM ? M - m_lo : kGemmMaxM);
+    for (int i0 = 0; i0 < n; i0 += kGemmMaxGroup) {
+      const int cnt = n - i0 < kGemmMaxGroup ? n - i0 : kGemmMaxGroup;
+      void* ys[kGemmMaxGroup];
+      for (int i = 0; i < cnt; ++i) ys[i] = reinterpret_cast<uint8_t*>(y[i0 + i]) + (size_t)m_lo * mats[i0 + i]->d_out * esz;
+      const int rc = launch_gemm(rt, mats + i0, cnt, xb + (size_t)m_lo * m0->d_in * 2, mc, ys, y_dtype);
+      if (rc) return rc;
+    }
+  }
+  return LLVQ_OK;
+}
+
+int llvq_hip_gemm_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, int M, void* const* y, int y_dtype) {
+  if (!rt || !mats || !y || n < 0 || M < 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_group: bad argument");
+  if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_group: unknown output dtype");
+  for (int i = 0; i < n; ++i) {
+    if (!mats[i]) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_group: null matrix");
+    if (mats[i]->d_in != mats[0]->d_in)
+      return fail(LLVQ_ERR_INVALID_ARGUMENT, mats[i]->name + ": projections of one group must share d_in");
+  }
+  if (M == 0 || n == 0) return LLVQ_OK;  // no rows: nothing is read or written, so the pointers may be null
+  if (!x) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_group: null activation");
+  for (int i = 0; i < n; ++i)
+    if (!y[i]) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_group: null output");
+  HIP_TRY(hipSetDevice(rt->device));
+  // consecutive matrices that share a basis go into one launch; the activation is rotated once per basis
+  for (int i0 = 0; i0 < n;) {
+    int i1 = i0 + 1;
+    while (i1 < n && mats[i1]->has_rotation == mats[i0]->has_rotation && (!mats[i0]->has_rotation || mats[i1]->rot == mats[i0]->rot)) ++i1;
+    const int rc = gemm_same_basis(rt, mats + i0, i1 - i0, x, M, y + i0, y_dtype);
+    if (rc) return rc;
+    i0 = i1;
+  }
+  return LLVQ_OK;
+}
+
 int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y, int y_dtype) {
   if (!rt || !m || M < 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: bad argument");
   if (M == 0) return LLVQ_OK;  // no rows: nothing is read or written, so the pointers may be null
   if (!x || !y) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: null activation or output");
-  if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: unknown output dtype");
-  HIP_TRY(hipSetDevice(rt->device));
-  const size_t esz = y_dtype == LLVQ_F32 ? 4 : 2;
-  const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
-  uint8_t* yb = reinterpret_cast<uint8_t*>(y);
-  // The matrix-core kernel reads activations as 16-byte vectors; a single row,
-  // or a shape that breaks that alignment, runs as GEMV launches instead.
-  if (m->has_rotation && M >= 2 && m->d_in % 8 == 0 && m->nblocks > 0) {
-    // rows are rotated (f32 inside) and narrowed to the binary16 the matrix cores take
-    const size_t need = (size_t)M * m->d_in;
-    if (need > rt->rot_rows_elems) {
-      (void)hipFree(rt->rot_rows);
-      rt->rot_rows = nullptr;
-      rt->rot_rows_elems = 0;
-      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&rt->rot_rows), need * sizeof(__half)));
-      rt->rot_rows_elems = need;
-    }
-    const int rc = launch_rotate(rt, m->rot, x, (uint32_t)M, rt->rot_rows, true);
-    if (rc) return rc;
-    xb = reinterpret_cast<const uint8_t*>(rt->rot_rows);
-    for (int m0 = 0; m0 < M; m0 += kGemmMaxM) {
-      const uint32_t mc = (uint32_t)(M - m0 < kGemmMaxM ? M - m0 : kGemmMaxM);
-      const int rc2 = launch_gemm(rt, m, xb + (size_t)m0 * m->d_in * 2, mc, yb + (size_t)m0 * m->d_out * esz, y_dtype);
-      if (rc2) return rc2;
-    }
-    return LLVQ_OK;
-  }
-  const bool mfma_ok = M >= 2 && m->d_in % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && m->nblocks > 0;
-  if (!mfma_ok) {
-    for (int r = 0; r < M; ++r) {
-      const int rc = launch_gemv(rt, m, xb + (size_t)r * m->d_in * 2, yb + (size_t)r * m->d_out * esz, y_dtype);
-      if (rc) return rc;
-    }
-    return LLVQ_OK;
-  }
-  for (int m0 = 0; m0 < M; m0 += kGemmMaxM) {
-    const uint32_t mc = (uint32_t)(M - m0 < kGemmMaxM ? M - m0 : kGemmMaxM);
-    const int rc = launch_gemm(rt, m, xb + (size_t)m0 * m->d_in * 2, mc, yb + (size_t)m0 * m->d_out * esz, y_dtype);
-    if (rc) return rc;
-  }
-  return LLVQ_OK;
+  return llvq_hip_gemm_group(rt, &m, 1, x, M, &y, y_dtype);
 }
 
 int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks, int8_t* points_dev,
@@ -1835,9 +1856,8 @@ int decoder_prefill_pass(llvq_decoder* d, uint32_t n, bool want_logits, uint32_t
     hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(kNormThreads), 0, st, d->ph, L ? d->pdown : (const __half*)nullptr,
                        d->ln1 + (size_t)L * d->hidden, L ? d->ph_alt : (__half*)nullptr, d->pnormed, d->hidden, d->eps);
     if (L) std::swap(d->ph, d->ph_alt);
-    int rc = rows(P[0], d->pnormed, d->pq);
-    if (!rc) rc = rows(P[1], d->pnormed, d->pk);
-    if (!rc) rc = rows(P[2], d->pnormed, d->pv);
+    void* const qkv[3] = {d->pq, d->pk, d->pv};
+    int rc = llvq_hip_gemm_group(rt, P, 3, d->pnormed, (int)n, qkv, LLVQ_F16);
     if (rc) return rc;
     KvQ8 lq8 = d->q8;
     if (d->kv_q8) {
@@ -1879,8 +1899,8 @@ int decoder_prefill_pass(llvq_decoder* d, uint32_t n, bool want_logits, uint32_t
     hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(kNormThreads), 0, st, d->ph, d->po, d->ln2 + (size_t)L * d->hidden, d->ph_alt,
                        d->pnormed, d->hidden, d->eps);
     std::swap(d->ph, d->ph_alt);
-    rc = rows(P[4], d->pnormed, d->pgate);
-    if (!rc) rc = rows(P[5], d->pnormed, d->pup);
+    void* const gate_up[2] = {d->pgate, d->pup};
+    rc = llvq_hip_gemm_group(rt, P + 4, 2, d->pnormed, (int)n, gate_up, LLVQ_F16);
     if (rc) return rc;
     const uint32_t na = n * d->inter;
     hipLaunchKernelGGL(silu_mul_kernel, dim3((na + 255) / 256 < 4096u ? (na + 255) / 256 : 4096u), dim3(256), 0, st, d->pgate, d->pup, d->pact, na);

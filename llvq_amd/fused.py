@@ -261,6 +261,26 @@ class FusedRuntime:
         _ffi.check(_ffi.lib().llvq_hip_gemm(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
         return y
 
+    def forward_batched_group_into(self, projs, x, ys):
+        """Rows of `x` [M, d_in] through the projections of one group (q/k/v, gate/up) into caller-owned
+        [M, d_out_i] tensors of one dtype: one batched launch per run of projections that share a basis
+        (the row loop of group_forward, model.rs:497-536)."""
+        torch = self._torch
+        if len(projs) != len(ys) or not projs:
+            raise ValueError("one output per projection")
+        if x.dtype != torch.float16 or not x.is_contiguous() or x.dim() != 2:
+            raise ValueError("the activation must be a contiguous f16 [M, d_in] tensor")
+        for p, y in zip(projs, ys):
+            if p.d_in != x.shape[1]:
+                raise ValueError(f"{p.name} expects d_in {p.d_in}, got {x.shape[1]}")
+            if tuple(y.shape) != (x.shape[0], p.d_out) or not y.is_contiguous() or y.dtype != ys[0].dtype:
+                raise ValueError(f"{p.name}: output must be contiguous [M, {p.d_out}], one dtype for the group")
+        mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
+        outs = (C.c_void_p * len(projs))(*[y.data_ptr() for y in ys])
+        code = _ffi.F16 if ys[0].dtype == torch.float16 else _ffi.F32
+        _ffi.check(_ffi.lib().llvq_hip_gemm_group(self.handle, mats, len(projs), x.data_ptr(), x.shape[0], outs, code))
+        return ys
+
     def decode_blocks(self, codes):
         """Parity probe: packed 6-byte records (uint8 tensor on the device) →
         (points int8 [n,24], gains uint8 [n], shells uint8 [n])."""

@@ -171,3 +171,35 @@ def test_gemm_qwen3_8b_shapes(gpu_rt, orc, site, d_out, d_in, M):
     Y_ref, A_ref = _reference(orc, raw, X[pick])
     _check(Y[pick], Y_ref, A_ref)
     assert np.isfinite(Y).all()
+
+
+def test_gemm_group_matches_the_oracle_and_the_single_calls(gpu_rt, orc):
+    """Five projections that share their activation rows (more than one launch holds), as one call:
+    every output against the oracle, and against the same projection called on its own (the two may
+    split the block range differently, so they agree to rounding, not bit for bit)."""
+    import torch
+
+    d_in, M = 488, 70
+    d_outs = [192, 72, 8, 64, 130]
+    raws = [synth.make_matrix(f"model.layers.0.group{i}.weight", d, d_in, seed=40 + i) for i, d in enumerate(d_outs)]
+    X = synth.make_activation(d_in, seed=9, rows=M)
+    projs = [gpu_rt.upload(r) for r in raws]
+    try:
+        xd = _x16(X)
+        for dtype in (torch.float32, torch.float16):
+            ys = [torch.empty((M, d), dtype=dtype, device="cuda") for d in d_outs]
+            gpu_rt.forward_batched_group_into(projs, xd, ys)
+            for raw, p, y in zip(raws, projs, ys):
+                Y_ref, A_ref = _reference(orc, raw, X)
+                _check(y.float().cpu().numpy(), Y_ref, A_ref, out_rounding=0.0 if dtype == torch.float32 else 2.0 ** -11)
+                single = gpu_rt.forward_batched(p, xd, out_dtype=dtype)
+                assert (single.float() - y.float()).abs().max().item() <= 2e-3 * y.float().abs().max().item()
+        with pytest.raises(Exception):
+            other = gpu_rt.upload(synth.make_matrix("model.layers.0.other_width.weight", 8, 496, seed=1))
+            try:
+                gpu_rt.forward_batched_group_into([projs[0], other], xd, [ys[0], torch.empty((M, 8), dtype=ys[0].dtype, device="cuda")])
+            finally:
+                gpu_rt.free(other)
+    finally:
+        for p in projs:
+            gpu_rt.free(p)
