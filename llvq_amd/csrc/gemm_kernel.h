@@ -187,11 +187,16 @@ __global__ __launch_bounds__(256) void tile_activations_kernel(const __half* x, 
   xt[idx] = (m < M && col < kcols) ? *reinterpret_cast<const uint4*>(x + (size_t)m * ldx + col) : make_uint4(0, 0, 0, 0);
 }
 
-// Position of a role in the workgroup's sequence of (unit, slice) pairs.  Both roles
-// step through the same sequence, the consumers one stage behind.
+// The launch's slices are numbered band by band, and the workgroups share that sequence out
+// evenly: workgroup c walks slices [g_lo(c), g_hi(c)), `base` or `base + 1` of them, so that the
+// chip is busy whatever the matrix's shape.  A band whose slices fall to several workgroups gets
+// one partial sum from each ("pieces", numbered in workgroup order).  Both roles step through the
+// same slices, the consumers one stage behind.
 struct SliceWalk {
-  uint32_t unit, si, n_slices, sj;  // sj: the slice walked at step si (units start at a band-dependent offset)
-  uint32_t band, split, mat, r0, rows, kb_lo, kb_hi;  // r0: the band's first row in matrix `mat`
+  uint32_t g;                   // slice number in the launch's sequence (band-major), valid below the workgroup's g_hi
+  uint32_t band, j;             // band, and the slice's place in it: blocks [16 j, 16 j + 16) of every row
+  uint32_t mat, r0, rows;       // the band's matrix, its first row there, its row count
+  uint32_t piece;               // which of the band's partial sums this workgroup's run of slices feeds
 };
 
 #ifdef LLVQ_PHASE_TIMING
@@ -214,13 +219,25 @@ struct GemmMat {
 struct GemmArgs {
   GlobalTables tables;
   const __half* xt;       // [n_steps, m_pad, 32]: tile_activations_kernel's output
-  float* ws;              // [S * kparts, n_bands, M, 64] partial sums
+  float* ws;              // [n_bands, max_pieces, kparts, M, 64] partial sums
   GemmMat mat[kGemmMaxGroup];
   uint32_t n_mats;
   uint32_t M, m_pad, nblocks;
-  uint32_t n_bands, S, bps;  // bands of all matrices, split count, blocks per split (a multiple of the slice)
+  uint32_t n_bands;          // bands of all matrices
+  uint32_t spb;              // slices per band
+  uint32_t base, rem;        // workgroup c walks base + (c < rem) slices
+  uint32_t max_pieces;       // workspace slots per band
   uint32_t ct_shift;         // log2 of the 64-row activation tiles the consumers spread over
 };
+
+// The workgroup that walks slice g, and the first slice of workgroup c.
+__host__ __device__ inline uint32_t gemm_owner(uint32_t g, uint32_t base, uint32_t rem) {
+  const uint32_t head = rem * (base + 1u);
+  return g < head ? g / (base + 1u) : rem + (g - head) / base;
+}
+__host__ __device__ inline uint32_t gemm_first_slice(uint32_t c, uint32_t base, uint32_t rem) {
+  return c * base + (c < rem ? c : rem);
+}
 
 // PW = producer wavefronts (8 or 12); the other 16 - PW consume.
 template <int PW>
@@ -240,29 +257,34 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
   const uint32_t nb = a.nblocks;
-  const uint32_t n_units = a.n_bands * a.S;
+  const uint32_t g_lo = gemm_first_slice(blockIdx.x, a.base, a.rem), g_hi = gemm_first_slice(blockIdx.x + 1u, a.base, a.rem);
 
-  auto open_unit = [&](SliceWalk& w, uint32_t unit) {
-    w.unit = unit;
-    w.si = 0;
-    if (unit >= n_units) return;
-    w.band = unit / a.S;
-    w.split = unit - w.band * a.S;
+  auto enter_band = [&](SliceWalk& w) {
     w.mat = 0;
 #pragma unroll
     for (uint32_t k = 1; k < (uint32_t)kGemmMaxGroup; ++k)
       if (k < a.n_mats && w.band >= a.mat[k].band_begin) w.mat = k;
     w.r0 = (w.band - a.mat[w.mat].band_begin) * kGemmRows;
     w.rows = min((uint32_t)kGemmRows, a.mat[w.mat].d_out - w.r0);
-    w.kb_lo = min(nb, w.split * a.bps);
-    w.kb_hi = min(nb, w.kb_lo + a.bps);
-    w.n_slices = (w.kb_hi - w.kb_lo + kGemmKb - 1) / kGemmKb;  // >= 1: the host leaves no split empty
-    w.sj = (w.band * 5u) % w.n_slices;
+  };
+  auto start_walk = [&](SliceWalk& w) {
+    w.g = g_lo;
+    w.band = g_lo / a.spb;
+    w.j = g_lo - w.band * a.spb;
+    w.piece = blockIdx.x - gemm_owner(w.band * a.spb, a.base, a.rem);
+    enter_band(w);
   };
   auto advance = [&](SliceWalk& w) {
-    w.sj = w.sj + 1 == w.n_slices ? 0u : w.sj + 1;
-    if (++w.si == w.n_slices) open_unit(w, w.unit + gridDim.x);
+    ++w.g;
+    if (++w.j == a.spb) {
+      w.j = 0;
+      ++w.band;
+      w.piece = 0;  // this workgroup is the first to reach the next band
+      if (w.g < g_hi) enter_band(w);
+    }
   };
+  auto live = [&](const SliceWalk& w) { return w.g < g_hi; };
+  auto slice_blocks = [&](const SliceWalk& w) { return min((uint32_t)kGemmKb, nb - w.j * kGemmKb); };
 
   // Both W buffers start as zeros: a slice shorter than 16 blocks per row leaves columns the
   // consumers still multiply (by zero activations), which must therefore be finite.
@@ -276,8 +298,8 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     // classification, whose dependent table reads then overlap the others' arithmetic.
     // Buffers: code bytes and counters of slice s in set s mod 3, queues and W in set s mod 2.
     auto prefetch = [&](const SliceWalk& w, uint4& pre) {
-      if (w.unit >= n_units) return;
-      const uint32_t k0 = w.kb_lo + w.sj * kGemmKb, kb = min((uint32_t)kGemmKb, w.kb_hi - k0);
+      if (!live(w)) return;
+      const uint32_t k0 = w.j * kGemmKb, kb = slice_blocks(w);
       const uint32_t row = tid / kGemmRowChunks, j = tid - row * kGemmRowChunks;
       if (row < w.rows) {
         const size_t byte0 = ((size_t)(w.r0 + row) * nb + k0) * 6;
@@ -296,8 +318,8 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     };
     auto view = [&](const SliceWalk& w, uint32_t s) {
       SliceView v;
-      v.k0 = w.kb_lo + w.sj * kGemmKb;
-      v.kb = min((uint32_t)kGemmKb, w.kb_hi - v.k0);
+      v.k0 = w.j * kGemmKb;
+      v.kb = slice_blocks(w);
       v.r0 = w.r0;
       v.nblk = w.rows * v.kb;
       v.inv_kb = (65536u + v.kb - 1u) / v.kb;  // floor(f / kb) = (f * inv_kb) >> 16 for f < 2048, kb <= 32
@@ -328,19 +350,19 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
           });
     };
     SliceWalk w0, w1, w2, w3;  // slices g, g + 1, g + 2, g + 3
-    open_unit(w0, blockIdx.x);
+    start_walk(w0);
     w1 = w0;
     advance(w1);
     w2 = w1;
-    if (w2.unit < n_units) advance(w2);
+    if (live(w2)) advance(w2);
     w3 = w2;
-    if (w3.unit < n_units) advance(w3);
+    if (live(w3)) advance(w3);
     uint4 pre = make_uint4(0, 0, 0, 0);
     prefetch(w0, pre);
     stage_raw(0, pre);
     prefetch(w1, pre);
     wg_barrier();  // slice 0's code bytes and the table image are in LDS
-    if (w1.unit < n_units) stage_raw(1, pre);
+    if (live(w1)) stage_raw(1, pre);
     prefetch(w2, pre);
     classify(view(w0, 0));
     wg_barrier();
@@ -348,16 +370,16 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 #ifdef LLVQ_PHASE_TIMING
     uint32_t stage_no = 0;
 #endif
-    while (w0.unit < n_units) {
+    while (live(w0)) {
 #ifdef LLVQ_PHASE_TIMING
       ++stage_no;
 #endif
       LLVQ_GSTAMP(0, 0);
-      if (w2.unit < n_units) stage_raw((g + 2u) % 3u, pre);
+      if (live(w2)) stage_raw((g + 2u) % 3u, pre);
       prefetch(w3, pre);
       unrank(view(w0, g));
       LLVQ_GSTAMP(0, 1);
-      if (w1.unit < n_units) classify(view(w1, g + 1u));
+      if (live(w1)) classify(view(w1, g + 1u));
       LLVQ_GSTAMP(0, 2);
       wg_barrier();
       LLVQ_GSTAMP(0, 3);
@@ -365,7 +387,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       w0 = w1;
       w1 = w2;
       w2 = w3;
-      if (w3.unit < n_units) advance(w3);
+      if (live(w3)) advance(w3);
     }
     wg_barrier();  // the consumers' last stage
   } else {
@@ -387,8 +409,8 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     const size_t step_bytes = (size_t)a.m_pad * 64u;
     const size_t own_bytes = (size_t)kparts * step_bytes;  // between two of this consumer's K-steps
     const uint32_t n_own = (uint32_t)(kGemmKb * 24 / 32) / kparts;  // 12, 6 or 3 K-steps
-    auto slice_base = [&](const SliceWalk& w) {  // 24 k0 / 32 K-steps precede the slice; k0 is a multiple of 4
-      return reinterpret_cast<const uint8_t*>(a.xt) + (size_t)((w.kb_lo + w.sj * kGemmKb) * 3u / 4u + kpart) * step_bytes;
+    auto slice_base = [&](const SliceWalk& w) {  // twelve K-steps per slice
+      return reinterpret_cast<const uint8_t*>(a.xt) + (size_t)(w.j * (uint32_t)(kGemmKb * 24 / 32) + kpart) * step_bytes;
     };
     half8_t ring[2][2][2];
     auto fetch = [&](const uint8_t* step, half8_t (&dst)[2][2]) {
@@ -399,7 +421,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     };
 
     SliceWalk w, ahead;
-    open_unit(w, blockIdx.x);
+    start_walk(w);
     ahead = w;
     advance(ahead);
     const uint8_t* xs = slice_base(w);
@@ -424,12 +446,12 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 #ifdef LLVQ_PHASE_TIMING
     uint32_t stage_no = 1;
 #endif
-    while (w.unit < n_units) {
+    while (live(w)) {
 #ifdef LLVQ_PHASE_TIMING
       ++stage_no;
 #endif
       LLVQ_GSTAMP(256, 0);
-      const bool last_of_unit = w.si + 1 == w.n_slices;
+      const bool last_of_unit = w.j + 1 == a.spb || w.g + 1 == g_hi;  // the band ends, or this workgroup's share of it
       // The loads run ahead into the unit's next slice.  At the unit's end they re-read this
       // slice (the ring starts afresh behind the epilogue, which needs the registers).
       const uint8_t* xs_next = last_of_unit ? xs : slice_base(ahead);
@@ -469,7 +491,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       const SliceWalk done = w;
       w = ahead;
       advance(ahead);
-      xs = slice_base(w);  // past the last unit: an address that is not read
+      xs = slice_base(w);  // past the last slice: an address that is not read
       buf ^= 1u;
       if (last_of_unit) {
         // the unit's sums: acc[rt][ct][j] belongs to weight row r0 + 32 rt + 8 (j / 4) + 4 lh + j % 4
@@ -479,7 +501,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
           for (int ct = 0; ct < 2; ++ct) {
             const uint32_t my_m = m0 + 32u * ct + l32;
             if (my_m < a.M) {
-              float* dst = a.ws + (((size_t)(done.split * kparts + kpart) * a.n_bands + done.band) * a.M + my_m) * kGemmRows;
+              float* dst = a.ws + ((((size_t)done.band * a.max_pieces + done.piece) * kparts + kpart) * a.M + my_m) * kGemmRows;
 #pragma unroll
               for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
@@ -490,7 +512,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
           }
         }
         clear_acc();
-        if (w.unit < n_units) fetch(xs, ring[0]);
+        if (live(w)) fetch(xs, ring[0]);
       }
     }
   }
@@ -508,11 +530,12 @@ struct GemmReduceMat {
   uint32_t d_out, band_begin;
 };
 struct GemmReduceArgs {
-  const float* ws;  // [S, n_bands, M, 64]
+  const float* ws;  // [n_bands, max_pieces, kparts, M, 64]
   const __half* x;  // [M, ldx]
   GemmReduceMat mat[kGemmMaxGroup];
   uint32_t n_mats;
-  uint32_t M, ldx, nblocks, tail_w, S, n_bands;
+  uint32_t M, ldx, nblocks, tail_w, n_bands;
+  uint32_t spb, base, rem, max_pieces, kparts;  // as in GemmArgs: which workgroups fed a band
 };
 
 constexpr int kReduceRowsM = 16;  // activation rows per workgroup
@@ -542,17 +565,19 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
   }
   __syncthreads();
   if (m >= a.M || row >= rows) return;
-  const size_t sstride = (size_t)a.n_bands * a.M * kGemmRows;
-  const float* src = a.ws + ((size_t)band * a.M + m) * kGemmRows + row;
+  // the band's partial sums: one per workgroup that walked some of its slices, times the K-step shares
+  const uint32_t n_sums = (gemm_owner((band + 1u) * a.spb - 1u, a.base, a.rem) - gemm_owner(band * a.spb, a.base, a.rem) + 1u) * a.kparts;
+  const size_t sstride = (size_t)a.M * kGemmRows;
+  const float* src = a.ws + ((size_t)band * a.max_pieces * a.kparts * a.M + m) * kGemmRows + row;
   float sum[4] = {0.f, 0.f, 0.f, 0.f};
-  for (uint32_t s0 = 0; s0 < a.S; s0 += 8) {
+  for (uint32_t s0 = 0; s0 < n_sums; s0 += 8) {
     float4 p[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u)
-      p[u] = s0 + u < a.S ? *reinterpret_cast<const float4*>(src + (size_t)(s0 + u) * sstride) : make_float4(0.f, 0.f, 0.f, 0.f);
+      p[u] = s0 + u < n_sums ? *reinterpret_cast<const float4*>(src + (size_t)(s0 + u) * sstride) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int u = 0; u < 8; ++u)
-      if (s0 + u < a.S) {
+      if (s0 + u < n_sums) {
         sum[0] += p[u].x;
         sum[1] += p[u].y;
         sum[2] += p[u].z;

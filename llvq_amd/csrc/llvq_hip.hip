@@ -1473,33 +1473,6 @@ int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   return forward_group(rt, mats, n, x, y, y_dtype);
 }
 
-// Split of a matrix's block range over work units: the count that minimises a
-// coarse time model (rounds of units over the CUs x per-unit time), so that a
-// matrix with few 64-row bands still occupies the chip.  A slice of 16 blocks per
-// row costs what its unranking costs (the matrix-core work of the slice before runs
-// beside it), a unit pays one more stage to drain, and every launch ends in the
-// chip-wide sum.  Splits are whole slices, so every slice starts on a 32-column
-// K-step of the tiled activations.
-static void pick_gemm_split(uint32_t n_bands, uint32_t nblocks, uint32_t M, uint32_t kparts, uint32_t grid,
-                            uint32_t* S_out, uint32_t* bps_out) {
-  double best = 1e30;
-  const uint32_t total_slices = (nblocks + kGemmKb - 1) / kGemmKb;
-  uint32_t best_s = 1, best_bps = total_slices * kGemmKb;
-  const double stage_us = 7.5;
-  for (uint32_t per = total_slices; per >= 1; --per) {  // slices per split
-    const uint32_t S = (total_slices + per - 1) / per;
-    if (S > 64) break;
-    if ((total_slices + S - 1) / S != per) continue;  // the same S with a smaller last split: already seen
-    const double unit_us = 2.0 + (per + 1) * stage_us + 0.004 * M;
-    const uint64_t units = (uint64_t)n_bands * S;
-    const double reduce_us = 6.0 + (double)S * kparts * M * 64.0 * n_bands * 4.0 / 2.0e6;
-    const double t = (double)((units + grid - 1) / grid) * unit_us + reduce_us;
-    if (t < best * 0.999) { best = t; best_s = S; best_bps = per * kGemmKb; }
-  }
-  *S_out = best_s;
-  *bps_out = best_bps;
-}
-
 // Grows a device buffer of the runtime to `need` bytes (contents are not kept).
 static int grow_buffer(void** buf, size_t* have, size_t need) {
   if (need <= *have) return LLVQ_OK;
@@ -1540,10 +1513,17 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   a.ct_shift = 0;
   while (((uint32_t)kGemmColTile << a.ct_shift) < M) ++a.ct_shift;
   const uint32_t kparts = consumers >> a.ct_shift;
-  pick_gemm_split(a.n_bands, m0->nblocks, M, kparts, grid_cap, &a.S, &a.bps);
-  const uint32_t n_partials = a.S * kparts;
+  // The launch's slices, band by band, are shared out evenly over the workgroups (one per CU): a
+  // band whose slices fall to several of them leaves one partial sum per workgroup.
+  a.spb = (m0->nblocks + kGemmKb - 1) / kGemmKb;
+  const uint64_t total = (uint64_t)a.n_bands * a.spb;
+  if (total > 0xFFFFFFFFull) return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": too many K-slices for one batched launch");
+  const uint32_t n_wg = total < grid_cap ? (uint32_t)total : grid_cap;
+  a.base = (uint32_t)(total / n_wg);
+  a.rem = (uint32_t)(total % n_wg);
+  a.max_pieces = (a.spb + a.base - 1) / a.base + 1;
   int rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes,
-                       (size_t)n_partials * a.n_bands * M * kGemmRows * sizeof(float));
+                       (size_t)a.n_bands * a.max_pieces * kparts * M * kGemmRows * sizeof(float));
   if (rc) return rc;
   // every slice has all its twelve K-steps in the tiled copy, zeros past the matrix's last block
   const uint32_t n_steps = (m0->nblocks + kGemmKb - 1) / kGemmKb * (kGemmKb * 24 / 32);
@@ -1555,8 +1535,7 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   HIP_TRY(hipGetLastError());
   a.xt = rt->gemm_xt;
   a.ws = rt->gemm_ws;
-  const uint32_t units = a.n_bands * a.S;
-  const dim3 grid(units < grid_cap ? units : grid_cap), wg(kWgThreads);
+  const dim3 grid(n_wg), wg(kWgThreads);
   if (consumers == 4) hipLaunchKernelGGL(gemm_tiles_kernel<12>, grid, wg, gemm_lds_bytes(), rt->stream, a);
   else hipLaunchKernelGGL(gemm_tiles_kernel<8>, grid, wg, gemm_lds_bytes(), rt->stream, a);
   HIP_TRY(hipGetLastError());
@@ -1566,8 +1545,12 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   r.ldx = m0->d_in;
   r.nblocks = m0->nblocks;
   r.tail_w = m0->tail_w;
-  r.S = n_partials;
   r.n_bands = a.n_bands;
+  r.spb = a.spb;
+  r.base = a.base;
+  r.rem = a.rem;
+  r.max_pieces = a.max_pieces;
+  r.kparts = kparts;
   const uint32_t rgrid = a.n_bands * ((M + kReduceRowsM - 1) / kReduceRowsM);
   if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3(rgrid), dim3(256), 0, rt->stream, r);
   else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3(rgrid), dim3(256), 0, rt->stream, r);
