@@ -193,8 +193,9 @@ __global__ __launch_bounds__(256) void tile_activations_kernel(const __half* x, 
 // one partial sum from each ("pieces", numbered in workgroup order).  Both roles step through the
 // same slices, the consumers one stage behind.
 struct SliceWalk {
-  uint32_t g;                   // slice number in the launch's sequence (band-major), valid below the workgroup's g_hi
+  uint32_t g;                   // slices walked before this one, counted from the launch's first; valid below the workgroup's g_hi
   uint32_t band, j;             // band, and the slice's place in it: blocks [16 j, 16 j + 16) of every row
+  uint32_t run_lo, run_len, si; // this workgroup's slices of the band, and how many of them are done
   uint32_t mat, r0, rows;       // the band's matrix, its first row there, its row count
   uint32_t piece;               // which of the band's partial sums this workgroup's run of slices feeds
 };
@@ -267,20 +268,31 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     w.r0 = (w.band - a.mat[w.mat].band_begin) * kGemmRows;
     w.rows = min((uint32_t)kGemmRows, a.mat[w.mat].d_out - w.r0);
   };
+  // A workgroup's slices of one band are walked from a band-dependent starting point, round the
+  // run: workgroups that hold the same slices of different bands then do not all pull the same
+  // activation columns through the same L2 channels at the same time.
+  auto enter_run = [&](SliceWalk& w) {
+    w.run_len = min(a.spb - w.run_lo, g_hi - w.g);
+    w.si = 0;
+    w.j = w.run_lo + (w.band * 5u) % w.run_len;
+    enter_band(w);
+  };
   auto start_walk = [&](SliceWalk& w) {
     w.g = g_lo;
     w.band = g_lo / a.spb;
-    w.j = g_lo - w.band * a.spb;
+    w.run_lo = g_lo - w.band * a.spb;
     w.piece = blockIdx.x - gemm_owner(w.band * a.spb, a.base, a.rem);
-    enter_band(w);
+    enter_run(w);
   };
   auto advance = [&](SliceWalk& w) {
     ++w.g;
-    if (++w.j == a.spb) {
-      w.j = 0;
+    if (++w.si == w.run_len) {
       ++w.band;
+      w.run_lo = 0;
       w.piece = 0;  // this workgroup is the first to reach the next band
-      if (w.g < g_hi) enter_band(w);
+      if (w.g < g_hi) enter_run(w);
+    } else {
+      w.j = w.j + 1 == w.run_lo + w.run_len ? w.run_lo : w.j + 1;
     }
   };
   auto live = [&](const SliceWalk& w) { return w.g < g_hi; };
@@ -451,7 +463,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       ++stage_no;
 #endif
       LLVQ_GSTAMP(256, 0);
-      const bool last_of_unit = w.j + 1 == a.spb || w.g + 1 == g_hi;  // the band ends, or this workgroup's share of it
+      const bool last_of_unit = w.si + 1 == w.run_len;  // the band ends, or this workgroup's share of it
       // The loads run ahead into the unit's next slice.  At the unit's end they re-read this
       // slice (the ring starts afresh behind the epilogue, which needs the registers).
       const uint8_t* xs_next = last_of_unit ? xs : slice_base(ahead);
