@@ -7,11 +7,11 @@
 // (llvq-llm/src/model.rs:521-529); this kernel decodes every block once for
 // all M rows instead.
 //
-// Work unit: a band of 64 weight rows x a range of blocks of those rows, walked
-// in K-slices of 16 blocks per row (384 columns = 12 K-steps of 32, 1024 blocks)
-// by one persistent 1024-lane workgroup per CU.  Its 16 wavefronts split into two
-// roles, and the unranking and the contraction of consecutive slices run at the
-// same time:
+// The work is cut into K-slices: 16 blocks per row of a band of 64 weight rows (384
+// columns = 12 K-steps of 32, 1024 blocks).  The launch's slices, numbered band by band,
+// are shared out evenly over one persistent 1024-lane workgroup per CU.  A workgroup's
+// 16 wavefronts split into two roles, and the unranking and the contraction of
+// consecutive slices run at the same time:
 //   producers (the first 8 or 12) slice g: code bytes -> LDS (loads issued two
 //                                slices ahead), classify and bin the blocks (odd /
 //                                even / generic queues), unrank; every block writes
@@ -21,9 +21,9 @@
 //   consumers (the other 8 or 4) v_mfma_f32_32x32x16_f16 over slice g - 1 from
 //                                W[(g - 1) & 1]: every consumer owns all 64 weight
 //                                rows x 64 activation rows (64 accumulator
-//                                registers, live across the unit's slices), A
+//                                registers, live across a band's slices), A
 //                                fragments from LDS, B fragments from global
-//                                memory / L2, three K-steps in flight.
+//                                memory / L2, two K-steps in flight.
 // The unranking is integer and f64 VALU work and the contraction runs on the
 // matrix cores, so the two overlap on every SIMD.  Because the roles are separate
 // branches of one kernel, the accumulators and the decode state are never live
@@ -31,17 +31,16 @@
 // wavefront (one wavefront doing both in turn spills beyond 32 accumulators).
 // A narrow batch leaves the matrix cores little to do, and 12 wavefronts unrank.
 //
-// A stage has two workgroup barriers (after the classification, after the
-// unranking); the consumers cross the same two while they work through their
-// K-steps, so the W buffer written in stage g is complete before it is read in
-// stage g + 1 and is not overwritten before stage g + 2.
+// A stage ends in one workgroup barrier.  In stage g the producers unrank slice g
+// and then classify slice g + 1 (three sets of code bytes and counters, two sets of
+// queues), the consumers multiply slice g - 1; so the W buffer written in stage g is
+// complete before it is read in stage g + 1 and is not overwritten before stage g + 2.
 //
-// Every consumer writes its sums to the workspace [split x K-share][band][m][64]
-// (consumers left over by a batch of few 64-row tiles take the same tile on
-// interleaved K-steps; matrices with few bands split their block range over
-// several units so that the chip is occupied); gemm_reduce_kernel adds the
-// partial sums in that fixed order and applies row scale and the f32 tail
-// columns, so the result does not depend on scheduling.
+// Every consumer writes its sums to the workspace [band][piece][K-share][m][64]: a
+// band whose slices fell to several workgroups has one piece from each, and consumers
+// left over by a batch of few 64-row tiles take the same tile on interleaved K-steps.
+// gemm_reduce_kernel adds the partial sums in that fixed order and applies row scale
+// and the f32 tail columns, so the result does not depend on scheduling.
 #pragma once
 
 namespace llvq {
