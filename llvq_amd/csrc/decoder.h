@@ -388,6 +388,189 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const __half* __restrict_
       }
 }
 
+// The same causal attention for 32 rows at a time on the matrix cores (head_dim = 128).
+// Workgroup (kv head, block of 32 rows); wavefront w serves query head w of the group and all
+// 32 rows.  The cache is walked in tiles of 32 positions, staged in LDS once for all heads:
+// K as stored ([position][dim]), V transposed ([dim][position], positions in the order the
+// second product wants them).  Per tile and wavefront:
+//   S^T = K Q^T      8 x v_mfma_f32_32x32x16_f16; A = K rows from LDS, B = the wavefront's
+//                    query rows, held in registers for the whole walk.  Lane (q, h) of the
+//                    result holds row q's scores of positions 8a + 4h + b (a, b < 4);
+//   online softmax   per row in its two lanes: running maximum and sum in f32, one exchange
+//                    between the halves of the wavefront; the causal mask is applied here;
+//   O^T += V^T P^T   8 x the same MFMA; B = the probabilities just computed, rounded to
+//                    binary16 in the lanes that hold them (no cross-lane movement: the K
+//                    index of the product is permuted to match, V^T is stored in that order).
+// Scores, maxima, sums and O stay in f32; the context is rounded once.  The next tile's K and
+// V rows are requested before the current tile is multiplied.  Positions past the pass's last
+// row are read as that row (their probabilities are zero; the values must be finite).
+constexpr int kAttnTile = 32;
+constexpr int kAttnKPitch = 128 + 8;   // binary16 elements per K row in LDS
+constexpr int kAttnVPitch = 32 + 8;    // per V^T row
+template <bool Q8, int G>
+__global__ __launch_bounds__(G * 64) void attn_rows_mfma_kernel(const __half* __restrict__ q, const __half* __restrict__ kcache,
+                                                                const __half* __restrict__ vcache, KvQ8 q8,
+                                                                __half* __restrict__ ctx, uint32_t n_heads, uint32_t n_kv,
+                                                                uint32_t pos0, uint32_t n_rows, uint32_t max_pos, float scale) {
+  typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+  typedef float f16v __attribute__((ext_vector_type(16)));
+  constexpr uint32_t kDimH = 128, kThreads = G * 64;
+  constexpr int CH = (kAttnTile * kDimH / 8 + kThreads - 1) / kThreads;  // 16-byte pieces of a tile per lane
+  __shared__ __align__(16) _Float16 kt[kAttnTile * kAttnKPitch];
+  __shared__ __align__(16) _Float16 vt[kDimH * kAttnVPitch];
+  const uint32_t kvh = blockIdx.x, row0 = blockIdx.y * kAttnTile;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t groups = n_heads / n_kv;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  const bool has_head = wave < groups;
+  const uint32_t head = kvh * groups + min(wave, groups - 1u);
+  const uint32_t my_row = min(row0 + l32, n_rows - 1u);      // rows past the pass repeat its last row and store nothing
+  const uint32_t qpos = pos0 + my_row;
+  const uint32_t last_pos = pos0 + n_rows - 1u;              // last cached position
+  const uint32_t t_end = pos0 + min(row0 + kAttnTile - 1u, n_rows - 1u);
+  const uint32_t n_tiles = t_end / kAttnTile + 1u;
+  const size_t base = (size_t)kvh * max_pos;
+  constexpr uint32_t kvgroups = kDimH / kKvGroup;
+
+  // query rows: B fragments of the first product, dims [16 s + 8 h, +8) of row q
+  h8 qf[8];
+  {
+    const __half* qrow = q + ((size_t)my_row * n_heads + head) * kDimH + lh * 8u;
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) qf[s8] = *reinterpret_cast<const h8*>(qrow + s8 * 16);
+  }
+  f16v o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) o[dt][j] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // staging, 16-byte pieces: piece c of K = position c / 16, dims [8 (c % 16), +8) (rows are read and
+  // stored whole); piece c of V = position c % 32, dims [8 (c / 32), +8) (the transposing 2-byte stores
+  // of a wavefront then fall into different LDS banks)
+  uint4 kreg[CH], vreg[CH];
+  float ksc[CH], kbi[CH], vsc[CH], vbi[CH];
+  auto request = [&](uint32_t tile) {
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      const uint32_t c = tid + (uint32_t)u * kThreads;
+      if (c < kAttnTile * kDimH / 8) {
+        const uint32_t kpos = min(tile * kAttnTile + c / 16u, last_pos), kd0 = (c & 15u) * 8u;
+        const uint32_t vpos = min(tile * kAttnTile + (c & 31u), last_pos), vd0 = (c >> 5) * 8u;
+        if constexpr (Q8) {
+          const uint2 kc = *reinterpret_cast<const uint2*>(q8.kq + (base + kpos) * kDimH + kd0);
+          const uint2 vc = *reinterpret_cast<const uint2*>(q8.vq + (base + vpos) * kDimH + vd0);
+          const size_t kgi = (base + kpos) * kvgroups + kd0 / kKvGroup, vgi = (base + vpos) * kvgroups + vd0 / kKvGroup;
+          kreg[u] = make_uint4(kc.x, kc.y, 0, 0);
+          vreg[u] = make_uint4(vc.x, vc.y, 0, 0);
+          ksc[u] = __half2float(q8.ks[kgi]); kbi[u] = __half2float(q8.kb[kgi]);
+          vsc[u] = __half2float(q8.vs[vgi]); vbi[u] = __half2float(q8.vb[vgi]);
+        } else {
+          kreg[u] = *reinterpret_cast<const uint4*>(kcache + (base + kpos) * kDimH + kd0);
+          vreg[u] = *reinterpret_cast<const uint4*>(vcache + (base + vpos) * kDimH + vd0);
+        }
+      }
+    }
+  };
+  auto deposit = [&]() {
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      const uint32_t c = tid + (uint32_t)u * kThreads;
+      if (c < kAttnTile * kDimH / 8) {
+        const uint32_t kp = c / 16u, kd0 = (c & 15u) * 8u, p = c & 31u, vd0 = (c >> 5) * 8u;
+        h8 kv8, vv8;
+        if constexpr (Q8) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            kv8[t] = (_Float16)kv_dequant((kreg[u].x >> (8 * t)) & 0xFFu, ksc[u], kbi[u]);
+            kv8[4 + t] = (_Float16)kv_dequant((kreg[u].y >> (8 * t)) & 0xFFu, ksc[u], kbi[u]);
+            vv8[t] = (_Float16)kv_dequant((vreg[u].x >> (8 * t)) & 0xFFu, vsc[u], vbi[u]);
+            vv8[4 + t] = (_Float16)kv_dequant((vreg[u].y >> (8 * t)) & 0xFFu, vsc[u], vbi[u]);
+          }
+        } else {
+          kv8 = __builtin_bit_cast(h8, kreg[u]);
+          vv8 = __builtin_bit_cast(h8, vreg[u]);
+        }
+        *reinterpret_cast<h8*>(kt + kp * kAttnKPitch + kd0) = kv8;
+        // position p = 16 hh + 8 a + 4 h + b sits at column 16 hh + 8 h + 4 a + b of its V^T row
+        const uint32_t col = (p & 16u) + ((p >> 2) & 1u) * 8u + ((p >> 3) & 1u) * 4u + (p & 3u);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) vt[(vd0 + t) * kAttnVPitch + col] = vv8[t];
+      }
+    }
+  };
+
+  request(0);
+  for (uint32_t tile = 0; tile < n_tiles; ++tile) {
+    __syncthreads();  // the previous tile has been read by every wavefront
+    deposit();
+    __syncthreads();
+    if (tile + 1 < n_tiles) request(tile + 1);
+    // S^T = K Q^T
+    f16v sacc;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) sacc[j] = 0.f;
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) {
+      const h8 kf = *reinterpret_cast<const h8*>(kt + l32 * kAttnKPitch + s8 * 16 + lh * 8u);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s8], sacc, 0, 0, 0);
+    }
+    // online softmax of row q over this tile's positions (16 of them in this lane, 16 in lane ^ 32)
+    float sc[16], mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t pos = tile * kAttnTile + 8u * (j >> 2) + 4u * lh + (j & 3);
+      sc[j] = pos <= qpos ? sacc[j] * scale : -INFINITY;
+      mx = fmaxf(mx, sc[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen nothing yet
+    const float alpha = __expf(m_run - m_use);              // 0 while m_run = -inf
+    float psum = 0.f;
+    h8 pf[2];  // the probabilities as the second product's B fragments
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float pj = __expf(sc[j] - m_use);
+      psum += pj;
+      pf[j >> 3][j & 7] = (_Float16)pj;
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = fmaf(l_run, alpha, psum);
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) o[dt][j] *= alpha;
+    // O^T += V^T P^T: K index e of half hh <-> position 16 hh + 8 (e / 4) + 4 h + e % 4 = this lane's score 8 hh + e
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        const h8 vf = *reinterpret_cast<const h8*>(vt + (dt * 32 + l32) * kAttnVPitch + hh * 16 + lh * 8u);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[hh], o[dt], 0, 0, 0);
+      }
+    }
+  }
+  // o[dt][j] = O[q = l32][dim 32 dt + 8 (j / 4) + 4 h + j % 4]
+  if (has_head && row0 + l32 < n_rows) {
+    const float inv = 1.0f / l_run;
+    __half* dst = ctx + ((size_t)my_row * n_heads + head) * kDimH;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const __half2 lo = __float22half2_rn(make_float2(o[dt][4 * a] * inv, o[dt][4 * a + 1] * inv));
+        const __half2 hi = __float22half2_rn(make_float2(o[dt][4 * a + 2] * inv, o[dt][4 * a + 3] * inv));
+        uint2 pk;
+        pk.x = *reinterpret_cast<const uint32_t*>(&lo);
+        pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+        *reinterpret_cast<uint2*>(dst + dt * 32 + 8 * a + 4 * lh) = pk;
+      }
+  }
+}
+
 // Attention of one query position over the cache (model.rs:812-822), split over
 // the cache: workgroup (kv head, split) takes a contiguous range of positions
 // for all query heads that share the kv head, so every K and V row is fetched

@@ -1862,17 +1862,33 @@ int decoder_prefill_pass(llvq_decoder* d, uint32_t n, bool want_logits, uint32_t
       hipLaunchKernelGGL(kernel, agrid, dim3(64), 0, st, d->pq, kc, vc, lq8, d->pctx, d->n_heads, d->n_kv, d->head_dim, d->pos, d->max_pos, scale);
     };
     const uint32_t grp = d->n_heads / d->n_kv;
+    // 32 rows per workgroup on the matrix cores where the head width is the one that kernel is built for
+    const bool on_mfma = d->head_dim == 128 && grp <= (uint32_t)kAttnMaxGroup;
+    const dim3 mgrid(d->n_kv, (n + kAttnTile - 1) / kAttnTile);
+    auto attend_mfma = [&](auto kernel, uint32_t waves) {
+      hipLaunchKernelGGL(kernel, mgrid, dim3(waves * 64), 0, st, d->pq, kc, vc, lq8, d->pctx, d->n_heads, d->n_kv, d->pos, n, d->max_pos, scale);
+    };
     if (d->kv_q8) {
       hipLaunchKernelGGL(norm_rope_append_rows_kernel<true>, hgrid, dim3(64), 0, st, d->pq, d->pk, d->pv, nw, lq8, d->n_heads, d->n_kv,
                          d->head_dim, d->pos, d->max_pos);
-      if (grp <= 2) attend(attn_rows_kernel<true, 2>);
+      if (on_mfma) {
+        if (grp <= 2) attend_mfma(attn_rows_mfma_kernel<true, 2>, 2);
+        else if (grp <= 4) attend_mfma(attn_rows_mfma_kernel<true, 4>, 4);
+        else if (grp <= 5) attend_mfma(attn_rows_mfma_kernel<true, 5>, 5);
+        else attend_mfma(attn_rows_mfma_kernel<true, kAttnMaxGroup>, kAttnMaxGroup);
+      } else if (grp <= 2) attend(attn_rows_kernel<true, 2>);
       else if (grp <= 4) attend(attn_rows_kernel<true, 4>);
       else if (grp <= 5) attend(attn_rows_kernel<true, 5>);
       else attend(attn_rows_kernel<true, kAttnMaxGroup>);
     } else {
       hipLaunchKernelGGL(norm_rope_append_rows_kernel<false>, hgrid, dim3(64), 0, st, d->pq, d->pk, d->pv, nw, lq8, d->n_heads, d->n_kv,
                          d->head_dim, d->pos, d->max_pos);
-      if (grp <= 2) attend(attn_rows_kernel<false, 2>);
+      if (on_mfma) {
+        if (grp <= 2) attend_mfma(attn_rows_mfma_kernel<false, 2>, 2);
+        else if (grp <= 4) attend_mfma(attn_rows_mfma_kernel<false, 4>, 4);
+        else if (grp <= 5) attend_mfma(attn_rows_mfma_kernel<false, 5>, 5);
+        else attend_mfma(attn_rows_mfma_kernel<false, kAttnMaxGroup>, kAttnMaxGroup);
+      } else if (grp <= 2) attend(attn_rows_kernel<false, 2>);
       else if (grp <= 4) attend(attn_rows_kernel<false, 4>);
       else if (grp <= 5) attend(attn_rows_kernel<false, 5>);
       else attend(attn_rows_kernel<false, kAttnMaxGroup>);

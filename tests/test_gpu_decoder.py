@@ -269,3 +269,37 @@ def test_generate_edge_cases(gpu_rt, orc):
         assert full.size == 11
     finally:
         dec.close()
+
+
+def _wide(heads, kv, kv_mode="f16"):
+    return decoder.Qwen3Config(num_hidden_layers=2, hidden_size=256, num_attention_heads=heads, num_key_value_heads=kv,
+                               head_dim=128, intermediate_size=384, vocab_size=400, rope_theta=1e6, rms_norm_eps=1e-6,
+                               max_positions=128, tie_word_embeddings=True, kv_mode=kv_mode)
+
+
+@pytest.mark.parametrize("heads,kv,kv_mode,seed", [(4, 2, "f16", 11), (4, 1, "f16", 12), (10, 2, "q8", 13), (8, 1, "q8", 14),
+                                                   (6, 2, "f16", 15)])
+def test_prompt_attention_on_the_matrix_cores(gpu_rt, orc, heads, kv, kv_mode, seed):
+    """Heads of 128 take the matrix-core attention of the batched prompt path: 2, 4, 5 and 8 query heads
+    per kv head (3 runs on the instantiation for 4 with a wavefront idle), both caches.  100 positions in
+    passes of 48: row blocks of 32 and 16, a last pass of 4, up to four cache tiles per block.  The last
+    row's logits and six decoded positions over the cache the passes left, against the oracle and against
+    the position-by-position path of the same decoder."""
+    cfg = _wide(heads, kv, kv_mode)
+    dec, ref = _build(gpu_rt, orc, cfg, seed, prefill_rows=48)
+    try:
+        tokens = np.random.default_rng(seed).integers(0, cfg.vocab_size, size=100)
+        more = np.random.default_rng(seed + 100).integers(0, cfg.vocab_size, size=6)
+        want = [ref.forward_token(int(t)) for t in tokens][-1:] + [ref.forward_token(int(t)) for t in more]
+        one_by_one = [dec.forward_token(int(t))[0] for t in tokens][-1:] + [dec.forward_token(int(t))[0] for t in more]
+        dec.reset()
+        got, best = dec.prefill(tokens)
+        assert dec.position == len(tokens) and best == int(np.argmax(got))
+        batched = [got] + [dec.forward_token(int(t))[0] for t in more]
+        for w, o, b in zip(want, one_by_one, batched):
+            top = np.abs(w).max()
+            # observed: 1e-4 (a binary16 ulp of a logit); a wrong score, mask or V row shows at 1e-2 and more
+            assert np.abs(b - w).max() < 2e-3 * top, f"batched vs oracle {np.abs(b - w).max() / top:.3e}"
+            assert np.abs(b - o).max() < 2e-3 * top, f"batched vs position by position {np.abs(b - o).max() / top:.3e}"
+    finally:
+        dec.close()
