@@ -43,6 +43,8 @@
 // and the f32 tail columns, so the result does not depend on scheduling.
 #pragma once
 
+#include "gemm_share.h"
+
 namespace llvq {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -230,14 +232,6 @@ struct GemmArgs {
   uint32_t ct_shift;         // log2 of the 64-row activation tiles the consumers spread over
 };
 
-// The workgroup that walks slice g, and the first slice of workgroup c.
-__host__ __device__ inline uint32_t gemm_owner(uint32_t g, uint32_t base, uint32_t rem) {
-  const uint32_t head = rem * (base + 1u);
-  return g < head ? g / (base + 1u) : rem + (g - head) / base;
-}
-__host__ __device__ inline uint32_t gemm_first_slice(uint32_t c, uint32_t base, uint32_t rem) {
-  return c * base + (c < rem ? c : rem);
-}
 
 // PW = producer wavefronts (8 or 12); the other 16 - PW consume.
 template <int PW>

@@ -1518,10 +1518,11 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   a.spb = (m0->nblocks + kGemmKb - 1) / kGemmKb;
   const uint64_t total = (uint64_t)a.n_bands * a.spb;
   if (total > 0xFFFFFFFFull) return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": too many K-slices for one batched launch");
-  const uint32_t n_wg = total < grid_cap ? (uint32_t)total : grid_cap;
-  a.base = (uint32_t)(total / n_wg);
-  a.rem = (uint32_t)(total % n_wg);
-  a.max_pieces = (a.spb + a.base - 1) / a.base + 1;
+  const GemmShare share = gemm_share(total, a.spb, grid_cap);
+  const uint32_t n_wg = share.n_wg;
+  a.base = share.base;
+  a.rem = share.rem;
+  a.max_pieces = share.max_pieces;
   int rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes,
                        (size_t)a.n_bands * a.max_pieces * kparts * M * kGemmRows * sizeof(float));
   if (rc) return rc;

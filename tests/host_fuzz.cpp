@@ -14,6 +14,7 @@
 
 #include "../llvq_amd/csrc/artifact.hpp"
 #include "../llvq_amd/csrc/codebook.hpp"
+#include "../llvq_amd/csrc/gemm_share.h"
 #include "../llvq_amd/csrc/rotation.hpp"
 
 using namespace llvq;
@@ -117,6 +118,27 @@ int main(int argc, char** argv) {
     if (!(after > 0.999 * before && after < 1.001 * before)) { std::fprintf(stderr, "rotation of width %u does not keep the norm\n", n); return 4; }
     ++rotations;
   }
-  std::printf("ok: %zu records in the whole file, %zu hostile inputs, %zu decodable ranks, %zu rotations\n", whole, cases, valid, rotations);
+  // the batched launch's work sharing: every slice has exactly one owner, workgroups hold consecutive
+  // slices, loads differ by at most one, and no band receives more partial sums than the workspace holds
+  size_t shares = 0;
+  for (uint32_t cap : {1u, 3u, 256u, 304u})
+    for (uint32_t spb : {1u, 2u, 7u, 11u, 26u, 32u, 46u})
+      for (uint32_t bands : {1u, 2u, 5u, 16u, 40u, 96u, 192u, 255u, 256u, 257u, 304u, 1000u}) {
+        const uint64_t total = (uint64_t)bands * spb;
+        const GemmShare sh = gemm_share(total, spb, cap);
+        if (sh.n_wg == 0 || sh.n_wg > cap || sh.n_wg > total || sh.base == 0) { std::fprintf(stderr, "share: bad workgroup count\n"); return 5; }
+        if (gemm_first_slice(0, sh.base, sh.rem) != 0 || gemm_first_slice(sh.n_wg, sh.base, sh.rem) != total) { std::fprintf(stderr, "share: slices not covered\n"); return 5; }
+        for (uint32_t c = 0; c < sh.n_wg; ++c) {
+          const uint32_t lo = gemm_first_slice(c, sh.base, sh.rem), hi = gemm_first_slice(c + 1, sh.base, sh.rem);
+          if (hi - lo != sh.base + (c < sh.rem ? 1u : 0u)) { std::fprintf(stderr, "share: uneven load\n"); return 5; }
+          if (gemm_owner(lo, sh.base, sh.rem) != c || gemm_owner(hi - 1, sh.base, sh.rem) != c) { std::fprintf(stderr, "share: owner of a slice\n"); return 5; }
+        }
+        for (uint32_t b = 0; b < bands; ++b) {
+          const uint32_t pieces = gemm_owner((b + 1) * spb - 1, sh.base, sh.rem) - gemm_owner(b * spb, sh.base, sh.rem) + 1;
+          if (pieces > sh.max_pieces) { std::fprintf(stderr, "share: %u pieces in a band, %u slots\n", pieces, sh.max_pieces); return 5; }
+        }
+        ++shares;
+      }
+  std::printf("ok: %zu records in the whole file, %zu hostile inputs, %zu decodable ranks, %zu rotations, %zu work shares\n", whole, cases, valid, rotations, shares);
   return 0;
 }
