@@ -213,10 +213,14 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
 def bench_gemm(args, torch, llvq_amd, synth, dev):
-    """Batched dequant-GEMM: the seven projections of `--layers` (default 4 here) Qwen3-8B-shaped
-    layers against M activation rows.  A step is one pass over all of them."""
-    n_layers = min(args.layers, 4)
-    M = args.M
+    """`--workload gemm`: its own JSON line."""
+    print(json.dumps(measure_gemm(args, torch, llvq_amd, synth, dev, args.M, min(args.layers, 4), args.steps, args.warmup)),
+          flush=True)
+
+
+def measure_gemm(args, torch, llvq_amd, synth, dev, M, n_layers, steps, warmup):
+    """Batched dequant-GEMM: the seven projections of n_layers Qwen3-8B-shaped layers against M
+    activation rows.  A step is one pass over all of them."""
     rt = llvq_amd.FusedRuntime(device=0)
     mats = [synth.layer_matrices(layer, args.seed, QWEN3_8B_LAYER) for layer in range(n_layers)]
     projs = [[rt.upload(m) for m in layer] for layer in mats]
@@ -249,28 +253,28 @@ def bench_gemm(args, torch, llvq_amd, synth, dev):
         us = e0.elapsed_time(e1) * 1e3 / 5
         per_shape[f"{p.d_out}x{p.d_in}"] = {"us": round(us, 1),
                                             "TFLOPs": round(2.0 * M * p.d_out * p.d_in / us / 1e6, 1)}
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     ev1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     dev_s = ev0.elapsed_time(ev1) * 1e-3
-    tflops = flops * args.steps / wall / 1e12
+    tflops = flops * steps / wall / 1e12
     n_launch = n_layers * 4
     out = {
         "metric": "dequant_gemm_TFLOPs",
         "value": round(tflops, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(wall * 1e3 / args.steps, 4),
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(wall * 1e3 / steps, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -280,24 +284,24 @@ def bench_gemm(args, torch, llvq_amd, synth, dev):
                                f"layers = {n_layers * 7} LLVQ matrices in {n_launch} group calls (q/k/v, o, gate/up, down), "
                                f"M = {M} activation rows, f16 in / f16 out",
                    "layers": n_layers, "M": M, "seed": args.seed},
-        "encoded_weight_GBps": round(enc_bytes * args.steps / wall / 1e9, 2),
-        "blocks_per_s": round(n_blocks * args.steps / wall, 1),
+        "encoded_weight_GBps": round(enc_bytes * steps / wall / 1e9, 2),
+        "blocks_per_s": round(n_blocks * steps / wall, 1),
         "per_shape": per_shape,
         "roofline": {
             "kernel": "gemm_tiles_kernel",
             "bound": "mfma",
-            "achieved": round(flops * args.steps / dev_s / 1e12, 2),
+            "achieved": round(flops * steps / dev_s / 1e12, 2),
             "peak": MFMA_F16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
-            "frac": round(flops * args.steps / dev_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 5),
+            "frac": round(flops * steps / dev_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 5),
             "traffic": None,
-            "avg_launch_us": round(dev_s * 1e6 / (args.steps * n_launch), 2),
+            "avg_launch_us": round(dev_s * 1e6 / (steps * n_launch), 2),
             "launches_per_step": n_launch,
             "algorithmic_flops_per_launch": round(flops / n_launch, 1),
         },
     }
     rt.close()
-    print(json.dumps(out), flush=True)
+    return out
 
 
 def main():
@@ -441,6 +445,10 @@ def main():
     }
     if not args.no_decode and args.layers == 36:
         out["decode"] = decode_leg(rt, projs, args.seed)
+        # BASELINE config 3 beside it, shortened: two Qwen3-8B-shaped layers, M = 256 (the full sweep is --workload gemm)
+        g = measure_gemm(args, torch, llvq_amd, synth, dev, 256, 2, 3, 1)
+        out["batched"] = {"M": 256, "TFLOPs": g["value"], "mfma_peak_frac": g["roofline"]["frac"],
+                          "ms_per_step": g["ms_per_step"], "workload": g["config"]["workload"]}
     if args.copy_probe:
         src = torch.arange(1 << 26, dtype=torch.int32, device=dev)  # 256 MiB
         dst = torch.empty_like(src)
