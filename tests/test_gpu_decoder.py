@@ -303,3 +303,34 @@ def test_prompt_attention_on_the_matrix_cores(gpu_rt, orc, heads, kv, kv_mode, s
             assert np.abs(b - o).max() < 2e-3 * top, f"batched vs position by position {np.abs(b - o).max() / top:.3e}"
     finally:
         dec.close()
+
+
+def test_full_size_greedy_tokens_match_the_oracle_fixture(gpu_rt):
+    """BASELINE config 2 at full size: 36 layers at the Qwen3-4B widths, a 512-token prompt, 256 greedy
+    tokens.  The expected tokens are the CPU oracle runner's over the same synthetic weights
+    (tests/golden/qwen3_4b_synthetic_greedy.json, written by tests/golden/make_full_size_tokens.py; the
+    oracle needs a quarter of an hour and 30 GB for them, the device loop seconds).  The fixture also
+    holds the gap between the oracle's two largest logits at every step: the smallest is one binary16
+    ulp of a logit of magnitude 10 (2^-7), no step is a tie, so the tokens must be identical — position
+    by position, and with the prompt through the batched path."""
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "qwen3_4b_synthetic_greedy.json")) as f:
+        fixture = json.load(f)
+    want = np.array(fixture["tokens"], np.uint32)
+    assert min(fixture["top_two_gap"]) > 1e-4  # the bar below allows no exception
+    cfg = decoder.QWEN3_4B
+    raws = decoder.synthetic_projections(cfg, fixture["prompt_seed"])
+    weights = decoder.synthetic_weights(cfg, fixture["prompt_seed"])
+    dec = decoder.Decoder(gpu_rt, cfg, raws, weights, prefill_rows=512)
+    try:
+        prompt = np.random.default_rng(fixture["prompt_seed"]).integers(0, cfg.vocab_size, size=fixture["prompt_tokens"])
+        for batched in (False, True):
+            got = dec.generate(prompt, len(want), batched_prefill=batched)
+            same = want == got
+            assert same.all(), f"batched_prefill={batched}: first divergence at step {int(np.argmin(same))}: " \
+                               f"oracle {want[int(np.argmin(same))]}, device {got[int(np.argmin(same))]}, " \
+                               f"oracle gap {fixture['top_two_gap'][int(np.argmin(same))]}"
+    finally:
+        dec.close()
