@@ -2,7 +2,7 @@
 36-layer Qwen3-4B-shaped model over synthetic LLVQ weights of seed 0, a 512-token prompt, 256 new tokens)
 as the CPU oracle runner produces them, with the gap between the two largest logits of every step.
 
-Needs no GPU; takes the oracle about a quarter of an hour and 30 GB of memory (the 252 matrices are
+Needs no GPU; takes the oracle about four minutes on 16 host threads and 30 GB of memory (the 252 matrices are
 decoded to dense f32 on the CPU first).  Run from the repository root:
     python tests/golden/make_full_size_tokens.py
 tests/test_gpu_decoder.py::test_full_size_greedy_tokens_match_the_oracle_fixture compares the device

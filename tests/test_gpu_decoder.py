@@ -309,7 +309,7 @@ def test_full_size_greedy_tokens_match_the_oracle_fixture(gpu_rt):
     """BASELINE config 2 at full size: 36 layers at the Qwen3-4B widths, a 512-token prompt, 256 greedy
     tokens.  The expected tokens are the CPU oracle runner's over the same synthetic weights
     (tests/golden/qwen3_4b_synthetic_greedy.json, written by tests/golden/make_full_size_tokens.py; the
-    oracle needs a quarter of an hour and 30 GB for them, the device loop seconds).  The fixture also
+    oracle needs four minutes and 30 GB for them, the device loop seconds).  The fixture also
     holds the gap between the oracle's two largest logits at every step: the smallest is one binary16
     ulp of a logit of magnitude 10 (2^-7), no step is a tie, so the tokens must be identical — position
     by position, and with the prompt through the batched path."""
