@@ -305,25 +305,32 @@ def test_prompt_attention_on_the_matrix_cores(gpu_rt, orc, heads, kv, kv_mode, s
         dec.close()
 
 
-def test_full_size_greedy_tokens_match_the_oracle_fixture(gpu_rt):
-    """BASELINE config 2 at full size: 36 layers at the Qwen3-4B widths, a 512-token prompt, 256 greedy
-    tokens.  The expected tokens are the CPU oracle runner's over the same synthetic weights
-    (tests/golden/qwen3_4b_synthetic_greedy.json, written by tests/golden/make_full_size_tokens.py; the
-    oracle needs four minutes and 30 GB for them, the device loop seconds).  The fixture also
-    holds the gap between the oracle's two largest logits at every step: the smallest is one binary16
-    ulp of a logit of magnitude 10 (2^-7), no step is a tie, so the tokens must be identical — position
-    by position, and with the prompt through the batched path."""
+@pytest.mark.parametrize("fixture_name,cfg,max_positions", [
+    ("qwen3_4b_synthetic_greedy.json", decoder.QWEN3_4B, 768),
+    ("qwen3_14b_q8kv_synthetic_greedy.json", decoder.QWEN3_14B, 128),
+])
+def test_full_size_greedy_tokens_match_the_oracle_fixture(gpu_rt, fixture_name, cfg, max_positions):
+    """The full-size models.  BASELINE config 2: 36 layers at the Qwen3-4B widths, a 512-token prompt, 256
+    greedy tokens.  BASELINE config 4's model: 40 layers at the Qwen3-14B widths (5 query heads per kv
+    head, 17 408-wide down_proj rows, int8 KV cache), a 96-token prompt and 32 tokens.  The expected tokens
+    are the CPU oracle runner's over the same synthetic weights (tests/golden/*.json, written by
+    tests/golden/make_full_size_tokens.py; the oracle needs minutes and tens of GB for them, the device
+    loop seconds).  The fixtures also hold the gap between the oracle's two largest logits at every step:
+    the smallest is one binary16 ulp of a logit (2^-7), no step is a tie, so the tokens must be identical —
+    position by position, and with the prompt through the batched path."""
+    import dataclasses
     import json
     import os
 
-    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "qwen3_4b_synthetic_greedy.json")) as f:
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", fixture_name)) as f:
         fixture = json.load(f)
     want = np.array(fixture["tokens"], np.uint32)
     assert min(fixture["top_two_gap"]) > 1e-4  # the bar below allows no exception
-    cfg = decoder.QWEN3_4B
+    cfg = dataclasses.replace(cfg, max_positions=max_positions)
     raws = decoder.synthetic_projections(cfg, fixture["prompt_seed"])
     weights = decoder.synthetic_weights(cfg, fixture["prompt_seed"])
-    dec = decoder.Decoder(gpu_rt, cfg, raws, weights, prefill_rows=512)
+    dec = decoder.Decoder(gpu_rt, cfg, raws, weights, prefill_rows=min(512, fixture["prompt_tokens"]))
+    del raws
     try:
         prompt = np.random.default_rng(fixture["prompt_seed"]).integers(0, cfg.vocab_size, size=fixture["prompt_tokens"])
         for batched in (False, True):
