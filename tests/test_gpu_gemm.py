@@ -157,6 +157,8 @@ def test_gemm_matches_gemv_rows(gpu_rt):
     ("self_attn.k_proj", 1024, 4096, 64),     # few bands: the block range is split over units
     ("mlp.down_proj", 4096, 12288, 16),
     ("mlp.gate_proj", 12288, 4096, 256),
+    ("self_attn.o_proj", 4096, 4096, 512),    # eight consumer wavefronts, bands shared between workgroups
+    ("mlp.down_proj", 4096, 12288, 512),
 ])
 def test_gemm_qwen3_8b_shapes(gpu_rt, orc, site, d_out, d_in, M):
     """BASELINE config 3 shapes; checked on a sample of activation rows to keep the f64 reference short."""
@@ -167,7 +169,7 @@ def test_gemm_qwen3_8b_shapes(gpu_rt, orc, site, d_out, d_in, M):
     proj = gpu_rt.upload(raw)
     Y = gpu_rt.forward_batched(proj, _x16(X), out_dtype=torch.float32).cpu().numpy()
     gpu_rt.free(proj)
-    pick = sorted({0, 1, M // 2, M - 1})
+    pick = sorted({0, 1, 63, 64, M // 2, M - 65, M - 1} & set(range(M)))  # rows of every 64-row tile's ends
     Y_ref, A_ref = _reference(orc, raw, X[pick])
     _check(Y[pick], Y_ref, A_ref)
     assert np.isfinite(Y).all()
