@@ -154,6 +154,48 @@ def test_long_cache_takes_the_merge_kernel(gpu_rt, orc):
         dec.close()
 
 
+def test_context_of_8192_positions_int8_cache(gpu_rt):
+    """BASELINE config 4's regime for the attention: an int8 KV cache filled to 8192 positions, heads of
+    128, 5 query heads per kv head (a small model otherwise, so that the oracle can follow).  The cache is
+    filled once position by position (split-KV attention over up to 64 ranges and the merge kernel) and once
+    by the batched path (matrix-core attention over up to 256 cache tiles, int8 rows rebuilt in LDS); the
+    logits of the last prompt position and of six more positions are compared with the oracle's, which are
+    a fixture (tests/golden/qwen3_small_q8kv_8192_logits.npz, written by make_long_context_logits.py: the
+    oracle takes minutes over the 8192 positions)."""
+    import os
+
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("make_long_context_logits", os.path.join(golden, "make_long_context_logits.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)  # the model description and seeds the fixture was made with (runs nothing)
+    with np.load(os.path.join(golden, "qwen3_small_q8kv_8192_logits.npz")) as f:
+        want = f["logits"].astype(np.float64)
+        assert (int(f["model_seed"]), int(f["prompt_seed"]), int(f["more_seed"]), int(f["n_prompt"])) == \
+            (gen.MODEL_SEED, gen.PROMPT_SEED, gen.MORE_SEED, gen.N_PROMPT)
+    cfg = gen.CFG
+    dec = decoder.Decoder(gpu_rt, cfg, decoder.synthetic_projections(cfg, gen.MODEL_SEED), decoder.synthetic_weights(cfg, gen.MODEL_SEED),
+                          prefill_rows=512)
+    try:
+        tokens = np.random.default_rng(gen.PROMPT_SEED).integers(0, cfg.vocab_size, size=gen.N_PROMPT)
+        more = np.random.default_rng(gen.MORE_SEED).integers(0, cfg.vocab_size, size=gen.N_MORE)
+        for batched in (False, True):
+            dec.reset()
+            if batched:
+                got = [dec.prefill(tokens)[0]]
+            else:
+                for t in tokens[:-1]:
+                    dec.forward_token(int(t), want_logits=False)
+                got = [dec.forward_token(int(tokens[-1]))[0]]
+            got += [dec.forward_token(int(t))[0] for t in more]
+            assert dec.position == 8192
+            worst = max(float(np.abs(g - w).max() / np.abs(w).max()) for g, w in zip(got, want))
+            assert worst < 5e-3, f"batched={batched}: max |dlogit| / max|logit| = {worst:.3e}"
+    finally:
+        dec.close()
+
+
 def test_greedy_tokens_match_oracle(gpu_rt, orc):
     dec, ref = _build(gpu_rt, orc, SMALL, 3)
     try:
