@@ -191,7 +191,7 @@ def test_context_of_8192_positions_int8_cache(gpu_rt):
             got += [dec.forward_token(int(t))[0] for t in more]
             assert dec.position == 8192
             worst = max(float(np.abs(g - w).max() / np.abs(w).max()) for g, w in zip(got, want))
-            assert worst < 5e-3, f"batched={batched}: max |dlogit| / max|logit| = {worst:.3e}"
+            assert worst < 1e-3, f"batched={batched}: max |dlogit| / max|logit| = {worst:.3e}"  # observed: 1.2e-4, a binary16 ulp
     finally:
         dec.close()
 
