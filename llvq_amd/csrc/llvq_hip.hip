@@ -7,6 +7,7 @@
 // reciprocals) that every workgroup copies into LDS.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
+#include <type_traits>
 
 #include <cstdio>
 #include <cmath>
@@ -70,7 +71,20 @@ __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const Global
   const uint4* src = reinterpret_cast<const uint4*>(g.image);
   uint4* dst = reinterpret_cast<uint4*>(smem);
   constexpr size_t kBytes = kFull ? sizeof(TableImage) : (kLut ? kLdsImageBytesLean : kLdsImageBytesLeanest);
-  for (uint32_t i = threadIdx.x; i < kBytes / 16; i += blockDim.x) dst[i] = src[i];
+  // five loads per lane in flight at a time (one pass for a 1024-lane workgroup): a load and its
+  // store per loop iteration would pay the L2 latency once per iteration
+  constexpr uint32_t kUnits = (uint32_t)(kBytes / 16), kLast = kUnits - 1u;
+  const uint32_t st = blockDim.x;
+  for (uint32_t i0 = threadIdx.x; i0 < kUnits; i0 += 5u * st) {
+    const uint32_t i1 = i0 + st, i2 = i1 + st, i3 = i2 + st, i4 = i3 + st;
+    const uint4 r0 = src[i0], r1 = src[min(i1, kLast)], r2 = src[min(i2, kLast)], r3 = src[min(i3, kLast)], r4 = src[min(i4, kLast)];
+    __builtin_amdgcn_sched_barrier(0);  // keep the loads together, ahead of the first store
+    dst[i0] = r0;
+    if (i1 < kUnits) dst[i1] = r1;
+    if (i2 < kUnits) dst[i2] = r2;
+    if (i3 < kUnits) dst[i3] = r3;
+    if (i4 < kUnits) dst[i4] = r4;
+  }
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
   const TableImage* far = kFull ? s : g.image;
   return DecodeTables{far->golay, g.cls, s->fast, s->starts, kLut ? s->lut : g.image->lut, s->rcp, far->on_lut, g.off_lut,
@@ -414,8 +428,10 @@ __device__ __forceinline__ void prefetch_tile(const GroupArgs& a, uint32_t tile,
   const uint32_t off = (uint32_t)(byte0 & 15);
   const uint4* src = reinterpret_cast<const uint4*>(M.codes + (byte0 - off));
   const uint32_t n16 = (off + rows * a.nblocks * 6 + 15) >> 4;
-  if (tid < n16) p0 = src[tid];
-  if (tid + kWgThreads < n16) p1 = src[tid + kWgThreads];
+  // unconditional (a lane past the tile's end re-reads its last unit, which is never stored): a
+  // guarded load is merged with the old value right away, and that merge waits for the load
+  p0 = src[min(tid, n16 - 1u)];
+  p1 = src[min(tid + kWgThreads, n16 - 1u)];
 }
 
 // Phase timestamps for tuning builds (-DLLVQ_PHASE_TIMING): wave 0 of each
@@ -531,6 +547,12 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   constexpr int kRawBytes = TILE * 6 + 32;
   extern __shared__ __align__(16) uint8_t smem[];
   const DecodeTables T = stage_tables<!LEAN && (LLVQ_LDS_GOLAY != 0)>(smem, a.tables);
+  // The code bytes of a tile travel HBM -> registers -> LDS; the next tile's loads are issued
+  // while the current one is being decoded.  The first tile's are issued right behind the
+  // loads of the activation: the memory counter retires in order, so whatever is requested
+  // after them would wait for HBM with them, and they are not needed before the activation is.
+  uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0;
+  auto request_first_tile = [&]() { prefetch_tile(a, blockIdx.x, threadIdx.x, pre0, pre1); };
   const uint32_t nb = a.nblocks;
   uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + (LEAN ? kLdsImageBytesLean : kLdsImageBytes));
   float* xscale = reinterpret_cast<float*>(xplanes + (size_t)nb * kPlaneDwords);
@@ -541,12 +563,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   uint32_t* gqueue = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
   uint32_t* ctrl = gqueue + kGenericSlots;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  // The code bytes of a tile travel HBM -> registers -> LDS; the first tile's
-  // loads are issued before the tables and the activation are staged, the next
-  // tile's while the current one is being decoded.
   static_assert(kRawBytes <= 2 * 16 * kWgThreads, "two 16-byte registers per lane hold a tile's code bytes");
-  uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0;
-  prefetch_tile(a, blockIdx.x, tid, pre0, pre1);
   const __half* xsrc = a.x;
   // A launch over matrices stored in a rotated basis rotates its activation itself: the
   // values go, signs applied, as f32 to the area the first tile's code bytes, queues and
@@ -560,51 +577,80 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     // instead of waiting for a kernel of its own; it is staged, as binary16, where
     // the tile's code bytes will go.
     __half* xs = reinterpret_cast<__half*>(raw);
-    if (a.prologue == kPrologueSiluMul) {
-      for (uint32_t i = tid; i < d_in; i += kWgThreads) {
-        const float g = __half2float(a.x2[i]);
-        const float sg = __half2float(__float2half_rn(g / (1.0f + __expf(-g))));
-        const __half h = __float2half_rn(sg * __half2float(a.x[i]));
-        if (rotated) xf[i] = signed_f32(i, __half2float(h));
-        else xs[i] = h;
-      }
-    } else {
-      float* red = partial + kTileBlocks - kWaves;  // the end of the partial sums: beyond the f32 staging of a rotated launch
-      constexpr int kPer = (kRawBytes / 2 + kWgThreads - 1) / kWgThreads;
-      float v[kPer];
-      float ss = 0.f;
+    // All of a lane's values are requested before the first is used (a load and its use per loop
+    // iteration would pay the memory latency once per iteration): the rounds are counted at compile
+    // time (3 covers 3072 values, 6 and 12 the wider rows), their loads are unconditional (a lane past
+    // the row's end reads its last value) and a scheduling barrier keeps them ahead of the arithmetic.
+    constexpr int kPerMax = (kRawBytes / 2 + kWgThreads - 1) / kWgThreads;
+    const bool silu = a.prologue == kPrologueSiluMul;
+    const __half* src1 = a.x2 ? a.x2 : a.x;
+    const __half* src2 = silu ? a.x : a.norm_w;
+    auto derive = [&](auto rounds) {
+      constexpr int kPer = decltype(rounds)::value;
+      __half in0[kPer], in1[kPer], in2[kPer];
 #pragma unroll
       for (int k = 0; k < kPer; ++k) {
-        const uint32_t i = tid + (uint32_t)k * kWgThreads;
-        v[k] = 0.f;
-        if (i < d_in) {
-          float r = __half2float(a.x[i]);
-          if (a.x2) r = __half2float(__float2half_rn(r + __half2float(a.x2[i])));
-          if (a.resid_out && blockIdx.x == 0) a.resid_out[i] = __float2half_rn(r);
-          v[k] = r;
-          ss += r * r;
+        const uint32_t i = min(tid + (uint32_t)k * kWgThreads, d_in - 1u);
+        in0[k] = a.x[i];
+        in1[k] = src1[i];
+        in2[k] = src2[i];
+      }
+      request_first_tile();
+      __builtin_amdgcn_sched_barrier(0);
+      if (silu) {
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+          const uint32_t i = tid + (uint32_t)k * kWgThreads;
+          if (i < d_in) {
+            const float g = __half2float(in1[k]);
+            const float sg = __half2float(__float2half_rn(g / (1.0f + __expf(-g))));
+            const __half h = __float2half_rn(sg * __half2float(in0[k]));
+            if (rotated) xf[i] = signed_f32(i, __half2float(h));
+            else xs[i] = h;
+          }
+        }
+      } else {
+        float* red = partial + kTileBlocks - kWaves;  // the end of the partial sums: beyond the f32 staging of a rotated launch
+        float v[kPer];
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+          const uint32_t i = tid + (uint32_t)k * kWgThreads;
+          v[k] = 0.f;
+          if (i < d_in) {
+            float r = __half2float(in0[k]);
+            if (a.x2) r = __half2float(__float2half_rn(r + __half2float(in1[k])));
+            if (a.resid_out && blockIdx.x == 0) a.resid_out[i] = __float2half_rn(r);
+            v[k] = r;
+            ss += r * r;
+          }
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) total += red[w];
+        const float inv = 1.0f / sqrtf(total / (float)d_in + a.eps);
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+          const uint32_t i = tid + (uint32_t)k * kWgThreads;
+          if (i < d_in) {
+            const __half h = __float2half_rn(v[k] * inv * __half2float(in2[k]));
+            if (rotated) xf[i] = signed_f32(i, __half2float(h));
+            else xs[i] = h;
+          }
         }
       }
-      ss = wave_sum(ss);
-      if (lane == 0) red[wave] = ss;
-      __syncthreads();
-      float total = 0.f;
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) total += red[w];
-      const float inv = 1.0f / sqrtf(total / (float)d_in + a.eps);
-#pragma unroll
-      for (int k = 0; k < kPer; ++k) {
-        const uint32_t i = tid + (uint32_t)k * kWgThreads;
-        if (i < d_in) {
-          const __half h = __float2half_rn(v[k] * inv * __half2float(a.norm_w[i]));
-          if (rotated) xf[i] = signed_f32(i, __half2float(h));
-          else xs[i] = h;
-        }
-      }
-    }
+    };
+    const uint32_t n_per = (d_in + kWgThreads - 1) / kWgThreads;
+    if (n_per <= 3) derive(std::integral_constant<int, kPerMax < 3 ? kPerMax : 3>{});
+    else if (n_per <= 6) derive(std::integral_constant<int, kPerMax < 6 ? kPerMax : 6>{});
+    else derive(std::integral_constant<int, kPerMax>{});
     __syncthreads();
     xsrc = xs;
   } else if (rotated) {
+    request_first_tile();
     // eight values per lane and pass; a width that is not a multiple of eight ends one value at a time
     const uint32_t n8 = d_in & ~7u;
     for (uint32_t i = tid * 8u; i < n8; i += kWgThreads * 8u) {
@@ -628,14 +674,34 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     for (uint32_t col = tid; col < nb; col += kWgThreads)
       quantize_block_f32(xf + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     if (tid < a.tail_w) xtail[tid] = xf[(size_t)nb * kDim + tid];
-  } else if (a.x_f32) {
-    for (uint32_t col = tid; col < nb; col += kWgThreads)
-      quantize_block_f32(a.x_f32 + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
-    if (tid < a.tail_w) xtail[tid] = a.x_f32[(size_t)nb * kDim + tid];
-  } else {
+  } else if (a.prologue != kPrologueNone) {
     for (uint32_t col = tid; col < nb; col += kWgThreads)
       quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     if (tid < a.tail_w) xtail[tid] = __half2float(xsrc[(size_t)nb * kDim + tid]);
+  } else {
+    // a finished activation from global memory: this lane's block is requested, then the first tile's
+    // code bytes, then the block is quantised (rows wider than 1024 blocks take further rounds)
+    float v[kDim];
+#pragma unroll
+    for (int j = 0; j < kDim; ++j) v[j] = 0.f;
+    if (nb) {  // a row of tail columns only has no block to read
+      const uint32_t c0 = min(tid, nb - 1u);
+      if (a.x_f32) {
+#pragma unroll
+        for (int j = 0; j < kDim; ++j) v[j] = a.x_f32[(size_t)c0 * kDim + j];
+      } else {
+        load_block_f16(xsrc + (size_t)c0 * kDim, v);
+      }
+    }
+    const float tail_v = tid < a.tail_w ? (a.x_f32 ? a.x_f32[(size_t)nb * kDim + tid] : __half2float(xsrc[(size_t)nb * kDim + tid])) : 0.f;
+    request_first_tile();
+    __builtin_amdgcn_sched_barrier(0);
+    if (tid < nb) quantize_values(v, xplanes + (size_t)tid * kPlaneDwords, xscale + tid);
+    if (tid < a.tail_w) xtail[tid] = tail_v;
+    for (uint32_t col = tid + kWgThreads; col < nb; col += kWgThreads) {
+      if (a.x_f32) quantize_block_f32(a.x_f32 + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+      else quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+    }
   }
   if (a.prologue != kPrologueNone || rotated) __syncthreads();  // the staging area becomes the code-byte buffer
 
