@@ -305,13 +305,14 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     auto prefetch = [&](const SliceWalk& w, uint4& pre) {
       if (!live(w)) return;
       const uint32_t k0 = w.j * kGemmKb, kb = slice_blocks(w);
-      const uint32_t row = tid / kGemmRowChunks, j = tid - row * kGemmRowChunks;
-      if (row < w.rows) {
-        const size_t byte0 = ((size_t)(w.r0 + row) * nb + k0) * 6;
-        const uint32_t off = (uint32_t)(byte0 & 15);
-        const uint32_t n16 = (off + kb * 6 + 15) >> 4;
-        if (j < n16) pre = reinterpret_cast<const uint4*>(a.mat[w.mat].codes + (byte0 - off))[j];
-      }
+      // Unconditional: a lane past the band's rows or the row's units repeats the last ones (what it
+      // stores is never read).  A guarded load is merged with the register's old value at once, and
+      // that merge waits for the load, which is meant to stay in flight for a stage.
+      const uint32_t row_raw = tid / kGemmRowChunks, row = min(row_raw, w.rows - 1u), j = tid - row_raw * kGemmRowChunks;
+      const size_t byte0 = ((size_t)(w.r0 + row) * nb + k0) * 6;
+      const uint32_t off = (uint32_t)(byte0 & 15);
+      const uint32_t n16 = (off + kb * 6 + 15) >> 4;
+      pre = reinterpret_cast<const uint4*>(a.mat[w.mat].codes + (byte0 - off))[min(j, n16 - 1u)];
     };
     auto stage_raw = [&](uint32_t set, const uint4& pre) {
       if (tid < 4) ctrl0[set * 4 + tid] = 0;
