@@ -684,7 +684,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     float v[kDim];
 #pragma unroll
     for (int j = 0; j < kDim; ++j) v[j] = 0.f;
-    if (nb) {  // a row of tail columns only has no block to read
+    if ((tid & ~63u) < nb) {  // wavefronts with a block to read (a row of tail columns only has none)
       const uint32_t c0 = min(tid, nb - 1u);
       if (a.x_f32) {
 #pragma unroll
