@@ -207,6 +207,7 @@ constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = kAttnThreads / 64;
 constexpr int kAttnMaxSplits = 64;  // the cache is cut into at most this many ranges (host picks by length; 128 was measured slower at 8188 positions)
 constexpr int kAttnMaxGroup = 8;    // query heads per kv head
+constexpr int kAttnInlineSplits = 16;  // up to this many ranges, the workgroup that finishes last merges them itself
 
 // ---- rows of positions at once (prompt processing through the batched product) ----
 // One wavefront per (head, row): q heads are normed and rotated in place, k heads are
@@ -613,8 +614,42 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
   const __half* Vb = q8.vb + (size_t)kvh * max_pos * kvgroups;
   const uint32_t stride = head_dim + 2;  // floats per partial: max, sum, head_dim sums
 
-  // the query heads of this kv head: norm, rotate, scale
   const uint32_t pos = T - 1;  // the position being decoded
+  const bool has_new = nj > 0 && j1 == T;
+  const uint32_t newj = has_new ? pos : 0xFFFFFFFFu;
+  // Lane (pj, sub) = (lane / 16, lane % 16) of wavefront w holds dims [8 sub, 8 sub + 8) of the
+  // positions of class c = 4 w + pj: jj = c, c + 16, ...  U rows of K and of V are requested
+  // together.  The loads are unconditional (a lane with no row, or with the row this launch
+  // appends, re-reads a valid one and ignores it): a guarded load would be waited for where it
+  // is issued, and the first batch is issued here, ahead of the work on the query heads, which
+  // then runs beside the cache's latency.
+  const uint32_t sub = lane & 15u, pj = lane >> 4, i0 = sub * 8u, c = wave * 4u + pj;
+  const bool active = i0 < head_dim;
+  const uint32_t i0c = active ? i0 : 0u;
+  constexpr int U = 4;
+  uint4 kraw[U], vraw[U];
+  float ksc[U], kbi[U], vsc[U], vbi[U];
+  auto request = [&](uint32_t jb) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t j = min(j0 + jb + 16u * u, pos);
+      if constexpr (Q8) {
+        const uint2 kc = *reinterpret_cast<const uint2*>(Kq + (size_t)j * head_dim + i0c);
+        const uint2 vc = *reinterpret_cast<const uint2*>(Vq + (size_t)j * head_dim + i0c);
+        const size_t gi = (size_t)j * kvgroups + i0c / kKvGroup;
+        kraw[u] = make_uint4(kc.x, kc.y, 0, 0);
+        vraw[u] = make_uint4(vc.x, vc.y, 0, 0);
+        ksc[u] = __half2float(Ks[gi]); kbi[u] = __half2float(Kb[gi]);
+        vsc[u] = __half2float(Vs[gi]); vbi[u] = __half2float(Vb[gi]);
+      } else {
+        kraw[u] = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0c);
+        vraw[u] = *reinterpret_cast<const uint4*>(V + (size_t)j * head_dim + i0c);
+        ksc[u] = kbi[u] = vsc[u] = vbi[u] = 0.f;
+      }
+    }
+  };
+  request(c);
+  // the query heads of this kv head: norm, rotate, scale
   for (uint32_t g = wave; g < groups; g += kAttnWaves) {
     norm_rope_wave(nw.q_raw + (size_t)(kvh * groups + g) * head_dim, nw.qn, nw.cos_t, nw.sin_t, pos, head_dim, nw.eps,
                    stage[wave], lane);
@@ -624,8 +659,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
   // The range that ends at the new position owns its k and v: they go to the
   // cache for later positions, and to LDS, in the form the cache gives back,
   // for this one (nothing else reads that cache row during this launch).
-  const bool has_new = nj > 0 && j1 == T;
-  const uint32_t newj = has_new ? pos : 0xFFFFFFFFu;
   if (has_new && wave == 0) {
     norm_rope_wave(nw.k_raw + (size_t)kvh * head_dim, nw.kn, nw.cos_t, nw.sin_t, pos, head_dim, nw.eps, stage[0], lane);
     const size_t row = (size_t)kvh * max_pos + pos;
@@ -672,12 +705,9 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
   __syncthreads();
 
   // ---- one pass over the range: scores, running maxima and weighted V sums together ----
-  // Lane (pj, sub) = (lane / 16, lane % 16) of wavefront w holds dims [8 sub, 8 sub + 8) of the
-  // positions of class c = 4 w + pj: jj = c, c + 16, ...  Each class keeps its own running
-  // maximum, sum of exponentials and weighted V sum (f32); U rows of K and of V are requested
-  // together, their scores are formed first (independent cross-lane sums), then folded in order.
-  const uint32_t sub = lane & 15u, pj = lane >> 4, i0 = sub * 8u, c = wave * 4u + pj;
-  const bool active = i0 < head_dim;
+  // Each position class keeps its own running maximum, sum of exponentials and weighted V sum
+  // (f32); the scores of a batch are formed first (independent cross-lane sums), then folded in
+  // order, with the next batch's rows already requested.
   float qv[G][8], acc[G][8], m[G], l[G];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
@@ -689,30 +719,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
       qv[g][t] = ((uint32_t)g < groups && active) ? qs[g * head_dim + i0 + t] : 0.f;
     }
   }
-  constexpr int U = 4;
   for (uint32_t jb = c; jb < nj; jb += 16u * U) {
-    uint4 kraw[U], vraw[U];
-    float ksc[U], kbi[U], vsc[U], vbi[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t jj = jb + 16u * u, j = j0 + jj;
-      kraw[u] = vraw[u] = make_uint4(0, 0, 0, 0);
-      ksc[u] = kbi[u] = vsc[u] = vbi[u] = 0.f;
-      if (active && jj < nj && j != newj) {
-        if constexpr (Q8) {
-          const uint2 kc = *reinterpret_cast<const uint2*>(Kq + (size_t)j * head_dim + i0);
-          const uint2 vc = *reinterpret_cast<const uint2*>(Vq + (size_t)j * head_dim + i0);
-          const size_t gi = (size_t)j * kvgroups + i0 / kKvGroup;
-          kraw[u].x = kc.x; kraw[u].y = kc.y;
-          vraw[u].x = vc.x; vraw[u].y = vc.y;
-          ksc[u] = __half2float(Ks[gi]); kbi[u] = __half2float(Kb[gi]);
-          vsc[u] = __half2float(Vs[gi]); vbi[u] = __half2float(Vb[gi]);
-        } else {
-          kraw[u] = *reinterpret_cast<const uint4*>(K + (size_t)j * head_dim + i0);
-          vraw[u] = *reinterpret_cast<const uint4*>(V + (size_t)j * head_dim + i0);
-        }
-      }
-    }
     float sc[U][G], vfs[U][8];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -750,6 +757,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
         sc[u][g] = row16_sum(d);
       }
     }
+    if (jb + 16u * U < nj) request(jb + 16u * U);
 #pragma unroll
     for (int u = 0; u < U; ++u)
       if (jb + 16u * u < nj) {
@@ -817,50 +825,58 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnNew nw, c
   if (tid == 0) arrived = __hip_atomic_fetch_add(&counters[kvh], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   if (arrived != n_splits - 1) return;
-  // Merge.  The (max, sum) pairs of every (head, split) are fetched in one pass
-  // and turned into weights in LDS; the weighted sums then read the partial
-  // vectors with many loads in flight (they come from the other XCDs' writes,
-  // i.e. from memory, so latency is what matters here).
-  float* wts = att_smem;                     // [groups][n_splits] weights (the staging of this launch is dead)
-  float* Ls = wts + groups * n_splits;       // [groups]
-  for (uint32_t o = tid; o < groups * n_splits; o += kAttnThreads) {
-    const uint32_t g = o / n_splits, sp = o - g * n_splits;
-    wts[o] = part[((size_t)(kvh * groups + g) * n_splits + sp) * stride];  // the split's running max
-  }
-  __syncthreads();
-  if (tid < groups) {
-    float M = -INFINITY;
-    for (uint32_t sp = 0; sp < n_splits; ++sp) M = fmaxf(M, wts[tid * n_splits + sp]);
-    Ls[tid] = M;
-  }
-  __syncthreads();
-  for (uint32_t o = tid; o < groups * n_splits; o += kAttnThreads) {
-    const uint32_t g = o / n_splits;
-    wts[o] = __expf(wts[o] - Ls[g]);  // 0 for an empty range
-  }
-  __syncthreads();
-  if (tid < groups) {
-    float L = 0.f;
-    for (uint32_t sp = 0; sp < n_splits; ++sp)
-      L = fmaf(part[((size_t)(kvh * groups + tid) * n_splits + sp) * stride + 1], wts[tid * n_splits + sp], L);
-    Ls[tid] = L;
-  }
-  __syncthreads();
-  for (uint32_t o = tid; o < groups * head_dim; o += kAttnThreads) {
+  // Merge (at most kAttnInlineSplits ranges).  The partials come from the other XCDs' writes,
+  // i.e. from memory, so latency is what matters: the (max, sum) pairs and the first partial
+  // vectors are requested together, every load unconditional (a lane past the end re-reads a
+  // valid element and gives it weight zero).  Each lane then forms its head's weights from
+  // the pairs in LDS for itself; sums run in range order.
+  float* mx = att_smem;                // [groups][n_splits] running maxima (the staging of this launch is dead)
+  float* sm = mx + groups * n_splits;  // [groups][n_splits] sums of exponentials
+  const uint32_t n_pairs = groups * n_splits, n_out = groups * head_dim;
+  auto fetch = [&](uint32_t o, float (&v)[kAttnInlineSplits]) {
+    o = min(o, n_out - 1u);
     const uint32_t g = o / head_dim, i = o - g * head_dim;
-    const uint32_t head = kvh * groups + g;
-    const float* src = part + (size_t)head * n_splits * stride + 2 + i;
-    float A = 0.f;
-    uint32_t sp = 0;
-    for (; sp + 8 <= n_splits; sp += 8) {
-      float v[8];
+    const float* src = part + (size_t)(kvh * groups + g) * n_splits * stride + 2 + i;
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(sp + u) * stride];
+    for (int u = 0; u < kAttnInlineSplits; ++u) v[u] = src[(size_t)min((uint32_t)u, n_splits - 1u) * stride];
+  };
+  float v[kAttnInlineSplits], vn[kAttnInlineSplits];
+  float2 pair[(kAttnMaxGroup * kAttnInlineSplits + kAttnThreads - 1) / kAttnThreads];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) A = fmaf(v[u], wts[g * n_splits + sp + u], A);  // split order
+  for (uint32_t r = 0; r < sizeof(pair) / sizeof(pair[0]); ++r) {
+    const uint32_t o = min(tid + r * kAttnThreads, n_pairs - 1u);
+    const uint32_t g = o / n_splits, sp = o - g * n_splits;
+    pair[r] = *reinterpret_cast<const float2*>(part + ((size_t)(kvh * groups + g) * n_splits + sp) * stride);
+  }
+  fetch(tid, v);
+#pragma unroll
+  for (uint32_t r = 0; r < sizeof(pair) / sizeof(pair[0]); ++r) {
+    const uint32_t o = tid + r * kAttnThreads;
+    if (o < n_pairs) {
+      mx[o] = pair[r].x;
+      sm[o] = pair[r].y;
     }
-    for (; sp < n_splits; ++sp) A = fmaf(src[(size_t)sp * stride], wts[g * n_splits + sp], A);
-    ctx[(size_t)head * head_dim + i] = __float2half_rn(A / Ls[g]);
+  }
+  __syncthreads();
+  for (uint32_t o = tid; o < n_out; o += kAttnThreads) {
+    fetch(o + kAttnThreads, vn);
+    const uint32_t g = o / head_dim, i = o - g * head_dim;
+    float w[kAttnInlineSplits], M = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < kAttnInlineSplits; ++u) {
+      w[u] = mx[g * n_splits + min((uint32_t)u, n_splits - 1u)];
+      M = fmaxf(M, w[u]);
+    }
+    float L = 0.f, A = 0.f;
+#pragma unroll
+    for (int u = 0; u < kAttnInlineSplits; ++u) {
+      w[u] = (uint32_t)u < n_splits ? __expf(w[u] - M) : 0.f;  // 0 for an empty range too
+      L = fmaf(sm[g * n_splits + min((uint32_t)u, n_splits - 1u)], w[u], L);
+      A = fmaf(v[u], w[u], A);
+    }
+    ctx[(size_t)(kvh * groups + g) * head_dim + i] = __float2half_rn(A / L);
+#pragma unroll
+    for (int u = 0; u < kAttnInlineSplits; ++u) v[u] = vn[u];
   }
   if (tid == 0) counters[kvh] = 0;  // ready for the next launch
 }

@@ -1777,11 +1777,11 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   const uint32_t groups_per_kv = d->n_heads / d->n_kv;
   // the queries and the sixteen position classes' running results
   size_t attn_lds = ((size_t)groups_per_kv * d->head_dim + (size_t)16 * groups_per_kv * (d->head_dim + 2)) * sizeof(float);
-  const size_t merge_lds = (size_t)groups_per_kv * (n_splits + 1) * sizeof(float);  // the merge reuses the staging area
+  const size_t merge_lds = (size_t)groups_per_kv * 2 * n_splits * sizeof(float);  // the merge reuses the staging area
   if (attn_lds < merge_lds) attn_lds = merge_lds;
   const size_t group_layer = cache_layer / kKvGroup;
   // few partials: the last workgroup of a kv head merges them; many: a chip-wide merge kernel does
-  const uint32_t merge_inline = n_splits <= 16 ? 1u : 0u;
+  const uint32_t merge_inline = n_splits <= (uint32_t)kAttnInlineSplits ? 1u : 0u;
   // Projections in the natural basis derive their activation in the launch's
   // prologue; a rotated basis needs the activation as a tensor first (it goes
   // through the rotation kernel), and so do rows too wide for the staging area:
