@@ -94,6 +94,9 @@ static_assert(sizeof(FastClass) == 48, "FastClass must stay 48 bytes");
 constexpr int kMetaPathShift = 17;         // bits 17..18: which decoder a class takes
 constexpr int kMetaGolayShift = 20;        // bits 20..31: first codeword of the weight bucket
 enum : uint32_t { kPathOdd = 0, kPathEven = 1, kPathGeneric = 2 };
+constexpr int kTailSlots = 8;             // slots of the odd-coset walk that are looked up, not walked
+constexpr int kTailMetaSlots = 732;       // 9^3 threshold triples, padded to a multiple of four
+constexpr int kTailCodeSlots = 65536 + 2520;  // 4^8 arrangements, and the padding
 
 struct Codebook {
   uint32_t golay[4096];
@@ -110,6 +113,15 @@ struct Codebook {
   // step[(m * 25 + c) * 2 + {0,1}] = {m / c, 1 - m / c}: the odd-coset walk's per-slot
   // update t' + 1 = (t + 1 - lo) * (m / c) + (1 - m / c), m = slots left after this one
   double step[24 * 25 * 2];
+  // The last kTailSlots slots of the odd-coset walk are one table read.  With eight slots left the
+  // walk's state is the three thresholds T1 <= T2 <= T3 <= 8 (counts of the four kinds still to
+  // place) and a rank below the remaining multiset's arrangement count M <= 2520:
+  // tail_meta[T1 + 9 T2 + 81 T3] = M | first entry << 12, and tail_codes[first + rank] holds the
+  // eight slots' table codes (3 - kind), one per byte, first slot in the lowest byte — what the
+  // walk itself produces, which is how the table is filled.  Padded so that any rank below 2520
+  // stays inside the table.
+  uint32_t tail_meta[kTailMetaSlots];
+  std::vector<uint64_t> tail_codes;
   uint64_t n12 = 0;                       // points in the cap-12 ball (47-bit field)
   // fast paths
   FastClass fast[kClassSlots];

@@ -63,7 +63,9 @@ struct DecodeTables {
   const uint32_t* off_lut;  // even coset, off-support arrangements
   const uint32_t* expand;   // 8 dwords per codeword: deposit masks for the word and for its complement
   const uint8_t* pdep4;     // 4-bit deposit table
-  const double* step;       // {m/c, 1 - m/c} pairs, see Codebook::step
+  const double* step;       // {m/c, 1 - m/c} pairs, see Codebook::step (rows m >= kTailSlots are read)
+  const uint32_t* tail_meta;   // the walk's last kTailSlots slots, see Codebook::tail_meta
+  const uint64_t* tail_codes;
 };
 
 // Threshold packing: field f (bits 6f..6f+4) holds T_{4-f}; bit 6f+5 is the
@@ -153,22 +155,40 @@ LLVQ_HD uint32_t odd_walk_slot(const DecodeTables& T, uint32_t n, double& t1, ui
   return jj;
 }
 
+// The first sixteen slots of the walk (n = 24 .. 9 slots left) as they are produced; ends with
+// the state the table of the last eight slots is entered with.
 template <class OnCodes>
-LLVQ_HD void odd_codes(const DecodeTables& T, const FastClass& f, uint64_t li, OnCodes&& on_codes) {
+LLVQ_HD void odd_walk_head(const DecodeTables& T, const FastClass& f, uint64_t li, uint32_t& ncw, double& t1, uint32_t& tg,
+                           OnCodes&& on_codes) {
   const double local = (double)li;
   const double g = floor64((local + 0.5) * f.inv0);
   const double r = fma64(-g, f.d1, local);
-  double t1 = fma64((r + 0.5) * f.inv0, 24.0, 1.0);
-  const uint32_t ncw = ~T.golay[(uint32_t)g & 4095u];
-  uint32_t tg = f.u0;
+  t1 = fma64((r + 0.5) * f.inv0, 24.0, 1.0);
+  ncw = ~T.golay[(uint32_t)g & 4095u];
+  tg = f.u0;
 #pragma unroll
-  for (int q = 0; q < 6; ++q) {
+  for (int q = 0; q < (kDim - kTailSlots) / 4; ++q) {
     uint32_t sel = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) sel |= odd_walk_slot(T, (uint32_t)(kDim - 4 * q - j), t1, tg) << (8 * j);
     // table index = jj - 1 (kinds 0..3 <-> jj 4..1), bit 2 = off the codeword's support
     on_codes(q, (sel - 0x01010101u) | ((((ncw >> (4 * q)) & 15u) * kSpread2) & 0x04040404u));
   }
+}
+
+template <class OnCodes>
+LLVQ_HD void odd_codes(const DecodeTables& T, const FastClass& f, uint64_t li, OnCodes&& on_codes) {
+  uint32_t ncw, tg;
+  double t1;
+  odd_walk_head(T, f, li, ncw, t1, tg, on_codes);
+  // The last eight slots.  t1 - 1 = 8 rho with rho = (rank + 1/2) / M for the M arrangements of
+  // what is left, so rank = floor(rho M); the thresholds T3, T2, T1 sit in fields 1, 2, 3.
+  const uint32_t th = tg >> 6;
+  const uint32_t me = T.tail_meta[(th & 15u) * 81u + ((th >> 6) & 15u) * 9u + ((th >> 12) & 15u)];
+  const uint32_t rank = (uint32_t)(fma64(t1, 0.125, -0.125) * (double)(me & 0xFFFu));
+  const uint64_t codes = T.tail_codes[(me >> 12) + rank];
+  on_codes(4, (uint32_t)codes | ((((ncw >> 16) & 15u) * kSpread2) & 0x04040404u));
+  on_codes(5, (uint32_t)(codes >> 32) | ((((ncw >> 20) & 15u) * kSpread2) & 0x04040404u));
 }
 
 // ---- even coset, fast path --------------------------------------------------------

@@ -40,8 +40,9 @@ struct TableImage {
   FastClass fast[kClassSlots];
   uint64_t starts[kStartsLds];
   double rcp[32];
-  double step[24 * 25 * 2];
+  double step[(24 - kTailSlots) * 25 * 2];  // rows m >= kTailSlots: the walk's last slots are looked up
   uint8_t pdep4[256];
+  uint32_t tail_meta[kTailMetaSlots];
   uint16_t lut[2048];        // a 47-bit field only reaches the lower half of the host table
   uint32_t golay[4096];
   uint32_t on_lut[kOnLutSlots];
@@ -55,6 +56,7 @@ struct GlobalTables {
   const DevClass* cls;
   const uint32_t* off_lut;
   const uint32_t* expand;
+  const uint64_t* tail_codes;
 };
 
 constexpr size_t kLdsImageBytesLean = offsetof(TableImage, golay);  // without the Golay words and the support-arrangement table
@@ -88,7 +90,7 @@ __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const Global
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
   const TableImage* far = kFull ? s : g.image;
   return DecodeTables{far->golay, g.cls, s->fast, s->starts, kLut ? s->lut : g.image->lut, s->rcp, far->on_lut, g.off_lut,
-                      g.expand, s->pdep4, s->step};
+                      g.expand, s->pdep4, s->step - kTailSlots * 25 * 2, s->tail_meta, g.tail_codes};
 }
 
 // 6-byte big-endian record at a 2-byte-aligned offset of a 4-byte-aligned buffer
@@ -1022,12 +1024,14 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   hipError_t e = hipGetDeviceProperties(&prop, device);
   if (e != hipSuccess) { delete rt; return hip_fail(e, "hipGetDeviceProperties"); }
   rt->cu_count = prop.multiProcessorCount;
-  // one blob: LDS image | generic class records | off-support table | deposit masks
+  // one blob: LDS image | generic class records | off-support table | deposit masks | walk-tail codes
   if (cb.on_lut.size() > (size_t)kOnLutSlots) { delete rt; return fail(LLVQ_ERR_UNSUPPORTED, "support-arrangement table outgrew its LDS slot"); }
   const size_t off_cls = sizeof(TableImage);
   const size_t off_lut = off_cls + sizeof(cb.dev_classes);
   const size_t off_exp = (off_lut + cb.off_lut.size() * 4 + 15) & ~(size_t)15;
-  const size_t total = off_exp + sizeof(cb.expand);
+  const size_t off_tail = off_exp + sizeof(cb.expand);
+  static_assert(sizeof(cb.expand) % 16 == 0, "the walk-tail codes are read as 8-byte units");
+  const size_t total = off_tail + cb.tail_codes.size() * 8;
   std::vector<uint8_t> host(total, 0);
   auto* img = reinterpret_cast<TableImage*>(host.data());
   std::memcpy(img->golay, cb.golay, sizeof img->golay);
@@ -1035,12 +1039,14 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   std::memcpy(img->starts, cb.starts, sizeof img->starts);
   std::memcpy(img->lut, cb.lut, sizeof img->lut);
   std::memcpy(img->rcp, cb.rcp, sizeof img->rcp);
-  std::memcpy(img->step, cb.step, sizeof img->step);
+  std::memcpy(img->step, cb.step + kTailSlots * 25 * 2, sizeof img->step);
+  std::memcpy(img->tail_meta, cb.tail_meta, sizeof img->tail_meta);
   std::memcpy(img->pdep4, cb.pdep4, sizeof img->pdep4);
   std::memcpy(img->on_lut, cb.on_lut.data(), cb.on_lut.size() * 4);
   std::memcpy(host.data() + off_cls, cb.dev_classes, sizeof(cb.dev_classes));
   std::memcpy(host.data() + off_lut, cb.off_lut.data(), cb.off_lut.size() * 4);
   std::memcpy(host.data() + off_exp, cb.expand, sizeof(cb.expand));
+  std::memcpy(host.data() + off_tail, cb.tail_codes.data(), cb.tail_codes.size() * 8);
   e = hipMalloc(reinterpret_cast<void**>(&rt->blob), total);
   if (e != hipSuccess) { delete rt; return hip_fail(e, "hipMalloc(tables)"); }
   e = hipMemcpy(rt->blob, host.data(), total, hipMemcpyHostToDevice);
@@ -1049,6 +1055,7 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   rt->tables.cls = reinterpret_cast<const DevClass*>(rt->blob + off_cls);
   rt->tables.off_lut = reinterpret_cast<const uint32_t*>(rt->blob + off_lut);
   rt->tables.expand = reinterpret_cast<const uint32_t*>(rt->blob + off_exp);
+  rt->tables.tail_codes = reinterpret_cast<const uint64_t*>(rt->blob + off_tail);
   // the activation tile of a wide matrix pushes dynamic LDS past the 64 KB default
   const int max_lds = 160 * 1024;
   for_each_gemv_kernel([&](const void* kernel) { (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds); });
