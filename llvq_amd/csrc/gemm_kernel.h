@@ -155,7 +155,7 @@ static_assert(kGemmMaxM <= (kWgThreads - kGemmMinProducers) / 64 * kGemmColTile,
 
 // table image | code bytes of three slices | two block queues | two generic queues | three counter sets | two W buffers
 constexpr size_t gemm_lds_bytes() {
-  return kGemmImageBytes + 3 * (size_t)kGemmRows * kGemmRowBytes + 2 * (size_t)kGemmTile * 4 + 2 * kGenericSlots * 4 + 48 +
+  return kGemmImageBytes + 3 * (size_t)kGemmRows * kGemmRowBytes + 2 * (size_t)kGemmTile * 4 + 2 * kGenericSlots * 4 + 96 +
          2 * (size_t)kGemmRows * kGemmWStride * 2;
 }
 static_assert(gemm_lds_bytes() <= 160 * 1024, "GEMM workgroup state must fit one CU's LDS");
@@ -237,7 +237,6 @@ struct GemmArgs {
 template <int PW>
 __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   constexpr int kProducers = PW * 64, kConsumers = 16 - PW;
-  constexpr int kP1Blocks = (kGemmTile + kProducers - 1) / kProducers;
   static_assert(kProducers >= kGemmMinProducers && (kConsumers == 8 || kConsumers == 4), "roles");
   extern __shared__ __align__(16) uint8_t smem[];
   const DecodeTables T = stage_tables<false, false>(smem, a.tables);
@@ -245,8 +244,8 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   constexpr uint32_t kRawBuf = kGemmRows * kGemmRowBytes;
   uint32_t* queue0 = reinterpret_cast<uint32_t*>(raw0 + 3 * kRawBuf);
   uint32_t* gqueue0 = queue0 + 2 * kGemmTile;
-  uint32_t* ctrl0 = gqueue0 + 2 * kGenericSlots;  // three sets of four counters
-  _Float16* W0 = reinterpret_cast<_Float16*>(ctrl0 + 12);
+  uint32_t* ctrl0 = gqueue0 + 2 * kGenericSlots;  // three sets of eight counters: queue lengths, unrank ticket, classify ticket
+  _Float16* W0 = reinterpret_cast<_Float16*>(ctrl0 + 24);
   constexpr uint32_t kWBuf = kGemmRows * kGemmWStride;  // elements per W buffer
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -315,7 +314,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       pre = reinterpret_cast<const uint4*>(a.mat[w.mat].codes + (byte0 - off))[min(j, n16 - 1u)];
     };
     auto stage_raw = [&](uint32_t set, const uint4& pre) {
-      if (tid < 4) ctrl0[set * 4 + tid] = 0;
+      if (tid < 8) ctrl0[set * 8 + tid] = 0;
       if (tid < (uint32_t)(kGemmRows * kGemmRowChunks)) reinterpret_cast<uint4*>(raw0 + set * kRawBuf)[tid] = pre;
     };
     struct SliceView {  // what the phases of one slice need
@@ -337,19 +336,34 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     };
     auto classify = [&](const SliceView& v) {  // P1.  An origin block is queued like any other: its 24 zero weights must be written.
       const uint8_t* raw = raw0 + v.set3 * kRawBuf;
-      classify_and_bin<kP1Blocks, kProducers>(
-          T, v.nblk, kGemmTile, queue0 + v.set2 * kGemmTile, gqueue0 + v.set2 * kGenericSlots, ctrl0 + v.set3 * 4,
-          [&](uint32_t f) {
-            const uint32_t row = (f * v.inv_kb) >> 16, b = f - row * v.kb;
-            const uint32_t off = ((((v.r0 + row) * nb + v.k0) & 7u) * 6u) & 15u;  // (6 n) mod 16 depends on n mod 8 only
-            return read_record(raw, row * kGemmRowBytes + off + 6u * b);
-          },
-          [](uint32_t) { return true; });
+      uint32_t* ctrl = ctrl0 + v.set3 * 8;
+      auto record = [&](uint32_t f) {
+        const uint32_t row = (f * v.inv_kb) >> 16, b = f - row * v.kb;
+        const uint32_t off = ((((v.r0 + row) * nb + v.k0) & 7u) * 6u) & 15u;  // (6 n) mod 16 depends on n mod 8 only
+        return read_record(raw, row * kGemmRowBytes + off + 6u * b);
+      };
+      auto origin = [](uint32_t) { return true; };
+      uint32_t* queue = queue0 + v.set2 * kGemmTile;
+      uint32_t* gqueue = gqueue0 + v.set2 * kGenericSlots;
+      if constexpr (kGemmTile % kProducers == 0) {
+        // the slice's blocks divide evenly over the producers, and so do its sixteen chunks to unrank
+        classify_and_bin<kGemmTile / kProducers, kProducers>(T, v.nblk, kGemmTile, queue, gqueue, ctrl, record, origin);
+      } else {
+        // 64 blocks at a time, handed out by a counter: the wavefronts that drew fewer chunks to
+        // unrank arrive first and take more of this, so the stage ends for all at about the same time
+        for (;;) {
+          uint32_t unit = 0;
+          if (lane == 0) unit = atomicAdd(&ctrl[4], 1u);
+          unit = (uint32_t)__builtin_amdgcn_readfirstlane((int)unit);
+          if (unit * 64u >= v.nblk) break;
+          classify_and_bin<1, 64>(T, v.nblk, kGemmTile, queue, gqueue, ctrl, record, origin, unit * 64u + lane);
+        }
+      }
     };
     auto unrank = [&](const SliceView& v) {  // P2
       const uint8_t* raw = raw0 + v.set3 * kRawBuf;
       unrank_queues_to_slice<kGemmTile, kGemmWStride>(
-          T, queue0 + v.set2 * kGemmTile, gqueue0 + v.set2 * kGenericSlots, ctrl0 + v.set3 * 4, v.kb, v.inv_kb, v.g0, v.g1,
+          T, queue0 + v.set2 * kGemmTile, gqueue0 + v.set2 * kGenericSlots, ctrl0 + v.set3 * 8, v.kb, v.inv_kb, v.g0, v.g1,
           W0 + v.set2 * kWBuf, [&](uint32_t row, uint32_t b) -> uint64_t {
             const uint32_t off = ((((v.r0 + row) * nb + v.k0) & 7u) * 6u) & 15u;
             return read_record(raw, row * kGemmRowBytes + off + 6u * b);

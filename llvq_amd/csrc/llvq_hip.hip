@@ -449,7 +449,9 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 #endif
 
 // P1 of the GEMV and GEMM kernels: each of the LANES lanes taking part (the first
-// LANES of the workgroup) classifies up to NB blocks of the tile and bins them.  `record(f)` returns the 48-bit record of tile slot f < nblk;
+// LANES of the workgroup) classifies up to NB blocks of the tile and bins them: slots first, first + LANES, ...
+// (`first` is the lane's index in the workgroup unless the caller hands out the slots itself).
+// `record(f)` returns the 48-bit record of tile slot f < nblk;
 // `origin(f)` is called for an origin block (index 0) and returns whether the
 // block must still be queued (flagged, with the odd-coset blocks) or is settled.
 // Queue entry: slot (12 bits) | class << 16 | gain << 25 | origin << 30 | generic walk << 31.
@@ -460,8 +462,9 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 constexpr uint32_t kEntryOrigin = 0x40000000u, kEntryGeneric = 0x80000000u;
 template <int NB, int LANES = kWgThreads, typename RecordFn, typename OriginFn>
 __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t nblk, uint32_t capacity, uint32_t* queue,
-                                                 uint32_t* gqueue, uint32_t* ctrl, RecordFn record, OriginFn origin) {
-  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+                                                 uint32_t* gqueue, uint32_t* ctrl, RecordFn record, OriginFn origin,
+                                                 uint32_t first = threadIdx.x) {
+  const uint32_t tid = first, lane = threadIdx.x & 63u;
   uint32_t entry[NB], ci[NB];
   uint64_t zi[NB];  // zero-based index, ~0 when the lane has no block / an origin
   bool queued_origin[NB];
