@@ -4,6 +4,7 @@
 // the index decoder the kernels share with the host runs on class boundaries and random 48-bit ranks, and the
 // rotation tables are built and applied for served and awkward widths.
 // Each input lives in a heap block of exactly its size, so a read past the end is reported.
+#include <algorithm>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -103,6 +104,32 @@ int main(int argc, char** argv) {
   const uint64_t edges[] = {0, 1, 2, 196560, 196561, kN13 - 1, kN13, kN13 + 1, (1ULL << 47) - 1, 1ULL << 47, (1ULL << 48) - 1, ~0ULL};
   for (uint64_t e : edges) valid += host_decode(e, pt, &shell) ? 1 : 0;
   for (size_t m = 0; m < 200000; ++m) valid += host_decode(next_u64() >> 16, pt, &shell) ? 1 : 0;
+  // The table that stands for the last eight slots of the odd-coset walk, against an independent
+  // enumeration: for every multiset of four kinds over eight slots, entry r must be the r-th
+  // arrangement in lexicographic order (kind 0 first; index.rs:97-117), as codes 3 - kind, first
+  // slot in the lowest byte, and the multisets' entries must follow one another without gaps.
+  {
+    const Codebook& cb = codebook();
+    size_t entries = 0;
+    for (int t3 = 0; t3 <= 8; ++t3)
+      for (int t2 = 0; t2 <= t3; ++t2)
+        for (int t1 = 0; t1 <= t2; ++t1) {
+          const uint32_t me = cb.tail_meta[t1 + 9 * t2 + 81 * t3];
+          if ((me >> 12) != entries) { std::fprintf(stderr, "walk tail: multiset %d %d %d starts at %u, not %zu\n", t1, t2, t3, me >> 12, entries); return 6; }
+          int seq[8];
+          for (int i = 0; i < 8; ++i) seq[i] = i < t1 ? 0 : i < t2 ? 1 : i < t3 ? 2 : 3;
+          uint32_t r = 0;
+          do {
+            uint64_t want = 0;
+            for (int i = 0; i < 8; ++i) want |= (uint64_t)(3 - seq[i]) << (8 * i);
+            if (cb.tail_codes[entries + r] != want) { std::fprintf(stderr, "walk tail: multiset %d %d %d, rank %u\n", t1, t2, t3, r); return 6; }
+            ++r;
+          } while (std::next_permutation(seq, seq + 8));
+          if (r != (me & 0xFFFu)) { std::fprintf(stderr, "walk tail: multiset %d %d %d has %u arrangements, table says %u\n", t1, t2, t3, r, me & 0xFFFu); return 6; }
+          entries += r;
+        }
+    if (entries != 65536) { std::fprintf(stderr, "walk tail: %zu entries\n", entries); return 6; }
+  }
   // rotation tables of served and awkward widths (an odd factor above 32 is a refusal, not a fault)
   size_t rotations = 0;
   for (uint32_t n : {1u, 8u, 24u, 104u, 256u, 1000u, 2560u, 2568u, 4096u, 9728u, 17408u}) {

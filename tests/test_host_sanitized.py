@@ -1,6 +1,7 @@
 """The library's host code under AddressSanitizer and UBSan (host only; no GPU): the file readers on
 every prefix and on corrupted copies of a sealed file, the shared index decoder on boundaries and
-random ranks, the rotation tables on served and awkward widths.  Reader refusals are pinned case by case elsewhere; this run is about never faulting."""
+random ranks, the rotation tables on served and awkward widths, the batched launch's work sharing, and the
+table behind the last eight slots of the odd-coset walk against an independent lexicographic enumeration.  Reader refusals are pinned case by case elsewhere; this run is about never faulting."""
 import os
 import subprocess
 
