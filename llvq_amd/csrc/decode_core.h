@@ -96,6 +96,11 @@ LLVQ_HD int mad24(int a, int b, int c) {
 }
 
 LLVQ_HD double floor64(double v) { return __builtin_floor(v); }
+// x < 2^52 as a double, exactly: the integer dropped into the mantissa of 2^52, which is then
+// taken away (two instructions; the compiler's general conversion of a 64-bit integer takes four)
+LLVQ_HD double small_u64_to_double(uint64_t x) {
+  return __builtin_bit_cast(double, x | 0x4330000000000000ULL) - 4503599627370496.0;
+}
 LLVQ_HD double fma64(double a, double b, double c) { return __builtin_fma(a, b, c); }
 LLVQ_HD uint32_t bfi32(uint32_t mask, uint32_t a, uint32_t b) { return (a & mask) | (b & ~mask); }
 
@@ -142,7 +147,7 @@ LLVQ_HD uint32_t find_class(const DecodeTables& T, uint64_t i) {
 // One slot of the walk: n slots are left, the kind's code 4 - kind is returned.
 LLVQ_HD uint32_t odd_walk_slot(const DecodeTables& T, uint32_t n, double& t1, uint32_t& tg) {
   const uint32_t ti1 = (uint32_t)t1;                      // floor(t) + 1
-  const uint32_t ltg = (uint32_t)mad24(-(int)ti1, (int)kFieldOnes, (int)tg) & kFieldGuard;  // guard survives iff T_m > floor(t)
+  const uint32_t ltg = (uint32_t)mad24((int)ti1, -(int)kFieldOnes, (int)tg) & kFieldGuard;  // guard survives iff T_m > floor(t)
   const uint32_t jj = popc32(ltg);                        // 4 - kind
   const uint32_t sh = jj * 6u;
   const uint32_t lo = (tg >> sh) & 31u;
@@ -160,7 +165,7 @@ LLVQ_HD uint32_t odd_walk_slot(const DecodeTables& T, uint32_t n, double& t1, ui
 template <class OnCodes>
 LLVQ_HD void odd_walk_head(const DecodeTables& T, const FastClass& f, uint64_t li, uint32_t& ncw, double& t1, uint32_t& tg,
                            OnCodes&& on_codes) {
-  const double local = (double)li;
+  const double local = small_u64_to_double(li);
   const double g = floor64((local + 0.5) * f.inv0);
   const double r = fma64(-g, f.d1, local);
   t1 = fma64((r + 0.5) * f.inv0, 24.0, 1.0);
@@ -218,7 +223,7 @@ LLVQ_HD void even_codes(const DecodeTables& T, const FastClass& f, uint64_t li, 
   li >>= sf;
   const uint32_t r_sw = (uint32_t)li & ((1u << sw) - 1u);
   li >>= sw;
-  const double rest = (double)li;
+  const double rest = small_u64_to_double(li);
   const double q1 = floor64((rest + 0.5) * f.inv0);
   const uint32_t r_off = (uint32_t)fma64(-q1, (double)f.a_off, rest);
   const double g = floor64((q1 + 0.5) * f.d1);

@@ -756,10 +756,9 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     prefetch_tile(a, tile + gridDim.x, tid, pre0, pre1);
 
     // P2: unrank and reduce.  Chunks of 64 queued blocks are handed out through a
-    // counter: the generic chunk first (longest), then odd, then even.
+    // counter: the generic chunk first (longest), then even, then odd (the shortest last).
     const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
     const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
-    // the ticket counter hands out the generic chunk first (longest), then odd, then even chunks
     auto ticket = [&]() {
       uint32_t t = 0;
       if (lane == 0) t = atomicAdd(&ctrl[3], 1u);
@@ -791,8 +790,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       chunk = ticket();
     }
     for (; chunk < c_gen + c_odd + c_even; chunk = ticket()) {
-      if (chunk < c_gen + c_odd) {
-        const uint32_t k = (chunk - c_gen) * 64u + lane;
+      if (chunk >= c_gen + c_even) {
+        const uint32_t k = (chunk - c_gen - c_even) * 64u + lane;
         const uint32_t entry = k < n_odd ? queue[k] : kEntryGeneric;
         if (!(entry >> 31)) {  // generic blocks that found the small queue full wait for the pass below
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
@@ -813,7 +812,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
           partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * g);
         }
       } else {
-        const uint32_t k = (chunk - c_gen - c_odd) * 64u + lane;
+        const uint32_t k = (chunk - c_gen) * 64u + lane;
         if (k < n_even) {
           const uint32_t entry = queue[kTileBlocks - 1 - k];
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
