@@ -468,6 +468,12 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
   uint32_t entry[NB], ci[NB];
   uint64_t zi[NB];  // zero-based index, ~0 when the lane has no block / an origin
   bool queued_origin[NB];
+  // Every LDS read of this phase is unconditional (a lane without a block reads a valid slot and
+  // ignores it), so that the NB reads of a step go out together: a guarded read is waited for
+  // where it is issued, and the phase is a chain of dependent reads.
+  uint64_t recs[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) recs[i] = record(min(tid + (uint32_t)i * LANES, nblk - 1u));
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     const uint32_t f = tid + (uint32_t)i * LANES;
@@ -476,7 +482,7 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
     ci[i] = 0;
     queued_origin[i] = false;
     if (f < nblk) {
-      const uint64_t rec = record(f);
+      const uint64_t rec = recs[i];
       entry[i] = f | ((uint32_t)(rec & 1) << 25);
       if ((rec >> 1) == 0) {  // the origin decodes to zero whatever the gain (index.rs:335-337)
         queued_origin[i] = origin(f);
@@ -487,11 +493,14 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
     }
   }
   uint32_t kbits[NB], kmax = 0;  // kbits = 2^k: how many classes the bucket's search spans
+  uint32_t probe[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) probe[i] = T.lut[(uint32_t)(zi[i] >> kLutShift) & 2047u];
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     kbits[i] = 0;
     if (zi[i] != ~0ULL) {
-      const uint32_t e = T.lut[(uint32_t)(zi[i] >> kLutShift)];
+      const uint32_t e = probe[i];
       ci[i] = e & 511u;
       kbits[i] = 1u << ((e >> 9) & 7u);
       kmax = max(kmax, kbits[i]);
@@ -503,14 +512,19 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
 #pragma unroll
   for (uint32_t t = 1; t <= 6; ++t) kw = __any(kmax >= (1u << t)) ? (1u << t) : kw;
   for (uint32_t step = kw >> 1; step; step >>= 1) {
+    uint64_t first[NB];  // ci + step stays inside the padded table whatever the lane holds
+#pragma unroll
+    for (int i = 0; i < NB; ++i) first[i] = T.starts[ci[i] + step];
 #pragma unroll
     for (int i = 0; i < NB; ++i)
-      if (step < kbits[i] && T.starts[ci[i] + step] <= zi[i]) ci[i] += step;
+      if (step < kbits[i] && first[i] <= zi[i]) ci[i] += step;
   }
-  uint32_t path[NB], odd_rank[NB], even_rank[NB], n_o = 0, n_e = 0;
+  uint32_t path[NB], odd_rank[NB], even_rank[NB], n_o = 0, n_e = 0, meta[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) meta[i] = T.fast[ci[i]].meta;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    path[i] = zi[i] != ~0ULL ? ((T.fast[ci[i]].meta >> kMetaPathShift) & 3u) : (queued_origin[i] ? (uint32_t)kPathOdd : 3u);
+    path[i] = zi[i] != ~0ULL ? ((meta[i] >> kMetaPathShift) & 3u) : (queued_origin[i] ? (uint32_t)kPathOdd : 3u);
     entry[i] |= ci[i] << 16;
     if (path[i] == kPathGeneric) {
       entry[i] |= kEntryGeneric;
