@@ -28,8 +28,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 
-# (6997.5 KiB fetched x 2.000 + 23.8 KiB written) per gemv_tiles_kernel launch on the default workload
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = round((6997.5 * 2.000 + 23.8) * 1024)
+# (7013.5 KiB fetched x 2.000 + 23.8 KiB written) per gemv_tiles_kernel launch on the default workload
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = round((7013.5 * 2.000 + 23.8) * 1024)
 
 
 def log(*a):
