@@ -770,7 +770,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     prefetch_tile(a, tile + gridDim.x, tid, pre0, pre1);
 
     // P2: unrank and reduce.  Chunks of 64 queued blocks are handed out through a
-    // counter: the generic chunk first (longest), then even, then odd (the shortest last).
+    // counter: the generic chunk first (longest), then even and odd ones in turn.
     const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
     const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
     auto ticket = [&]() {
@@ -803,9 +803,16 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       if (lane < n_gen) generic_block(gqueue[lane]);
       chunk = ticket();
     }
+    // even and odd chunks alternate while both queues last: the even coset waits for tables in L2,
+    // the odd one issues arithmetic, and wavefronts on either kind at the same time overlap the two
+    const uint32_t c_pair = min(c_odd, c_even);
     for (; chunk < c_gen + c_odd + c_even; chunk = ticket()) {
-      if (chunk >= c_gen + c_even) {
-        const uint32_t k = (chunk - c_gen - c_even) * 64u + lane;
+      const uint32_t t = chunk - c_gen;
+      const bool paired = t < 2u * c_pair;
+      const bool is_odd = paired ? (t & 1u) != 0u : c_odd > c_even;
+      const uint32_t ordinal = paired ? t >> 1 : t - c_pair;
+      if (is_odd) {
+        const uint32_t k = ordinal * 64u + lane;
         const uint32_t entry = k < n_odd ? queue[k] : kEntryGeneric;
         if (!(entry >> 31)) {  // generic blocks that found the small queue full wait for the pass below
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
@@ -826,7 +833,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
           partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * g);
         }
       } else {
-        const uint32_t k = (chunk - c_gen) * 64u + lane;
+        const uint32_t k = ordinal * 64u + lane;
         if (k < n_even) {
           const uint32_t entry = queue[kTileBlocks - 1 - k];
           const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
