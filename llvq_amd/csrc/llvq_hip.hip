@@ -134,7 +134,15 @@ __global__ __launch_bounds__(256) void decode_blocks_kernel(GlobalTables g, cons
   __syncthreads();
   for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < nblocks;
        b += (size_t)gridDim.x * blockDim.x) {
-    const uint64_t rec = read_record(codes, 6 * b);
+    // the stream's last record is read byte by byte: the two-dword read would touch up to two
+    // bytes past a buffer the caller sized to 6 * nblocks
+    uint64_t rec;
+    if (b + 1 < nblocks) {
+      rec = read_record(codes, 6 * b);
+    } else {
+      rec = 0;
+      for (int k = 0; k < 6; ++k) rec = (rec << 8) | codes[6 * b + k];
+    }
     int8_t* out = points + b * kDim;
     const int ci = decode_index(T, rec >> 1, [&](int p, int v) { out[p] = (int8_t)v; });
     if (gains) gains[b] = (uint8_t)(rec & 1);
@@ -422,7 +430,7 @@ __device__ __forceinline__ void tile_of(const GroupArgs& a, uint32_t tile, MatAr
 // Issues the loads of a tile's code bytes (16-byte units, from the aligned
 // address at or below the tile's first byte) into two registers per lane.
 __device__ __forceinline__ void prefetch_tile(const GroupArgs& a, uint32_t tile, uint32_t tid, uint4& p0, uint4& p1) {
-  if (tile >= a.n_tiles) return;
+  if (tile >= a.n_tiles || a.nblocks == 0) return;  // rows of tail columns only have no code bytes
   MatArg M;
   uint32_t r0, rows;
   tile_of(a, tile, M, r0, rows);
@@ -758,8 +766,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     __syncthreads();
     LLVQ_STAMP(1);
 
-    // P1: classify and bin
-    classify_and_bin<kP1Blocks>(
+    // P1: classify and bin (a tile of tail-only rows has no blocks: its queues stay empty)
+    if (nblk != 0) classify_and_bin<kP1Blocks>(
         T, nblk, kTileBlocks, queue, gqueue, ctrl, [&](uint32_t f) { return read_record(raw, off + 6 * f); },
         [&](uint32_t f) {
           partial[f] = 0.f;

@@ -162,6 +162,16 @@ class FusedRuntime:
             raise ValueError(f"{proj.name} expects d_in={proj.d_in}, got {x.shape[-1]}")
         return x.to(torch.float16).contiguous()
 
+    def _out_code(self, dtype):
+        """The kernels store binary16 or f32 outputs and nothing else: any other dtype would be
+        written with the wrong element size."""
+        torch = self._torch
+        if dtype == torch.float16:
+            return _ffi.F16
+        if dtype == torch.float32:
+            return _ffi.F32
+        raise ValueError(f"outputs are torch.float16 or torch.float32, not {dtype}")
+
     def rotate(self, proj: FusedProj, x):
         """FusedRuntime::rotate (fused_cuda.rs:362): one f16 activation [.., d_in] into the
         basis the projection was quantized in, as f32 [1, d_in].  Natural-basis matrices
@@ -192,7 +202,7 @@ class FusedRuntime:
         dims = list(out_dims if out_dims is not None else xr.shape)
         dims[-1] = proj.d_out
         y = torch.empty(dims, dtype=out_dtype, device=xr.device)  # uninitialised: every row is stored
-        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        code = self._out_code(out_dtype)
         _ffi.check(_ffi.lib().llvq_hip_gemv_rotated(self.handle, proj.handle, xr.data_ptr(), y.data_ptr(), code))
         return y
 
@@ -206,7 +216,7 @@ class FusedRuntime:
         dims = list(x.shape)
         dims[-1] = proj.d_out
         y = torch.empty(dims, dtype=out_dtype, device=x.device)
-        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        code = self._out_code(out_dtype)
         _ffi.check(_ffi.lib().llvq_hip_gemv(self.handle, proj.handle, x.data_ptr(), y.data_ptr(), code))
         return y
 
@@ -226,7 +236,7 @@ class FusedRuntime:
         ys = [torch.empty(list(x.shape[:-1]) + [p.d_out], dtype=out_dtype, device=x.device) for p in projs]
         mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
         outs = (C.c_void_p * len(projs))(*[y.data_ptr() for y in ys])
-        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        code = self._out_code(out_dtype)
         fn = _ffi.lib().llvq_hip_gemv_group
         rt, n, xp = self.handle, len(projs), C.c_void_p(x.data_ptr())
         keep = (x, ys, mats, outs)
@@ -246,7 +256,7 @@ class FusedRuntime:
         x = x.to(torch.float16).contiguous()
         out_dtype = out_dtype or torch.float16
         y = torch.empty((x.shape[0], proj.d_out), dtype=out_dtype, device=x.device)
-        code = _ffi.F16 if out_dtype == torch.float16 else _ffi.F32
+        code = self._out_code(out_dtype)
         _ffi.check(_ffi.lib().llvq_hip_gemm(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
         return y
 
@@ -257,7 +267,7 @@ class FusedRuntime:
             raise ValueError(f"{proj.name} expects a contiguous f16 [M, {proj.d_in}] activation")
         if tuple(y.shape) != (x.shape[0], proj.d_out) or not y.is_contiguous():
             raise ValueError(f"{proj.name}: output must be contiguous [M, {proj.d_out}]")
-        code = _ffi.F16 if y.dtype == torch.float16 else _ffi.F32
+        code = self._out_code(y.dtype)
         _ffi.check(_ffi.lib().llvq_hip_gemm(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
         return y
 
@@ -277,7 +287,7 @@ class FusedRuntime:
                 raise ValueError(f"{p.name}: output must be contiguous [M, {p.d_out}], one dtype for the group")
         mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
         outs = (C.c_void_p * len(projs))(*[y.data_ptr() for y in ys])
-        code = _ffi.F16 if ys[0].dtype == torch.float16 else _ffi.F32
+        code = self._out_code(ys[0].dtype)
         _ffi.check(_ffi.lib().llvq_hip_gemm_group(self.handle, mats, len(projs), x.data_ptr(), x.shape[0], outs, code))
         return ys
 

@@ -240,3 +240,19 @@ int main(void) {
     want = [C.sizeof(_ffi.MatrixDesc), C.sizeof(_ffi.DecoderDesc), C.sizeof(_ffi.QuantRows), C.sizeof(_ffi.RawInfo),
             C.sizeof(_ffi.BlobInfo), _ffi.DecoderDesc.kv_mode.offset, _ffi.DecoderDesc.prefill_rows.offset]
     assert got == want
+
+
+def test_output_dtype_is_checked():
+    """Outputs are binary16 or f32; anything else (bfloat16: two bytes written as four) is refused
+    before a kernel sees the pointer."""
+    import torch
+
+    from llvq_amd import _ffi, fused
+
+    rt = fused.FusedRuntime.__new__(fused.FusedRuntime)
+    rt._torch, rt.handle, rt.projs = torch, None, []
+    assert rt._out_code(torch.float16) == _ffi.F16
+    assert rt._out_code(torch.float32) == _ffi.F32
+    for bad in (torch.bfloat16, torch.float64, torch.int8):
+        with pytest.raises(ValueError):
+            rt._out_code(bad)
