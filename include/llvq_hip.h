@@ -177,6 +177,18 @@ int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, int M, 
 int llvq_hip_gemm_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x_f16_dev, int M,
                         void* const* y_dev, int y_dtype);
 
+/* llvq_hip_gemm for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart
+ * in the reference.  Same kernels and results as llvq_hip_gemm; the partial sums, the tiled
+ * copy of the activations and (rotated matrices) the rotated rows live in one static device
+ * array of LLVQ_STATIC_SCRATCH_BYTES per GPU instead of buffers the runtime grows, and the
+ * call makes no hipMalloc / hipFree.  A shape whose workspaces do not fit is refused with
+ * LLVQ_ERR_UNSUPPORTED (the message names the bytes needed).  Every call on a GPU shares that
+ * GPU's array: calls that overlap on one GPU (two streams, two runtimes) race. */
+#define LLVQ_STATIC_SCRATCH_BYTES (64u << 20)
+int llvq_hip_gemm_static(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, int M, void* y_dev,
+                         int y_dtype);
+
 /* Parity probe (the role of decode_probe, llvq-cuda/kernels/preflight.cu:39):
  * unrank packed 6-byte records on the device.  points: 24 int8 per block;
  * gains: one byte per block; shells (may be NULL): one byte per block. */

@@ -977,6 +977,7 @@ struct llvq_rt {
   int device = 0;
   hipStream_t stream = nullptr;
   uint8_t* blob = nullptr;  // one device allocation holding every table
+  uint8_t* static_scratch = nullptr;  // this device's copy of `scratch` (kStaticScratchBytes)
   GlobalTables tables{};
   int cu_count = 0;
   // rotations by (width, seed) — shared by every matrix that consumes the same activation
@@ -1017,6 +1018,14 @@ struct llvq_mat {
 
 static thread_local std::string g_last_error;
 
+// Workspace of llvq_hip_gemm_static: device memory the library never allocates or frees.  The
+// array's name is only a host-side handle; its device address differs per GPU and is asked for
+// once per device, with that device current, at llvq_hip_runtime_create.
+constexpr size_t kStaticScratchBytes = (size_t)LLVQ_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static uint8_t* g_scratch_ptr[kMaxDevices] = {};
+
 static int fail(int code, const std::string& msg) {
   g_last_error = msg;
   return code;
@@ -1055,6 +1064,15 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   hipError_t e = hipGetDeviceProperties(&prop, device);
   if (e != hipSuccess) { delete rt; return hip_fail(e, "hipGetDeviceProperties"); }
   rt->cu_count = prop.multiProcessorCount;
+  if (device >= 0 && device < kMaxDevices) {
+    if (!g_scratch_ptr[device]) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess) { delete rt; return hip_fail(e, "hipGetSymbolAddress(scratch)"); }
+      g_scratch_ptr[device] = reinterpret_cast<uint8_t*>(p);
+    }
+    rt->static_scratch = g_scratch_ptr[device];
+  }
   // one blob: LDS image | generic class records | off-support table | deposit masks | walk-tail codes
   if (cb.on_lut.size() > (size_t)kOnLutSlots) { delete rt; return fail(LLVQ_ERR_UNSUPPORTED, "support-arrangement table outgrew its LDS slot"); }
   const size_t off_cls = sizeof(TableImage);
@@ -1592,10 +1610,32 @@ static int grow_buffer(void** buf, size_t* have, size_t need) {
 // twelve of the sixteen wavefronts unrank and four multiply (four consumers cover 256 rows).
 constexpr uint32_t kGemmNarrowRows = 256;
 
+// Where a batched call's device workspaces come from: the runtime's buffers, grown with
+// hipMalloc on first use of a larger shape, or (fixed != null) a region the caller of this
+// file's helpers provides, which is carved up and never outgrown.
+struct GemmWorkspace {
+  uint8_t* fixed = nullptr;
+  size_t fixed_bytes = 0, used = 0;
+};
+static int workspace_take(llvq_rt* rt, GemmWorkspace* w, void** runtime_buf, size_t* runtime_have, size_t need, void** out) {
+  if (!w || !w->fixed) {
+    const int rc = grow_buffer(runtime_buf, runtime_have, need);
+    *out = *runtime_buf;
+    return rc;
+  }
+  const size_t at = (w->used + 255) & ~(size_t)255;
+  if (need > w->fixed_bytes || at > w->fixed_bytes - need)
+    return fail(LLVQ_ERR_UNSUPPORTED, "gemm_static: this shape needs " + std::to_string(at + need) +
+                                          " bytes of workspace, the static one holds " + std::to_string(w->fixed_bytes));
+  *out = w->fixed + at;
+  w->used = at + need;
+  return LLVQ_OK;
+}
+
 // One launch over n <= kGemmMaxGroup matrices of equal d_in that take the same activations
 // (already in the matrices' basis), M <= kGemmMaxM rows.
 static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, uint32_t M, void* const* y,
-                       int y_dtype) {
+                       int y_dtype, GemmWorkspace* wsp = nullptr) {
   const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
   const bool f32 = y_dtype == LLVQ_F32;
   const llvq_mat* m0 = mats[0];
@@ -1627,19 +1667,23 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   a.base = share.base;
   a.rem = share.rem;
   a.max_pieces = share.max_pieces;
-  int rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes,
-                       (size_t)a.n_bands * a.max_pieces * kparts * M * kGemmRows * sizeof(float));
+  void* ws_buf = nullptr;
+  void* xt_buf = nullptr;
+  const size_t mark = wsp ? wsp->used : 0;  // a launch's carvings are released when it has been enqueued: the stream orders the next
+  int rc = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes,
+                          (size_t)a.n_bands * a.max_pieces * kparts * M * kGemmRows * sizeof(float), &ws_buf);
   if (rc) return rc;
   // every slice has all its twelve K-steps in the tiled copy, zeros past the matrix's last block
   const uint32_t n_steps = (m0->nblocks + kGemmKb - 1) / kGemmKb * (kGemmKb * 24 / 32);
   const size_t xt_bytes = (size_t)n_steps * a.m_pad * 64;
-  rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_xt), &rt->gemm_xt_bytes, xt_bytes);
+  rc = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->gemm_xt), &rt->gemm_xt_bytes, xt_bytes, &xt_buf);
   if (rc) return rc;
+  if (wsp) wsp->used = mark;
   hipLaunchKernelGGL(tile_activations_kernel, dim3((uint32_t)((xt_bytes / 16 + 255) / 256)), dim3(256), 0, rt->stream, xh, M,
-                     m0->d_in, m0->nblocks * 24u, a.m_pad, n_steps, reinterpret_cast<uint4*>(rt->gemm_xt));
+                     m0->d_in, m0->nblocks * 24u, a.m_pad, n_steps, reinterpret_cast<uint4*>(xt_buf));
   HIP_TRY(hipGetLastError());
-  a.xt = rt->gemm_xt;
-  a.ws = rt->gemm_ws;
+  a.xt = reinterpret_cast<__half*>(xt_buf);
+  a.ws = reinterpret_cast<float*>(ws_buf);
   const dim3 grid(n_wg), wg(kWgThreads);
   if (consumers == 4) hipLaunchKernelGGL(gemm_tiles_kernel<12>, grid, wg, gemm_lds_bytes(), rt->stream, a);
   else hipLaunchKernelGGL(gemm_tiles_kernel<8>, grid, wg, gemm_lds_bytes(), rt->stream, a);
@@ -1665,7 +1709,8 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
 
 // Matrices [0, n) of one group: same d_in, same basis.  The matrix-core kernel reads activations as
 // 16-byte vectors; a single row, or a shape that breaks that alignment, runs as GEMV launches instead.
-static int gemm_same_basis(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, int M, void* const* y, int y_dtype) {
+static int gemm_same_basis(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, int M, void* const* y, int y_dtype,
+                           GemmWorkspace* wsp = nullptr) {
   const llvq_mat* m0 = mats[0];
   const size_t esz = y_dtype == LLVQ_F32 ? 4 : 2;
   const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
@@ -1680,11 +1725,13 @@ static int gemm_same_basis(llvq_rt* rt, const llvq_mat* const* mats, int n, cons
   }
   if (m0->has_rotation) {
     // rows are rotated (f32 inside) and narrowed to the binary16 the matrix cores take
-    const int rc0 = grow_buffer(reinterpret_cast<void**>(&rt->rot_rows), &rt->rot_rows_bytes, (size_t)M * m0->d_in * sizeof(__half));
+    void* rows = nullptr;
+    const int rc0 = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->rot_rows), &rt->rot_rows_bytes,
+                                   (size_t)M * m0->d_in * sizeof(__half), &rows);
     if (rc0) return rc0;
-    const int rc = launch_rotate(rt, m0->rot, x, (uint32_t)M, rt->rot_rows, true);
+    const int rc = launch_rotate(rt, m0->rot, x, (uint32_t)M, rows, true);
     if (rc) return rc;
-    xb = reinterpret_cast<const uint8_t*>(rt->rot_rows);
+    xb = reinterpret_cast<const uint8_t*>(rows);
   }
   for (int m_lo = 0; m_lo < M; m_lo += kGemmMaxM) {
     const uint32_t mc = (uint32_t)(M - m_lo < kGemmMaxM ? M - m_lo : kGemmMaxM);
@@ -1692,7 +1739,7 @@ static int gemm_same_basis(llvq_rt* rt, const llvq_mat* const* mats, int n, cons
       const int cnt = n - i0 < kGemmMaxGroup ? n - i0 : kGemmMaxGroup;
       void* ys[kGemmMaxGroup];
       for (int i = 0; i < cnt; ++i) ys[i] = reinterpret_cast<uint8_t*>(y[i0 + i]) + (size_t)m_lo * mats[i0 + i]->d_out * esz;
-      const int rc = launch_gemm(rt, mats + i0, cnt, xb + (size_t)m_lo * m0->d_in * 2, mc, ys, y_dtype);
+      const int rc = launch_gemm(rt, mats + i0, cnt, xb + (size_t)m_lo * m0->d_in * 2, mc, ys, y_dtype, wsp);
       if (rc) return rc;
     }
   }
@@ -1728,6 +1775,19 @@ int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y,
   if (M == 0) return LLVQ_OK;  // no rows: nothing is read or written, so the pointers may be null
   if (!x || !y) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm: null activation or output");
   return llvq_hip_gemm_group(rt, &m, 1, x, M, &y, y_dtype);
+}
+
+int llvq_hip_gemm_static(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y, int y_dtype) {
+  if (!rt || !m || M < 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_static: bad argument");
+  if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_static: unknown output dtype");
+  if (M == 0) return LLVQ_OK;
+  if (!x || !y) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_static: null activation or output");
+  if (!rt->static_scratch) return fail(LLVQ_ERR_UNSUPPORTED, "gemm_static: no static workspace on this device");
+  HIP_TRY(hipSetDevice(rt->device));
+  GemmWorkspace w;
+  w.fixed = rt->static_scratch;
+  w.fixed_bytes = kStaticScratchBytes;
+  return gemm_same_basis(rt, &m, 1, x, M, &y, y_dtype, &w);
 }
 
 int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks, int8_t* points_dev,

@@ -271,6 +271,18 @@ class FusedRuntime:
         _ffi.check(_ffi.lib().llvq_hip_gemm(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
         return y
 
+    def forward_batched_static_into(self, proj: FusedProj, x, y):
+        """`forward_batched_into` through llvq_hip_gemm_static: the call allocates no device memory
+        (its workspaces are a static device array); shapes beyond that array raise Unsupported."""
+        torch = self._torch
+        if x.dtype != torch.float16 or not x.is_contiguous() or x.dim() != 2 or x.shape[1] != proj.d_in:
+            raise ValueError(f"{proj.name} expects a contiguous f16 [M, {proj.d_in}] activation")
+        if tuple(y.shape) != (x.shape[0], proj.d_out) or not y.is_contiguous():
+            raise ValueError(f"{proj.name}: output must be contiguous [M, {proj.d_out}]")
+        code = self._out_code(y.dtype)
+        _ffi.check(_ffi.lib().llvq_hip_gemm_static(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
+        return y
+
     def forward_batched_group_into(self, projs, x, ys):
         """Rows of `x` [M, d_in] through the projections of one group (q/k/v, gate/up) into caller-owned
         [M, d_out_i] tensors of one dtype: one batched launch per run of projections that share a basis
