@@ -2,15 +2,34 @@
 a small Qwen3-architecture model with random LLVQ projections.
 
 Bars: with the oracle's tokens fed to both (teacher forcing) the logits agree to
-a few binary16 steps at every position; free-running greedy tokens are identical
+a few binary16 steps at every position.  Each bar below is at most four times the
+largest error observed for that model (printed by the test as OBSERVED ...): a
+real regression (a wrong rounding point, a dropped tail column, a mis-scaled
+block) moves logits by 1e-2 and more.  Free-running greedy tokens are identical
 up to the first position where the oracle's own top-two logits are closer than
-the observed logit error."""
+twice that logit error plus 1e-4 (ties below 1e-4 are the only ones the
+reference's own runner comparison excuses, llvq-llm/src/bin/fusedrun.rs:263-278)."""
 import numpy as np
 import pytest
 
 from llvq_amd import artifact, decoder
 
 pytestmark = pytest.mark.gpu
+
+# max |dlogit| / max |logit| against the oracle, by model (observed -> bar)
+BAR_SMALL = 5e-4    # 1.2e-4: hidden 256, heads of 64
+BAR_RAGGED = 2e-3   # 5.3e-4: hidden 200, heads of 32, every projection with tail columns; few logits, so a binary16 step weighs more
+BAR_Q8 = 9e-4       # 1.3e-4 position by position, 2.3e-4 after a batched prompt: int8 KV cache
+
+
+def _bar(cfg):
+    return BAR_RAGGED if cfg.hidden_size == 200 else (BAR_Q8 if cfg.kv_mode == "q8" else BAR_SMALL)
+
+
+def _near_tie(trace_step, bar):
+    """Whether the oracle's own two largest logits at a step are closer than the logit error allows to resolve."""
+    l = np.sort(trace_step)[-2:]
+    return float(l[1] - l[0]) <= 2 * bar * float(np.abs(trace_step).max()) + 1e-4
 
 SMALL = decoder.Qwen3Config(num_hidden_layers=3, hidden_size=256, num_attention_heads=4, num_key_value_heads=2,
                             head_dim=64, intermediate_size=512, vocab_size=1000, rope_theta=1e6, rms_norm_eps=1e-6,
@@ -67,7 +86,8 @@ def test_teacher_forced_logits(gpu_rt, orc, cfg, seed, n):
                 agree += 1
             else:
                 assert top2[1] - top2[0] <= 2 * err + 1e-4, "argmax differs where the oracle's top two are well separated"
-        assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
+        print(f"OBSERVED teacher_forced {cfg.hidden_size}/{cfg.kv_mode}: {worst:.3e}")
+        assert worst < _bar(cfg), f"max |dlogit| / max|logit| = {worst:.3e}"
         assert agree >= len(tokens) - 2
         assert dec.position == len(tokens)
     finally:
@@ -86,7 +106,8 @@ def test_rotated_projections_in_the_loop(gpu_rt, orc):
             want = ref.forward_token(int(t))
             got, _ = dec.forward_token(int(t))
             worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
-        assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
+        print(f"OBSERVED rotated_loop: {worst:.3e}")
+        assert worst < BAR_SMALL, f"max |dlogit| / max|logit| = {worst:.3e}"
     finally:
         dec.close()
 
@@ -111,7 +132,8 @@ def test_batched_prefill_then_decode(gpu_rt, orc, cfg, seed, rotate):
             want = ref.forward_token(int(t))
             got, _ = dec.forward_token(int(t))
             worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
-        assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
+        print(f"OBSERVED batched_prefill {cfg.hidden_size}/{cfg.kv_mode}/rot={rotate}: {worst:.3e}")
+        assert worst < _bar(cfg), f"max |dlogit| / max|logit| = {worst:.3e}"
     finally:
         dec.close()
 
@@ -126,8 +148,7 @@ def test_generate_with_batched_prefill_matches_token_by_token(gpu_rt, orc):
         if not same.all():  # a flip needs a near-tie in the oracle's own logits at that step
             first = int(np.argmin(same))
             _, trace = ref.generate(prompt, first + 1)
-            l = np.sort(trace[first])[-2:]
-            assert l[1] - l[0] < 5e-2 * np.abs(trace[first]).max(), f"first divergence at step {first} without a near-tie"
+            assert _near_tie(trace[first], BAR_SMALL), f"first divergence at step {first} without a near-tie"
         with pytest.raises(Exception):
             decoder.Decoder(gpu_rt, SMALL, decoder.synthetic_projections(SMALL, 3), decoder.synthetic_weights(SMALL, 3)).prefill(prompt)
     finally:
@@ -149,7 +170,8 @@ def test_long_cache_takes_the_merge_kernel(gpu_rt, orc):
             got, _ = dec.forward_token(int(t), want_logits=i >= 1000)
             if i >= 1000:
                 worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
-        assert worst < 2e-2, f"max |dlogit| / max|logit| = {worst:.3e}"
+        print(f"OBSERVED long_cache_merge: {worst:.3e}")
+        assert worst < BAR_Q8, f"max |dlogit| / max|logit| = {worst:.3e}"
     finally:
         dec.close()
 
@@ -191,9 +213,63 @@ def test_context_of_8192_positions_int8_cache(gpu_rt):
             got += [dec.forward_token(int(t))[0] for t in more]
             assert dec.position == 8192
             worst = max(float(np.abs(g - w).max() / np.abs(w).max()) for g, w in zip(got, want))
-            assert worst < 1e-3, f"batched={batched}: max |dlogit| / max|logit| = {worst:.3e}"  # observed: 1.2e-4, a binary16 ulp
+            print(f"OBSERVED ctx8192 batched={batched}: {worst:.3e}")
+            assert worst < 5e-4, f"batched={batched}: max |dlogit| / max|logit| = {worst:.3e}"  # observed: 1.2e-4, a binary16 ulp
     finally:
         dec.close()
+
+
+def test_config4_as_stated_14b_int8_cache_8192_positions(gpu_rt):
+    """BASELINE config 4 as stated, in one run: the 40-layer model at the Qwen3-14B widths (280 LLVQ
+    matrices, 3.3 GB of codes resident), int8 KV cache, batch 1 at 8186+ cached positions — past 1024
+    positions the split attention leaves more than 16 partials per head, so the chip-wide merge kernel is
+    the path taken at every decoded position here.  The CPU oracle cannot follow at this size (hours), so
+    the checks are properties the reference states for its own cache (llvq-llm/tests/kv_cache.rs:222-262:
+    split prefill == whole prefill; llvq-llm/src/bin/run.rs:4-7: cached generation is repeatable):
+      * the cache filled by the batched path in passes of 512 rows and in passes of 384 rows gives the same
+        next-token logits to 1e-3 of the largest (different row blocks, cache tiles and partial-sum splits);
+      * six greedy tokens decoded over that cache are the same both times, and again after a reset;
+      * every logit is finite and the position ends at 8192.
+    The model's own arithmetic at these widths is pinned against the oracle at 128 positions by the
+    fixture test below, and the 8192-position attention against the oracle on a small model above."""
+    import dataclasses
+
+    cfg = dataclasses.replace(decoder.QWEN3_14B, max_positions=8192)
+    assert (cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.kv_mode) == (40, 5120, 17408, "q8")
+    n_prompt, n_new = 8186, 6
+    weights = decoder.synthetic_weights(cfg, 4)
+    projs = []
+    for layer in decoder.synthetic_projections(cfg, 4):
+        projs.append([gpu_rt.upload(m) for m in layer])
+    prompt = np.random.default_rng(4).integers(0, cfg.vocab_size, size=n_prompt)
+    runs = []
+    try:
+        for rows in (512, 384, 512):
+            dec = decoder.Decoder(gpu_rt, cfg, projs, weights, prefill_rows=rows)
+            try:
+                logits, best = dec.prefill(prompt)
+                assert dec.position == n_prompt and np.isfinite(logits).all() and best == int(np.argmax(logits))
+                toks, tok = [], best
+                for _ in range(n_new):
+                    step_logits, nxt = dec.forward_token(tok)
+                    assert np.isfinite(step_logits).all()
+                    toks.append(tok)
+                    tok = nxt
+                assert dec.position == n_prompt + n_new == 8192
+                runs.append((logits.astype(np.float64), toks))
+            finally:
+                dec.close()
+        (l512, t512), (l384, t384), (l512b, t512b) = runs
+        diff = float(np.abs(l512 - l384).max() / np.abs(l512).max())
+        print(f"OBSERVED config4 prefill 512 vs 384 rows: {diff:.3e}")
+        assert diff < 1e-3, f"passes of 512 vs 384 rows: max |dlogit| / max|logit| = {diff:.3e}"
+        assert np.array_equal(l512, l512b) and t512 == t512b, "the same run twice must give the same bits"
+        assert t512 == t384, (t512, t384)
+        assert len(set(t512)) > 1 or n_new == 1
+    finally:
+        for layer in projs:
+            for p in layer:
+                gpu_rt.free(p)
 
 
 def test_greedy_tokens_match_oracle(gpu_rt, orc):
@@ -205,9 +281,7 @@ def test_greedy_tokens_match_oracle(gpu_rt, orc):
         same = want == got
         if not same.all():
             first = int(np.argmin(same))
-            l = np.sort(trace[first])[-2:]
-            assert l[1] - l[0] < 5e-2 * np.abs(trace[first]).max(), (
-                f"first divergence at step {first}: oracle {want[first]}, device {got[first]}, top-two gap {l[1] - l[0]:.3e}")
+            assert _near_tie(trace[first], BAR_SMALL), f"first divergence at step {first}: oracle {want[first]}, device {got[first]}"
             assert first >= 8, "diverged almost at once"
         # generation is repeatable and independent of earlier state
         again = dec.generate(prompt, 40)
@@ -239,8 +313,7 @@ def test_full_width_layers_tokens_match_oracle(gpu_rt, orc):
             same = want == got
             if not same.all():  # only a near-tie of the oracle's own logits may flip a token
                 first = int(np.argmin(same))
-                l = np.sort(trace[first])[-2:]
-                assert l[1] - l[0] < 1e-2 * np.abs(trace[first]).max(), (batched, first, float(l[1] - l[0]))
+                assert _near_tie(trace[first], BAR_SMALL), (batched, first)
     finally:
         dec.close()
 

@@ -205,6 +205,36 @@ def test_gemv_config0_full_size(gpu_rt, orc):
     assert e < 1e-5
 
 
+def test_gemv_config1_full_size_groups(gpu_rt, orc):
+    """BASELINE config 1: the seven projections of one Qwen3-4B layer at full size, through the four
+    group launches a decode step makes (q/k/v, o, gate/up, down), f32 and binary16 outputs, against the
+    oracle's f64 fused product.  Bars: 1e-5 of sum|w_i x_i| for f32 outputs, 1e-3 for binary16 ones
+    (the reference's own, docs/mesures/e1v-cuda-2026-08-16.txt:95-96)."""
+    import torch
+
+    mats = synth.layer_matrices(0, seed=0)
+    assert sum(m.encoded_bytes() for m in mats) == 27_243_632
+    acts = {d: synth.make_activation(d, seed=0)[0] for d in (2560, 4096, 9728)}
+    projs = [gpu_rt.upload(m) for m in mats]
+    refs = [_oracle_matrix(orc, m).fused_product(acts[m.d_in].astype(np.float64)) for m in mats]
+    try:
+        worst = {}
+        for dtype, bar in ((torch.float32, 1e-5), (torch.float16, 1e-3)):
+            ys = []
+            for group in (projs[0:3], projs[3:4], projs[4:6], projs[6:7]):
+                ys += gpu_rt.forward_group(group, _x16(acts[group[0].d_in]), out_dtype=dtype)
+            worst[dtype] = 0.0
+            for m, y, (y_ref, a_ref) in zip(mats, ys, refs):
+                assert y.shape[-1] == m.d_out
+                e = np.abs(y.float().cpu().numpy().reshape(-1).astype(np.float64) - y_ref) / np.maximum(a_ref, 1e-30)
+                assert e.max() < bar, f"{m.name} {dtype}: max |dy|/sum|wx| = {e.max():.3e}"
+                worst[dtype] = max(worst[dtype], float(e.max()))
+        print(f"config 1 worst |dy|/sum|wx|: f32 {worst[torch.float32]:.2e}, f16 {worst[torch.float16]:.2e}")
+    finally:
+        for p in projs:
+            gpu_rt.free(p)
+
+
 def test_gemv_group_matches_single(gpu_rt, orc):
     import torch
 
