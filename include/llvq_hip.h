@@ -177,6 +177,16 @@ int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, int M, 
 int llvq_hip_gemm_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x_f16_dev, int M,
                         void* const* y_dev, int y_dtype);
 
+/* llvq_hip_gemm / llvq_hip_gemm_group keep their partial sums, a tiled copy of the activations and
+ * (rotated matrices) the rotated rows in buffers of the runtime, which they grow on first use of a
+ * larger shape — a hipFree + hipMalloc, i.e. a device-wide wait inside a call that otherwise only
+ * enqueues.  This sizes those buffers ahead of time for calls over `mats` (one group, as
+ * llvq_hip_gemm_group takes it) with up to max_rows rows; later calls within that bound allocate
+ * nothing and return without synchronising.  llvq_hip_decoder_create does the same for its
+ * projections when prefill_rows > 0.  No counterpart in the reference, whose l > 1 path is a row
+ * loop of matrix-vector launches (model.rs:521-529). */
+int llvq_hip_reserve_batched(llvq_rt* rt, const llvq_mat* const* mats, int n, int max_rows);
+
 /* llvq_hip_gemm for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart
  * in the reference.  Same kernels and results as llvq_hip_gemm; the partial sums, the tiled
@@ -268,6 +278,15 @@ int llvq_hip_decoder_prefill(llvq_decoder* dec, const uint32_t* tokens, size_t n
 /* llvq_hip_decoder_generate with the prompt taken through llvq_hip_decoder_prefill. */
 int llvq_hip_decoder_generate_prefilled(llvq_decoder* dec, const uint32_t* prompt, size_t n_prompt, size_t max_new,
                                         uint32_t* out);
+
+/* Qwen3::generate_phased (model.rs:1116-1163, behind LLVQ_TIME_PHASES=1 in bin/fusedrun): the tokens
+ * of llvq_hip_decoder_generate, with every decode step's phases timed — phase_ms[4 * t + k] for
+ * token t, k = 0 final norm + head, 1 argmax, 2 embedding of that token, 3 the layers over it (2 and
+ * 3 are zero for the last token, which is not fed back).  The prompt is not phased.  Where the
+ * reference fences the device after each phase, this records events on the stream: the phases are
+ * device time and the run is not serialised by them.  A diagnostic, not the published rate. */
+int llvq_hip_decoder_generate_phased(llvq_decoder* dec, const uint32_t* prompt, size_t n_prompt, size_t max_new,
+                                     uint32_t* out, double* phase_ms);
 
 int llvq_hip_synchronize(llvq_rt* rt);
 const char* llvq_hip_last_error(void);

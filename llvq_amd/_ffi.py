@@ -121,6 +121,8 @@ def lib():
     L.llvq_hip_matrix_rotation.argtypes = [vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint64)]
     L.llvq_hip_gemv_group.argtypes = [vp, C.POINTER(vp), C.c_int, vp, C.POINTER(vp), C.c_int]
     L.llvq_hip_gemm.argtypes = [vp, vp, vp, C.c_int, vp, C.c_int]
+    L.llvq_hip_reserve_batched.argtypes = [vp, C.POINTER(vp), C.c_int, C.c_int]
+    L.llvq_hip_decoder_generate_phased.argtypes = [vp, vp, sz, sz, vp, vp]
     L.llvq_hip_gemm_static.argtypes = [vp, vp, vp, C.c_int, vp, C.c_int]
     L.llvq_hip_gemm_group.argtypes = [vp, C.POINTER(vp), C.c_int, vp, C.c_int, C.POINTER(vp), C.c_int]
     L.llvq_hip_decode_blocks.argtypes = [vp, vp, sz, vp, vp, vp]
@@ -151,7 +153,7 @@ EXPORTS = [
     "llvq_hip_host_decode", "llvq_hip_matrix_upload", "llvq_hip_read_header", "llvq_hip_parse_matrix_record",
     "llvq_hip_matrix_from_record", "llvq_hip_parse_raw_tensor", "llvq_hip_parse_blob",
     "llvq_hip_matrix_free", "llvq_hip_matrix_info", "llvq_hip_matrix_name", "llvq_hip_gemv",
-    "llvq_hip_gemv_group", "llvq_hip_gemm", "llvq_hip_gemm_static", "llvq_hip_gemm_group", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
+    "llvq_hip_gemv_group", "llvq_hip_gemm", "llvq_hip_gemm_static", "llvq_hip_reserve_batched", "llvq_hip_decoder_generate_phased", "llvq_hip_gemm_group", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
     "llvq_hip_last_error", "llvq_hip_version",
     "llvq_hip_host_rotate", "llvq_hip_rotate", "llvq_hip_gemv_rotated", "llvq_hip_matrix_rotation",
     "llvq_hip_decoder_create", "llvq_hip_decoder_destroy", "llvq_hip_decoder_reset", "llvq_hip_decoder_position", "llvq_hip_decoder_seek",

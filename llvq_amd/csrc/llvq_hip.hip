@@ -1632,6 +1632,60 @@ static int workspace_take(llvq_rt* rt, GemmWorkspace* w, void** runtime_buf, siz
   return LLVQ_OK;
 }
 
+// Workspace bytes of one batched launch (launch_gemm) over these matrices at M rows: the partial
+// sums and the K-step-tiled copy of the activations.
+static void gemm_workspace_bytes(const llvq_rt* rt, const llvq_mat* const* mats, int n, uint32_t M, size_t* ws_bytes, size_t* xt_bytes) {
+  const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
+  const llvq_mat* m0 = mats[0];
+  uint32_t n_bands = 0;
+  for (int i = 0; i < n; ++i) n_bands += (mats[i]->d_out + kGemmRows - 1) / kGemmRows;
+  const uint32_t consumers = M <= kGemmNarrowRows ? 4u : 8u;
+  uint32_t ct_shift = 0;
+  while (((uint32_t)kGemmColTile << ct_shift) < M) ++ct_shift;
+  const uint32_t kparts = consumers >> ct_shift;
+  const uint32_t spb = (m0->nblocks + kGemmKb - 1) / kGemmKb;
+  const uint64_t total = (uint64_t)n_bands * spb;
+  const GemmShare share = gemm_share(total ? total : 1, spb ? spb : 1, grid_cap);
+  const uint32_t m_pad = (M + kGemmColTile - 1) / kGemmColTile * kGemmColTile;
+  const uint32_t n_steps = spb * (kGemmKb * 24 / 32);
+  *ws_bytes = (size_t)n_bands * share.max_pieces * kparts * M * kGemmRows * sizeof(float);
+  *xt_bytes = (size_t)n_steps * m_pad * 64;
+}
+
+// Sizes the runtime's batched-path buffers for calls over these matrices (grouped as
+// llvq_hip_gemm_group groups them) at up to max_rows activation rows, so that those calls find
+// them large enough and allocate nothing.
+static int reserve_batched(llvq_rt* rt, const llvq_mat* const* mats, int n, uint32_t max_rows) {
+  if (n <= 0 || max_rows < 2) return LLVQ_OK;
+  size_t ws = 0, xt = 0, rows = 0;
+  const uint32_t chunk = max_rows < (uint32_t)kGemmMaxM ? max_rows : (uint32_t)kGemmMaxM;
+  for (int i0 = 0; i0 < n;) {
+    int i1 = i0 + 1;
+    while (i1 < n && i1 - i0 < kGemmMaxGroup && mats[i1]->has_rotation == mats[i0]->has_rotation &&
+           (!mats[i0]->has_rotation || mats[i1]->rot == mats[i0]->rot))
+      ++i1;
+    if (mats[i0]->nblocks) {
+      // every row count up to the chunk: the partial-sum layout is not monotone in M where the consumers' split changes
+      for (uint32_t M : {chunk, (uint32_t)64, (uint32_t)128, (uint32_t)256}) {
+        if (M > chunk) continue;
+        size_t w = 0, x = 0;
+        gemm_workspace_bytes(rt, mats + i0, i1 - i0, M, &w, &x);
+        ws = w > ws ? w : ws;
+        xt = x > xt ? x : xt;
+      }
+    }
+    if (mats[i0]->has_rotation) {
+      const size_t r = (size_t)max_rows * mats[i0]->d_in * sizeof(__half);
+      rows = r > rows ? r : rows;
+    }
+    i0 = i1;
+  }
+  int rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes, ws);
+  if (!rc) rc = grow_buffer(reinterpret_cast<void**>(&rt->gemm_xt), &rt->gemm_xt_bytes, xt);
+  if (!rc) rc = grow_buffer(reinterpret_cast<void**>(&rt->rot_rows), &rt->rot_rows_bytes, rows);
+  return rc;
+}
+
 // One launch over n <= kGemmMaxGroup matrices of equal d_in that take the same activations
 // (already in the matrices' basis), M <= kGemmMaxM rows.
 static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x, uint32_t M, void* const* y,
@@ -1670,12 +1724,15 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   void* ws_buf = nullptr;
   void* xt_buf = nullptr;
   const size_t mark = wsp ? wsp->used : 0;  // a launch's carvings are released when it has been enqueued: the stream orders the next
-  int rc = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes,
-                          (size_t)a.n_bands * a.max_pieces * kparts * M * kGemmRows * sizeof(float), &ws_buf);
+  size_t ws_bytes = 0, xt_bytes = 0;
+  gemm_workspace_bytes(rt, mats, n, M, &ws_bytes, &xt_bytes);
+  if (ws_bytes != (size_t)a.n_bands * a.max_pieces * kparts * M * kGemmRows * sizeof(float))
+    return fail(LLVQ_ERR_DEVICE, "gemm: workspace sizing disagrees with the launch");
+  int rc = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes, ws_bytes, &ws_buf);
   if (rc) return rc;
   // every slice has all its twelve K-steps in the tiled copy, zeros past the matrix's last block
   const uint32_t n_steps = (m0->nblocks + kGemmKb - 1) / kGemmKb * (kGemmKb * 24 / 32);
-  const size_t xt_bytes = (size_t)n_steps * a.m_pad * 64;
+  if (xt_bytes != (size_t)n_steps * a.m_pad * 64) return fail(LLVQ_ERR_DEVICE, "gemm: activation-copy sizing disagrees with the launch");
   rc = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->gemm_xt), &rt->gemm_xt_bytes, xt_bytes, &xt_buf);
   if (rc) return rc;
   if (wsp) wsp->used = mark;
@@ -1777,6 +1834,17 @@ int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y,
   return llvq_hip_gemm_group(rt, &m, 1, x, M, &y, y_dtype);
 }
 
+int llvq_hip_reserve_batched(llvq_rt* rt, const llvq_mat* const* mats, int n, int max_rows) {
+  if (!rt || !mats || n < 0 || max_rows < 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "reserve_batched: bad argument");
+  for (int i = 0; i < n; ++i) {
+    if (!mats[i]) return fail(LLVQ_ERR_INVALID_ARGUMENT, "reserve_batched: null matrix");
+    if (mats[i]->d_in != mats[0]->d_in)
+      return fail(LLVQ_ERR_INVALID_ARGUMENT, mats[i]->name + ": projections of one group must share d_in");
+  }
+  HIP_TRY(hipSetDevice(rt->device));
+  return reserve_batched(rt, mats, n, (uint32_t)max_rows);
+}
+
 int llvq_hip_gemm_static(llvq_rt* rt, const llvq_mat* m, const void* x, int M, void* y, int y_dtype) {
   if (!rt || !m || M < 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_static: bad argument");
   if (y_dtype != LLVQ_F32 && y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "gemm_static: unknown output dtype");
@@ -1840,9 +1908,17 @@ struct llvq_decoder {
   __half *ph = nullptr, *ph_alt = nullptr, *pnormed = nullptr, *pq = nullptr, *pk = nullptr, *pv = nullptr, *pctx = nullptr, *po = nullptr;
   __half *pgate = nullptr, *pup = nullptr, *pact = nullptr, *pdown = nullptr;
   uint32_t* ptokens = nullptr;
+  // llvq_hip_decoder_generate_phased: events recorded at the phase boundaries of a step (null otherwise)
+  std::vector<hipEvent_t>* marks = nullptr;
+  size_t next_mark = 0;
 };
 
 namespace {
+
+// A phase boundary of a timed step: the next event of the decoder's list goes onto the stream.
+void phase_mark(llvq_decoder* d) {
+  if (d->marks && d->next_mark < d->marks->size()) (void)hipEventRecord((*d->marks)[d->next_mark++], d->rt->stream);
+}
 
 // The head over dec->normed and the argmax, which overwrites *dec->token (and history[slot] when recording).
 void launch_head(llvq_decoder* d, uint32_t history_slot, bool record) {
@@ -1853,8 +1929,10 @@ void launch_head(llvq_decoder* d, uint32_t history_slot, bool record) {
   else
     hipLaunchKernelGGL(lm_head_kernel, dim3(d->head_grid), dim3(kHeadThreads), d->hidden * sizeof(float), st, d->head, d->normed,
                        d->vocab, d->hidden, d->logits, d->best_val, d->best_idx);
+  phase_mark(d);
   hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(1024), 0, st, d->best_val, d->best_idx,
                      d->head_grid * (kHeadThreads / 64), d->token, record ? d->history : (uint32_t*)nullptr, history_slot);
+  phase_mark(d);
 }
 
 // Enqueues one position: embeds *dec->token, runs the layers at position dec->pos,
@@ -1863,10 +1941,12 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   llvq_rt* rt = d->rt;
   hipStream_t st = rt->stream;
   if (d->pos >= d->max_pos) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder: position " + std::to_string(d->pos) + " is past max_positions");
+  phase_mark(d);
   if (d->embed_q8)
     hipLaunchKernelGGL(embed_q8_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed_q, d->token, d->vocab, d->hidden, d->h);
   else
     hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, d->h);
+  phase_mark(d);
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
   const uint32_t T = d->pos + 1;
   // about 64 cached positions per workgroup (one batch of four per position class), at most kAttnMaxSplits ranges
@@ -1976,6 +2056,7 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     rc = project(P + 6, 1, d->up, d_out, act);
     if (rc) return rc;
   }
+  phase_mark(d);
   if (want_logits) {
     hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->down, d->fnorm, d->h, d->normed, d->hidden, d->eps);
     launch_head(d, history_slot, record);
@@ -2245,6 +2326,16 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
     d->ph = PH(p_h); d->ph_alt = PH(p_h2); d->pnormed = PH(p_nm); d->pq = PH(p_q); d->pk = PH(p_k); d->pv = PH(p_v); d->pctx = PH(p_ctx);
     d->po = PH(p_o); d->pgate = PH(p_g); d->pup = PH(p_u); d->pact = PH(p_act); d->pdown = PH(p_dn);
     d->ptokens = reinterpret_cast<uint32_t*>(d->pblob + p_tok);
+    // the batched products of a pass find their workspaces sized: no allocation (and no implicit
+    // device synchronisation) between the launches of a prompt
+    for (uint32_t L = 0; L < c->n_layers; ++L) {
+      const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
+      int rc = reserve_batched(rt, P, 3, c->prefill_rows);
+      if (!rc) rc = reserve_batched(rt, P + 3, 1, c->prefill_rows);
+      if (!rc) rc = reserve_batched(rt, P + 4, 2, c->prefill_rows);
+      if (!rc) rc = reserve_batched(rt, P + 6, 1, c->prefill_rows);
+      if (rc) { (void)hipFree(d->pblob); (void)hipFree(d->blob); delete d; return rc; }
+    }
   }
   *out = d;
   return LLVQ_OK;
@@ -2288,7 +2379,7 @@ int llvq_hip_decoder_forward_token(llvq_decoder* d, uint32_t token, float* logit
 }
 
 static int generate_impl(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out, bool batched,
-                         const char* who) {
+                         const char* who, double* phase_ms = nullptr) {
   if (!d || (n_prompt && !prompt) || (max_new && !out)) return fail(LLVQ_ERR_INVALID_ARGUMENT, std::string(who) + ": null argument");
   if (max_new == 0) return LLVQ_OK;  // model.rs:1052-1054
   if (n_prompt == 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, std::string(who) + ": empty prompt");
@@ -2298,12 +2389,31 @@ static int generate_impl(llvq_decoder* d, const uint32_t* prompt, size_t n_promp
     if (prompt[i] >= d->vocab) return fail(LLVQ_ERR_INVALID_ARGUMENT, std::string(who) + ": prompt token outside the vocabulary");
   HIP_TRY(hipSetDevice(d->rt->device));
   d->pos = 0;
+  // Phase timing: five events per timed step (start, after the embedding, after the layers, after the
+  // head, after the argmax); the step that ends the prompt is the first timed one.
+  std::vector<hipEvent_t> marks;
+  struct MarksGuard {
+    llvq_decoder* d;
+    std::vector<hipEvent_t>* m;
+    ~MarksGuard() {
+      d->marks = nullptr;
+      for (hipEvent_t e : *m) (void)hipEventDestroy(e);
+    }
+  } guard{d, &marks};
+  if (phase_ms) {
+    marks.resize(5 * max_new);
+    for (auto& e : marks) {
+      e = nullptr;
+      HIP_TRY(hipEventCreate(&e));
+    }
+  }
   if (batched) {
     const int rc = decoder_prefill(d, prompt, n_prompt, 0, true);
     if (rc) return rc;
   } else {
     for (size_t i = 0; i < n_prompt; ++i) {
       hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(1), 0, d->rt->stream, d->token, prompt[i]);
+      if (phase_ms && i + 1 == n_prompt) { d->marks = &marks; d->next_mark = 0; }
       const int rc = decoder_step(d, i + 1 == n_prompt, 0, true);
       if (rc) return rc;
     }
@@ -2314,6 +2424,23 @@ static int generate_impl(llvq_decoder* d, const uint32_t* prompt, size_t n_promp
   }
   HIP_TRY(hipMemcpyAsync(out, d->history, max_new * sizeof(uint32_t), hipMemcpyDeviceToHost, d->rt->stream));
   HIP_TRY(hipStreamSynchronize(d->rt->stream));
+  if (phase_ms) {
+    auto between = [&](size_t a, size_t b, double* ms) -> int {
+      float f = 0.f;
+      HIP_TRY(hipEventElapsedTime(&f, marks[a], marks[b]));
+      *ms = (double)f;
+      return LLVQ_OK;
+    };
+    for (size_t t = 0; t < max_new; ++t) {
+      double* row = phase_ms + 4 * t;
+      row[0] = row[1] = row[2] = row[3] = 0.0;
+      int rc = between(5 * t + 2, 5 * t + 3, &row[0]);           // final norm + head of the step that chose token t
+      if (!rc) rc = between(5 * t + 3, 5 * t + 4, &row[1]);      // argmax
+      if (!rc && t + 1 < max_new) rc = between(5 * (t + 1), 5 * (t + 1) + 1, &row[2]);      // embedding of token t
+      if (!rc && t + 1 < max_new) rc = between(5 * (t + 1) + 1, 5 * (t + 1) + 2, &row[3]);  // the layers over it
+      if (rc) return rc;
+    }
+  }
   return LLVQ_OK;
 }
 
@@ -2323,6 +2450,12 @@ int llvq_hip_decoder_generate(llvq_decoder* d, const uint32_t* prompt, size_t n_
 
 int llvq_hip_decoder_generate_prefilled(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out) {
   return generate_impl(d, prompt, n_prompt, max_new, out, true, "decoder_generate_prefilled");
+}
+
+int llvq_hip_decoder_generate_phased(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out,
+                                     double* phase_ms) {
+  if (max_new && !phase_ms) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_generate_phased: null phase array");
+  return generate_impl(d, prompt, n_prompt, max_new, out, false, "decoder_generate_phased", phase_ms);
 }
 
 int llvq_hip_decoder_prefill(llvq_decoder* d, const uint32_t* tokens, size_t n, float* logits_host, uint32_t* argmax_host) {

@@ -228,6 +228,17 @@ class Decoder:
         _ffi.check(fn(self.handle, prompt.ctypes.data, prompt.size, max_new, out.ctypes.data))
         return out
 
+    def generate_phased(self, prompt, max_new: int):
+        """Qwen3::generate_phased (model.rs:1116-1163): the tokens of `generate` and, per decoded token,
+        the device time of its phases in ms — columns head (final norm + head), rest (argmax), embed,
+        blocks (the layers); the last token's embed and blocks are zero (it is not fed back)."""
+        prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+        out = np.zeros(max_new, np.uint32)
+        phases = np.zeros((max_new, 4), np.float64)
+        _ffi.check(_ffi.lib().llvq_hip_decoder_generate_phased(self.handle, prompt.ctypes.data, prompt.size, max_new,
+                                                                out.ctypes.data, phases.ctypes.data))
+        return out, phases
+
     def close(self):
         if self.handle is not None:
             _ffi.lib().llvq_hip_decoder_destroy(self.handle)

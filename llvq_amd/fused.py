@@ -271,6 +271,12 @@ class FusedRuntime:
         _ffi.check(_ffi.lib().llvq_hip_gemm(self.handle, proj.handle, x.data_ptr(), x.shape[0], y.data_ptr(), code))
         return y
 
+    def reserve_batched(self, projs, max_rows: int):
+        """Sizes the runtime's batched-path workspaces for `forward_batched*` calls over this group with up
+        to max_rows rows, so that those calls allocate nothing and return without synchronising."""
+        mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
+        _ffi.check(_ffi.lib().llvq_hip_reserve_batched(self.handle, mats, len(projs), int(max_rows)))
+
     def forward_batched_static_into(self, proj: FusedProj, x, y):
         """`forward_batched_into` through llvq_hip_gemm_static: the call allocates no device memory
         (its workspaces are a static device array); shapes beyond that array raise Unsupported."""

@@ -256,3 +256,76 @@ def test_output_dtype_is_checked():
     for bad in (torch.bfloat16, torch.float64, torch.int8):
         with pytest.raises(ValueError):
             rt._out_code(bad)
+
+
+def _c_prototypes():
+    """name -> (return type, [argument types]) of every function include/llvq_hip.h declares, types
+    normalised to a small vocabulary shared with the Rust side."""
+    import re
+
+    text = open(os.path.join(ROOT, "include", "llvq_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    text = re.sub(r"^\s*#.*$", " ", text, flags=re.M)
+    protos = {}
+    for ret, name, args in re.findall(r"([A-Za-z_][\w \*]*?)\s*\b(llvq_hip_\w+)\s*\(([^;{}]*?)\)\s*;", text):
+        protos[name] = (_c_type(ret), [] if args.strip() in ("", "void") else [_c_type(a) for a in args.split(",")])
+    return protos
+
+
+def _c_type(decl):
+    import re
+
+    d = decl.strip()
+    d = re.sub(r"\[\d*\]\s*$", "*", d)                 # int8_t point[24] -> pointer
+    if "*" not in d or d.endswith("*"):
+        pass
+    stars = d.count("*")
+    base = d.replace("*", " ")
+    words = [w for w in base.split() if w not in ("const", "struct")]
+    # drop the parameter name, if there is one
+    known = {"void", "int", "char", "float", "double", "size_t", "uint8_t", "int8_t", "uint16_t", "uint32_t", "uint64_t",
+             "llvq_rt", "llvq_mat", "llvq_decoder", "llvq_matrix_desc", "llvq_record_info", "llvq_raw_info", "llvq_blob_info",
+             "llvq_decoder_desc"}
+    if len(words) > 1 and words[-1] not in known:
+        words = words[:-1]
+    ctype = " ".join(words)
+    table = {"int": "c_int", "char": "c_char", "float": "f32", "double": "f64", "size_t": "usize", "uint8_t": "u8", "int8_t": "i8",
+             "uint16_t": "u16", "uint32_t": "u32", "uint64_t": "u64", "void": "c_void", "llvq_rt": "LlvqRt", "llvq_mat": "LlvqMat",
+             "llvq_decoder": "LlvqDecoder", "llvq_matrix_desc": "LlvqMatrixDesc", "llvq_record_info": "LlvqRecordInfo",
+             "llvq_raw_info": "LlvqRawInfo", "llvq_blob_info": "LlvqBlobInfo", "llvq_decoder_desc": "LlvqDecoderDesc"}
+    return table[ctype] + "*" * stars if stars else ("()" if ctype == "void" else table[ctype])
+
+
+def _rust_prototypes():
+    import re
+
+    text = open(os.path.join(ROOT, "llvq-hip", "src", "lib.rs")).read()
+    block = re.search(r'extern\s+"C"\s*\{(.*?)\n\}', text, flags=re.S).group(1)
+    protos = {}
+    for name, args, ret in re.findall(r"fn\s+(llvq_hip_\w+)\s*\(([^)]*)\)\s*(?:->\s*([^;]+))?;", block):
+        types = []
+        for a in [a for a in args.split(",") if a.strip()]:
+            t = a.split(":", 1)[1].strip()
+            stars = len(re.findall(r"\*(?:const|mut)", t))
+            base = re.sub(r"\*(?:const|mut)\s*", "", t).strip()
+            types.append(base + "*" * stars)
+        r = (ret or "()").strip()
+        stars = len(re.findall(r"\*(?:const|mut)", r))
+        protos[name] = (re.sub(r"\*(?:const|mut)\s*", "", r).strip() + "*" * stars, types)
+    return protos
+
+
+def test_rust_crate_declares_the_header():
+    """llvq-hip/src/lib.rs (source only: there is no Rust toolchain to build it with here) binds every
+    function of include/llvq_hip.h with the header's argument and return types, and nothing else; the
+    ctypes mirror exports the same set."""
+    c, rust = _c_prototypes(), _rust_prototypes()
+    assert set(c) == set(rust), (sorted(set(c) - set(rust)), sorted(set(rust) - set(c)))
+    for name in sorted(c):
+        assert c[name] == rust[name], f"{name}: header {c[name]}, crate {rust[name]}"
+    assert set(_ffi.EXPORTS) == set(c), (sorted(set(c) - set(_ffi.EXPORTS)), sorted(set(_ffi.EXPORTS) - set(c)))
+    for name in c:
+        assert hasattr(_ffi.lib(), name)
+    # the crate's repr(C) mirror of the one struct a Rust caller fills in field by field
+    text = open(os.path.join(ROOT, "llvq-hip", "src", "lib.rs")).read()
+    assert "pub const STATIC_SCRATCH_BYTES: usize = 64 << 20;" in text and _ffi.STATIC_SCRATCH_BYTES == 64 << 20
