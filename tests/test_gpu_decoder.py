@@ -290,6 +290,26 @@ def test_greedy_tokens_match_oracle(gpu_rt, orc):
         dec.close()
 
 
+def test_generate_phased_gives_the_tokens_of_generate(gpu_rt, orc):
+    """Qwen3::generate_phased (model.rs:1116-1163): the phased run must yield the tokens of the plain one
+    (the reference pins the same), one sample per phase and decoded token, nothing for the prompt."""
+    dec, _ = _build(gpu_rt, orc, SMALL, 3)
+    try:
+        prompt = np.random.default_rng(3).integers(0, SMALL.vocab_size, size=12)
+        plain = dec.generate(prompt, 10)
+        toks, phases = dec.generate_phased(prompt, 10)
+        assert np.array_equal(plain, toks)
+        assert phases.shape == (10, 4) and np.isfinite(phases).all()
+        assert (phases[:, 0] > 0).all() and (phases[:, 1] > 0).all()       # head, argmax: every token
+        assert (phases[:-1, 2] > 0).all() and (phases[:-1, 3] > 0).all()   # embedding, layers: every token fed back
+        assert phases[-1, 2] == 0 and phases[-1, 3] == 0
+        assert phases[:-1, 3].min() > phases[:-1, 2].max()                  # three layers cost more than a gather
+        empty, none = dec.generate_phased(prompt, 0)
+        assert empty.size == 0 and none.shape == (0, 4)
+    finally:
+        dec.close()
+
+
 def test_full_width_layers_tokens_match_oracle(gpu_rt, orc):
     """Six layers at the Qwen3-4B widths (hidden 2560, 32/8 heads of 128, intermediate 9728, vocabulary
     151 936, untied f16 head): greedy tokens of the device loop, token by token and with the prompt through

@@ -205,3 +205,28 @@ def test_gemm_group_matches_the_oracle_and_the_single_calls(gpu_rt, orc):
     finally:
         for p in projs:
             gpu_rt.free(p)
+
+
+def test_reserved_workspaces_change_nothing(gpu_rt):
+    """llvq_hip_reserve_batched only sizes buffers: the products before and after it are identical, for
+    the group it was told about and at fewer rows than it was told."""
+    import torch
+
+    mats = [synth.make_matrix(f"model.layers.0.reserve.{i}.weight", do, 1000, seed=31 + i) for i, do in enumerate((192, 64))]
+    projs = [gpu_rt.upload(m) for m in mats]
+    try:
+        X = _x16(synth.make_activation(1000, seed=5, rows=300))
+        before = [gpu_rt.forward_batched(p, X, out_dtype=torch.float32) for p in projs]
+        gpu_rt.reserve_batched(projs, 600)
+        ys = [torch.empty((300, p.d_out), dtype=torch.float32, device="cuda") for p in projs]
+        gpu_rt.forward_batched_group_into(projs, X, ys)
+        for b, y in zip(before, ys):
+            assert torch.equal(b, y)
+        few = [gpu_rt.forward_batched(p, X[:40].contiguous(), out_dtype=torch.float32) for p in projs]
+        for b, y in zip(before, few):
+            assert torch.equal(b[:40], y) or float((b[:40] - y).abs().max()) < 1e-3 * float(b.abs().max())
+        with pytest.raises(Exception):
+            gpu_rt.reserve_batched(projs, -1)
+    finally:
+        for p in projs:
+            gpu_rt.free(p)
