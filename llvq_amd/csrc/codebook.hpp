@@ -21,10 +21,23 @@ constexpr uint64_t kFingerprint = 0x338f420f11866319ULL;  // llvq-artifact/tests
 constexpr int kMaxShell = 13;
 constexpr int kClassSlots = 384;   // 383 classes + one sentinel, a power-of-two-friendly size
 constexpr int kStartsPadded = 512; // class starts, padded with UINT64_MAX past N(13)
-constexpr int kStartsLds = 448;    // what a bounded search from class <= 382 with k <= 6 can touch
+constexpr int kStartsLds = 320;    // what a 47-bit index can reach (class <= 317) plus its upper neighbour; the rare wide search reads the padded table
+constexpr int kFastLds = 320;      // fast-path class records a 47-bit index can reach
 constexpr int kLutShift = 36;      // class-find table is keyed on the zero-based index >> 36
 constexpr int kOnLutSlots = 4352;  // LDS slots for the support-arrangement table (4322 entries used)
 constexpr int kLutSize = 4096;     // covers every zero-based index < N(13) < 2^48 (a 47-bit field uses the lower half)
+constexpr int kLut2Shift = 31;     // second-level buckets of the class-find table
+constexpr int kLut2Span = 1 << (kLutShift - kLut2Shift);  // entries of a second-level table
+constexpr int kLut2Lds = 54 * kLut2Span;  // second-level entries the lower half of the first level refers to (53 tables)
+// Class-find table entries (16 bits).  First level, keyed on the zero-based index >> kLutShift:
+//   bit 15 set: bits 0..14 = a second-level table, keyed on (index >> kLut2Shift) % kLut2Span;
+//   else a final entry.  Final entry (either level): bits 0..8 = class c0 holding the bucket's first
+//   index; bit 13 clear: the bucket meets at most one class start, so the class is c0 or c0 + 1
+//   (one comparison with starts[c0 + 1]) and bits 9..10 / 11..12 are the decoders of c0 / c0 + 1
+//   (kLutKind*); bit 13 set: the bucket meets several class starts, bits 9..11 = k with the class
+//   at most 2^k - 1 further, found by a halving search.
+constexpr uint32_t kLutRedirect = 0x8000u, kLutWide = 0x2000u;
+enum : uint32_t { kLutKindOdd = 0, kLutKindEven = 1, kLutKindEvenSecond = 2, kLutKindGeneric = 3 };
 
 struct KindCount {
   int value;
@@ -92,6 +105,7 @@ struct alignas(16) FastClass {
 static_assert(sizeof(FastClass) == 48, "FastClass must stay 48 bytes");
 
 constexpr int kMetaPathShift = 17;         // bits 17..18: which decoder a class takes
+constexpr uint32_t kMetaSecondFree = 1u << 19;  // even-coset fast path: the class has a second non-zero off-support kind
 constexpr int kMetaGolayShift = 20;        // bits 20..31: first codeword of the weight bucket
 enum : uint32_t { kPathOdd = 0, kPathEven = 1, kPathGeneric = 2 };
 constexpr int kTailSlots = 8;             // slots of the odd-coset walk that are looked up, not walked
@@ -105,10 +119,8 @@ struct Codebook {
   // device-shaped tables
   DevClass dev_classes[kClassSlots];
   uint64_t starts[kStartsPadded];         // starts[c] = offset of class c, starts[383] = N(13), then UINT64_MAX
-  // lut[key]: low 9 bits = class holding zero-based index (key << kLutShift), clamped to 382;
-  // bits 9..11 = k, where the class of any index of the bucket is at most 2^k - 1 classes further;
-  // bits 12..13 = decoder path of that class (meaningful when k = 0)
-  uint16_t lut[kLutSize];
+  uint16_t lut[kLutSize];                 // first level of the class-find table (see kLutRedirect)
+  std::vector<uint16_t> lut2;             // its second-level tables, those of the lowest keys first
   double rcp[32];                         // rcp[c] = 1/c, rcp[0] unused
   // step[(m * 25 + c) * 2 + {0,1}] = {m / c, 1 - m / c}: the odd-coset walk's per-slot
   // update t' + 1 = (t + 1 - lo) * (m / c) + (1 - m / c), m = slots left after this one

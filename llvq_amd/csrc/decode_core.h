@@ -56,8 +56,10 @@ struct DecodeTables {
   const uint32_t* golay;    // 4096 codewords, canonical order
   const DevClass* cls;      // generic-walk class records
   const FastClass* fast;    // fast-path class records
-  const uint64_t* starts;   // starts[c] = first zero-based index of class c; starts[383] = N(13)
-  const uint16_t* lut;      // lut[i >> kLutShift] = class holding zero-based index (key << kLutShift)
+  const uint64_t* starts;   // starts[c] = first zero-based index of class c; starts[383] = N(13) (a kernel's copy may end at kStartsLds)
+  const uint64_t* starts_far;  // the whole padded table, for the wide search
+  const uint16_t* lut;      // class-find table, first level (kLutRedirect in codebook.hpp)
+  const uint16_t* lut2;     // its second-level tables
   const double* rcp;        // rcp[c] = 1/c for c in 1..24
   const uint32_t* on_lut;   // even coset, support arrangements
   const uint32_t* off_lut;  // even coset, off-support arrangements
@@ -125,16 +127,23 @@ LLVQ_HD uint32_t walk_step(double& rho, uint32_t& tg, uint32_t n, const double* 
   return jj;
 }
 
-// Class of the zero-based index i < N(13): one table probe on the top bits,
-// then a halving search over at most 2^k classes (k = 0 for 96 % of uniformly
-// drawn indices, k <= 6 always).  starts[] is padded with UINT64_MAX.
-LLVQ_HD uint32_t find_class(const DecodeTables& T, uint64_t i) {
-  const uint32_t e = T.lut[(uint32_t)(i >> kLutShift)];
+// Final class-find entry of the zero-based index i < N(13): one table probe on the top bits and,
+// where that bucket meets several class starts, one on the bits below.
+LLVQ_HD uint32_t class_entry(const DecodeTables& T, uint64_t i) {
+  uint32_t e = T.lut[(uint32_t)(i >> kLutShift)];
+  if (e & kLutRedirect) e = T.lut2[(e & 0x7FFFu) * (uint32_t)kLut2Span + ((uint32_t)(i >> kLut2Shift) & (uint32_t)(kLut2Span - 1))];
+  return e;
+}
+// The class from its entry: one comparison, or (0.09 % of uniformly drawn indices) a halving
+// search over at most 2^k classes.  starts_far is padded with UINT64_MAX.
+LLVQ_HD uint32_t class_from_entry(const DecodeTables& T, uint32_t e, uint64_t i) {
   uint32_t ci = e & 511u;
+  if (!(e & kLutWide)) return ci + (T.starts_far[ci + 1u] <= i ? 1u : 0u);
   for (uint32_t step = (1u << ((e >> 9) & 7u)) >> 1; step; step >>= 1)
-    if (T.starts[ci + step] <= i) ci += step;
+    if (T.starts_far[ci + step] <= i) ci += step;
   return ci;
 }
+LLVQ_HD uint32_t find_class(const DecodeTables& T, uint64_t i) { return class_from_entry(T, class_entry(T, i), i); }
 
 // ---- odd coset, fast path (at most four magnitudes) ------------------------------
 // local = g * m_arr + r_arr (index.rs:33-36).  Calls on_codes(q, sel) for q = 0..5:
@@ -214,7 +223,9 @@ LLVQ_HD uint32_t expand24(uint32_t x, const uint32_t* e) {
 // Calls on_codes(q, sel, sel2) for q = 0..5: byte j of sel is
 // on-support | primary-kind << 1 | minus << 2 of coordinate 4q + j (FastClass::tab);
 // byte j of sel2 is second-free-kind | minus << 2.
-template <class OnCodes>
+// SEC = false is for classes without a second free kind (FastClass::meta & kMetaSecondFree clear): their
+// off-support table entries have an empty high half, and sel2 is passed as zero.
+template <bool SEC = true, class OnCodes>
 LLVQ_HD void even_codes(const DecodeTables& T, const FastClass& f, uint64_t li, OnCodes&& on_codes) {
   const uint32_t p_req = (f.meta >> kMetaPreqShift) & 1u;
   const uint32_t sf = (f.meta >> kMetaSfShift) & 31u;
@@ -238,7 +249,7 @@ LLVQ_HD void even_codes(const DecodeTables& T, const FastClass& f, uint64_t li, 
   // the parity rule (index.rs:375-388)
   const uint32_t signs_on = r_sw | (((popc32(r_sw) & 1u) ^ p_req) << sw);
   // free signs go to the nonzero off-support slots in slot order (index.rs:403-415)
-  const uint32_t nz = (off_e | (off_e >> 16)) & 0xFFFFu;
+  const uint32_t nz = SEC ? (off_e | (off_e >> 16)) & 0xFFFFu : off_e & 0xFFFFu;
   uint32_t signs_off = 0, r = r_sf;
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
@@ -247,14 +258,14 @@ LLVQ_HD void even_codes(const DecodeTables& T, const FastClass& f, uint64_t li, 
     r >>= popc32(m4);
   }
   const uint32_t prim = bfi32(cw, expand24(on_e & 0xFFFFu, e_on), expand24(off_e & 0xFFFFu, e_off));
-  const uint32_t sec = expand24(off_e >> 16, e_off) & ~cw;
+  const uint32_t sec = SEC ? expand24(off_e >> 16, e_off) & ~cw : 0u;
   const uint32_t sign = bfi32(cw, expand24(signs_on, e_on), expand24(signs_off, e_off));
 #pragma unroll
   for (int q = 0; q < 6; ++q) {
     const uint32_t s2 = (((sign >> (4 * q)) & 15u) * kSpread2) & 0x04040404u;
     const uint32_t sel = ((((cw >> (4 * q)) & 15u) * kSpread0) & 0x01010101u) |
                          ((((prim >> (4 * q)) & 15u) * kSpread1) & 0x02020202u) | s2;
-    const uint32_t sel2 = ((((sec >> (4 * q)) & 15u) * kSpread0) & 0x01010101u) | s2;
+    const uint32_t sel2 = SEC ? ((((sec >> (4 * q)) & 15u) * kSpread0) & 0x01010101u) | s2 : 0u;
     on_codes(q, sel, sel2);
   }
 }
@@ -340,13 +351,16 @@ LLVQ_HD int decode_index(const DecodeTables& T, uint64_t idx, Emit&& emit) {
     });
   } else if (path == kPathEven) {
     const int fv1 = (int)(f.u0 >> 16);
-    even_codes(T, f, li, [&](int q, uint32_t sel, uint32_t sel2) {
+    auto on_codes = [&](int q, uint32_t sel, uint32_t sel2) {
       for (int j = 0; j < 4; ++j) {
         const uint32_t c2 = (sel2 >> (8 * j)) & 7u;
         const int second = (c2 & 1u) ? ((c2 & 4u) ? -fv1 : fv1) : 0;
         emit(4 * q + j, table_byte(f.tab_lo, f.tab_hi, (sel >> (8 * j)) & 7u) + second);
       }
-    });
+    };
+    // the two instantiations the GEMV kernel bins even-coset blocks into
+    if (f.meta & kMetaSecondFree) even_codes<true>(T, f, li, on_codes);
+    else even_codes<false>(T, f, li, on_codes);
   } else {
     const DevClass c = T.cls[ci];
     if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);

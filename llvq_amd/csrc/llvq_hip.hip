@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 #include <type_traits>
 
+#include <algorithm>
 #include <cstdio>
 #include <cmath>
 #include <cstring>
@@ -37,13 +38,14 @@ namespace llvq {
 #define LLVQ_LDS_GOLAY 1   // 1: Golay words and the support-arrangement table live in LDS; 0: read through L2
 #endif
 struct TableImage {
-  FastClass fast[kClassSlots];
+  FastClass fast[kFastLds];
   uint64_t starts[kStartsLds];
   double rcp[32];
   double step[(24 - kTailSlots) * 25 * 2];  // rows m >= kTailSlots: the walk's last slots are looked up
   uint8_t pdep4[256];
   uint32_t tail_meta[kTailMetaSlots];
   uint16_t lut[2048];        // a 47-bit field only reaches the lower half of the host table
+  uint16_t lut2[kLut2Lds];   // the second-level tables that half refers to
   uint32_t golay[4096];
   uint32_t on_lut[kOnLutSlots];
 };
@@ -53,6 +55,7 @@ static_assert(kLdsImageBytes % 16 == 0, "LDS part of the table image is copied i
 
 struct GlobalTables {
   const TableImage* image;
+  const uint64_t* starts;  // the padded table of class starts (kStartsPadded)
   const DevClass* cls;
   const uint32_t* off_lut;
   const uint32_t* expand;
@@ -89,7 +92,7 @@ __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const Global
   }
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
   const TableImage* far = kFull ? s : g.image;
-  return DecodeTables{far->golay, g.cls, s->fast, s->starts, kLut ? s->lut : g.image->lut, s->rcp, far->on_lut, g.off_lut,
+  return DecodeTables{far->golay, g.cls, s->fast, s->starts, g.starts, kLut ? s->lut : g.image->lut, kLut ? s->lut2 : g.image->lut2, s->rcp, far->on_lut, g.off_lut,
                       g.expand, s->pdep4, s->step - kTailSlots * 25 * 2, s->tail_meta, g.tail_codes};
 }
 
@@ -122,6 +125,18 @@ __device__ __forceinline__ float wave_sum(float v) {
   v = row16_sum(v);
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16)) +
          __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+}
+
+// Inclusive prefix sum over the wavefront's lanes: four shifts inside each row of 16 lanes, then the
+// rows' totals are handed on (row 0 to row 1 and row 2 to row 3, then rows 0-1 to rows 2-3).
+__device__ __forceinline__ uint32_t wave_prefix_sum(uint32_t v) {
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xF, 0xF, true);  // row_shr:1
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xF, 0xF, true);  // row_shr:2
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xF, 0xF, true);  // row_shr:4
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xF, 0xF, true);  // row_shr:8
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xA, 0xF, true);  // row_bcast:15 into rows 1 and 3
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xC, 0xF, true);  // row_bcast:31 into rows 2 and 3
+  return v;
 }
 
 // ---- parity probe: unrank records to points -----------------------------------
@@ -328,10 +343,15 @@ __device__ __forceinline__ void rotate_lds(float* v, uint32_t n, uint32_t m, uin
 }
 
 constexpr int kSmallTileBlocks = 2048;  // tile of the variant for rows too wide for the full tile's LDS
+constexpr int kSecSlots = 384;          // queue of even-coset blocks whose class has a second free kind (7.6 % of uniform draws)
+// Per queue slot an 8-byte entry and its 2-byte block number, per tile slot a partial sum; the 32
+// bytes between them keep the area at least as large as a derived activation's staging needs it
+// (see prologue_fits / rotation_fits).
+__host__ __device__ constexpr size_t gemv_stage_bytes(uint32_t tile) { return ((size_t)tile + kSecSlots) * 10 + 32 + (size_t)tile * 4; }
 __host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks, uint32_t tile = kTileBlocks,
                                                     size_t image_bytes = kLdsImageBytes) {
-  return image_bytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + ((size_t)tile * 6 + 32) +
-         (size_t)tile * 4 * 2 + kGenericSlots * 4 + 16;
+  return image_bytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + gemv_stage_bytes(tile) +
+         2 * (size_t)kGenericSlots * 10 + 32;
 }
 
 template <typename OutT>
@@ -427,21 +447,55 @@ __device__ __forceinline__ void tile_of(const GroupArgs& a, uint32_t tile, MatAr
   rows = min(a.rows_per_tile, M.d_out - r0);
 }
 
-// Issues the loads of a tile's code bytes (16-byte units, from the aligned
-// address at or below the tile's first byte) into two registers per lane.
-__device__ __forceinline__ void prefetch_tile(const GroupArgs& a, uint32_t tile, uint32_t tid, uint4& p0, uint4& p1) {
+// A lane's share of a tile's code bytes: NB consecutive 6-byte records, 3 NB / 2 dwords, from the
+// byte the first of them starts at.  A tile starts on a row boundary, i.e. at an even byte (a
+// multiple of four whenever rows-per-tile x blocks-per-row is even), so these are vector loads at
+// two- or four-byte alignment; consecutive lanes read consecutive memory.  Unconditional: a lane
+// past the tile's end reads the tile's first records again and ignores them — a guarded load is
+// merged with the register's old value at once, and that merge waits for the load.
+template <int NB>
+struct LaneRecords {
+  static_assert(NB == 2 || NB == 4, "a lane takes two or four records");
+  uint32_t w[NB * 3 / 2];
+};
+typedef uint32_t dwords4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t dwords3_a2 __attribute__((ext_vector_type(3), aligned(2)));
+typedef uint32_t dwords2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+template <int NB>
+__device__ __forceinline__ void prefetch_records(const GroupArgs& a, uint32_t tile, uint32_t tid, LaneRecords<NB>& r) {
   if (tile >= a.n_tiles || a.nblocks == 0) return;  // rows of tail columns only have no code bytes
   MatArg M;
   uint32_t r0, rows;
   tile_of(a, tile, M, r0, rows);
-  const size_t byte0 = (size_t)r0 * a.nblocks * 6;
-  const uint32_t off = (uint32_t)(byte0 & 15);
-  const uint4* src = reinterpret_cast<const uint4*>(M.codes + (byte0 - off));
-  const uint32_t n16 = (off + rows * a.nblocks * 6 + 15) >> 4;
-  // unconditional (a lane past the tile's end re-reads its last unit, which is never stored): a
-  // guarded load is merged with the old value right away, and that merge waits for the load
-  p0 = src[min(tid, n16 - 1u)];
-  p1 = src[min(tid + kWgThreads, n16 - 1u)];
+  // a lane whose records all lie past the tile's end re-reads the tile's first ones: every byte read lies
+  // inside the tile or within 6 NB bytes behind it, which the 64 bytes of slack behind a matrix's last
+  // record cover
+  const uint32_t share = (uint32_t)NB * 6u;
+  const uint32_t at = tid * (uint32_t)NB < rows * a.nblocks ? tid * share : 0u;
+  const uint8_t* src = M.codes + (size_t)r0 * a.nblocks * 6 + at;
+  if constexpr (NB == 4) {
+    const dwords4_a2 lo = *reinterpret_cast<const dwords4_a2*>(src);
+    const dwords2_a2 hi = *reinterpret_cast<const dwords2_a2*>(src + 16);
+    r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w; r.w[4] = hi.x; r.w[5] = hi.y;
+  } else {
+    const dwords3_a2 v = *reinterpret_cast<const dwords3_a2*>(src);
+    r.w[0] = v.x; r.w[1] = v.y; r.w[2] = v.z;
+  }
+}
+
+// Record j of a lane's share as the 48-bit big-endian number it is: one byte permute for its
+// low 32 bits, one for its high 16.
+template <int NB>
+__device__ __forceinline__ void lane_record(const LaneRecords<NB>& r, int j, uint32_t& lo32, uint32_t& hi16) {
+  const int d = 3 * (j / 2) + (j & 1);
+  const uint32_t a = r.w[d], b = r.w[d + 1];  // the record's bytes lie in these two dwords
+  if (j & 1) {  // starts at byte 2 of a
+    lo32 = __builtin_amdgcn_perm(b, a, 0x04050607u);
+    hi16 = __builtin_amdgcn_perm(b, a, 0x0c0c0203u);
+  } else {      // starts at byte 0 of a
+    lo32 = __builtin_amdgcn_perm(b, a, 0x02030405u);
+    hi16 = __builtin_amdgcn_perm(b, a, 0x0c0c0001u);
+  }
 }
 
 // Phase timestamps for tuning builds (-DLLVQ_PHASE_TIMING): wave 0 of each
@@ -455,6 +509,54 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 #else
 #define LLVQ_STAMP(k) do {} while (0)
 #endif
+
+// Classes of NB zero-based indices (< 2^47) side by side: the class, its first index and its decoder
+// (kLutKind*).  Two table probes and one comparison each, every read unconditional so that the NB
+// reads of a step go out together; the indices whose bucket meets several class starts (0.09 % of
+// uniform draws) take the halving search afterwards, under a wavefront-wide test.
+template <int NB>
+__device__ __forceinline__ void find_classes(const DecodeTables& T, const uint32_t (&zlo)[NB], const uint32_t (&zhi)[NB],
+                                             uint32_t (&ci)[NB], uint64_t (&start)[NB], uint32_t (&kind)[NB]) {
+  uint32_t e[NB], e2[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) e[i] = T.lut[(zhi[i] >> (kLutShift - 32)) & 2047u];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const uint32_t sub = __builtin_amdgcn_alignbit(zhi[i], zlo[i], kLut2Shift) & (uint32_t)(kLut2Span - 1);
+    const uint32_t at = (e[i] & 0x7FFFu) * (uint32_t)kLut2Span + sub;
+    e2[i] = T.lut2[(e[i] & kLutRedirect) ? at : 0u];
+  }
+  uint64_t s0[NB], s1[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    e[i] = (e[i] & kLutRedirect) ? e2[i] : e[i];
+    s0[i] = T.starts[e[i] & 511u];
+    s1[i] = T.starts[(e[i] & 511u) + 1u];
+  }
+  uint32_t wide = 0;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const uint64_t z = ((uint64_t)zhi[i] << 32) | zlo[i];
+    const bool up = s1[i] <= z;
+    ci[i] = (e[i] & 511u) + (up ? 1u : 0u);
+    start[i] = up ? s1[i] : s0[i];
+    kind[i] = (e[i] >> (up ? 11 : 9)) & 3u;
+    wide |= e[i] & kLutWide;
+  }
+  if (__any(wide != 0u)) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+      if (e[i] & kLutWide) {
+        const uint32_t c = class_from_entry(T, e[i], ((uint64_t)zhi[i] << 32) | zlo[i]);
+        const uint32_t meta = T.fast[c].meta, path = (meta >> kMetaPathShift) & 3u;
+        ci[i] = c;
+        start[i] = T.starts_far[c];
+        kind[i] = path == kPathOdd ? (uint32_t)kLutKindOdd
+                                   : path == kPathEven ? ((meta & kMetaSecondFree) ? (uint32_t)kLutKindEvenSecond : (uint32_t)kLutKindEven)
+                                                       : (uint32_t)kLutKindGeneric;
+      }
+  }
+}
 
 // P1 of the GEMV and GEMM kernels: each of the LANES lanes taking part (the first
 // LANES of the workgroup) classifies up to NB blocks of the tile and bins them: slots first, first + LANES, ...
@@ -500,39 +602,19 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
       }
     }
   }
-  uint32_t kbits[NB], kmax = 0;  // kbits = 2^k: how many classes the bucket's search spans
-  uint32_t probe[NB];
+  uint32_t zlo[NB], zhi[NB], kind[NB];
+  uint64_t start[NB];
 #pragma unroll
-  for (int i = 0; i < NB; ++i) probe[i] = T.lut[(uint32_t)(zi[i] >> kLutShift) & 2047u];
+  for (int i = 0; i < NB; ++i) {  // a lane without a block, or with an origin, walks the tables with index 0
+    zlo[i] = zi[i] != ~0ULL ? (uint32_t)zi[i] : 0u;
+    zhi[i] = zi[i] != ~0ULL ? (uint32_t)(zi[i] >> 32) : 0u;
+  }
+  find_classes<NB>(T, zlo, zhi, ci, start, kind);
+  uint32_t path[NB], odd_rank[NB], even_rank[NB], n_o = 0, n_e = 0;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    kbits[i] = 0;
-    if (zi[i] != ~0ULL) {
-      const uint32_t e = probe[i];
-      ci[i] = e & 511u;
-      kbits[i] = 1u << ((e >> 9) & 7u);
-      kmax = max(kmax, kbits[i]);
-    }
-  }
-  // the wavefront runs as many halving steps as its widest bucket needs; a
-  // lane only reads the table on the steps its own bucket needs
-  uint32_t kw = 1;
-#pragma unroll
-  for (uint32_t t = 1; t <= 6; ++t) kw = __any(kmax >= (1u << t)) ? (1u << t) : kw;
-  for (uint32_t step = kw >> 1; step; step >>= 1) {
-    uint64_t first[NB];  // ci + step stays inside the padded table whatever the lane holds
-#pragma unroll
-    for (int i = 0; i < NB; ++i) first[i] = T.starts[ci[i] + step];
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-      if (step < kbits[i] && first[i] <= zi[i]) ci[i] += step;
-  }
-  uint32_t path[NB], odd_rank[NB], even_rank[NB], n_o = 0, n_e = 0, meta[NB];
-#pragma unroll
-  for (int i = 0; i < NB; ++i) meta[i] = T.fast[ci[i]].meta;
-#pragma unroll
-  for (int i = 0; i < NB; ++i) {
-    path[i] = zi[i] != ~0ULL ? ((meta[i] >> kMetaPathShift) & 3u) : (queued_origin[i] ? (uint32_t)kPathOdd : 3u);
+    const uint32_t decoder = kind[i] == kLutKindOdd ? (uint32_t)kPathOdd : kind[i] == kLutKindGeneric ? (uint32_t)kPathGeneric : (uint32_t)kPathEven;
+    path[i] = zi[i] != ~0ULL ? decoder : (queued_origin[i] ? (uint32_t)kPathOdd : 3u);
     entry[i] |= ci[i] << 16;
     if (path[i] == kPathGeneric) {
       entry[i] |= kEntryGeneric;
@@ -562,6 +644,127 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
   }
 }
 
+// ---- P1 of the GEMV kernel --------------------------------------------------------------
+// Each lane classifies the NB consecutive records it loaded itself and queues them with
+// everything P2 needs, so that the record is parsed once:
+//   qa[slot] = { local rank, bits 0..31;  local rank, bits 32..44 | class << 13 | gain << 22 | flags }
+//   qf[slot] = the block's number in the tile (row * blocks per row + column)
+// (the largest class holds fewer than 2^45 indices).  Three queues — the odd coset from the bottom
+// of qa / qf, the even coset from their top, and even-coset classes with a second free kind in a
+// small queue of their own (what does not fit there rides in the even queue, flagged) — because the
+// three are different straight-line programs.  Blocks of the rare generic classes go to two small
+// queues, by coset; what does not fit rides in the odd queue, flagged.
+constexpr uint32_t kQaClassShift = 13, kQaGainShift = 22;
+constexpr uint32_t kQaSecond = 0x40000000u, kQaGeneric = 0x80000000u;
+enum : uint32_t { kCtrlOdd = 0, kCtrlEven = 1, kCtrlGenOdd = 2, kCtrlTicket = 3, kCtrlSec = 4, kCtrlGenEven = 5, kCtrlWords = 8 };
+
+struct GemvQueues {
+  uint2* qa;        // [tile + kSecSlots]: the odd queue from 0 up, the even queue from tile - 1 down, the small even queue from tile up
+  uint16_t* qf;     // [tile + kSecSlots]
+  uint2* gqa;       // [2][kGenericSlots]: odd-coset generic blocks, then even-coset ones
+  uint16_t* gqf;
+  uint32_t* ctrl;   // [kCtrlWords]
+  float* partial;   // [tile]
+};
+
+template <int NB>
+__device__ __forceinline__ void classify_stream(const DecodeTables& T, const LaneRecords<NB>& rec, uint32_t nblk, uint32_t capacity,
+                                                const GemvQueues& Q) {
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  // Every LDS read below is unconditional, from a valid slot, so that the NB reads of a step go
+  // out together (a guarded read is waited for where it is issued).  A lane past the tile's end
+  // walks the tables with whatever bytes follow the tile and queues nothing.
+  uint32_t zlo[NB], zhi[NB], gain[NB], ci[NB], kind[NB];
+  uint64_t start[NB];
+  bool live[NB];  // a block of the tile that is not the origin (which decodes to zero whatever the gain, index.rs:335-337)
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const uint32_t f = tid * NB + (uint32_t)i;
+    uint32_t lo32, hi16;
+    lane_record(rec, i, lo32, hi16);
+    gain[i] = lo32 & 1u;
+    const uint32_t ilo = __builtin_amdgcn_alignbit(hi16, lo32, 1), ihi = hi16 >> 1;  // the 47-bit index
+    const bool origin = (ilo | ihi) == 0u;
+    live[i] = f < nblk && !origin;
+    if (f < nblk && origin) Q.partial[f] = 0.f;
+    const uint64_t z = (((uint64_t)ihi << 32) | ilo) - 1u;  // zero-based
+    zlo[i] = (uint32_t)z;
+    zhi[i] = (uint32_t)(z >> 32) & 0x7FFFu;  // an origin wraps to all ones: keep it a 47-bit index
+  }
+  find_classes<NB>(T, zlo, zhi, ci, start, kind);
+  // Which queue a block joins: 0 odd, 1 even, 2 the small even queue, 3 none.  A generic block rides in
+  // the odd queue, flagged, unless its coset's small queue has room (rare: settled under a wavefront-wide test).
+  uint32_t kq[NB], e0[NB], e1[NB];
+  uint32_t any_generic = 0;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const uint64_t li = (((uint64_t)zhi[i] << 32) | zlo[i]) - start[i];
+    const uint32_t generic = kind[i] == kLutKindGeneric ? 1u : 0u;
+    e0[i] = (uint32_t)li;
+    e1[i] = (uint32_t)(li >> 32) | (ci[i] << kQaClassShift) | (gain[i] << kQaGainShift) | (generic << 31);
+    kq[i] = live[i] ? (generic ? 0u : kind[i]) : 3u;
+    any_generic |= live[i] ? generic : 0u;
+  }
+  if (__any(any_generic != 0u)) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+      if (kq[i] == 0u && (e1[i] >> 31)) {
+        const uint32_t even = (T.fast[ci[i]].meta & kMetaOdd) ? 0u : 1u;
+        const uint32_t slot = atomicAdd(&Q.ctrl[even ? kCtrlGenEven : kCtrlGenOdd], 1u);
+        if (slot < (uint32_t)kGenericSlots) {
+          Q.gqa[even * kGenericSlots + slot] = make_uint2(e0[i], e1[i]);
+          Q.gqf[even * kGenericSlots + slot] = (uint16_t)(tid * NB + (uint32_t)i);
+          kq[i] = 3u;  // placed
+        }
+      }
+  }
+  // A block's rank in its queue among the wavefront's blocks.  Three 10-bit counters packed in a
+  // dword (a wavefront classifies at most 256 blocks): a lane's own blocks in order, behind the
+  // blocks of the lanes below it — one prefix sum over the wavefront by lane shifts.
+  uint32_t sh[NB], running[NB], total = 0;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    sh[i] = kq[i] * 10u;
+    running[i] = total;
+    total += kq[i] < 3u ? 1u << sh[i] : 0u;
+  }
+  const uint32_t through = wave_prefix_sum(total);  // this lane's blocks included
+  const uint32_t below = through - total;
+  const uint32_t all = (uint32_t)__builtin_amdgcn_readlane((int)through, 63);
+  const uint32_t n_o = all & 1023u, n_e = (all >> 10) & 1023u, n_s = (all >> 20) & 1023u;
+  uint32_t base_o = 0, base_e = 0, base_s = 0;
+  if (lane == 0) {
+    base_o = atomicAdd(&Q.ctrl[kCtrlOdd], n_o);
+    base_s = atomicAdd(&Q.ctrl[kCtrlSec], n_s);
+    // what the small queue cannot take rides in the even queue behind this wavefront's own entries
+    const uint32_t spill = base_s + n_s > (uint32_t)kSecSlots ? base_s + n_s - max(base_s, (uint32_t)kSecSlots) : 0u;
+    base_e = atomicAdd(&Q.ctrl[kCtrlEven], n_e + spill);
+  }
+  base_o = __builtin_amdgcn_readfirstlane(base_o);
+  base_e = __builtin_amdgcn_readfirstlane(base_e);
+  base_s = __builtin_amdgcn_readfirstlane(base_s);
+  // odd from the bottom, even from the top, the small queue behind both
+  const uint32_t top = capacity - 1u - base_e, small = capacity + base_s;
+  const bool spills = base_s + n_s > (uint32_t)kSecSlots;  // wavefront-uniform, rare
+  const uint32_t fits = base_s >= (uint32_t)kSecSlots ? 0u : (uint32_t)kSecSlots - base_s;  // small-queue ranks below this fit
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const uint32_t rank = ((below + running[i]) >> sh[i]) & 1023u;
+    const uint32_t up = base_o + rank, down = top - rank, behind = small + rank;
+    uint32_t pos = kq[i] == 1u ? down : up;
+    pos = kq[i] == 2u ? behind : pos;
+    if (spills) {
+      const bool out = kq[i] == 2u && rank >= fits;
+      pos = out ? top - (n_e + (rank - fits)) : pos;
+      e1[i] |= out ? kQaSecond : 0u;
+    }
+    if (kq[i] != 3u) {
+      Q.qa[pos] = make_uint2(e0[i], e1[i]);
+      Q.qf[pos] = (uint16_t)(tid * NB + (uint32_t)i);
+    }
+  }
+}
+
 // LEAN: the Golay words and the support-arrangement table stay in L2, which leaves
 // room for the full tile beside the activation planes of a very wide row.
 // ROT: the launch can rotate its own activation (GroupArgs::rot_m); kept out of the other
@@ -571,26 +774,37 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   // the tile capacity of this instantiation (these shadow the namespace-level defaults)
   constexpr int kTileBlocks = TILE;
   constexpr int kP1Blocks = TILE / kWgThreads;
-  constexpr int kRawBytes = TILE * 6 + 32;
+  constexpr int kRawBytes = TILE * 6 + 32;  // what a derived binary16 activation may take of the staging area
   extern __shared__ __align__(16) uint8_t smem[];
+#ifdef LLVQ_PHASE_TIMING
+  if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 3] = wall_clock64();
+#endif
   const DecodeTables T = stage_tables<!LEAN && (LLVQ_LDS_GOLAY != 0)>(smem, a.tables);
-  // The code bytes of a tile travel HBM -> registers -> LDS; the next tile's loads are issued
-  // while the current one is being decoded.  The first tile's are issued right behind the
+  // A lane loads the records it classifies itself, HBM -> registers; the next tile's loads are
+  // issued while the current one is being decoded.  The first tile's are issued right behind the
   // loads of the activation: the memory counter retires in order, so whatever is requested
   // after them would wait for HBM with them, and they are not needed before the activation is.
-  uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0;
-  auto request_first_tile = [&]() { prefetch_tile(a, blockIdx.x, threadIdx.x, pre0, pre1); };
+  LaneRecords<kP1Blocks> pre;
+#pragma unroll
+  for (int k = 0; k < kP1Blocks * 3 / 2; ++k) pre.w[k] = 0;
+  auto request_first_tile = [&]() { prefetch_records(a, blockIdx.x, threadIdx.x, pre); };
   const uint32_t nb = a.nblocks;
   uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + (LEAN ? kLdsImageBytesLean : kLdsImageBytes));
   float* xscale = reinterpret_cast<float*>(xplanes + (size_t)nb * kPlaneDwords);
   float* xtail = xscale + nb;
+  // queue entries | block numbers | 32 bytes | partial sums: also the staging area of a derived or rotated activation
   uint8_t* raw = reinterpret_cast<uint8_t*>(xtail + 32);
-  uint32_t* queue = reinterpret_cast<uint32_t*>(raw + kRawBytes);
-  float* partial = reinterpret_cast<float*>(queue + kTileBlocks);
-  uint32_t* gqueue = reinterpret_cast<uint32_t*>(partial + kTileBlocks);
-  uint32_t* ctrl = gqueue + kGenericSlots;
+  GemvQueues Q;
+  Q.qa = reinterpret_cast<uint2*>(raw);
+  Q.qf = reinterpret_cast<uint16_t*>(Q.qa + kTileBlocks + kSecSlots);
+  Q.partial = reinterpret_cast<float*>(Q.qf + kTileBlocks + kSecSlots + 16);
+  Q.gqa = reinterpret_cast<uint2*>(Q.partial + kTileBlocks);
+  Q.gqf = reinterpret_cast<uint16_t*>(Q.gqa + 2 * kGenericSlots);
+  Q.ctrl = reinterpret_cast<uint32_t*>(Q.gqf + 2 * kGenericSlots);
+  float* partial = Q.partial;
+  uint32_t* ctrl = Q.ctrl;
+  static_assert((kTileBlocks + kSecSlots) % 4 == 0 && kGenericSlots % 2 == 0, "the arrays behind the 16-bit ones stay 8-byte aligned");
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  static_assert(kRawBytes <= 2 * 16 * kWgThreads, "two 16-byte registers per lane hold a tile's code bytes");
   const __half* xsrc = a.x;
   // A launch over matrices stored in a rotated basis rotates its activation itself: the
   // values go, signs applied, as f32 to the area the first tile's code bytes, queues and
@@ -741,16 +955,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     uint32_t r0, rows;
     tile_of(a, tile, M, r0, rows);
     const uint32_t nblk = rows * nb;
-    const size_t byte0 = (size_t)r0 * nb * 6;
-    const uint32_t off = (uint32_t)(byte0 & 15);
 
-    // P0: code bytes registers -> LDS
-    if (tid < 4) ctrl[tid] = 0;
-    {
-      const uint32_t n16 = (off + nblk * 6 + 15) >> 4;
-      if (tid < n16) reinterpret_cast<uint4*>(raw)[tid] = pre0;
-      if (tid + kWgThreads < n16) reinterpret_cast<uint4*>(raw)[tid + kWgThreads] = pre1;
-    }
+    if (tid < (uint32_t)kCtrlWords) ctrl[tid] = 0;
     // P3 operands (row scales, tail weights): fetched now, used after the decode
     const uint32_t sub = lane >> 4, l16 = lane & 15u;
     constexpr int kP3Rounds = 2;  // 64 rows per round cover every tile of the usual shapes
@@ -767,109 +973,132 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     LLVQ_STAMP(1);
 
     // P1: classify and bin (a tile of tail-only rows has no blocks: its queues stay empty)
-    if (nblk != 0) classify_and_bin<kP1Blocks>(
-        T, nblk, kTileBlocks, queue, gqueue, ctrl, [&](uint32_t f) { return read_record(raw, off + 6 * f); },
-        [&](uint32_t f) {
-          partial[f] = 0.f;
-          return false;
-        });
+    if (nblk != 0) classify_stream<kP1Blocks>(T, pre, nblk, kTileBlocks, Q);
     __syncthreads();
     LLVQ_STAMP(2);
-    prefetch_tile(a, tile + gridDim.x, tid, pre0, pre1);
+    prefetch_records(a, tile + gridDim.x, tid, pre);
 
-    // P2: unrank and reduce.  Chunks of 64 queued blocks are handed out through a
-    // counter: the generic chunk first (longest), then even and odd ones in turn.
-    const uint32_t n_odd = ctrl[0], n_even = ctrl[1], n_gen = min(ctrl[2], (uint32_t)kGenericSlots);
-    const uint32_t c_gen = n_gen ? 1u : 0u, c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6;
+    // P2: unrank and reduce.  Chunks of 64 queued blocks are handed out through a counter: the two
+    // generic chunks first (longest), then the chunks of the three fast decoders.
+    const uint32_t n_odd = ctrl[kCtrlOdd], n_even = ctrl[kCtrlEven], n_sec = min(ctrl[kCtrlSec], (uint32_t)kSecSlots);
+    const uint32_t n_gen_o = min(ctrl[kCtrlGenOdd], (uint32_t)kGenericSlots), n_gen_e = min(ctrl[kCtrlGenEven], (uint32_t)kGenericSlots);
+    const uint32_t c_gen_o = n_gen_o ? 1u : 0u, c_gen_e = n_gen_e ? 1u : 0u, c_gen = c_gen_o + c_gen_e;
+    const uint32_t c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6, c_sec = (n_sec + 63u) >> 6;
     auto ticket = [&]() {
       uint32_t t = 0;
-      if (lane == 0) t = atomicAdd(&ctrl[3], 1u);
+      if (lane == 0) t = atomicAdd(&ctrl[kCtrlTicket], 1u);
       return (uint32_t)__shfl(t, 0, 64);
     };
-    // generic walk of one queued block (rare classes), scalar reduction against the planes
-    auto generic_block = [&](uint32_t entry) {
-      const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
-      const uint64_t rec = read_record(raw, off + 6 * f);
-      const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+    // what every decoder starts from: the block's local rank, class, column and scale
+    struct Block {
+      uint64_t li;
+      uint32_t f, ci, col;
+      float g;
+    };
+    auto open_block = [&](uint2 e, uint32_t f) {
+      Block b;
+      b.li = ((uint64_t)(e.y & 0x1FFFu) << 32) | e.x;
+      b.ci = (e.y >> kQaClassShift) & 0x1FFu;
+      b.f = f;
       const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
-      const uint32_t col = f - row * nb;
-      const uint8_t* xb = reinterpret_cast<const uint8_t*>(xplanes + (size_t)col * kPlaneDwords);
-      const float g = (entry >> 25) & 1u ? M.g1 : M.g0;
-      const DevClass c = T.cls[ci];
+      b.col = f - row * nb;
+      b.g = (e.y >> kQaGainShift) & 1u ? M.g1 : M.g0;
+      return b;
+    };
+    // generic walk of one queued block (rare classes): coordinates packed four to a dword, then
+    // the same integer dot products as the fast paths
+    auto generic_block = [&](uint2 e, uint32_t f) {
+      const Block b = open_block(e, f);
+      const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+      const DevClass c = T.cls[b.ci];
+      uint32_t w[6] = {0, 0, 0, 0, 0, 0};
+      auto emit = [&](int p, int v) { w[p >> 2] |= ((uint32_t)v & 0xFFu) << (8 * (p & 3)); };
+      if (c.meta & kMetaOdd) decode_odd(T, c, b.li, emit);
+      else decode_even(T, c, b.li, emit);
       int d0 = 0, d1 = 0, d2 = 0;
-      auto emit = [&](int p, int v) {
-        d0 += v * (int)(int8_t)xb[p];
-        d1 += v * (int)(int8_t)xb[24 + p];
-        d2 += v * (int)(int8_t)xb[48 + p];
-      };
-      if (c.meta & kMetaOdd) decode_odd(T, c, li, emit);
-      else decode_even(T, c, li, emit);
-      partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (c.inv_norm * g);
+#pragma unroll
+      for (int q = 0; q < 6; ++q) {
+        d0 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[q], d0, false);
+        d1 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[6 + q], d1, false);
+        d2 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[12 + q], d2, false);
+      }
+      partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (c.inv_norm * b.g);
+    };
+    auto odd_block = [&](uint2 e, uint32_t f) {
+      const Block b = open_block(e, f);
+      const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+      const FastClass fc = T.fast[b.ci];
+      int d0 = 0, d1 = 0, d2 = 0;
+      odd_codes(T, fc, b.li, [&](int q, uint32_t sel) {
+        const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+        d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+        d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+        d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+      });
+      partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
+    };
+    auto even_block = [&](uint2 e, uint32_t f, auto second) {
+      constexpr bool kSecond = decltype(second)::value;
+      const Block b = open_block(e, f);
+      const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+      const FastClass fc = T.fast[b.ci];
+      const uint32_t fv1 = fc.u0 >> 16;
+      const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
+      int d0 = 0, d1 = 0, d2 = 0;
+      even_codes<kSecond>(T, fc, b.li, [&](int q, uint32_t sel, uint32_t sel2) {
+        int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+        if (kSecond) w |= (int)__builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2);
+        d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+        d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+        d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+      });
+      partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
     };
     uint32_t chunk = ticket();
-    if (c_gen && chunk == 0) {  // kept out of the loop below: its code and registers are not the hot path's
-      if (lane < n_gen) generic_block(gqueue[lane]);
+    // the generic chunks, kept out of the loop below: their code and registers are not the hot path's
+    while (chunk < c_gen) {
+      const uint32_t even = (chunk == 1u || !c_gen_o) ? 1u : 0u;
+      if (lane < (even ? n_gen_e : n_gen_o)) generic_block(Q.gqa[even * kGenericSlots + lane], Q.gqf[even * kGenericSlots + lane]);
       chunk = ticket();
     }
-    // even and odd chunks alternate while both queues last: the even coset waits for tables in L2,
-    // the odd one issues arithmetic, and wavefronts on either kind at the same time overlap the two
+    // Even and odd chunks alternate while both queues last: the even coset waits for tables in L2,
+    // the odd one issues arithmetic, and wavefronts on either kind at the same time overlap the two.
+    // The chunks of the small even queue come first (their queue ends in a partial chunk as well).
     const uint32_t c_pair = min(c_odd, c_even);
-    for (; chunk < c_gen + c_odd + c_even; chunk = ticket()) {
-      const uint32_t t = chunk - c_gen;
+    for (; chunk < c_gen + c_sec + c_odd + c_even; chunk = ticket()) {
+      const uint32_t ts = chunk - c_gen;
+      if (ts < c_sec) {
+        const uint32_t k = ts * 64u + lane;
+        if (k < n_sec) even_block(Q.qa[kTileBlocks + k], Q.qf[kTileBlocks + k], std::true_type{});
+        continue;
+      }
+      const uint32_t t = ts - c_sec;
       const bool paired = t < 2u * c_pair;
       const bool is_odd = paired ? (t & 1u) != 0u : c_odd > c_even;
       const uint32_t ordinal = paired ? t >> 1 : t - c_pair;
+      const uint32_t k = ordinal * 64u + lane;
       if (is_odd) {
-        const uint32_t k = ordinal * 64u + lane;
-        const uint32_t entry = k < n_odd ? queue[k] : kEntryGeneric;
-        if (!(entry >> 31)) {  // generic blocks that found the small queue full wait for the pass below
-          const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
-          const uint64_t rec = read_record(raw, off + 6 * f);
-          const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
-          const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
-          const uint32_t col = f - row * nb;
-          const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
-          const float g = (entry >> 25) & 1u ? M.g1 : M.g0;
-          const FastClass fc = T.fast[ci];
-          int d0 = 0, d1 = 0, d2 = 0;
-          odd_codes(T, fc, li, [&](int q, uint32_t sel) {
-            const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
-            d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
-            d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-            d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
-          });
-          partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * g);
-        }
+        const uint32_t at = min(k, (uint32_t)kTileBlocks - 1u);
+        const uint2 e = Q.qa[at];
+        // generic blocks that found their small queue full wait for the pass below
+        if (k < n_odd && !(e.y >> 31)) odd_block(e, Q.qf[at]);
       } else {
-        const uint32_t k = ordinal * 64u + lane;
-        if (k < n_even) {
-          const uint32_t entry = queue[kTileBlocks - 1 - k];
-          const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
-          const uint64_t rec = read_record(raw, off + 6 * f);
-          const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
-          const FastClass fc = T.fast[ci];
-          const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
-          const uint32_t col = f - row * nb;
-          const uint32_t* xp = xplanes + (size_t)col * kPlaneDwords;
-          const uint32_t fv1 = fc.u0 >> 16;
-          const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
-          int d0 = 0, d1 = 0, d2 = 0;
-          even_codes(T, fc, li, [&](int q, uint32_t sel, uint32_t sel2) {
-            const int w = (int)(__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel) |
-                                __builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2));
-            d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
-            d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-            d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
-          });
-          partial[f] = planes_to_float(d0, d1, d2) * xscale[col] * (fc.inv_norm * ((entry >> 25) ? M.g1 : M.g0));
+        const uint32_t at = kTileBlocks - 1 - min(k, (uint32_t)kTileBlocks - 1u);
+        const uint2 e = Q.qa[at];
+        const bool mine = k < n_even;
+        // blocks with a second free kind that found their queue full ride here, flagged
+        if (__any(mine && (e.y & kQaSecond))) {
+          if (mine) even_block(e, Q.qf[at], std::true_type{});
+        } else {
+          if (mine) even_block(e, Q.qf[at], std::false_type{});
         }
       }
     }
-    if (ctrl[2] > (uint32_t)kGenericSlots) {
-      // more generic blocks than the small queue holds (hostile input): the rest sit flagged in the odd queue
+    if (ctrl[kCtrlGenOdd] > (uint32_t)kGenericSlots || ctrl[kCtrlGenEven] > (uint32_t)kGenericSlots) {
+      // more generic blocks than the small queues hold (hostile input): the rest sit flagged in the odd queue
       for (uint32_t k = tid; k < n_odd; k += kWgThreads) {
-        const uint32_t entry = queue[k];
-        if (entry >> 31) generic_block(entry);
+        const uint2 e = Q.qa[k];
+        if (e.y >> 31) generic_block(e, Q.qf[k]);
       }
     }
     LLVQ_STAMP(4);
@@ -1075,7 +1304,9 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   }
   // one blob: LDS image | generic class records | off-support table | deposit masks | walk-tail codes
   if (cb.on_lut.size() > (size_t)kOnLutSlots) { delete rt; return fail(LLVQ_ERR_UNSUPPORTED, "support-arrangement table outgrew its LDS slot"); }
-  const size_t off_cls = sizeof(TableImage);
+  const size_t off_starts = sizeof(TableImage);
+  static_assert(sizeof(TableImage) % 8 == 0, "the class starts follow the image 8-byte aligned");
+  const size_t off_cls = (off_starts + sizeof(cb.starts) + 15) & ~(size_t)15;
   const size_t off_lut = off_cls + sizeof(cb.dev_classes);
   const size_t off_exp = (off_lut + cb.off_lut.size() * 4 + 15) & ~(size_t)15;
   const size_t off_tail = off_exp + sizeof(cb.expand);
@@ -1087,6 +1318,16 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   std::memcpy(img->fast, cb.fast, sizeof img->fast);
   std::memcpy(img->starts, cb.starts, sizeof img->starts);
   std::memcpy(img->lut, cb.lut, sizeof img->lut);
+  // a 47-bit index reaches no class past kFastLds - 2 and no second-level table past kLut2Lds
+  uint32_t lut2_used = 0;
+  for (uint16_t e : img->lut)
+    if (e & kLutRedirect) lut2_used = std::max<uint32_t>(lut2_used, ((e & 0x7FFFu) + 1u) * kLut2Span);
+  if (lut2_used > (uint32_t)kLut2Lds || lut2_used > cb.lut2.size() || cb.starts[kFastLds - 1] < (1ULL << 47)) {
+    delete rt;
+    return fail(LLVQ_ERR_UNSUPPORTED, "class-find tables outgrew their LDS slots");
+  }
+  std::memcpy(img->lut2, cb.lut2.data(), (size_t)lut2_used * 2);
+  std::memcpy(host.data() + off_starts, cb.starts, sizeof(cb.starts));
   std::memcpy(img->rcp, cb.rcp, sizeof img->rcp);
   std::memcpy(img->step, cb.step + kTailSlots * 25 * 2, sizeof img->step);
   std::memcpy(img->tail_meta, cb.tail_meta, sizeof img->tail_meta);
@@ -1101,6 +1342,7 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   e = hipMemcpy(rt->blob, host.data(), total, hipMemcpyHostToDevice);
   if (e != hipSuccess) { (void)hipFree(rt->blob); delete rt; return hip_fail(e, "hipMemcpy(tables)"); }
   rt->tables.image = reinterpret_cast<const TableImage*>(rt->blob);
+  rt->tables.starts = reinterpret_cast<const uint64_t*>(rt->blob + off_starts);
   rt->tables.cls = reinterpret_cast<const DevClass*>(rt->blob + off_cls);
   rt->tables.off_lut = reinterpret_cast<const uint32_t*>(rt->blob + off_lut);
   rt->tables.expand = reinterpret_cast<const uint32_t*>(rt->blob + off_exp);
