@@ -16,6 +16,7 @@ timed on the host cores on one layer of the same workload.
 import argparse
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -28,8 +29,24 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 
-# (7013.5 KiB fetched x 2.000 + 23.8 KiB written) per gemv_tiles_kernel launch on the default workload
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = round((7013.5 * 2.000 + 23.8) * 1024)
+# HBM-side bytes per gemv_tiles_kernel launch come from rocprofv3 --pmc runs of this command (FETCH_SIZE,
+# WRITE_SIZE); the summary of those runs is this file, whose machine-readable lines bench.py reads back
+TRAFFIC_PROFILE = os.path.join("profiles", "gemv_tiles_kernel_qwen3-4b-projections_counters.txt")
+
+
+def profiled(path=None):
+    """`key = value` lines of the committed counter summary: traffic_bytes_per_launch, kernel_avg_us,
+    valu_slots_per_block, valu_busy_frac.  Missing file or key: None."""
+    out = {}
+    try:
+        with open(path or os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_PROFILE)) as f:
+            for line in f:
+                m = re.match(r"\s*([a-z_]+)\s*=\s*([0-9.eE+-]+)\s*$", line)
+                if m:
+                    out[m.group(1)] = float(m.group(2))
+    except OSError:
+        pass
+    return out
 
 
 def log(*a):
@@ -93,7 +110,7 @@ def cpu_baseline(layer_mats, acts, threads, y_device=None):
     }
 
 
-def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
+def decode_leg(rt, projs, seed, n_prompt=512, n_new=256, q8_head=False):
     """BASELINE config 2: the whole Qwen3-4B-architecture loop (36 layers over the projections already on the
     device, f16 embedding tied to the head, vocabulary 151936): a 512-token random prompt, then 256 greedy
     tokens.  Decode rate = (time of prompt + 256 tokens) - (time of prompt + 1 token), over 255 steps."""
@@ -102,8 +119,13 @@ def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
     cfg = decoder.QWEN3_4B
     t0 = time.time()
     weights = decoder.synthetic_weights(cfg, seed)
-    dec = decoder.Decoder(rt, cfg, projs, weights, prefill_rows=n_prompt)
-    log(f"[bench] decoder built in {time.time() - t0:.1f}s")
+    if q8_head:
+        # the embedding and the head as the int8 g64 tensors of a sealed file (Embed::Q8 / Head::Q8, model.rs:546-575):
+        # the f16 head is 778 MB per token, as much as all 252 projections together
+        weights.embed = decoder.quantize_rows_q8("model.embed_tokens.weight", weights.embed)
+        weights.lm_head = decoder.quantize_rows_q8("lm_head.weight", weights.lm_head)
+    dec = decoder.Decoder(rt, cfg, projs, weights, prefill_rows=0 if q8_head else n_prompt)
+    log(f"[bench] decoder built in {time.time() - t0:.1f}s ({'int8' if q8_head else 'f16'} embedding and head)")
     prompt = np.random.default_rng(seed).integers(0, cfg.vocab_size, size=n_prompt)
     dec.generate(prompt[:8], 4)  # warm-up
     t0 = time.perf_counter()
@@ -111,14 +133,21 @@ def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
     t1 = time.perf_counter()
     toks = dec.generate(prompt, n_new)
     t2 = time.perf_counter()
+    assert toks[0] == first[0]
+    step_s = ((t2 - t1) - (t1 - t0)) / (n_new - 1)
+    if q8_head:
+        dec.close()
+        return {"tokens_per_s": round(1.0 / step_s, 2), "ms_per_token": round(step_s * 1e3, 4), "prompt_tokens": n_prompt,
+                "new_tokens": n_new, "embedding_and_head": "int8 g64", "distinct_tokens": int(np.unique(toks).size)}
+    # where a decode token's time goes (Qwen3::generate_phased, model.rs:1116-1163): device time per phase, medians
+    _, phases = dec.generate_phased(prompt[:64], 33)
+    med = np.median(phases[:-1], axis=0)
     # the same prompt through the batched product (matrix cores, all positions of the prompt at once)
     dec.generate(prompt, 1, batched_prefill=True)
     t3 = time.perf_counter()
     batched_first = dec.generate(prompt, 1, batched_prefill=True)
     t4 = time.perf_counter()
     dec.close()
-    assert toks[0] == first[0]
-    step_s = ((t2 - t1) - (t1 - t0)) / (n_new - 1)
     return {
         "tokens_per_s": round(1.0 / step_s, 2),
         "ms_per_token": round(step_s * 1e3, 4),
@@ -129,6 +158,9 @@ def decode_leg(rt, projs, seed, n_prompt=512, n_new=256):
         "batched_prefill_tokens_per_s": round(n_prompt / (t4 - t3), 1),
         "batched_prefill_first_token_agrees": bool(batched_first[0] == first[0]),
         "distinct_tokens": int(np.unique(toks).size),
+        "embedding_and_head": "f16",
+        "phase_ms_median": {"head": round(float(med[0]), 4), "argmax": round(float(med[1]), 4), "embed": round(float(med[2]), 4),
+                            "blocks": round(float(med[3]), 4), "at_positions": "64..96"},
     }
 
 
@@ -403,6 +435,11 @@ def main():
 
     avg_launch_us = dev_ms * 1e3 / (args.steps * n_kernels)
     achieved = enc_bytes * args.steps / (dev_ms * 1e-3) / 1e9
+    # traffic and the VALU figures are those of the committed counter summary, taken with this command; they
+    # only stand while this run's kernel time agrees with the profiled one (5 %) on the profiled workload
+    prof = profiled()
+    prof_ok = bool(prof) and (args.layers, args.seed) == (36, 0) and "kernel_avg_us" in prof and \
+        abs(prof["kernel_avg_us"] - avg_launch_us) <= 0.05 * avg_launch_us
     out = {
         "metric": "dequant_gemv_encoded_weight_GBps",
         "value": round(gbps, 3),
@@ -414,7 +451,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f32",  # int8 x int8 -> int32 dot products per block (exact), f32 scales and accumulation; f16 in, f16 out
         "data": "synthetic",
         "config": {
             "workload": f"Qwen3-4B decoder-layer projections at batch 1 (BASELINE config 1 shapes), "
@@ -436,8 +473,14 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 5),
             # L2-miss bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command,
-            # each scaled by its reading for a 256 MiB device copy (x2.000 and x1.000); profiles/ holds both
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (args.layers, args.seed) == (36, 0) else None,
+            # each scaled by its reading for a 256 MiB device copy; null when the profile is not of this kernel time
+            "traffic": int(prof["traffic_bytes_per_launch"]) if prof_ok and "traffic_bytes_per_launch" in prof else None,
+            "traffic_source": TRAFFIC_PROFILE if prof_ok else None,
+            "profiled_kernel_avg_us": prof.get("kernel_avg_us"),
+            # what actually binds: the unranking arithmetic on the vector ALUs, not HBM (rocprofv3 SQ counters, same file)
+            "limited_by": "valu",
+            "valu_slots_per_block": prof.get("valu_slots_per_block") if prof_ok else None,
+            "valu_busy_frac": prof.get("valu_busy_frac") if prof_ok else None,
             "avg_launch_us": round(avg_launch_us, 3),
             "launches_per_step": n_kernels,
             "algorithmic_bytes_per_launch": round(enc_bytes / n_kernels, 1),
@@ -445,6 +488,7 @@ def main():
     }
     if not args.no_decode and args.layers == 36:
         out["decode"] = decode_leg(rt, projs, args.seed)
+        out["decode_q8_head"] = decode_leg(rt, projs, args.seed, q8_head=True)
         # BASELINE config 3 beside it, shortened: two Qwen3-8B-shaped layers, M = 256 (the full sweep is --workload gemm)
         g = measure_gemm(args, torch, llvq_amd, synth, dev, 256, 2, 3, 1)
         out["batched"] = {"M": 256, "TFLOPs": g["value"], "mfma_peak_frac": g["roofline"]["frac"],
@@ -456,8 +500,12 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
     if not args.no_cpu:
-        threads = min(16, os.cpu_count() or 1)
+        # a one-GPU box's share of the host is 16 cores whatever the machine has; both are reported
+        host_cores = os.cpu_count() or 1
+        threads = min(16, host_cores)
         out["cpu_baseline"] = cpu_baseline(layers[0], acts_np, threads, y_layer0)
+        out["cpu_baseline"]["host_cores"] = host_cores
+        out["cpu_baseline"]["cores_note"] = "threads used = min(16, host cores): 16 is the CPU share of a one-GPU box"
     rt.close()
     print(json.dumps(out), flush=True)
 

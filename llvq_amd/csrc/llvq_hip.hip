@@ -473,12 +473,13 @@ __device__ __forceinline__ void prefetch_records(const GroupArgs& a, uint32_t ti
   const uint32_t share = (uint32_t)NB * 6u;
   const uint32_t at = tid * (uint32_t)NB < rows * a.nblocks ? tid * share : 0u;
   const uint8_t* src = M.codes + (size_t)r0 * a.nblocks * 6 + at;
+  // streaming loads: the code bytes are read once, and must not push the decode tables out of L2
   if constexpr (NB == 4) {
-    const dwords4_a2 lo = *reinterpret_cast<const dwords4_a2*>(src);
-    const dwords2_a2 hi = *reinterpret_cast<const dwords2_a2*>(src + 16);
+    const dwords4_a2 lo = __builtin_nontemporal_load(reinterpret_cast<const dwords4_a2*>(src));
+    const dwords2_a2 hi = __builtin_nontemporal_load(reinterpret_cast<const dwords2_a2*>(src + 16));
     r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w; r.w[4] = hi.x; r.w[5] = hi.y;
   } else {
-    const dwords3_a2 v = *reinterpret_cast<const dwords3_a2*>(src);
+    const dwords3_a2 v = __builtin_nontemporal_load(reinterpret_cast<const dwords3_a2*>(src));
     r.w[0] = v.x; r.w[1] = v.y; r.w[2] = v.z;
   }
 }
