@@ -1618,20 +1618,36 @@ int llvq_hip_matrix_info(const llvq_mat* m, uint32_t* d_out, uint32_t* d_in, uin
 
 const char* llvq_hip_matrix_name(const llvq_mat* m) { return m ? m->name.c_str() : ""; }
 
-// Rows per tile: as even a split over the CUs as the tile capacity allows.
+// Rows per tile.  The workgroups take tiles in rounds of `grid`; a launch lasts rounds x (a tile's
+// blocks + what a tile costs whatever its size: barriers, row sums, the wait for its first code
+// bytes, taken as kTileFixedBlocks blocks' worth).  For k = 1, 2, ... rounds the best tile is the
+// smallest that needs no more than k rounds; the cheapest of those that fit the tile capacity wins
+// (7168 rows of 213 blocks on 256 CUs: 14 rows in exactly 2 rounds, not 19 rows in 1.5).
+constexpr uint32_t kTileFixedBlocks = 400;
 static uint32_t pick_rows_per_tile(const llvq_mat* const* mats, int n, uint32_t nblocks, uint32_t grid, uint32_t tile) {
-  const uint32_t cap = nblocks ? tile / nblocks : 0xFFFFFFFFu;
+  const uint32_t cap = nblocks ? (tile / nblocks ? tile / nblocks : 1u) : 0xFFFFFFFFu;
   uint64_t total = 0;
   for (int i = 0; i < n; ++i) total += mats[i]->d_out;
-  uint32_t r = (uint32_t)((total + grid - 1) / grid);
-  if (r < 1) r = 1;
-  for (uint32_t tries = 0; tries < 64 && r < cap; ++tries, ++r) {
-    uint64_t tiles = 0;
-    for (int i = 0; i < n; ++i) tiles += (mats[i]->d_out + r - 1) / r;
-    if (tiles <= grid) break;
+  auto tiles_at = [&](uint32_t r) {
+    uint64_t t = 0;
+    for (int i = 0; i < n; ++i) t += (mats[i]->d_out + r - 1) / r;
+    return t;
+  };
+  uint32_t best = cap == 0xFFFFFFFFu ? (uint32_t)((total + grid - 1) / grid) : cap;
+  if (best < 1) best = 1;
+  uint64_t best_cost = ((tiles_at(best) + grid - 1) / grid) * ((uint64_t)best * nblocks + kTileFixedBlocks);
+  for (uint32_t k = 1; k <= 16; ++k) {
+    uint32_t r = (uint32_t)((total + (uint64_t)k * grid - 1) / ((uint64_t)k * grid));
+    if (r < 1) r = 1;
+    for (uint32_t tries = 0; tries < 64 && r <= cap && tiles_at(r) > (uint64_t)k * grid; ++tries) ++r;
+    if (r > cap || tiles_at(r) > (uint64_t)k * grid) continue;
+    const uint64_t cost = (uint64_t)k * ((uint64_t)r * nblocks + kTileFixedBlocks);
+    if (cost < best_cost || (cost == best_cost && r > best)) {
+      best_cost = cost;
+      best = r;
+    }
   }
-  if (r > cap) r = cap;
-  return r < 1 ? 1 : r;
+  return best;
 }
 
 // Whether a launch over rows of this width can stage a derived activation where

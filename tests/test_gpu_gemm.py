@@ -175,6 +175,56 @@ def test_gemm_qwen3_8b_shapes(gpu_rt, orc, site, d_out, d_in, M):
     assert np.isfinite(Y).all()
 
 
+def test_gemm_2048_rows_in_chunks(gpu_rt, orc):
+    """More activation rows than one launch holds: four launches of 512 rows, each row of the
+    result against the oracle's on a sample that touches every chunk and its ends."""
+    import torch
+
+    d_out, d_in, M = 1024, 4096, 2048
+    raw = synth.make_matrix("model.layers.0.self_attn.k_proj.weight", d_out, d_in, seed=21)
+    X = synth.make_activation(d_in, seed=2048, rows=M)
+    proj = gpu_rt.upload(raw)
+    try:
+        Y32 = gpu_rt.forward_batched(proj, _x16(X), out_dtype=torch.float32).cpu().numpy()
+        Y16 = gpu_rt.forward_batched(proj, _x16(X)).cpu().numpy()
+    finally:
+        gpu_rt.free(proj)
+    pick = sorted({0, 1, 511, 512, 513, 1023, 1024, 1500, 1535, 1536, 2046, 2047})
+    Y_ref, A_ref = _reference(orc, raw, X[pick])
+    e = _check(Y32[pick], Y_ref, A_ref)
+    print(f"OBSERVED M=2048 max |dy|/sum|wx| = {e:.3e}")
+    assert e < 3e-4
+    _check(Y16[pick].astype(np.float32), Y_ref, A_ref, out_rounding=2.0 ** -11)
+    assert np.isfinite(Y32).all() and np.isfinite(Y16.astype(np.float32)).all()
+
+
+def test_gemm_partial_sums_of_the_call_before_do_not_leak(gpu_rt, orc):
+    """Bands that several workgroups share are summed from a workspace.  Two matrices of one shape
+    take turns, so the workspace holds the other one's partial sums at the same addresses whenever a
+    call starts: every result must be that of the first call, bit for bit, and the first calls are
+    checked against the oracle."""
+    import torch
+
+    d_out, d_in, M = 4096, 4096, 256  # 64 bands of 11 slices over 256 workgroups: every band has several pieces
+    raws = [synth.make_matrix(f"model.layers.{i}.self_attn.o_proj.weight", d_out, d_in, seed=60 + i) for i in range(2)]
+    Xs = [synth.make_activation(d_in, seed=70 + i, rows=M) for i in range(2)]
+    projs = [gpu_rt.upload(r) for r in raws]
+    try:
+        xd = [_x16(X) for X in Xs]
+        first = [gpu_rt.forward_batched(p, x, out_dtype=torch.float32) for p, x in zip(projs, xd)]
+        for rounds in range(6):
+            for i in (0, 1):
+                again = gpu_rt.forward_batched(projs[i], xd[i], out_dtype=torch.float32)
+                assert torch.equal(again, first[i]), f"round {rounds}, matrix {i}"
+        pick = [0, 63, 64, 200, 255]
+        for i in (0, 1):
+            Y_ref, A_ref = _reference(orc, raws[i], Xs[i][pick])
+            _check(first[i].cpu().numpy()[pick], Y_ref, A_ref)
+    finally:
+        for p in projs:
+            gpu_rt.free(p)
+
+
 def test_gemm_group_matches_the_oracle_and_the_single_calls(gpu_rt, orc):
     """Five projections that share their activation rows (more than one launch holds), as one call:
     every output against the oracle, and against the same projection called on its own (the two may
