@@ -28,15 +28,6 @@ namespace llvq {
 // ---- table image --------------------------------------------------------------
 // What every workgroup copies into LDS.  The rarely used generic class records
 // and the large even-coset tables stay in HBM (they live in L2).
-#ifndef LLVQ_WG_THREADS
-#define LLVQ_WG_THREADS 1024
-#endif
-#ifndef LLVQ_TILE_BLOCKS
-#define LLVQ_TILE_BLOCKS 4096
-#endif
-#ifndef LLVQ_LDS_GOLAY
-#define LLVQ_LDS_GOLAY 1   // 1: Golay words and the support-arrangement table live in LDS; 0: read through L2
-#endif
 struct TableImage {
   FastClass fast[kFastLds];
   uint64_t starts[kStartsLds];
@@ -50,7 +41,7 @@ struct TableImage {
   uint32_t on_lut[kOnLutSlots];
 };
 static_assert(sizeof(TableImage) % 16 == 0, "table image is copied in 16-byte units");
-constexpr size_t kLdsImageBytes = LLVQ_LDS_GOLAY ? sizeof(TableImage) : offsetof(TableImage, golay);
+constexpr size_t kLdsImageBytes = sizeof(TableImage);  // Golay words and the support-arrangement table included
 static_assert(kLdsImageBytes % 16 == 0, "LDS part of the table image is copied in 16-byte units");
 
 struct GlobalTables {
@@ -70,7 +61,7 @@ static_assert(kLdsImageBytesLeanest % 16 == 0, "LDS part of the table image is c
 // kFull: the whole image goes to LDS; otherwise its last two tables (33 KB) are
 // read through L2, for a kernel that needs the LDS for something else.  kLut = false
 // leaves the 4 KB class lookup table (one read per block) in L2 as well.
-template <bool kFull = (LLVQ_LDS_GOLAY != 0), bool kLut = true>
+template <bool kFull = true, bool kLut = true>
 __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const GlobalTables& g) {
   static_assert(kLut || !kFull, "the tables that stay in L2 are the image's last ones");
   const uint4* src = reinterpret_cast<const uint4*>(g.image);
@@ -187,9 +178,9 @@ __global__ __launch_bounds__(256) void decode_blocks_kernel(GlobalTables g, cons
 // value within 2^12 of its block's largest is exact and the rest round at
 // 2^-23 of that largest.  Integer sums of 24 products are exact; the three
 // plane sums are combined and scaled in f32.
-constexpr int kWgThreads = LLVQ_WG_THREADS;
+constexpr int kWgThreads = 1024;
 constexpr int kWaves = kWgThreads / 64;
-constexpr int kTileBlocks = LLVQ_TILE_BLOCKS;  // default tile capacity; the kernel is instantiated per capacity
+constexpr int kTileBlocks = 4096;  // default tile capacity; the kernel is instantiated per capacity
 constexpr int kMaxGroup = 4;
 constexpr int kPlaneDwords = 18;  // 3 planes x 6 dwords per 24-column block
 constexpr int kGenericSlots = 64; // queue of blocks that take the generic walk
@@ -770,7 +761,7 @@ __device__ __forceinline__ void classify_stream(const DecodeTables& T, const Lan
 // room for the full tile beside the activation planes of a very wide row.
 // ROT: the launch can rotate its own activation (GroupArgs::rot_m); kept out of the other
 // instantiations, whose hot loop it would otherwise cost registers and a few per cent.
-template <typename OutT, int TILE = LLVQ_TILE_BLOCKS, bool LEAN = false, bool ROT = false>
+template <typename OutT, int TILE = kTileBlocks, bool LEAN = false, bool ROT = false>
 __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   // the tile capacity of this instantiation (these shadow the namespace-level defaults)
   constexpr int kTileBlocks = TILE;
@@ -780,7 +771,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 #ifdef LLVQ_PHASE_TIMING
   if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 3] = wall_clock64();
 #endif
-  const DecodeTables T = stage_tables<!LEAN && (LLVQ_LDS_GOLAY != 0)>(smem, a.tables);
+  const DecodeTables T = stage_tables<!LEAN>(smem, a.tables);
   // A lane loads the records it classifies itself, HBM -> registers; the next tile's loads are
   // issued while the current one is being decoded.  The first tile's are issued right behind the
   // loads of the activation: the memory counter retires in order, so whatever is requested
@@ -1139,8 +1130,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 // The instantiations of gemv_tiles_kernel by (f32 output, tile, lean image, in-launch rotation).
 template <typename OutT, bool ROT>
 __host__ const void* gemv_kernel_of(uint32_t tile, bool lean) {
-  if (lean) return reinterpret_cast<const void*>(gemv_tiles_kernel<OutT, LLVQ_TILE_BLOCKS, true, ROT>);
-  if (tile == (uint32_t)LLVQ_TILE_BLOCKS) return reinterpret_cast<const void*>(gemv_tiles_kernel<OutT, LLVQ_TILE_BLOCKS, false, ROT>);
+  if (lean) return reinterpret_cast<const void*>(gemv_tiles_kernel<OutT, kTileBlocks, true, ROT>);
+  if (tile == (uint32_t)kTileBlocks) return reinterpret_cast<const void*>(gemv_tiles_kernel<OutT, kTileBlocks, false, ROT>);
   return reinterpret_cast<const void*>(gemv_tiles_kernel<OutT, kSmallTileBlocks, false, ROT>);
 }
 __host__ const void* gemv_kernel(bool f32, uint32_t tile, bool lean, bool rot) {
@@ -1151,9 +1142,9 @@ template <class Fn>
 __host__ void for_each_gemv_kernel(Fn&& fn) {
   for (int f32 = 0; f32 < 2; ++f32)
     for (int rot = 0; rot < 2; ++rot) {
-      fn(gemv_kernel(f32, LLVQ_TILE_BLOCKS, false, rot));
+      fn(gemv_kernel(f32, kTileBlocks, false, rot));
       fn(gemv_kernel(f32, kSmallTileBlocks, false, rot));
-      fn(gemv_kernel(f32, LLVQ_TILE_BLOCKS, true, rot));
+      fn(gemv_kernel(f32, kTileBlocks, true, rot));
     }
 }
 
@@ -2200,11 +2191,13 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   llvq_rt* rt = d->rt;
   hipStream_t st = rt->stream;
   if (d->pos >= d->max_pos) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder: position " + std::to_string(d->pos) + " is past max_positions");
+  // the two residual buffers, by local name: a step that fails part-way leaves the decoder as it found it
+  __half *h = d->h, *h_alt = d->h_alt;
   phase_mark(d);
   if (d->embed_q8)
-    hipLaunchKernelGGL(embed_q8_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed_q, d->token, d->vocab, d->hidden, d->h);
+    hipLaunchKernelGGL(embed_q8_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed_q, d->token, d->vocab, d->hidden, h);
   else
-    hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, d->h);
+    hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256), dim3(256), 0, st, d->embed, d->token, d->vocab, d->hidden, h);
   phase_mark(d);
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim;
   const uint32_t T = d->pos + 1;
@@ -2252,12 +2245,12 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     ln1.eps = d->eps;
     if (L) {
       ln1.x2 = d->down;
-      ln1.resid_out = d->h_alt;
+      ln1.resid_out = h_alt;
     }
     void* qkv_out[3] = {d->q, d->k, d->v};
-    int rc = project(P, 3, d->h, qkv_out, ln1);
+    int rc = project(P, 3, h, qkv_out, ln1);
     if (rc) return rc;
-    if (L) std::swap(d->h, d->h_alt);
+    if (L) std::swap(h, h_alt);
     KvQ8 lq8 = d->q8;
     if (d->kv_q8) {
       lq8.kq += L * cache_layer; lq8.vq += L * cache_layer;
@@ -2303,11 +2296,11 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     ln2.norm_w = d->ln2 + (size_t)L * d->hidden;
     ln2.eps = d->eps;
     ln2.x2 = d->o;
-    ln2.resid_out = d->h_alt;
+    ln2.resid_out = h_alt;
     void* gu_out[2] = {d->gate, d->up};
-    rc = project(P + 4, 2, d->h, gu_out, ln2);
+    rc = project(P + 4, 2, h, gu_out, ln2);
     if (rc) return rc;
-    std::swap(d->h, d->h_alt);
+    std::swap(h, h_alt);
     Prologue act;
     act.kind = kPrologueSiluMul;
     act.x2 = d->gate;
@@ -2317,7 +2310,7 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
   }
   phase_mark(d);
   if (want_logits) {
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->h, d->down, d->fnorm, d->h, d->normed, d->hidden, d->eps);
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, h, d->down, d->fnorm, h, d->normed, d->hidden, d->eps);
     launch_head(d, history_slot, record);
   }
   HIP_TRY(hipGetLastError());
@@ -2331,19 +2324,20 @@ int decoder_prefill_pass(llvq_decoder* d, uint32_t n, bool want_logits, uint32_t
   hipStream_t st = rt->stream;
   if (d->pos + n > d->max_pos) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_prefill: positions past max_positions");
   const uint32_t qd = d->n_heads * d->head_dim;
+  __half *ph = d->ph, *ph_alt = d->ph_alt;  // by local name: a pass that fails part-way leaves the decoder as it found it
   if (d->embed_q8)
-    hipLaunchKernelGGL(embed_q8_kernel, dim3((d->hidden + 255) / 256, n), dim3(256), 0, st, d->embed_q, d->ptokens, d->vocab, d->hidden, d->ph);
+    hipLaunchKernelGGL(embed_q8_kernel, dim3((d->hidden + 255) / 256, n), dim3(256), 0, st, d->embed_q, d->ptokens, d->vocab, d->hidden, ph);
   else
-    hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256, n), dim3(256), 0, st, d->embed, d->ptokens, d->vocab, d->hidden, d->ph);
+    hipLaunchKernelGGL(embed_kernel, dim3((d->hidden + 255) / 256, n), dim3(256), 0, st, d->embed, d->ptokens, d->vocab, d->hidden, ph);
   const size_t cache_layer = (size_t)d->n_kv * d->max_pos * d->head_dim, group_layer = cache_layer / kKvGroup;
   const float scale = 1.0f / sqrtf((float)d->head_dim);
   auto rows = [&](const llvq_mat* m, const __half* x, __half* y) { return llvq_hip_gemm(rt, m, x, (int)n, y, LLVQ_F16); };
   for (uint32_t L = 0; L < d->n_layers; ++L) {
     const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
     // residual + previous MLP branch, then the input norm (the branch of layer 0 is absent)
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(kNormThreads), 0, st, d->ph, L ? d->pdown : (const __half*)nullptr,
-                       d->ln1 + (size_t)L * d->hidden, L ? d->ph_alt : (__half*)nullptr, d->pnormed, d->hidden, d->eps);
-    if (L) std::swap(d->ph, d->ph_alt);
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(kNormThreads), 0, st, ph, L ? d->pdown : (const __half*)nullptr,
+                       d->ln1 + (size_t)L * d->hidden, L ? ph_alt : (__half*)nullptr, d->pnormed, d->hidden, d->eps);
+    if (L) std::swap(ph, ph_alt);
     void* const qkv[3] = {d->pq, d->pk, d->pv};
     int rc = llvq_hip_gemm_group(rt, P, 3, d->pnormed, (int)n, qkv, LLVQ_F16);
     if (rc) return rc;
@@ -2400,9 +2394,9 @@ int decoder_prefill_pass(llvq_decoder* d, uint32_t n, bool want_logits, uint32_t
     }
     rc = rows(P[3], d->pctx, d->po);
     if (rc) return rc;
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(kNormThreads), 0, st, d->ph, d->po, d->ln2 + (size_t)L * d->hidden, d->ph_alt,
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(kNormThreads), 0, st, ph, d->po, d->ln2 + (size_t)L * d->hidden, ph_alt,
                        d->pnormed, d->hidden, d->eps);
-    std::swap(d->ph, d->ph_alt);
+    std::swap(ph, ph_alt);
     void* const gate_up[2] = {d->pgate, d->pup};
     rc = llvq_hip_gemm_group(rt, P + 4, 2, d->pnormed, (int)n, gate_up, LLVQ_F16);
     if (rc) return rc;
@@ -2413,7 +2407,7 @@ int decoder_prefill_pass(llvq_decoder* d, uint32_t n, bool want_logits, uint32_t
   }
   if (want_logits) {
     const size_t last = (size_t)(n - 1) * d->hidden;
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, d->ph + last, d->pdown + last, d->fnorm, d->h, d->normed,
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, ph + last, d->pdown + last, d->fnorm, d->h, d->normed,
                        d->hidden, d->eps);
     launch_head(d, history_slot, record);
   }
