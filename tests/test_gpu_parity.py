@@ -153,33 +153,47 @@ def test_gemv_origin_and_shell13_blocks(gpu_rt, orc):
     _check_gemv(orc, y, raw, x)
 
 
-def test_gemv_tiles_full_of_rare_class_blocks(gpu_rt, orc):
-    """Every block from a class that takes the generic walk (odd with five magnitudes, support weight 0 or
-    24, three word kinds): 640 of them in one tile, ten times what the kernel's queue for such blocks holds,
-    so the overflow path runs too.  Uniform draws meet these classes 0.07 % of the time."""
-    import torch
-
+def _class_ranges(orc, want):
+    """Zero-based rank ranges [lo, hi) of the cap-12 classes that `want(odd, w, vals)` picks."""
     ranges = []
     for ci in range(383):
         info = orc.class_info(ci)
         vals, _, _ = orc.class_levels(ci)
-        if info["shell"] > 12:
-            continue
-        if info["odd"]:
-            rare = len(vals) > 4
-        else:
-            rare = not (info["w"] in (8, 12, 16) and len([v for v in vals if abs(v) % 4 == 2]) <= 2)
-        if rare:
+        if info["shell"] <= 12 and want(info["odd"], info["w"], vals):
             ranges.append((info["lo"], info["hi"]))
-    assert len(ranges) == 30
-    d_out, nb = 16, 40
-    rng = np.random.default_rng(11)
+    return ranges
+
+
+def _is_rare(odd, w, vals):
+    """The classes the kernels unrank by the generic walk: odd with five magnitudes, support weight 0 or 24,
+    three word kinds."""
+    if odd:
+        return len(vals) > 4
+    return not (w in (8, 12, 16) and len([v for v in vals if abs(v) % 4 == 2]) <= 2)
+
+
+def _matrix_of_classes(ranges, d_out, nb, seed, name):
+    rng = np.random.default_rng(seed)
     pick = rng.integers(0, len(ranges), size=d_out * nb)
-    idx = np.array([1 + int(rng.integers(ranges[p][0], ranges[p][1])) for p in pick], np.uint64)  # index = 1 + zero-based rank
+    lo = np.array([r[0] for r in ranges], np.uint64)[pick]
+    span = np.array([r[1] - r[0] for r in ranges], np.uint64)[pick]
+    idx = lo + (rng.integers(0, 1 << 62, size=pick.size, dtype=np.uint64) % span) + np.uint64(1)  # index = 1 + zero-based rank
     gains = rng.integers(0, 2, size=idx.size).astype(np.uint8)
-    raw = artifact.RawMatrix("model.layers.0.rare.weight", d_out, nb * 24, 12, [0.8, 1.25], np.exp(rng.normal(size=d_out)),
-                             np.zeros(0, np.float32), artifact.pack_codes(idx, gains))
-    x = synth.make_activation(nb * 24, seed=12)[0]
+    return artifact.RawMatrix(name, d_out, nb * 24, 12, [0.8, 1.25], np.exp(rng.normal(size=d_out)),
+                              np.zeros(0, np.float32), artifact.pack_codes(idx, gains))
+
+
+def test_gemv_tiles_full_of_rare_class_blocks(gpu_rt, orc):
+    """Every block from a class that takes the generic walk.  2560 rows of 40 blocks make tiles of ten rows:
+    400 such blocks in a tile, six times what the kernel's two side queues for them hold, so the overflow
+    path (the blocks ride in the odd queue, flagged) runs in every tile.  Uniform draws meet these classes
+    0.07 % of the time."""
+    import torch
+
+    ranges = _class_ranges(orc, _is_rare)
+    assert len(ranges) == 30
+    raw = _matrix_of_classes(ranges, 2560, 40, 11, "model.layers.0.rare.weight")
+    x = synth.make_activation(40 * 24, seed=12)[0]
     proj = gpu_rt.upload(raw)
     try:
         y = gpu_rt.forward(proj, _x16(x), out_dtype=torch.float32).cpu().numpy()
@@ -188,7 +202,39 @@ def test_gemv_tiles_full_of_rare_class_blocks(gpu_rt, orc):
     finally:
         gpu_rt.free(proj)
     assert _check_gemv(orc, y, raw, x) < 1e-5
-    _check_gemv(orc, Y[1], raw, x)
+    # the batched path rounds the weights to binary16: 1e-3 of sum|w x|, as tests/test_gpu_gemm.py states it
+    y_ref, a_ref = _oracle_matrix(orc, raw).fused_product(x.astype(np.float64))
+    assert (np.abs(Y[1].astype(np.float64) - y_ref) / np.maximum(a_ref, 1e-30)).max() < 1e-3
+
+
+@pytest.mark.parametrize("share", [1.0, 0.5])
+def test_gemv_tiles_full_of_second_free_kind_blocks(gpu_rt, orc, share):
+    """Even-coset classes whose off-support slots hold two magnitudes besides zero have a decoder and a
+    384-slot queue of their own (6 to 8 % of uniform draws, about 300 of a full tile).  2560 rows of 100 blocks
+    make tiles of 1000 blocks: with every block from such a class 616 of them overflow into the even queue,
+    flagged, in every tile; with half of them plain even-coset blocks the even queue's chunks mix the two."""
+    import torch
+
+    second = _class_ranges(orc, lambda odd, w, vals: not odd and not _is_rare(odd, w, vals)
+                           and len([v for v in vals if v != 0 and abs(v) % 4 == 0]) > 1)
+    plain = _class_ranges(orc, lambda odd, w, vals: not odd and not _is_rare(odd, w, vals)
+                          and len([v for v in vals if v != 0 and abs(v) % 4 == 0]) <= 1)
+    assert second and plain
+    d_out, nb = 2560, 100
+    raw = _matrix_of_classes(second, d_out, nb, 21, "model.layers.0.second.weight")
+    if share < 1.0:
+        other = _matrix_of_classes(plain, d_out, nb, 22, "x")
+        keep = np.random.default_rng(23).random(d_out * nb) < share
+        codes = raw.codes.reshape(-1, 6).copy()
+        codes[~keep] = other.codes.reshape(-1, 6)[~keep]
+        raw = artifact.RawMatrix(raw.name, d_out, nb * 24, 12, [0.8, 1.25], raw.row_scales, np.zeros(0, np.float32), codes.reshape(-1))
+    x = synth.make_activation(nb * 24, seed=24)[0]
+    proj = gpu_rt.upload(raw)
+    try:
+        y = gpu_rt.forward(proj, _x16(x), out_dtype=torch.float32).cpu().numpy()
+    finally:
+        gpu_rt.free(proj)
+    assert _check_gemv(orc, y, raw, x) < 1e-5
 
 
 def test_gemv_config0_full_size(gpu_rt, orc):
