@@ -36,11 +36,13 @@
 // queues), the consumers multiply slice g - 1; so the W buffer written in stage g is
 // complete before it is read in stage g + 1 and is not overwritten before stage g + 2.
 //
-// Every consumer writes its sums to the workspace [band][piece][K-share][m][64]: a
+// A band one workgroup walked alone, by consumers that own a 64-row tile each, is finished
+// where its sums are: row scale, the f32 tail columns (on the matrix cores, f32 operands),
+// the store to y.  Every other sum goes to the workspace [band][piece][K-share][m][64]: a
 // band whose slices fell to several workgroups has one piece from each, and consumers
 // left over by a batch of few 64-row tiles take the same tile on interleaved K-steps.
-// gemm_reduce_kernel adds the partial sums in that fixed order and applies row scale
-// and the f32 tail columns, so the result does not depend on scheduling.
+// gemm_reduce_kernel adds those partial sums in that fixed order and applies row scale
+// and the tail, so the result does not depend on scheduling.
 #pragma once
 
 #include "gemm_share.h"
@@ -188,13 +190,13 @@ __global__ __launch_bounds__(256) void tile_activations_kernel(const __half* x, 
   xt[idx] = (m < M && col < kcols) ? *reinterpret_cast<const uint4*>(x + (size_t)m * ldx + col) : make_uint4(0, 0, 0, 0);
 }
 
-// The launch's slices are numbered band by band, and the workgroups share that sequence out
-// evenly: workgroup c walks slices [g_lo(c), g_hi(c)), `base` or `base + 1` of them, so that the
-// chip is busy whatever the matrix's shape.  A band whose slices fall to several workgroups gets
+// The workgroups share the launch's slices out evenly (gemm_share.h): whole bands first, where there
+// are at least as many bands as workgroups, then consecutive slices of the bands left over, so that
+// the chip is busy whatever the matrix's shape.  A band whose slices fall to several workgroups gets
 // one partial sum from each ("pieces", numbered in workgroup order).  Both roles step through the
 // same slices, the consumers one stage behind.
 struct SliceWalk {
-  uint32_t g;                   // slices walked before this one, counted from the launch's first; valid below the workgroup's g_hi
+  uint32_t t;                   // slices this workgroup walked before this one; valid below its slice count
   uint32_t band, j;             // band, and the slice's place in it: blocks [16 j, 16 j + 16) of every row
   uint32_t run_lo, run_len, si; // this workgroup's slices of the band, and how many of them are done
   uint32_t mat, r0, rows;       // the band's matrix, its first row there, its row count
@@ -215,20 +217,26 @@ struct SliceWalk {
 constexpr int kGemmMaxGroup = 4;
 struct GemmMat {
   const uint8_t* codes;
+  const float* rscale;  // d_out row scales and 64 floats of slack
+  const float* tail;
+  void* y;
   float g0, g1;
   uint32_t d_out, band_begin;
 };
 struct GemmArgs {
   GlobalTables tables;
   const __half* xt;       // [n_steps, m_pad, 32]: tile_activations_kernel's output
-  float* ws;              // [n_bands, max_pieces, kparts, M, 64] partial sums
+  float* ws;              // [n_bands - ws_band0, max_pieces, kparts, M, 64] partial sums
+  const __half* x;        // [M, ldx] the activations as the caller gave them (the tail columns are read from here)
   GemmMat mat[kGemmMaxGroup];
   uint32_t n_mats;
+  uint32_t y_f32;            // output type: binary32, else binary16
+  uint32_t ldx, tail_w;
   uint32_t M, m_pad, nblocks;
   uint32_t n_bands;          // bands of all matrices
   uint32_t spb;              // slices per band
-  uint32_t base, rem;        // workgroup c walks base + (c < rem) slices
-  uint32_t max_pieces;       // workspace slots per band
+  GemmShare share;           // which workgroup walks what (gemm_share.h)
+  uint32_t ws_band0;         // the first band with a place in the workspace
   uint32_t ct_shift;         // log2 of the 64-row activation tiles the consumers spread over
 };
 
@@ -250,7 +258,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
   const uint32_t nb = a.nblocks;
-  const uint32_t g_lo = gemm_first_slice(blockIdx.x, a.base, a.rem), g_hi = gemm_first_slice(blockIdx.x + 1u, a.base, a.rem);
+  const uint32_t n_mine = gemm_slices_of(a.share, a.spb, blockIdx.x);  // slices this workgroup walks
 
   auto enter_band = [&](SliceWalk& w) {
     w.mat = 0;
@@ -264,30 +272,28 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   // run: workgroups that hold the same slices of different bands then do not all pull the same
   // activation columns through the same L2 channels at the same time.
   auto enter_run = [&](SliceWalk& w) {
-    w.run_len = min(a.spb - w.run_lo, g_hi - w.g);
+    const GemmRun r = gemm_run_at(a.share, a.spb, blockIdx.x, w.t);
+    w.band = r.band;
+    w.run_lo = r.lo;
+    w.run_len = r.len;
+    w.piece = r.piece;
     w.si = 0;
     w.j = w.run_lo + (w.band * 5u) % w.run_len;
     enter_band(w);
   };
   auto start_walk = [&](SliceWalk& w) {
-    w.g = g_lo;
-    w.band = g_lo / a.spb;
-    w.run_lo = g_lo - w.band * a.spb;
-    w.piece = blockIdx.x - gemm_owner(w.band * a.spb, a.base, a.rem);
+    w.t = 0;
     enter_run(w);
   };
   auto advance = [&](SliceWalk& w) {
-    ++w.g;
+    ++w.t;
     if (++w.si == w.run_len) {
-      ++w.band;
-      w.run_lo = 0;
-      w.piece = 0;  // this workgroup is the first to reach the next band
-      if (w.g < g_hi) enter_run(w);
+      if (w.t < n_mine) enter_run(w);
     } else {
       w.j = w.j + 1 == w.run_lo + w.run_len ? w.run_lo : w.j + 1;
     }
   };
-  auto live = [&](const SliceWalk& w) { return w.g < g_hi; };
+  auto live = [&](const SliceWalk& w) { return w.t < n_mine; };
   auto slice_blocks = [&](const SliceWalk& w) { return min((uint32_t)kGemmKb, nb - w.j * kGemmKb); };
 
   // Both W buffers start as zeros: a slice shorter than 16 blocks per row leaves columns the
@@ -433,7 +439,12 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       return reinterpret_cast<const uint8_t*>(a.xt) + (size_t)(w.j * (uint32_t)(kGemmKb * 24 / 32) + kpart) * step_bytes;
     };
     half8_t ring[2][2][2];
-    auto fetch = [&](const uint8_t* step, half8_t (&dst)[2][2]) {
+    auto fetch = [&](const uint8_t* step_any, half8_t (&dst)[2][2]) {
+      // the step's address is the same in every lane: said so, it stays in scalar registers and the
+      // loads take it with a 32-bit lane offset
+      const uint64_t bits = reinterpret_cast<uint64_t>(step_any);
+      const uint8_t* step = reinterpret_cast<const uint8_t*>(
+          ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(bits >> 32)) << 32) | (uint32_t)__builtin_amdgcn_readfirstlane((int)bits));
 #pragma unroll
       for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
@@ -517,17 +528,99 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
         // the unit's sums: acc[rt][ct][j] belongs to weight row r0 + 32 rt + 8 (j / 4) + 4 lh + j % 4
         // and activation row m0 + 32 ct + l32
         if (tile_live) {
+          // this lane's activation row and its place in a 64-row result, worked out here: offsets kept
+          // from the kernel's start would cost registers through every stage
+          uint32_t ln;  // this lane's number, asked for here
+          asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+          const uint32_t lane_l = ln & 31u, lane_h = ln >> 5, lane_m = m0 + lane_l, lane_r = 4u * lane_h;
+          if (done.band >= a.ws_band0) {
+            // one of several partial sums of its band: to the workspace
 #pragma unroll
-          for (int ct = 0; ct < 2; ++ct) {
-            const uint32_t my_m = m0 + 32u * ct + l32;
-            if (my_m < a.M) {
-              float* dst = a.ws + ((((size_t)done.band * a.max_pieces + done.piece) * kparts + kpart) * a.M + my_m) * kGemmRows;
+            for (int ct = 0; ct < 2; ++ct) {
+              const uint32_t my_m = lane_m + 32u * ct;
+              if (my_m < a.M) {
+                float* dst = a.ws + ((((size_t)(done.band - a.ws_band0) * a.share.max_pieces + done.piece) * kparts + kpart) * a.M + my_m) * kGemmRows;
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                  for (int j4 = 0; j4 < 4; ++j4)
+                    *reinterpret_cast<float4*>(dst + rt * 32u + 8u * j4 + lane_r) =
+                        make_float4(acc[rt][ct][4 * j4], acc[rt][ct][4 * j4 + 1], acc[rt][ct][4 * j4 + 2], acc[rt][ct][4 * j4 + 3]);
+              }
+            }
+          } else {
+            // the band's only sums (walked alone, and this consumer owns its tile's every K-step): finished here
+            const GemmMat& mt = a.mat[done.mat];
+            // row scale, four rows at a time (past a short last band's rows the array has 64 floats of slack)
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+              for (int j4 = 0; j4 < 4; ++j4) {
+                const float4 rs = *reinterpret_cast<const float4*>(mt.rscale + done.r0 + 32u * rt + 8u * j4 + lane_r);
+#pragma unroll
+                for (int ct = 0; ct < 2; ++ct) {
+                  acc[rt][ct][4 * j4] *= rs.x;
+                  acc[rt][ct][4 * j4 + 1] *= rs.y;
+                  acc[rt][ct][4 * j4 + 2] *= rs.z;
+                  acc[rt][ct][4 * j4 + 3] *= rs.w;
+                }
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+            // the f32 tail columns, two at a time: v_mfma_f32_32x32x2_f32 takes row l32, column lh of
+            // the weights and column l32, row lh of the activations
+            const uint32_t tw = a.tail_w;
+            for (uint32_t t0 = 0; t0 < tw; t0 += 2) {
+              const uint32_t t = t0 + lane_h;
+              float av[2], bv[2];
+#pragma unroll
+              for (int rt = 0; rt < 2; ++rt) {
+                const uint32_t r = 32u * rt + lane_l;
+                av[rt] = (t < tw && r < done.rows) ? mt.tail[(done.r0 + r) * tw + t] : 0.f;
+              }
+#pragma unroll
+              for (int ct = 0; ct < 2; ++ct) {
+                const uint32_t my_m = lane_m + 32u * ct;
+                bv[ct] = (t < tw && my_m < a.M) ? __half2float(a.x[my_m * a.ldx + nb * 24u + t]) : 0.f;
+              }
 #pragma unroll
               for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-                for (int j4 = 0; j4 < 4; ++j4)
-                  *reinterpret_cast<float4*>(dst + rt * 32u + 8u * j4 + 4u * lh) =
-                      make_float4(acc[rt][ct][4 * j4], acc[rt][ct][4 * j4 + 1], acc[rt][ct][4 * j4 + 2], acc[rt][ct][4 * j4 + 3]);
+                for (int ct = 0; ct < 2; ++ct) acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[rt], bv[ct], acc[rt][ct], 0, 0, 0);
+            }
+            const bool vec = (mt.d_out & 3u) == 0;
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct) {
+              const uint32_t my_m = lane_m + 32u * ct;
+              if (my_m < a.M) {
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                  for (int j4 = 0; j4 < 4; ++j4) {
+                    const uint32_t row = 32u * rt + 8u * j4 + lane_r;
+                    const size_t at = (size_t)my_m * mt.d_out + done.r0 + row;
+                    const float v0 = acc[rt][ct][4 * j4], v1 = acc[rt][ct][4 * j4 + 1], v2 = acc[rt][ct][4 * j4 + 2], v3 = acc[rt][ct][4 * j4 + 3];
+                    if (vec && row + 3u < done.rows) {
+                      if (a.y_f32) {
+                        *reinterpret_cast<float4*>(reinterpret_cast<float*>(mt.y) + at) = make_float4(v0, v1, v2, v3);
+                      } else {
+                        const __half2 lo = __float22half2_rn(make_float2(v0, v1)), hi = __float22half2_rn(make_float2(v2, v3));
+                        uint2 pk;
+                        pk.x = *reinterpret_cast<const uint32_t*>(&lo);
+                        pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+                        *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(mt.y) + at) = pk;
+                      }
+                    } else {
+                      const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+                      for (int i = 0; i < 4; ++i)
+                        if (row + i < done.rows) {
+                          if (a.y_f32) store_y<float>(mt.y, at + i, v[i]);
+                          else store_y<__half>(mt.y, at + i, v[i]);
+                        }
+                    }
+                  }
+              }
             }
           }
         }
@@ -538,8 +631,8 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
   }
 }
 
-// Second pass of a split launch: y[m][r] = (sum over splits, in split order, of the
-// partial sums) * rscale[r] + tail[r] . x_tail[m].  One workgroup per (band, 16
+// Second pass, for the bands that have partial sums in the workspace: y[m][r] = (their sum, in
+// index order) * rscale[r] + tail[r] . x_tail[m].  One workgroup per (band, 16
 // activation rows), one lane per four consecutive weight rows of one activation row;
 // the band's tail weights and the activation tails are staged in LDS once, and the
 // partial sums are read with all their loads in flight (eight splits at a time).
@@ -550,12 +643,13 @@ struct GemmReduceMat {
   uint32_t d_out, band_begin;
 };
 struct GemmReduceArgs {
-  const float* ws;  // [n_bands, max_pieces, kparts, M, 64]
+  const float* ws;  // [n_bands - ws_band0, max_pieces, kparts, M, 64]
   const __half* x;  // [M, ldx]
   GemmReduceMat mat[kGemmMaxGroup];
   uint32_t n_mats;
   uint32_t M, ldx, nblocks, tail_w, n_bands;
-  uint32_t spb, base, rem, max_pieces, kparts;  // as in GemmArgs: which workgroups fed a band
+  uint32_t spb, kparts, ws_band0;  // as in GemmArgs: which workgroups fed a band, and the bands that have partial sums
+  GemmShare share;
 };
 
 constexpr int kReduceRowsM = 16;  // activation rows per workgroup
@@ -565,7 +659,7 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
   __shared__ float tl[kGemmRows * kDim];            // [row][pitch], pitch odd
   __shared__ float xt[kReduceRowsM * (kDim - 1)];   // [m][tail_w]
   const uint32_t mchunks = (a.M + kReduceRowsM - 1) / kReduceRowsM;
-  const uint32_t band = blockIdx.x / mchunks, mc = blockIdx.x - band * mchunks;
+  const uint32_t wsb = blockIdx.x / mchunks, mc = blockIdx.x - wsb * mchunks, band = a.ws_band0 + wsb;
   uint32_t mi = 0;
 #pragma unroll
   for (uint32_t k = 1; k < (uint32_t)kGemmMaxGroup; ++k)
@@ -575,6 +669,15 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
   const uint32_t tw = a.tail_w, pitch = tw | 1u;
   const uint32_t tid = threadIdx.x, quad = tid & 15u, ml = tid >> 4;
   const uint32_t m = mc * kReduceRowsM + ml, row = quad * 4u;
+  // the band's partial sums: one per workgroup that walked some of its slices, times the K-step shares.
+  // The first eight are requested before the tail operands are staged (the two do not depend on each
+  // other, and each is a trip to memory); every load is unconditional, from a valid slot.
+  const uint32_t n_sums = gemm_pieces_of(a.share, a.spb, band) * a.kparts;
+  const size_t sstride = (size_t)a.M * kGemmRows;
+  const float* src = a.ws + ((size_t)wsb * a.share.max_pieces * a.kparts * a.M + min(m, a.M - 1u)) * kGemmRows + row;
+  float4 p[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) p[u] = *reinterpret_cast<const float4*>(src + (size_t)min((uint32_t)u, n_sums - 1u) * sstride);
   for (uint32_t o = tid; o < rows * tw; o += 256) {
     const uint32_t r = o / tw, t = o - r * tw;
     tl[r * pitch + t] = mt.tail[(size_t)r0 * tw + o];
@@ -585,16 +688,12 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
   }
   __syncthreads();
   if (m >= a.M || row >= rows) return;
-  // the band's partial sums: one per workgroup that walked some of its slices, times the K-step shares
-  const uint32_t n_sums = (gemm_owner((band + 1u) * a.spb - 1u, a.base, a.rem) - gemm_owner(band * a.spb, a.base, a.rem) + 1u) * a.kparts;
-  const size_t sstride = (size_t)a.M * kGemmRows;
-  const float* src = a.ws + ((size_t)band * a.max_pieces * a.kparts * a.M + m) * kGemmRows + row;
   float sum[4] = {0.f, 0.f, 0.f, 0.f};
   for (uint32_t s0 = 0; s0 < n_sums; s0 += 8) {
-    float4 p[8];
+    if (s0) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
-      p[u] = s0 + u < n_sums ? *reinterpret_cast<const float4*>(src + (size_t)(s0 + u) * sstride) : make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int u = 0; u < 8; ++u) p[u] = *reinterpret_cast<const float4*>(src + (size_t)min(s0 + u, n_sums - 1u) * sstride);
+    }
 #pragma unroll
     for (int u = 0; u < 8; ++u)
       if (s0 + u < n_sums) {

@@ -1481,12 +1481,14 @@ static int upload_impl(llvq_rt* rt, const std::string& name, uint32_t d_out, uin
   if ((e = hipMalloc(reinterpret_cast<void**>(&m->codes), code_alloc)) != hipSuccess) return cleanup(e, "hipMalloc(codes)");
   if ((e = hipMemset(m->codes, 0, code_alloc)) != hipSuccess) return cleanup(e, "hipMemset(codes)");
   if (code_len && (e = hipMemcpy(m->codes, codes, code_len, hipMemcpyHostToDevice)) != hipSuccess) return cleanup(e, "hipMemcpy(codes)");
-  if ((e = hipMalloc(reinterpret_cast<void**>(&m->rscale), d_out * sizeof(float))) != hipSuccess) return cleanup(e, "hipMalloc(rscale)");
-  if ((e = hipMemcpy(m->rscale, rs.data(), d_out * sizeof(float), hipMemcpyHostToDevice)) != hipSuccess) return cleanup(e, "hipMemcpy(rscale)");
+  // 64 floats of slack: the batched kernel reads the scales of a whole 64-row band, four at a time
+  rs.resize((size_t)d_out + 64, 0.f);
+  if ((e = hipMalloc(reinterpret_cast<void**>(&m->rscale), rs.size() * sizeof(float))) != hipSuccess) return cleanup(e, "hipMalloc(rscale)");
+  if ((e = hipMemcpy(m->rscale, rs.data(), rs.size() * sizeof(float), hipMemcpyHostToDevice)) != hipSuccess) return cleanup(e, "hipMemcpy(rscale)");
   // zero-length arrays become one-element dummies (fused_cuda.rs:1084-1098)
   if ((e = hipMalloc(reinterpret_cast<void**>(&m->tail), tail_len ? tail_len : sizeof(float))) != hipSuccess) return cleanup(e, "hipMalloc(tail)");
   if (tail_len && (e = hipMemcpy(m->tail, tail, tail_len, hipMemcpyHostToDevice)) != hipSuccess) return cleanup(e, "hipMemcpy(tail)");
-  m->device_bytes = code_alloc + d_out * sizeof(float) + (tail_len ? tail_len : sizeof(float));
+  m->device_bytes = code_alloc + rs.size() * sizeof(float) + (tail_len ? tail_len : sizeof(float));
   m->encoded_bytes = code_len + (uint64_t)d_out * 8 + tail_len + 16;
   *out = m;
   return LLVQ_OK;
@@ -1894,11 +1896,12 @@ static void gemm_workspace_bytes(const llvq_rt* rt, const llvq_mat* const* mats,
   while (((uint32_t)kGemmColTile << ct_shift) < M) ++ct_shift;
   const uint32_t kparts = consumers >> ct_shift;
   const uint32_t spb = (m0->nblocks + kGemmKb - 1) / kGemmKb;
-  const uint64_t total = (uint64_t)n_bands * spb;
-  const GemmShare share = gemm_share(total ? total : 1, spb ? spb : 1, grid_cap);
+  const GemmShare share = gemm_share(n_bands ? n_bands : 1, spb ? spb : 1, grid_cap);
+  // bands walked by one workgroup alone are finished in the launch when every consumer owns its tile's every K-step
+  const uint32_t ws_band0 = kparts == 1 ? share.shared0 : 0u;
   const uint32_t m_pad = (M + kGemmColTile - 1) / kGemmColTile * kGemmColTile;
   const uint32_t n_steps = spb * (kGemmKb * 24 / 32);
-  *ws_bytes = (size_t)n_bands * share.max_pieces * kparts * M * kGemmRows * sizeof(float);
+  *ws_bytes = (size_t)(n_bands - (ws_band0 < n_bands ? ws_band0 : n_bands)) * share.max_pieces * kparts * M * kGemmRows * sizeof(float);
   *xt_bytes = (size_t)n_steps * m_pad * 64;
 }
 
@@ -1949,10 +1952,14 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   a.tables = rt->tables;
   a.n_mats = r.n_mats = (uint32_t)n;
   for (int i = 0; i < n; ++i) {
-    a.mat[i] = GemmMat{mats[i]->codes, mats[i]->g[0], mats[i]->g[1], mats[i]->d_out, a.n_bands};
+    a.mat[i] = GemmMat{mats[i]->codes, mats[i]->rscale, mats[i]->tail, y[i], mats[i]->g[0], mats[i]->g[1], mats[i]->d_out, a.n_bands};
     r.mat[i] = GemmReduceMat{mats[i]->rscale, mats[i]->tail, y[i], mats[i]->d_out, a.n_bands};
     a.n_bands += (mats[i]->d_out + kGemmRows - 1) / kGemmRows;
   }
+  a.y_f32 = f32 ? 1u : 0u;
+  a.x = xh;
+  a.ldx = m0->d_in;
+  a.tail_w = m0->tail_w;
   a.M = M;
   a.m_pad = (M + kGemmColTile - 1) / kGemmColTile * kGemmColTile;
   a.nblocks = m0->nblocks;
@@ -1966,19 +1973,21 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   a.spb = (m0->nblocks + kGemmKb - 1) / kGemmKb;
   const uint64_t total = (uint64_t)a.n_bands * a.spb;
   if (total > 0xFFFFFFFFull) return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": too many K-slices for one batched launch");
-  const GemmShare share = gemm_share(total, a.spb, grid_cap);
+  const GemmShare share = gemm_share(a.n_bands, a.spb, grid_cap);
+  if (!gemm_share_exact(share, a.n_bands, a.spb)) return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": rows too wide for the batched launch's slice arithmetic");
   const uint32_t n_wg = share.n_wg;
-  a.base = share.base;
-  a.rem = share.rem;
-  a.max_pieces = share.max_pieces;
+  a.share = share;
+  a.ws_band0 = kparts == 1 ? share.shared0 : 0u;
+  const uint32_t ws_bands = a.n_bands - a.ws_band0;  // bands with partial sums in the workspace
   void* ws_buf = nullptr;
   void* xt_buf = nullptr;
   const size_t mark = wsp ? wsp->used : 0;  // a launch's carvings are released when it has been enqueued: the stream orders the next
   size_t ws_bytes = 0, xt_bytes = 0;
   gemm_workspace_bytes(rt, mats, n, M, &ws_bytes, &xt_bytes);
-  if (ws_bytes != (size_t)a.n_bands * a.max_pieces * kparts * M * kGemmRows * sizeof(float))
+  if (ws_bytes != (size_t)ws_bands * share.max_pieces * kparts * M * kGemmRows * sizeof(float))
     return fail(LLVQ_ERR_DEVICE, "gemm: workspace sizing disagrees with the launch");
-  int rc = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes, ws_bytes, &ws_buf);
+  int rc = LLVQ_OK;
+  if (ws_bytes) rc = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->gemm_ws), &rt->gemm_ws_bytes, ws_bytes, &ws_buf);
   if (rc) return rc;
   // every slice has all its twelve K-steps in the tiled copy, zeros past the matrix's last block
   const uint32_t n_steps = (m0->nblocks + kGemmKb - 1) / kGemmKb * (kGemmKb * 24 / 32);
@@ -2003,11 +2012,11 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   r.tail_w = m0->tail_w;
   r.n_bands = a.n_bands;
   r.spb = a.spb;
-  r.base = a.base;
-  r.rem = a.rem;
-  r.max_pieces = a.max_pieces;
+  r.share = share;
+  r.ws_band0 = a.ws_band0;
   r.kparts = kparts;
-  const uint32_t rgrid = a.n_bands * ((M + kReduceRowsM - 1) / kReduceRowsM);
+  if (ws_bands == 0) return LLVQ_OK;  // every band was finished by the workgroup that walked it
+  const uint32_t rgrid = ws_bands * ((M + kReduceRowsM - 1) / kReduceRowsM);
   if (f32) hipLaunchKernelGGL(gemm_reduce_kernel<float>, dim3(rgrid), dim3(256), 0, rt->stream, r);
   else hipLaunchKernelGGL(gemm_reduce_kernel<__half>, dim3(rgrid), dim3(256), 0, rt->stream, r);
   HIP_TRY(hipGetLastError());

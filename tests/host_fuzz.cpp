@@ -149,21 +149,46 @@ int main(int argc, char** argv) {
   // slices, loads differ by at most one, and no band receives more partial sums than the workspace holds
   size_t shares = 0;
   for (uint32_t cap : {1u, 3u, 256u, 304u})
-    for (uint32_t spb : {1u, 2u, 7u, 11u, 26u, 32u, 46u})
+    for (uint32_t spb : {1u, 2u, 7u, 11u, 26u, 32u, 46u, 683u})
       for (uint32_t bands : {1u, 2u, 5u, 16u, 40u, 96u, 192u, 255u, 256u, 257u, 304u, 1000u}) {
         const uint64_t total = (uint64_t)bands * spb;
-        const GemmShare sh = gemm_share(total, spb, cap);
-        if (sh.n_wg == 0 || sh.n_wg > cap || sh.n_wg > total || sh.base == 0) { std::fprintf(stderr, "share: bad workgroup count\n"); return 5; }
-        if (gemm_first_slice(0, sh.base, sh.rem) != 0 || gemm_first_slice(sh.n_wg, sh.base, sh.rem) != total) { std::fprintf(stderr, "share: slices not covered\n"); return 5; }
+        const GemmShare sh = gemm_share(bands, spb, cap);
+        if (sh.n_wg == 0 || sh.n_wg > cap || sh.n_wg > total) { std::fprintf(stderr, "share: bad workgroup count\n"); return 5; }
+        if (sh.shared0 != sh.whole * sh.n_wg || sh.shared0 > bands || bands - sh.shared0 >= sh.n_wg) { std::fprintf(stderr, "share: bands walked alone\n"); return 5; }
+        const uint64_t left = (uint64_t)(bands - sh.shared0) * spb;
+        if (!gemm_share_exact(sh, bands, spb)) { std::fprintf(stderr, "share: multipliers not exact\n"); return 5; }
+        // the multipliers against plain division, over every dividend the walk can form
+        for (uint32_t nq = 0; nq <= (uint32_t)left + spb; ++nq)
+          if (share_div(nq, sh.inv_spb) != nq / spb || share_div(nq, sh.inv_base1) != nq / (sh.base + 1u) ||
+              (sh.base && share_div(nq, sh.inv_base) != nq / sh.base)) { std::fprintf(stderr, "share: multiplier wrong at %u\n", nq); return 5; }
+        if (gemm_first_slice(0, sh.base, sh.rem) != 0 || gemm_first_slice(sh.n_wg, sh.base, sh.rem) != left) { std::fprintf(stderr, "share: slices not covered\n"); return 5; }
+        // every workgroup's walk, run by run as the kernel walks it: each slice of each band exactly once, pieces numbered
+        // 0.. in workgroup order, loads within one slice of each other
+        std::vector<uint8_t> seen((size_t)total, 0);
+        std::vector<uint32_t> pieces_seen(bands, 0);
+        uint32_t lo_load = ~0u, hi_load = 0;
         for (uint32_t c = 0; c < sh.n_wg; ++c) {
-          const uint32_t lo = gemm_first_slice(c, sh.base, sh.rem), hi = gemm_first_slice(c + 1, sh.base, sh.rem);
-          if (hi - lo != sh.base + (c < sh.rem ? 1u : 0u)) { std::fprintf(stderr, "share: uneven load\n"); return 5; }
-          if (gemm_owner(lo, sh.base, sh.rem) != c || gemm_owner(hi - 1, sh.base, sh.rem) != c) { std::fprintf(stderr, "share: owner of a slice\n"); return 5; }
+          const uint32_t n = gemm_slices_of(sh, spb, c);
+          lo_load = n < lo_load ? n : lo_load;
+          hi_load = n > hi_load ? n : hi_load;
+          for (uint32_t t = 0; t < n;) {
+            const GemmRun r = gemm_run_at(sh, spb, c, t);
+            if (r.band >= bands || r.len == 0 || r.lo + r.len > spb || t + r.len > n) { std::fprintf(stderr, "share: run out of range\n"); return 5; }
+            if (r.band < sh.shared0 && (r.lo != 0 || r.len != spb || r.piece != 0)) { std::fprintf(stderr, "share: a band walked alone is not whole\n"); return 5; }
+            if (r.piece != pieces_seen[r.band]++) { std::fprintf(stderr, "share: piece numbering\n"); return 5; }
+            for (uint32_t k = 0; k < r.len; ++k)
+              if (seen[(size_t)r.band * spb + r.lo + k]++) { std::fprintf(stderr, "share: slice walked twice\n"); return 5; }
+            t += r.len;
+          }
         }
-        for (uint32_t b = 0; b < bands; ++b) {
-          const uint32_t pieces = gemm_owner((b + 1) * spb - 1, sh.base, sh.rem) - gemm_owner(b * spb, sh.base, sh.rem) + 1;
-          if (pieces > sh.max_pieces) { std::fprintf(stderr, "share: %u pieces in a band, %u slots\n", pieces, sh.max_pieces); return 5; }
-        }
+        if (hi_load - lo_load > 1) { std::fprintf(stderr, "share: uneven load\n"); return 5; }
+        for (uint64_t k = 0; k < total; ++k)
+          if (!seen[(size_t)k]) { std::fprintf(stderr, "share: slice not walked\n"); return 5; }
+        for (uint32_t b = 0; b < bands; ++b)
+          if (pieces_seen[b] != gemm_pieces_of(sh, spb, b) || pieces_seen[b] > sh.max_pieces) {
+            std::fprintf(stderr, "share: %u pieces in band %u, formula %u, %u slots\n", pieces_seen[b], b, gemm_pieces_of(sh, spb, b), sh.max_pieces);
+            return 5;
+          }
         ++shares;
       }
   std::printf("ok: %zu records in the whole file, %zu hostile inputs, %zu decodable ranks, %zu rotations, %zu work shares\n", whole, cases, valid, rotations, shares);
