@@ -237,6 +237,65 @@ def test_gemv_tiles_full_of_second_free_kind_blocks(gpu_rt, orc, share):
     assert _check_gemv(orc, y, raw, x) < 1e-5
 
 
+def test_gemv_kernel_unranks_every_coordinate_exactly(gpu_rt, orc, boundary_indices):
+    """The lattice points as the product kernels themselves unrank them (their own class find, queues and
+    decoders, not the probe kernel's): one-hot activations read the matrix back column by column, and
+    every one of the 24 coordinates of 163 840 blocks must be the oracle's integer — class boundaries,
+    the rare classes, the classes with a second free kind, uniform cap-12 ranks and ranks over the whole
+    47-bit field (shell 13), origins, both gain bits."""
+    import torch
+
+    d_out, nb = 4096, 40
+    n = d_out * nb
+    rng = synth.SplitMix64(0x5EED)
+    idx = rng.take(n) % np.uint64(orc.N12 + 1)
+    wide = rng.take(n // 8) % np.uint64(1 << 47)
+    idx[: wide.size] = wide
+    b = boundary_indices[boundary_indices < (1 << 47)]
+    idx[wide.size: wide.size + b.size] = b
+    at = wide.size + b.size
+    for want, count in ((_is_rare, 4000), (lambda odd, w, vals: not odd and not _is_rare(odd, w, vals)
+                                           and len([v for v in vals if v != 0 and abs(v) % 4 == 0]) > 1, 8000)):
+        ranges = _class_ranges(orc, want)
+        pick = np.random.default_rng(count).integers(0, len(ranges), size=count)
+        lo = np.array([r[0] for r in ranges], np.uint64)[pick]
+        span = np.array([r[1] - r[0] for r in ranges], np.uint64)[pick]
+        idx[at: at + count] = lo + (rng.take(count) % span) + np.uint64(1)
+        at += count
+    idx[at: at + 64] = 0  # origins
+    perm = np.random.default_rng(9).permutation(n)  # every tile gets its share of every kind
+    idx = idx[perm]
+    gains = (rng.take(n) & np.uint64(1)).astype(np.uint8)
+    cent = [0.75, 1.5]
+    raw = artifact.RawMatrix("model.layers.0.coords.weight", d_out, nb * 24, 12, cent, np.ones(d_out), np.zeros(0, np.float32),
+                             artifact.pack_codes(idx, gains))
+    proj = gpu_rt.upload(raw)
+    try:
+        eye = torch.eye(nb * 24, dtype=torch.float16, device="cuda")
+        cols = [gpu_rt.forward(proj, eye[c], out_dtype=torch.float32).reshape(-1) for c in range(nb * 24)]
+        W = torch.stack(cols).t().contiguous().cpu().numpy().astype(np.float64)  # [d_out, d_in]
+        # the batched kernel's producers unrank on their own: the identity as 960 activation rows reads the matrix back too
+        Wb = gpu_rt.forward_batched(proj, eye, out_dtype=torch.float32).t().contiguous().cpu().numpy().astype(np.float64)
+    finally:
+        gpu_rt.free(proj)
+    pts = orc.decode_many(idx).astype(np.int64)  # [n, 24]
+    n2 = (pts * pts).sum(axis=1).astype(np.float64)
+    scale = np.where(n2 > 0, np.array(cent)[gains] / np.sqrt(np.maximum(n2, 1.0)), 0.0)
+    got = W.reshape(n, 24)
+    zero = n2 == 0
+    assert zero.sum() >= 64 and np.all(got[zero] == 0.0)
+    back = got[~zero] / scale[~zero, None]
+    assert np.abs(back - np.rint(back)).max() < 1e-3
+    assert np.array_equal(np.rint(back).astype(np.int64), pts[~zero])
+    # batched path: a weight is rounded once to binary16 (2^-11 relative, under 0.02 for coordinates below 32), so the
+    # integers are still unambiguous
+    gotb = Wb.reshape(n, 24)
+    assert np.all(gotb[zero] == 0.0)
+    backb = gotb[~zero] / scale[~zero, None]
+    assert np.abs(backb - np.rint(backb)).max() < 0.02
+    assert np.array_equal(np.rint(backb).astype(np.int64), pts[~zero])
+
+
 def test_gemv_config0_full_size(gpu_rt, orc):
     """BASELINE config 0: gate_proj 9728 x 2560, seed 0, against the oracle's f64 product."""
     import torch
