@@ -160,16 +160,19 @@ __global__ __launch_bounds__(256) void decode_blocks_kernel(GlobalTables g, cons
 // One persistent 1024-lane workgroup per CU.  The rows of up to four matrices
 // that share an activation are cut into tiles of at most kTileBlocks blocks; a
 // workgroup takes tiles round-robin and runs four phases on each:
-//   P0  copy the tile's code bytes from HBM to LDS with 16-byte loads;
-//   P1  one lane per block: find the block's class and push the block onto the
-//       odd-coset or the even-coset queue (the two decoders are different
-//       straight-line programs; binning keeps every lane of a wavefront on the
-//       same one); blocks of the rare generic classes are decoded on the spot;
+//   P0  every lane loads its own four consecutive 6-byte records from HBM into
+//       registers (issued a tile ahead; the records never pass through LDS);
+//   P1  the lane parses them, finds each block's class (two table probes and a
+//       comparison) and queues the block with its rank within the class: odd
+//       coset, even coset, and even-coset classes with a second free kind each
+//       have a queue, because they are different straight-line programs and
+//       binning keeps every lane of a wavefront on the same one; blocks of the
+//       rare generic classes go to two small side queues;
 //   P2  wavefronts take 64 queued blocks at a time, unrank them to 8-bit
 //       coordinates, reduce them against the activation with integer dot
 //       products and write one partial sum per block;
-//   P3  one wavefront per row adds the row's partial sums in a fixed order,
-//       applies the row scale and the tail columns, and stores y.
+//   P3  sixteen lanes per row add the row's partial sums in a fixed order,
+//       apply the row scale and the tail columns, and store y.
 // Results do not depend on the queue order, so they are reproducible.
 //
 // The activation is held in LDS as block-scaled fixed point: per 24-column
