@@ -467,7 +467,7 @@ __device__ __forceinline__ void prefetch_records(const GroupArgs& a, uint32_t ti
   const uint32_t share = (uint32_t)NB * 6u;
   const uint32_t at = tid * (uint32_t)NB < rows * a.nblocks ? tid * share : 0u;
   const uint8_t* src = M.codes + (size_t)r0 * a.nblocks * 6 + at;
-  // streaming loads: the code bytes are read once, and must not push the decode tables out of L2
+  // streaming loads: the code bytes are read once
   if constexpr (NB == 4) {
     const dwords4_a2 lo = __builtin_nontemporal_load(reinterpret_cast<const dwords4_a2*>(src));
     const dwords2_a2 hi = __builtin_nontemporal_load(reinterpret_cast<const dwords2_a2*>(src + 16));
@@ -802,7 +802,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const __half* xsrc = a.x;
   // A launch over matrices stored in a rotated basis rotates its activation itself: the
-  // values go, signs applied, as f32 to the area the first tile's code bytes, queues and
+  // values go, signs applied, as f32 to the area the first tile's queues and
   // partial sums will use (free until then), are rotated there and quantised from there.
   const bool rotated = ROT && a.rot_m != 0;
   float* xf = reinterpret_cast<float*>(raw);
@@ -811,7 +811,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   if (a.prologue != kPrologueNone) {
     // Every workgroup derives the activation for itself (a few thousand values)
     // instead of waiting for a kernel of its own; it is staged, as binary16, where
-    // the tile's code bytes will go.
+    // the tile's queues will go.
     __half* xs = reinterpret_cast<__half*>(raw);
     // All of a lane's values are requested before the first is used (a load and its use per loop
     // iteration would pay the memory latency once per iteration): the rounds are counted at compile
@@ -939,7 +939,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       else quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     }
   }
-  if (a.prologue != kPrologueNone || rotated) __syncthreads();  // the staging area becomes the code-byte buffer
+  if (a.prologue != kPrologueNone || rotated) __syncthreads();  // the staging area becomes the tile's queues
 
 #ifdef LLVQ_PHASE_TIMING
   if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 7] = wall_clock64();
@@ -1647,7 +1647,7 @@ static uint32_t pick_rows_per_tile(const llvq_mat* const* mats, int n, uint32_t 
 }
 
 // Whether a launch over rows of this width can stage a derived activation where
-// its tile's code bytes go.
+// its first tile's queues go.
 struct GemvShape {
   uint32_t tile;
   bool lean;
@@ -1669,7 +1669,7 @@ static bool prologue_fits(const llvq_mat* m0) {
 }
 
 // Whether a launch over rows of this width can rotate its own activation: the f32
-// values take the place of the first tile's code bytes, queue and partial sums.
+// values take the place of the first tile's queues and partial sums.
 static bool rotation_fits(const llvq_mat* m0) {
   const size_t tile = pick_gemv_shape(m0->nblocks).tile;
   return (size_t)m0->d_in * 4 + 64 <= tile * 6 + 32 + tile * 8;
