@@ -257,6 +257,37 @@ def test_gemm_group_matches_the_oracle_and_the_single_calls(gpu_rt, orc):
             gpu_rt.free(p)
 
 
+@pytest.mark.parametrize("M", [130, 257])
+def test_gemm_bands_finished_in_the_launch(gpu_rt, orc, M):
+    """More 64-row bands than workgroups: every workgroup walks whole bands alone and, where each
+    multiplying wavefront owns a tile's every K-step (M > 128), finishes them in the launch — row scale,
+    f32 tail, store — while the bands left over go through the workspace and the sum pass.  Three matrices
+    in one call (299 bands, the first 256 walked alone), so that a short last band (6 rows), row counts
+    that are no multiple of four (scalar stores) and tail columns all meet the in-launch epilogue, and a
+    57-row band the sum pass; f32 and f16 outputs against the oracle."""
+    import torch
+
+    d_in = 88  # three blocks and 16 tail columns: one slice per band
+    d_outs = [70, 16441, 2500]
+    raws = [synth.make_matrix(f"model.layers.0.alone{i}.weight", d, d_in, seed=80 + i) for i, d in enumerate(d_outs)]
+    X = synth.make_activation(d_in, seed=M, rows=M)
+    projs = [gpu_rt.upload(r) for r in raws]
+    try:
+        xd = _x16(X)
+        for dtype in (torch.float32, torch.float16):
+            ys = [torch.full((M, d), float("nan"), dtype=dtype, device="cuda") for d in d_outs]
+            gpu_rt.forward_batched_group_into(projs, xd, ys)
+            again = [torch.empty_like(y) for y in ys]
+            gpu_rt.forward_batched_group_into(projs, xd, again)
+            for raw, y, y2 in zip(raws, ys, again):
+                Y_ref, A_ref = _reference(orc, raw, X)
+                _check(y.float().cpu().numpy(), Y_ref, A_ref, out_rounding=0.0 if dtype == torch.float32 else 2.0 ** -11)
+                assert torch.equal(y, y2)
+    finally:
+        for p in projs:
+            gpu_rt.free(p)
+
+
 def test_reserved_workspaces_change_nothing(gpu_rt):
     """llvq_hip_reserve_batched only sizes buffers: the products before and after it are identical, for
     the group it was told about and at fewer rows than it was told."""
