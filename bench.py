@@ -29,9 +29,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 
-# HBM-side bytes per gemv_tiles_kernel launch come from rocprofv3 --pmc runs of this command (FETCH_SIZE,
+# HBM-side bytes per gemv_seq_kernel launch come from rocprofv3 --pmc runs of this command (FETCH_SIZE,
 # WRITE_SIZE); the summary of those runs is this file, whose machine-readable lines bench.py reads back
-TRAFFIC_PROFILE = os.path.join("profiles", "gemv_tiles_kernel_qwen3-4b-projections_counters.txt")
+TRAFFIC_PROFILE = os.path.join("profiles", "gemv_seq_kernel_qwen3-4b-projections_counters.txt")
 
 
 def profiled(path=None):
@@ -386,37 +386,50 @@ def main():
     n_blocks = code_bytes // 6
     n_launch = sum(len(p) for p in projs)
 
-    # one pre-bound launch per activation site: q/k/v, o, gate/up, down
-    launches, outputs = [], []
+    # one item per activation site: q/k/v, o, gate/up, down — bound once as a sequence (one persistent launch per
+    # step) and, for comparison, as one pre-bound launch each (the per-call entry point, 144 launches per step)
+    launches, outputs, items = [], [], []
     for lp in projs:
         q, k, v, o, gate, up, down = lp
         for group, d in (([q, k, v], 2560), ([o], 4096), ([gate, up], 2560), ([down], 9728)):
             launch, ys = rt.plan_group(group, acts[d])
             launches.append(launch)
             outputs.append(ys)
+            items.append((group, acts[d], False))
     n_kernels = len(launches)
-    # layer 0's results, taken before anything is timed, for the check against the CPU oracle
-    for launch in launches[:4]:
+    seq = rt.plan_sequence(items)
+    # layer 0's results, taken before anything is timed, for the check against the CPU oracle; the sequence
+    # must give the per-call results bit for bit
+    for launch in launches:
         launch()
-    torch.cuda.synchronize()
-    y_layer0 = [y.float().cpu().numpy() for ys in outputs[:4] for y in ys]
+    seq.run()
+    seq.status()
+    for ys, zs in zip(outputs, seq.outputs):
+        for y, z in zip(ys, zs):
+            if not torch.equal(y.view(torch.int16), z.view(torch.int16)):
+                raise SystemExit("[bench] the sequence's outputs differ from the per-call outputs")
+    y_layer0 = [y.float().cpu().numpy() for ys in seq.outputs[:4] for y in ys]
 
-    def step():
+    def timed(step_fn, steps, warmup):
+        for _ in range(warmup):
+            step_fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            step_fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, e0.elapsed_time(e1)
+
+    def per_call_step():
         for launch in launches:
             launch()
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    dev_ms = ev0.elapsed_time(ev1)
+    pc_wall, pc_dev_ms = timed(per_call_step, args.steps, args.warmup)
+    wall, dev_ms = timed(seq.run, args.steps, args.warmup)
+    seq.status()
     ms_per_step = wall * 1e3 / args.steps
     gbps = enc_bytes * args.steps / wall / 1e9
 
@@ -433,8 +446,9 @@ def main():
     torch.cuda.synchronize()
     cache_gbps = one_layer_bytes * reps / (c0.elapsed_time(c1) * 1e-3) / 1e9
 
-    avg_launch_us = dev_ms * 1e3 / (args.steps * n_kernels)
+    avg_launch_us = dev_ms * 1e3 / args.steps  # one launch of gemv_seq_kernel per step
     achieved = enc_bytes * args.steps / (dev_ms * 1e-3) / 1e9
+    pc_achieved = enc_bytes * args.steps / (pc_dev_ms * 1e-3) / 1e9
     # traffic and the VALU figures are those of the committed counter summary, taken with this command; they
     # only stand while this run's kernel time agrees with the profiled one (5 %) on the profiled workload
     prof = profiled()
@@ -466,7 +480,7 @@ def main():
         "projection_tokens_per_s": round(args.steps / wall * (36 / args.layers), 2),
         "cache_resident_one_layer_GBps": round(cache_gbps, 3),
         "roofline": {
-            "kernel": "gemv_tiles_kernel",
+            "kernel": "gemv_seq_kernel",
             "bound": "hbm",
             "achieved": round(achieved, 3),
             "peak": HBM_PEAK_GBPS,
@@ -482,10 +496,21 @@ def main():
             "valu_slots_per_block": prof.get("valu_slots_per_block") if prof_ok else None,
             "valu_busy_frac": prof.get("valu_busy_frac") if prof_ok else None,
             "avg_launch_us": round(avg_launch_us, 3),
+            "launches_per_step": 1,
+            "items_per_launch": n_kernels,
+            "algorithmic_bytes_per_launch": enc_bytes,
+        },
+        # the same items as separate llvq_hip_gemv_group calls (gemv_tiles_kernel, one launch per item)
+        "per_call": {
+            "GBps": round(enc_bytes * args.steps / pc_wall / 1e9, 3),
+            "ms_per_step": round(pc_wall * 1e3 / args.steps, 4),
+            "kernel": "gemv_tiles_kernel",
             "launches_per_step": n_kernels,
-            "algorithmic_bytes_per_launch": round(enc_bytes / n_kernels, 1),
+            "avg_launch_us": round(pc_dev_ms * 1e3 / (args.steps * n_kernels), 3),
+            "achieved_GBps_device_time": round(pc_achieved, 3),
         },
     }
+    seq.close()
     if not args.no_decode and args.layers == 36:
         out["decode"] = decode_leg(rt, projs, args.seed)
         out["decode_q8_head"] = decode_leg(rt, projs, args.seed, q8_head=True)

@@ -165,6 +165,43 @@ int llvq_hip_matrix_rotation(const llvq_mat* m, uint32_t* has_rotation, uint64_t
 int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const void* x_f16_dev,
                         void* const* y_dev, int y_dtype);
 
+/* A token's worth of group products as ONE launch.  The reference's FusedOp::cuda_fwd
+ * (llvq-llm/src/fused_cuda.rs:758-900) launches per projection, and group_forward
+ * (model.rs:497-536) calls it once per activation site, so a decode token is hundreds of
+ * launches whose latency the reference puts at about half the token (fused_cuda.rs:789-795).
+ * A sequence binds a list of items — each item is what one llvq_hip_gemv_group call would
+ * be: projections that share d_in, one activation, their outputs — once, and
+ * llvq_hip_sequence_run enqueues them all as one persistent kernel on the runtime's stream.
+ * Results are those of the separate calls, bit for bit.
+ *   after_previous = 0: the item's activation is complete before the run is enqueued.
+ *   after_previous = 1: the activation is (or depends on) an output of the item before it in
+ *     the list; the kernel orders the two on the device.  Such a sequence needs every
+ *     workgroup resident at once and is launched cooperatively.
+ * Matrices stored in a rotated basis, and rows wider than 24 576 columns, are refused with
+ * LLVQ_ERR_UNSUPPORTED (use the per-call entry points).  The pointers are captured at
+ * creation; the matrices and buffers must outlive the sequence.  Runs of one sequence must
+ * not overlap (they share its device-side counters). */
+typedef struct llvq_seq llvq_seq;
+typedef struct llvq_seq_item {
+  const llvq_mat* const* mats;
+  int n_mats;
+  const void* x_f16_dev;
+  void* const* y_dev;
+  int y_dtype;
+  int after_previous;
+} llvq_seq_item;
+int llvq_hip_sequence_create(llvq_rt* rt, const llvq_seq_item* items, int n_items, llvq_seq** out);
+int llvq_hip_sequence_run(llvq_rt* rt, llvq_seq* seq);
+/* Waits for the stream, then LLVQ_OK, or LLVQ_ERR_DEVICE if a workgroup of an earlier run gave
+ * up waiting for an item (its outputs are then incomplete). */
+int llvq_hip_sequence_status(llvq_rt* rt, llvq_seq* seq);
+void llvq_hip_sequence_destroy(llvq_rt* rt, llvq_seq* seq);
+/* How long an ordered item waits for the one before it: `spin_limit` polls (0: the default, about
+ * a second).  hold_item >= 0 makes the NEXT run treat that item as never complete, so that the
+ * items behind it give up after spin_limit polls and llvq_hip_sequence_status reports it: how
+ * the give-up path is tested without a kernel that hangs.  No counterpart in the reference. */
+int llvq_hip_sequence_tune(llvq_seq* seq, uint32_t spin_limit, int hold_item);
+
 /* The row loop of group_forward (model.rs:521-529) as one batched product:
  * Y[M, d_out] = X[M, d_in] W^T, X row-major binary16. */
 int llvq_hip_gemm(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, int M, void* y_dev,

@@ -26,6 +26,21 @@ pub struct LlvqMat {
 pub struct LlvqDecoder {
     _p: [u8; 0],
 }
+#[repr(C)]
+pub struct LlvqSeq {
+    _p: [u8; 0],
+}
+
+/// llvq_seq_item: one group product of a sequence (what one llvq_hip_gemv_group call would be)
+#[repr(C)]
+pub struct LlvqSeqItem {
+    pub mats: *const *const LlvqMat,
+    pub n_mats: c_int,
+    pub x_f16_dev: *const c_void,
+    pub y_dev: *const *mut c_void,
+    pub y_dtype: c_int,
+    pub after_previous: c_int,
+}
 
 /// llvq_matrix_desc
 #[repr(C)]
@@ -150,6 +165,11 @@ extern "C" {
     pub fn llvq_hip_host_rotate(n: u32, seed: u64, v: *mut f64) -> c_int;
     pub fn llvq_hip_matrix_rotation(m: *const LlvqMat, has_rotation: *mut u32, seed: *mut u64) -> c_int;
     pub fn llvq_hip_gemv_group(rt: *mut LlvqRt, mats: *const *const LlvqMat, n: c_int, x_f16_dev: *const c_void, y_dev: *const *mut c_void, y_dtype: c_int) -> c_int;
+    pub fn llvq_hip_sequence_create(rt: *mut LlvqRt, items: *const LlvqSeqItem, n_items: c_int, out: *mut *mut LlvqSeq) -> c_int;
+    pub fn llvq_hip_sequence_run(rt: *mut LlvqRt, seq: *mut LlvqSeq) -> c_int;
+    pub fn llvq_hip_sequence_status(rt: *mut LlvqRt, seq: *mut LlvqSeq) -> c_int;
+    pub fn llvq_hip_sequence_destroy(rt: *mut LlvqRt, seq: *mut LlvqSeq);
+    pub fn llvq_hip_sequence_tune(seq: *mut LlvqSeq, spin_limit: u32, hold_item: c_int) -> c_int;
     pub fn llvq_hip_gemm(rt: *mut LlvqRt, m: *const LlvqMat, x_f16_dev: *const c_void, rows: c_int, y_dev: *mut c_void, y_dtype: c_int) -> c_int;
     pub fn llvq_hip_gemm_group(rt: *mut LlvqRt, mats: *const *const LlvqMat, n: c_int, x_f16_dev: *const c_void, rows: c_int, y_dev: *const *mut c_void, y_dtype: c_int) -> c_int;
     pub fn llvq_hip_reserve_batched(rt: *mut LlvqRt, mats: *const *const LlvqMat, n: c_int, max_rows: c_int) -> c_int;

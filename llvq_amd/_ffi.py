@@ -61,6 +61,11 @@ class QuantRows(C.Structure):
                 ("group", C.c_uint32)]
 
 
+class SeqItem(C.Structure):
+    _fields_ = [("mats", C.POINTER(C.c_void_p)), ("n_mats", C.c_int), ("x_f16_dev", C.c_void_p),
+                ("y_dev", C.POINTER(C.c_void_p)), ("y_dtype", C.c_int), ("after_previous", C.c_int)]
+
+
 class DecoderDesc(C.Structure):
     _fields_ = [
         ("n_layers", C.c_uint32), ("hidden", C.c_uint32), ("n_heads", C.c_uint32), ("n_kv_heads", C.c_uint32),
@@ -120,6 +125,12 @@ def lib():
     L.llvq_hip_gemv_rotated.argtypes = [vp, vp, vp, vp, C.c_int]
     L.llvq_hip_matrix_rotation.argtypes = [vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint64)]
     L.llvq_hip_gemv_group.argtypes = [vp, C.POINTER(vp), C.c_int, vp, C.POINTER(vp), C.c_int]
+    L.llvq_hip_sequence_create.argtypes = [vp, C.POINTER(SeqItem), C.c_int, C.POINTER(vp)]
+    L.llvq_hip_sequence_run.argtypes = [vp, vp]
+    L.llvq_hip_sequence_status.argtypes = [vp, vp]
+    L.llvq_hip_sequence_tune.argtypes = [vp, C.c_uint32, C.c_int]
+    L.llvq_hip_sequence_destroy.argtypes = [vp, vp]
+    L.llvq_hip_sequence_destroy.restype = None
     L.llvq_hip_gemm.argtypes = [vp, vp, vp, C.c_int, vp, C.c_int]
     L.llvq_hip_reserve_batched.argtypes = [vp, C.POINTER(vp), C.c_int, C.c_int]
     L.llvq_hip_decoder_generate_phased.argtypes = [vp, vp, sz, sz, vp, vp]
@@ -153,7 +164,8 @@ EXPORTS = [
     "llvq_hip_host_decode", "llvq_hip_matrix_upload", "llvq_hip_read_header", "llvq_hip_parse_matrix_record",
     "llvq_hip_matrix_from_record", "llvq_hip_parse_raw_tensor", "llvq_hip_parse_blob",
     "llvq_hip_matrix_free", "llvq_hip_matrix_info", "llvq_hip_matrix_name", "llvq_hip_gemv",
-    "llvq_hip_gemv_group", "llvq_hip_gemm", "llvq_hip_gemm_static", "llvq_hip_reserve_batched", "llvq_hip_decoder_generate_phased", "llvq_hip_gemm_group", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
+    "llvq_hip_gemv_group", "llvq_hip_sequence_create", "llvq_hip_sequence_run", "llvq_hip_sequence_status", "llvq_hip_sequence_tune",
+    "llvq_hip_sequence_destroy", "llvq_hip_gemm", "llvq_hip_gemm_static", "llvq_hip_reserve_batched", "llvq_hip_decoder_generate_phased", "llvq_hip_gemm_group", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
     "llvq_hip_last_error", "llvq_hip_version",
     "llvq_hip_host_rotate", "llvq_hip_rotate", "llvq_hip_gemv_rotated", "llvq_hip_matrix_rotation",
     "llvq_hip_decoder_create", "llvq_hip_decoder_destroy", "llvq_hip_decoder_reset", "llvq_hip_decoder_position", "llvq_hip_decoder_seek",

@@ -344,7 +344,7 @@ constexpr int kSecSlots = 384;          // queue of even-coset blocks whose clas
 __host__ __device__ constexpr size_t gemv_stage_bytes(uint32_t tile) { return ((size_t)tile + kSecSlots) * 10 + 32 + (size_t)tile * 4; }
 __host__ __device__ constexpr size_t gemv_lds_bytes(uint32_t nblocks, uint32_t tile = kTileBlocks,
                                                     size_t image_bytes = kLdsImageBytes) {
-  return image_bytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + 32 * 4 + gemv_stage_bytes(tile) +
+  return image_bytes + (size_t)nblocks * (kPlaneDwords + 1) * 4 + (32 + (nblocks & 1u)) * 4 + gemv_stage_bytes(tile) +
          2 * (size_t)kGenericSlots * 10 + 32;
 }
 
@@ -662,16 +662,27 @@ struct GemvQueues {
   float* partial;   // [tile]
 };
 
+// What a lane knows of its NB blocks after classification and before they are queued: the two
+// words of each block's queue entry and, packed in `where`, bits 2i..2i+1 = the queue block i joins
+// (0 odd, 1 even, 2 the small even queue, 3 none), bit 8 + i = block i is the origin, bit 12 + i =
+// block i is a generic block of the even coset.
 template <int NB>
-__device__ __forceinline__ void classify_stream(const DecodeTables& T, const LaneRecords<NB>& rec, uint32_t nblk, uint32_t capacity,
-                                                const GemvQueues& Q) {
-  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+struct Classified {
+  uint32_t e0[NB], e1[NB];
+  uint32_t where;
+};
+
+// First half of P1: table reads only, nothing is written — it may run while another tile's queues are in use.
+template <int NB>
+__device__ __forceinline__ void classify_records(const DecodeTables& T, const LaneRecords<NB>& rec, uint32_t nblk, Classified<NB>& c) {
+  const uint32_t tid = threadIdx.x;
   // Every LDS read below is unconditional, from a valid slot, so that the NB reads of a step go
   // out together (a guarded read is waited for where it is issued).  A lane past the tile's end
   // walks the tables with whatever bytes follow the tile and queues nothing.
   uint32_t zlo[NB], zhi[NB], gain[NB], ci[NB], kind[NB];
   uint64_t start[NB];
   bool live[NB];  // a block of the tile that is not the origin (which decodes to zero whatever the gain, index.rs:335-337)
+  uint32_t where = 0;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     const uint32_t f = tid * NB + (uint32_t)i;
@@ -681,33 +692,50 @@ __device__ __forceinline__ void classify_stream(const DecodeTables& T, const Lan
     const uint32_t ilo = __builtin_amdgcn_alignbit(hi16, lo32, 1), ihi = hi16 >> 1;  // the 47-bit index
     const bool origin = (ilo | ihi) == 0u;
     live[i] = f < nblk && !origin;
-    if (f < nblk && origin) Q.partial[f] = 0.f;
+    where |= (f < nblk && origin) ? 1u << (8 + i) : 0u;
     const uint64_t z = (((uint64_t)ihi << 32) | ilo) - 1u;  // zero-based
     zlo[i] = (uint32_t)z;
     zhi[i] = (uint32_t)(z >> 32) & 0x7FFFu;  // an origin wraps to all ones: keep it a 47-bit index
   }
   find_classes<NB>(T, zlo, zhi, ci, start, kind);
-  // Which queue a block joins: 0 odd, 1 even, 2 the small even queue, 3 none.  A generic block rides in
-  // the odd queue, flagged, unless its coset's small queue has room (rare: settled under a wavefront-wide test).
-  uint32_t kq[NB], e0[NB], e1[NB];
+  // Which queue a block joins.  A generic block rides in the odd queue, flagged, unless its coset's small
+  // queue has room (settled when the block is queued).
   uint32_t any_generic = 0;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     const uint64_t li = (((uint64_t)zhi[i] << 32) | zlo[i]) - start[i];
     const uint32_t generic = kind[i] == kLutKindGeneric ? 1u : 0u;
-    e0[i] = (uint32_t)li;
-    e1[i] = (uint32_t)(li >> 32) | (ci[i] << kQaClassShift) | (gain[i] << kQaGainShift) | (generic << 31);
-    kq[i] = live[i] ? (generic ? 0u : kind[i]) : 3u;
+    c.e0[i] = (uint32_t)li;
+    c.e1[i] = (uint32_t)(li >> 32) | (ci[i] << kQaClassShift) | (gain[i] << kQaGainShift) | (generic << 31);
+    where |= (live[i] ? (generic ? 0u : kind[i]) : 3u) << (2 * i);
     any_generic |= live[i] ? generic : 0u;
   }
   if (__any(any_generic != 0u)) {
 #pragma unroll
     for (int i = 0; i < NB; ++i)
-      if (kq[i] == 0u && (e1[i] >> 31)) {
-        const uint32_t even = (T.fast[ci[i]].meta & kMetaOdd) ? 0u : 1u;
+      if (((where >> (2 * i)) & 3u) == 0u && (c.e1[i] >> 31) && !(T.fast[ci[i]].meta & kMetaOdd)) where |= 1u << (12 + i);
+  }
+  c.where = where;
+}
+
+// Second half of P1: the lane's classified blocks go to the tile's queues (LDS writes and counters).
+template <int NB>
+__device__ __forceinline__ void queue_classified(Classified<NB>& c, uint32_t capacity, const GemvQueues& Q) {
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  uint32_t kq[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) kq[i] = (c.where >> (2 * i)) & 3u;
+  uint32_t any_generic = 0;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) any_generic |= (kq[i] == 0u) ? c.e1[i] >> 31 : 0u;
+  if (__any(any_generic != 0u)) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+      if (kq[i] == 0u && (c.e1[i] >> 31)) {
+        const uint32_t even = (c.where >> (12 + i)) & 1u;
         const uint32_t slot = atomicAdd(&Q.ctrl[even ? kCtrlGenEven : kCtrlGenOdd], 1u);
         if (slot < (uint32_t)kGenericSlots) {
-          Q.gqa[even * kGenericSlots + slot] = make_uint2(e0[i], e1[i]);
+          Q.gqa[even * kGenericSlots + slot] = make_uint2(c.e0[i], c.e1[i]);
           Q.gqf[even * kGenericSlots + slot] = (uint16_t)(tid * NB + (uint32_t)i);
           kq[i] = 3u;  // placed
         }
@@ -748,58 +776,222 @@ __device__ __forceinline__ void classify_stream(const DecodeTables& T, const Lan
     const uint32_t up = base_o + rank, down = top - rank, behind = small + rank;
     uint32_t pos = kq[i] == 1u ? down : up;
     pos = kq[i] == 2u ? behind : pos;
+    uint32_t e1 = c.e1[i];
     if (spills) {
       const bool out = kq[i] == 2u && rank >= fits;
       pos = out ? top - (n_e + (rank - fits)) : pos;
-      e1[i] |= out ? kQaSecond : 0u;
+      e1 |= out ? kQaSecond : 0u;
     }
     if (kq[i] != 3u) {
-      Q.qa[pos] = make_uint2(e0[i], e1[i]);
+      Q.qa[pos] = make_uint2(c.e0[i], e1);
       Q.qf[pos] = (uint16_t)(tid * NB + (uint32_t)i);
     }
   }
 }
 
-// LEAN: the Golay words and the support-arrangement table stay in L2, which leaves
-// room for the full tile beside the activation planes of a very wide row.
-// ROT: the launch can rotate its own activation (GroupArgs::rot_m); kept out of the other
-// instantiations, whose hot loop it would otherwise cost registers and a few per cent.
-template <typename OutT, int TILE = kTileBlocks, bool LEAN = false, bool ROT = false>
-__global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
-  // the tile capacity of this instantiation (these shadow the namespace-level defaults)
-  constexpr int kTileBlocks = TILE;
-  constexpr int kP1Blocks = TILE / kWgThreads;
-  constexpr int kRawBytes = TILE * 6 + 32;  // what a derived binary16 activation may take of the staging area
-  extern __shared__ __align__(16) uint8_t smem[];
-#ifdef LLVQ_PHASE_TIMING
-  if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 3] = wall_clock64();
-#endif
-  const DecodeTables T = stage_tables<!LEAN>(smem, a.tables);
-  // A lane loads the records it classifies itself, HBM -> registers; the next tile's loads are
-  // issued while the current one is being decoded.  The first tile's are issued right behind the
-  // loads of the activation: the memory counter retires in order, so whatever is requested
-  // after them would wait for HBM with them, and they are not needed before the activation is.
-  LaneRecords<kP1Blocks> pre;
+// The origin blocks of a lane's share decode to zero: their partial sums are written here.
+template <int NB>
+__device__ __forceinline__ void settle_origins(uint32_t where, float* partial) {
+  if (__any((where >> 8) & 15u)) {
 #pragma unroll
-  for (int k = 0; k < kP1Blocks * 3 / 2; ++k) pre.w[k] = 0;
-  auto request_first_tile = [&]() { prefetch_records(a, blockIdx.x, threadIdx.x, pre); };
-  const uint32_t nb = a.nblocks;
-  uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + (LEAN ? kLdsImageBytesLean : kLdsImageBytes));
-  float* xscale = reinterpret_cast<float*>(xplanes + (size_t)nb * kPlaneDwords);
-  float* xtail = xscale + nb;
-  // queue entries | block numbers | 32 bytes | partial sums: also the staging area of a derived or rotated activation
-  uint8_t* raw = reinterpret_cast<uint8_t*>(xtail + 32);
-  GemvQueues Q;
-  Q.qa = reinterpret_cast<uint2*>(raw);
-  Q.qf = reinterpret_cast<uint16_t*>(Q.qa + kTileBlocks + kSecSlots);
-  Q.partial = reinterpret_cast<float*>(Q.qf + kTileBlocks + kSecSlots + 16);
-  Q.gqa = reinterpret_cast<uint2*>(Q.partial + kTileBlocks);
-  Q.gqf = reinterpret_cast<uint16_t*>(Q.gqa + 2 * kGenericSlots);
-  Q.ctrl = reinterpret_cast<uint32_t*>(Q.gqf + 2 * kGenericSlots);
-  float* partial = Q.partial;
+    for (int i = 0; i < NB; ++i)
+      if ((where >> (8 + i)) & 1u) partial[threadIdx.x * NB + (uint32_t)i] = 0.f;
+  }
+}
+
+template <int NB>
+__device__ __forceinline__ void classify_stream(const DecodeTables& T, const LaneRecords<NB>& rec, uint32_t nblk, uint32_t capacity,
+                                                const GemvQueues& Q) {
+  Classified<NB> c;
+  classify_records<NB>(T, rec, nblk, c);
+  settle_origins<NB>(c.where, Q.partial);
+  queue_classified<NB>(c, capacity, Q);
+}
+
+// P2 of the GEMV kernels: unrank the tile's queued blocks and reduce them against the activation planes.
+// Chunks of 64 queued blocks are handed out through a counter: the two generic chunks first (longest),
+// then the chunks of the three fast decoders.  `hook(done, last, state)` (kHook) runs in every wavefront before
+// each of its chunks of the fast decoders, with the number it has finished, and once more (last = true) when
+// there is none left for it: where a caller puts work that does not depend on this tile and fills the issue
+// slots this tile's decoders leave.  `state` is 0 at first and then whatever the hook returned last; the
+// function returns the final one.
+struct UnrankOperands {
+  const uint32_t* xplanes;  // [nb][kPlaneDwords]
+  const float* xscale;      // [nb]
+  uint32_t nb;              // blocks per row
+  float inv_nb;             // 1 / nb, for the block -> column split
+  float g0, g1;             // the matrix's gain centroids
+};
+template <int TILE, bool kHook, class Hook>
+__device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const GemvQueues& Q, const UnrankOperands& op, Hook&& hook) {
+  constexpr int kTileBlocks = TILE;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
   uint32_t* ctrl = Q.ctrl;
-  static_assert((kTileBlocks + kSecSlots) % 4 == 0 && kGenericSlots % 2 == 0, "the arrays behind the 16-bit ones stay 8-byte aligned");
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  float* partial = Q.partial;
+  const uint32_t* xplanes = op.xplanes;
+  const float* xscale = op.xscale;
+  const uint32_t nb = op.nb;
+  const uint32_t n_odd = ctrl[kCtrlOdd], n_even = ctrl[kCtrlEven], n_sec = min(ctrl[kCtrlSec], (uint32_t)kSecSlots);
+  const uint32_t n_gen_o = min(ctrl[kCtrlGenOdd], (uint32_t)kGenericSlots), n_gen_e = min(ctrl[kCtrlGenEven], (uint32_t)kGenericSlots);
+  const uint32_t c_gen_o = n_gen_o ? 1u : 0u, c_gen_e = n_gen_e ? 1u : 0u, c_gen = c_gen_o + c_gen_e;
+  const uint32_t c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6, c_sec = (n_sec + 63u) >> 6;
+  auto ticket = [&]() {
+    uint32_t t = 0;
+    if (lane == 0) t = atomicAdd(&ctrl[kCtrlTicket], 1u);
+    return (uint32_t)__shfl(t, 0, 64);
+  };
+  // what every decoder starts from: the block's local rank, class, column and scale
+  struct Block {
+    uint64_t li;
+    uint32_t f, ci, col;
+    float g;
+  };
+  auto open_block = [&](uint2 e, uint32_t f) {
+    Block b;
+    b.li = ((uint64_t)(e.y & 0x1FFFu) << 32) | e.x;
+    b.ci = (e.y >> kQaClassShift) & 0x1FFu;
+    b.f = f;
+    const uint32_t row = (uint32_t)(((float)f + 0.5f) * op.inv_nb);
+    b.col = f - row * nb;
+    b.g = (e.y >> kQaGainShift) & 1u ? op.g1 : op.g0;
+    return b;
+  };
+  // generic walk of one queued block (rare classes): coordinates packed four to a dword, then
+  // the same integer dot products as the fast paths
+  auto generic_block = [&](uint2 e, uint32_t f) {
+    const Block b = open_block(e, f);
+    const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+    const DevClass c = T.cls[b.ci];
+    uint32_t w[6] = {0, 0, 0, 0, 0, 0};
+    auto emit = [&](int p, int v) { w[p >> 2] |= ((uint32_t)v & 0xFFu) << (8 * (p & 3)); };
+    if (c.meta & kMetaOdd) decode_odd(T, c, b.li, emit);
+    else decode_even(T, c, b.li, emit);
+    int d0 = 0, d1 = 0, d2 = 0;
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+      d0 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[q], d0, false);
+      d1 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[6 + q], d1, false);
+      d2 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[12 + q], d2, false);
+    }
+    partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (c.inv_norm * b.g);
+  };
+  auto odd_block = [&](uint2 e, uint32_t f) {
+    const Block b = open_block(e, f);
+    const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+    const FastClass fc = T.fast[b.ci];
+    int d0 = 0, d1 = 0, d2 = 0;
+    odd_codes(T, fc, b.li, [&](int q, uint32_t sel) {
+      const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+      d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+      d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+      d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+    });
+    partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
+  };
+  auto even_block = [&](uint2 e, uint32_t f, auto second) {
+    constexpr bool kSecond = decltype(second)::value;
+    const Block b = open_block(e, f);
+    const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+    const FastClass fc = T.fast[b.ci];
+    const uint32_t fv1 = fc.u0 >> 16;
+    const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
+    int d0 = 0, d1 = 0, d2 = 0;
+    even_codes<kSecond>(T, fc, b.li, [&](int q, uint32_t sel, uint32_t sel2) {
+      int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
+      if (kSecond) w |= (int)__builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2);
+      d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
+      d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
+      d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+    });
+    partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
+  };
+  uint32_t chunk = ticket();
+  // the generic chunks, kept out of the loop below: their code and registers are not the hot path's
+  while (chunk < c_gen) {
+    const uint32_t even = (chunk == 1u || !c_gen_o) ? 1u : 0u;
+    if (lane < (even ? n_gen_e : n_gen_o)) generic_block(Q.gqa[even * kGenericSlots + lane], Q.gqf[even * kGenericSlots + lane]);
+    chunk = ticket();
+  }
+  // Even and odd chunks alternate while both queues last: the even coset waits for tables in L2,
+  // the odd one issues arithmetic, and wavefronts on either kind at the same time overlap the two.
+  // The chunks of the small even queue come first (their queue ends in a partial chunk as well).
+  const uint32_t c_pair = min(c_odd, c_even);
+  const uint32_t c_all = c_gen + c_sec + c_odd + c_even;
+  uint32_t done = 0, hook_state = 0;
+  for (;; ++done, chunk = ticket()) {
+    if constexpr (kHook) hook_state = hook(done, chunk >= c_all, hook_state);
+    if (chunk >= c_all) break;
+    const uint32_t ts = chunk - c_gen;
+    if (ts < c_sec) {
+      const uint32_t k = ts * 64u + lane;
+      if (k < n_sec) even_block(Q.qa[kTileBlocks + k], Q.qf[kTileBlocks + k], std::true_type{});
+      continue;
+    }
+    const uint32_t t = ts - c_sec;
+    const bool paired = t < 2u * c_pair;
+    const bool is_odd = paired ? (t & 1u) != 0u : c_odd > c_even;
+    const uint32_t ordinal = paired ? t >> 1 : t - c_pair;
+    const uint32_t k = ordinal * 64u + lane;
+    if (is_odd) {
+      const uint32_t at = min(k, (uint32_t)kTileBlocks - 1u);
+      const uint2 e = Q.qa[at];
+      // generic blocks that found their small queue full wait for the pass below
+      if (k < n_odd && !(e.y >> 31)) odd_block(e, Q.qf[at]);
+    } else {
+      const uint32_t at = kTileBlocks - 1 - min(k, (uint32_t)kTileBlocks - 1u);
+      const uint2 e = Q.qa[at];
+      const bool mine = k < n_even;
+      // blocks with a second free kind that found their queue full ride here, flagged
+      if (__any(mine && (e.y & kQaSecond))) {
+        if (mine) even_block(e, Q.qf[at], std::true_type{});
+      } else {
+        if (mine) even_block(e, Q.qf[at], std::false_type{});
+      }
+    }
+  }
+  if (ctrl[kCtrlGenOdd] > (uint32_t)kGenericSlots || ctrl[kCtrlGenEven] > (uint32_t)kGenericSlots) {
+    // more generic blocks than the small queues hold (hostile input): the rest sit flagged in the odd queue
+    for (uint32_t k = tid; k < n_odd; k += kWgThreads) {
+      const uint2 e = Q.qa[k];
+      if (e.y >> 31) generic_block(e, Q.qf[k]);
+    }
+  }
+  return hook_state;
+}
+
+// Where a launch's activation comes from, and what it may do to produce it before the product.
+struct ActivationSource {
+  const __half* x;
+  const float* x_f32;  // when set, the activation is these f32 values (a rotated activation) and x is unused
+  const __half* x2;
+  const __half* norm_w;
+  __half* resid_out;
+  float eps;
+  uint32_t prologue;   // kPrologue*
+  uint32_t nb, tail_w;
+  const uint32_t* rot_signbits;
+  const float* rot_small;
+  float rot_inv;
+  uint32_t rot_m, rot_k;
+  bool writes_resid;   // this workgroup is the one that stores the new residual
+};
+
+// Fills the activation planes, scales and tail values in LDS from `a`, by every lane of the workgroup.
+// `raw` (the tile's queue entries, block numbers and partial sums, free at this point) is the staging
+// area of a derived or rotated activation; `request` is called once, right behind the loads of the
+// activation's operands (the caller's first code bytes go out there).  Returns whether the staging
+// area was used: the caller then needs a barrier before the area becomes queues again.  kInPlace: `raw` is the
+// planes' own memory (rows of at most as many blocks as the workgroup has lanes, natural basis only).
+template <int TILE, bool ROT, bool kInPlace = false, class Request>
+__device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint32_t* xplanes, float* xscale, float* xtail, uint8_t* raw,
+                                                 float* partial, Request&& request_first_tile) {
+  constexpr int kTileBlocks = TILE;
+  constexpr int kRawBytes = TILE * 6 + 32;  // what a derived binary16 activation may take of the staging area
+  uint32_t tid = threadIdx.x;
+  // staged from inside a loop over tiles: lane-derived indices are formed here, not carried through the loop in registers
+  if constexpr (kInPlace) asm volatile("" : "+v"(tid));
+  const uint32_t lane = tid & 63u, wave = tid >> 6;
+  const uint32_t nb = a.nb;
   const __half* xsrc = a.x;
   // A launch over matrices stored in a rotated basis rotates its activation itself: the
   // values go, signs applied, as f32 to the area the first tile's queues and
@@ -821,12 +1013,12 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     const bool silu = a.prologue == kPrologueSiluMul;
     const __half* src1 = a.x2 ? a.x2 : a.x;
     const __half* src2 = silu ? a.x : a.norm_w;
-    auto derive = [&](auto rounds) {
+    auto derive = [&](auto rounds, uint32_t base) {
       constexpr int kPer = decltype(rounds)::value;
       __half in0[kPer], in1[kPer], in2[kPer];
 #pragma unroll
       for (int k = 0; k < kPer; ++k) {
-        const uint32_t i = min(tid + (uint32_t)k * kWgThreads, d_in - 1u);
+        const uint32_t i = min(base + tid + (uint32_t)k * kWgThreads, d_in - 1u);
         in0[k] = a.x[i];
         in1[k] = src1[i];
         in2[k] = src2[i];
@@ -836,7 +1028,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       if (silu) {
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
-          const uint32_t i = tid + (uint32_t)k * kWgThreads;
+          const uint32_t i = base + tid + (uint32_t)k * kWgThreads;
           if (i < d_in) {
             const float g = __half2float(in1[k]);
             const float sg = __half2float(__float2half_rn(g / (1.0f + __expf(-g))));
@@ -851,12 +1043,12 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
         float ss = 0.f;
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
-          const uint32_t i = tid + (uint32_t)k * kWgThreads;
+          const uint32_t i = base + tid + (uint32_t)k * kWgThreads;
           v[k] = 0.f;
           if (i < d_in) {
             float r = __half2float(in0[k]);
             if (a.x2) r = __half2float(__float2half_rn(r + __half2float(in1[k])));
-            if (a.resid_out && blockIdx.x == 0) a.resid_out[i] = __float2half_rn(r);
+            if (a.resid_out && a.writes_resid) a.resid_out[i] = __float2half_rn(r);
             v[k] = r;
             ss += r * r;
           }
@@ -870,7 +1062,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
         const float inv = 1.0f / sqrtf(total / (float)d_in + a.eps);
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
-          const uint32_t i = tid + (uint32_t)k * kWgThreads;
+          const uint32_t i = base + tid + (uint32_t)k * kWgThreads;
           if (i < d_in) {
             const __half h = __float2half_rn(v[k] * inv * __half2float(in2[k]));
             if (rotated) xf[i] = signed_f32(i, __half2float(h));
@@ -880,9 +1072,17 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       }
     };
     const uint32_t n_per = (d_in + kWgThreads - 1) / kWgThreads;
-    if (n_per <= 3) derive(std::integral_constant<int, kPerMax < 3 ? kPerMax : 3>{});
-    else if (n_per <= 6) derive(std::integral_constant<int, kPerMax < 6 ? kPerMax : 6>{});
-    else derive(std::integral_constant<int, kPerMax>{});
+    if constexpr (kInPlace) {
+      // at most six rounds of operands in registers at a time: the wider SiLU rows go in runs of 6144 values
+      // (a row sum of squares over more than 6144 values is refused by the host for this variant)
+      if (n_per <= 3) derive(std::integral_constant<int, 3>{}, 0u);
+      else
+        for (uint32_t base = 0; base < d_in; base += 6u * kWgThreads) derive(std::integral_constant<int, 6>{}, base);
+    } else {
+      if (n_per <= 3) derive(std::integral_constant<int, kPerMax < 3 ? kPerMax : 3>{}, 0u);
+      else if (n_per <= 6) derive(std::integral_constant<int, kPerMax < 6 ? kPerMax : 6>{}, 0u);
+      else derive(std::integral_constant<int, kPerMax>{}, 0u);
+    }
     __syncthreads();
     xsrc = xs;
   } else if (rotated) {
@@ -911,9 +1111,19 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       quantize_block_f32(xf + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     if (tid < a.tail_w) xtail[tid] = xf[(size_t)nb * kDim + tid];
   } else if (a.prologue != kPrologueNone) {
-    for (uint32_t col = tid; col < nb; col += kWgThreads)
-      quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
-    if (tid < a.tail_w) xtail[tid] = __half2float(xsrc[(size_t)nb * kDim + tid]);
+    if constexpr (kInPlace) {
+      // the staging area is the planes' own: every lane reads its block before any lane writes (nb <= lanes)
+      float v[kDim];
+      load_block_f16(xsrc + (size_t)min(tid, nb ? nb - 1u : 0u) * kDim, v);
+      const float tail_v = tid < a.tail_w ? __half2float(xsrc[(size_t)nb * kDim + tid]) : 0.f;
+      __syncthreads();
+      if (tid < nb) quantize_values(v, xplanes + (size_t)tid * kPlaneDwords, xscale + tid);
+      if (tid < a.tail_w) xtail[tid] = tail_v;
+    } else {
+      for (uint32_t col = tid; col < nb; col += kWgThreads)
+        quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+      if (tid < a.tail_w) xtail[tid] = __half2float(xsrc[(size_t)nb * kDim + tid]);
+    }
   } else {
     // a finished activation from global memory: this lane's block is requested, then the first tile's
     // code bytes, then the block is quantised (rows wider than 1024 blocks take further rounds)
@@ -939,7 +1149,52 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
       else quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     }
   }
-  if (a.prologue != kPrologueNone || rotated) __syncthreads();  // the staging area becomes the tile's queues
+  return a.prologue != kPrologueNone || rotated;
+}
+
+// LEAN: the Golay words and the support-arrangement table stay in L2, which leaves
+// room for the full tile beside the activation planes of a very wide row.
+// ROT: the launch can rotate its own activation (GroupArgs::rot_m); kept out of the other
+// instantiations, whose hot loop it would otherwise cost registers and a few per cent.
+template <typename OutT, int TILE = kTileBlocks, bool LEAN = false, bool ROT = false>
+__global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
+  // the tile capacity of this instantiation (these shadow the namespace-level defaults)
+  constexpr int kTileBlocks = TILE;
+  constexpr int kP1Blocks = TILE / kWgThreads;
+  extern __shared__ __align__(16) uint8_t smem[];
+#ifdef LLVQ_PHASE_TIMING
+  if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 3] = wall_clock64();
+#endif
+  const DecodeTables T = stage_tables<!LEAN>(smem, a.tables);
+  // A lane loads the records it classifies itself, HBM -> registers; the next tile's loads are
+  // issued while the current one is being decoded.  The first tile's are issued right behind the
+  // loads of the activation: the memory counter retires in order, so whatever is requested
+  // after them would wait for HBM with them, and they are not needed before the activation is.
+  LaneRecords<kP1Blocks> pre;
+#pragma unroll
+  for (int k = 0; k < kP1Blocks * 3 / 2; ++k) pre.w[k] = 0;
+  auto request_first_tile = [&]() { prefetch_records(a, blockIdx.x, threadIdx.x, pre); };
+  const uint32_t nb = a.nblocks;
+  uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + (LEAN ? kLdsImageBytesLean : kLdsImageBytes));
+  float* xscale = reinterpret_cast<float*>(xplanes + (size_t)nb * kPlaneDwords);
+  float* xtail = xscale + nb;
+  // queue entries | block numbers | 32 bytes | partial sums: also the staging area of a derived or rotated activation
+  uint8_t* raw = reinterpret_cast<uint8_t*>(xtail + 32 + (nb & 1u));  // 8-byte aligned: the queue entries are read as 64-bit words
+  GemvQueues Q;
+  Q.qa = reinterpret_cast<uint2*>(raw);
+  Q.qf = reinterpret_cast<uint16_t*>(Q.qa + kTileBlocks + kSecSlots);
+  Q.partial = reinterpret_cast<float*>(Q.qf + kTileBlocks + kSecSlots + 16);
+  Q.gqa = reinterpret_cast<uint2*>(Q.partial + kTileBlocks);
+  Q.gqf = reinterpret_cast<uint16_t*>(Q.gqa + 2 * kGenericSlots);
+  Q.ctrl = reinterpret_cast<uint32_t*>(Q.gqf + 2 * kGenericSlots);
+  float* partial = Q.partial;
+  uint32_t* ctrl = Q.ctrl;
+  static_assert((kTileBlocks + kSecSlots) % 4 == 0 && kGenericSlots % 2 == 0, "the arrays behind the 16-bit ones stay 8-byte aligned");
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const ActivationSource src{a.x, a.x_f32, a.x2, a.norm_w, a.resid_out, a.eps, a.prologue, nb, a.tail_w,
+                             a.rot_signbits, a.rot_small, a.rot_inv, a.rot_m, a.rot_k, blockIdx.x == 0};
+  if (stage_activation<kTileBlocks, ROT>(src, xplanes, xscale, xtail, raw, partial, request_first_tile))
+    __syncthreads();  // the staging area becomes the tile's queues
 
 #ifdef LLVQ_PHASE_TIMING
   if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 7] = wall_clock64();
@@ -973,129 +1228,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     LLVQ_STAMP(2);
     prefetch_records(a, tile + gridDim.x, tid, pre);
 
-    // P2: unrank and reduce.  Chunks of 64 queued blocks are handed out through a counter: the two
-    // generic chunks first (longest), then the chunks of the three fast decoders.
-    const uint32_t n_odd = ctrl[kCtrlOdd], n_even = ctrl[kCtrlEven], n_sec = min(ctrl[kCtrlSec], (uint32_t)kSecSlots);
-    const uint32_t n_gen_o = min(ctrl[kCtrlGenOdd], (uint32_t)kGenericSlots), n_gen_e = min(ctrl[kCtrlGenEven], (uint32_t)kGenericSlots);
-    const uint32_t c_gen_o = n_gen_o ? 1u : 0u, c_gen_e = n_gen_e ? 1u : 0u, c_gen = c_gen_o + c_gen_e;
-    const uint32_t c_odd = (n_odd + 63u) >> 6, c_even = (n_even + 63u) >> 6, c_sec = (n_sec + 63u) >> 6;
-    auto ticket = [&]() {
-      uint32_t t = 0;
-      if (lane == 0) t = atomicAdd(&ctrl[kCtrlTicket], 1u);
-      return (uint32_t)__shfl(t, 0, 64);
-    };
-    // what every decoder starts from: the block's local rank, class, column and scale
-    struct Block {
-      uint64_t li;
-      uint32_t f, ci, col;
-      float g;
-    };
-    auto open_block = [&](uint2 e, uint32_t f) {
-      Block b;
-      b.li = ((uint64_t)(e.y & 0x1FFFu) << 32) | e.x;
-      b.ci = (e.y >> kQaClassShift) & 0x1FFu;
-      b.f = f;
-      const uint32_t row = (uint32_t)(((float)f + 0.5f) * a.inv_nblocks);
-      b.col = f - row * nb;
-      b.g = (e.y >> kQaGainShift) & 1u ? M.g1 : M.g0;
-      return b;
-    };
-    // generic walk of one queued block (rare classes): coordinates packed four to a dword, then
-    // the same integer dot products as the fast paths
-    auto generic_block = [&](uint2 e, uint32_t f) {
-      const Block b = open_block(e, f);
-      const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
-      const DevClass c = T.cls[b.ci];
-      uint32_t w[6] = {0, 0, 0, 0, 0, 0};
-      auto emit = [&](int p, int v) { w[p >> 2] |= ((uint32_t)v & 0xFFu) << (8 * (p & 3)); };
-      if (c.meta & kMetaOdd) decode_odd(T, c, b.li, emit);
-      else decode_even(T, c, b.li, emit);
-      int d0 = 0, d1 = 0, d2 = 0;
-#pragma unroll
-      for (int q = 0; q < 6; ++q) {
-        d0 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[q], d0, false);
-        d1 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[6 + q], d1, false);
-        d2 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[12 + q], d2, false);
-      }
-      partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (c.inv_norm * b.g);
-    };
-    auto odd_block = [&](uint2 e, uint32_t f) {
-      const Block b = open_block(e, f);
-      const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
-      const FastClass fc = T.fast[b.ci];
-      int d0 = 0, d1 = 0, d2 = 0;
-      odd_codes(T, fc, b.li, [&](int q, uint32_t sel) {
-        const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
-        d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
-        d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-        d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
-      });
-      partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
-    };
-    auto even_block = [&](uint2 e, uint32_t f, auto second) {
-      constexpr bool kSecond = decltype(second)::value;
-      const Block b = open_block(e, f);
-      const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
-      const FastClass fc = T.fast[b.ci];
-      const uint32_t fv1 = fc.u0 >> 16;
-      const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
-      int d0 = 0, d1 = 0, d2 = 0;
-      even_codes<kSecond>(T, fc, b.li, [&](int q, uint32_t sel, uint32_t sel2) {
-        int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
-        if (kSecond) w |= (int)__builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2);
-        d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
-        d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-        d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
-      });
-      partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
-    };
-    uint32_t chunk = ticket();
-    // the generic chunks, kept out of the loop below: their code and registers are not the hot path's
-    while (chunk < c_gen) {
-      const uint32_t even = (chunk == 1u || !c_gen_o) ? 1u : 0u;
-      if (lane < (even ? n_gen_e : n_gen_o)) generic_block(Q.gqa[even * kGenericSlots + lane], Q.gqf[even * kGenericSlots + lane]);
-      chunk = ticket();
-    }
-    // Even and odd chunks alternate while both queues last: the even coset waits for tables in L2,
-    // the odd one issues arithmetic, and wavefronts on either kind at the same time overlap the two.
-    // The chunks of the small even queue come first (their queue ends in a partial chunk as well).
-    const uint32_t c_pair = min(c_odd, c_even);
-    for (; chunk < c_gen + c_sec + c_odd + c_even; chunk = ticket()) {
-      const uint32_t ts = chunk - c_gen;
-      if (ts < c_sec) {
-        const uint32_t k = ts * 64u + lane;
-        if (k < n_sec) even_block(Q.qa[kTileBlocks + k], Q.qf[kTileBlocks + k], std::true_type{});
-        continue;
-      }
-      const uint32_t t = ts - c_sec;
-      const bool paired = t < 2u * c_pair;
-      const bool is_odd = paired ? (t & 1u) != 0u : c_odd > c_even;
-      const uint32_t ordinal = paired ? t >> 1 : t - c_pair;
-      const uint32_t k = ordinal * 64u + lane;
-      if (is_odd) {
-        const uint32_t at = min(k, (uint32_t)kTileBlocks - 1u);
-        const uint2 e = Q.qa[at];
-        // generic blocks that found their small queue full wait for the pass below
-        if (k < n_odd && !(e.y >> 31)) odd_block(e, Q.qf[at]);
-      } else {
-        const uint32_t at = kTileBlocks - 1 - min(k, (uint32_t)kTileBlocks - 1u);
-        const uint2 e = Q.qa[at];
-        const bool mine = k < n_even;
-        // blocks with a second free kind that found their queue full ride here, flagged
-        if (__any(mine && (e.y & kQaSecond))) {
-          if (mine) even_block(e, Q.qf[at], std::true_type{});
-        } else {
-          if (mine) even_block(e, Q.qf[at], std::false_type{});
-        }
-      }
-    }
-    if (ctrl[kCtrlGenOdd] > (uint32_t)kGenericSlots || ctrl[kCtrlGenEven] > (uint32_t)kGenericSlots) {
-      // more generic blocks than the small queues hold (hostile input): the rest sit flagged in the odd queue
-      for (uint32_t k = tid; k < n_odd; k += kWgThreads) {
-        const uint2 e = Q.qa[k];
-        if (e.y >> 31) generic_block(e, Q.qf[k]);
-      }
-    }
+    // P2: unrank and reduce
+    unrank_tile<kTileBlocks, false>(T, Q, UnrankOperands{xplanes, xscale, nb, a.inv_nblocks, M.g0, M.g1}, [](uint32_t, bool, uint32_t) { return 0u; });
     LLVQ_STAMP(4);
     __syncthreads();
     LLVQ_STAMP(5);
@@ -1189,6 +1323,7 @@ __global__ __launch_bounds__(1024) void rotate_kernel(RotArgs a) {
 
 }  // namespace llvq
 
+#include "gemv_seq.h"
 #include "gemm_kernel.h"
 #include "decoder.h"
 
@@ -1238,6 +1373,14 @@ struct llvq_mat {
   bool has_rotation = false;
   uint64_t rotation_seed = 0;
   const llvq_rt::DevRotation* rot = nullptr;  // owned by the runtime
+};
+
+struct llvq_seq {
+  uint8_t* blob = nullptr;  // one device allocation: tiles | items | counters | status
+  SeqArgs args{};
+  uint32_t tile = 0, grid = 0, n_items = 0;
+  bool lean = false, cooperative = false;
+  size_t lds = 0;
 };
 
 static thread_local std::string g_last_error;
@@ -1848,6 +1991,209 @@ int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   }
   HIP_TRY(hipSetDevice(rt->device));
   return forward_group(rt, mats, n, x, y, y_dtype);
+}
+
+// ---- sequences of group products in one launch (gemv_seq.h) -------------------------------
+// One item of a sequence as the library's own callers state it: what a launch_group call takes.
+struct SeqSpec {
+  const llvq_mat* const* mats = nullptr;
+  int n = 0;
+  const void* x = nullptr;
+  void* const* y = nullptr;
+  int y_dtype = LLVQ_F16;
+  bool after_previous = false;
+  Prologue pro{};
+};
+
+static const void* seq_kernel(uint32_t tile, bool lean) {
+  if (lean) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, true>);
+  if (tile == (uint32_t)kTileBlocks) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, false>);
+  return reinterpret_cast<const void*>(gemv_seq_kernel<kSmallTileBlocks, false>);
+}
+
+// The kernel variant for a sequence whose widest rows have max_nb blocks (as pick_gemv_shape).
+static GemvShape pick_seq_shape(uint32_t max_nb) {
+  GemvShape s{(uint32_t)kTileBlocks, false, gemv_seq_lds_bytes(max_nb, kTileBlocks, kLdsImageBytes)};
+  if (s.lds <= 160 * 1024) return s;
+  s = GemvShape{(uint32_t)kTileBlocks, true, gemv_seq_lds_bytes(max_nb, kTileBlocks, kLdsImageBytesLean)};
+  if (s.lds <= 160 * 1024) return s;
+  return GemvShape{(uint32_t)kSmallTileBlocks, false, gemv_seq_lds_bytes(max_nb, kSmallTileBlocks, kLdsImageBytes)};
+}
+
+constexpr uint32_t kSeqSpinLimit = 1u << 20;  // polls of a wait before it gives up (about a second)
+
+static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) {
+  if (n <= 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: no items");
+  uint32_t max_nb = 0;
+  bool dependent = false;
+  for (int i = 0; i < n; ++i) {
+    const SeqSpec& sp = specs[i];
+    if (!sp.mats || sp.n <= 0 || !sp.x || !sp.y) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: item " + std::to_string(i) + " has a null or empty field");
+    if (sp.y_dtype != LLVQ_F32 && sp.y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: unknown output dtype");
+    if (sp.after_previous && i == 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: the first item has no item before it");
+    for (int j = 0; j < sp.n; ++j) {
+      const llvq_mat* m = sp.mats[j];
+      if (!m || !sp.y[j]) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: null matrix or output in item " + std::to_string(i));
+      if (m->d_in != sp.mats[0]->d_in) return fail(LLVQ_ERR_INVALID_ARGUMENT, m->name + ": projections of one item must share d_in");
+      if (m->has_rotation) return fail(LLVQ_ERR_UNSUPPORTED, m->name + ": a sequence takes natural-basis matrices only");
+    }
+    if (sp.mats[0]->nblocks > 1024u) return fail(LLVQ_ERR_UNSUPPORTED, sp.mats[0]->name + ": rows wider than 24 576 columns do not fit a sequence");
+    max_nb = std::max(max_nb, sp.mats[0]->nblocks);
+    dependent |= sp.after_previous;
+  }
+  const GemvShape shape = pick_seq_shape(max_nb);
+  if (shape.lds > 160 * 1024 || max_nb > shape.tile) return fail(LLVQ_ERR_UNSUPPORTED, "sequence_create: the widest rows do not fit the LDS activation tile");
+  for (int i = 0; i < n; ++i)
+    if (specs[i].pro.kind == kPrologueAddRmsNorm && specs[i].mats[0]->d_in > 6u * kWgThreads)
+      return fail(LLVQ_ERR_UNSUPPORTED, specs[i].mats[0]->name + ": d_in too wide for a fused norm inside a sequence");
+  const uint32_t grid_cap = (uint32_t)(rt->cu_count > 0 ? rt->cu_count : 256);
+  std::vector<SeqTile> tiles;
+  std::vector<SeqItem> items((size_t)n);
+  for (int i = 0; i < n; ++i) {
+    const SeqSpec& sp = specs[i];
+    const llvq_mat* m0 = sp.mats[0];
+    const uint32_t nb = m0->nblocks;
+    // Ordered items are balanced one by one, like launches (everyone waits for an item's slowest workgroup);
+    // independent items fill their tiles, because the round-robin runs on across item boundaries.
+    uint32_t rpt = dependent ? pick_rows_per_tile(sp.mats, sp.n, nb, grid_cap, shape.tile) : (nb ? std::max(1u, shape.tile / nb) : 256u);
+    SeqItem& I = items[(size_t)i];
+    std::memset(&I, 0, sizeof I);
+    I.x = reinterpret_cast<const __half*>(sp.x);
+    I.x2 = reinterpret_cast<const __half*>(sp.pro.x2);
+    I.norm_w = reinterpret_cast<const __half*>(sp.pro.norm_w);
+    I.resid_out = reinterpret_cast<__half*>(sp.pro.resid_out);
+    I.eps = sp.pro.eps;
+    I.prologue = sp.pro.kind;
+    I.nb = nb;
+    I.tail_w = m0->tail_w;
+    I.inv_nb = nb ? 1.0f / (float)nb : 0.f;
+    I.y_f16 = sp.y_dtype == LLVQ_F16 ? 1u : 0u;
+    I.first_tile = (uint32_t)tiles.size();
+    I.wait_item = sp.after_previous ? (uint32_t)(i - 1) : kSeqNoWait;
+    I.signals = (i + 1 < n && specs[i + 1].after_previous) ? 1u : 0u;
+    const size_t ysz = sp.y_dtype == LLVQ_F16 ? 2 : 4;
+    for (int j = 0; j < sp.n; ++j) {
+      const llvq_mat* m = sp.mats[j];
+      for (uint32_t r0 = 0; r0 < m->d_out; r0 += rpt) {
+        SeqTile t{};
+        t.rows = std::min(rpt, m->d_out - r0);
+        t.nblk = t.rows * nb;
+        t.codes = m->codes + (size_t)r0 * nb * 6;
+        t.rscale = m->rscale + r0;
+        t.tail = m->tail + (size_t)r0 * m->tail_w;
+        t.y = reinterpret_cast<uint8_t*>(sp.y[j]) + (size_t)r0 * ysz;
+        t.g0 = m->g[0];
+        t.g1 = m->g[1];
+        t.item = (uint32_t)i;
+        tiles.push_back(t);
+      }
+    }
+  }
+  if (tiles.size() > 0x7FFFFFFFu) return fail(LLVQ_ERR_UNSUPPORTED, "sequence_create: too many tiles");
+  const uint32_t n_tiles = (uint32_t)tiles.size();
+  const uint32_t grid = std::min(n_tiles, grid_cap);
+  for (int i = 0; i < n; ++i) {
+    const uint32_t t0 = items[(size_t)i].first_tile, t1 = i + 1 < n ? items[(size_t)i + 1].first_tile : n_tiles;
+    items[(size_t)i].expected = std::min(t1 - t0, grid);
+  }
+  HIP_TRY(hipSetDevice(rt->device));
+  auto* q = new llvq_seq();
+  const size_t off_items = tiles.size() * sizeof(SeqTile);
+  const size_t off_counters = (off_items + items.size() * sizeof(SeqItem) + 255) & ~(size_t)255;
+  const size_t off_status = off_counters + (((size_t)n * 4 + 255) & ~(size_t)255);
+  const size_t total = off_status + 256;
+  hipError_t e = hipMalloc(reinterpret_cast<void**>(&q->blob), total);
+  if (e == hipSuccess) e = hipMemset(q->blob, 0, total);
+  if (e == hipSuccess) e = hipMemcpy(q->blob, tiles.data(), off_items, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(q->blob + off_items, items.data(), items.size() * sizeof(SeqItem), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(q->blob);
+    delete q;
+    return hip_fail(e, "sequence tables");
+  }
+  q->args.tables = rt->tables;
+  q->args.tiles = reinterpret_cast<const SeqTile*>(q->blob);
+  q->args.items = reinterpret_cast<const SeqItem*>(q->blob + off_items);
+  q->args.n_tiles = n_tiles;
+  q->args.max_nb = max_nb;
+  q->args.counters = reinterpret_cast<uint32_t*>(q->blob + off_counters);
+  q->args.status = reinterpret_cast<uint32_t*>(q->blob + off_status);
+  q->args.run = 0;
+  q->args.spin_limit = kSeqSpinLimit;
+  q->args.hold_item = kSeqNoWait;
+  q->tile = shape.tile;
+  q->lean = shape.lean;
+  q->lds = shape.lds;
+  q->grid = grid;
+  q->n_items = (uint32_t)n;
+  q->cooperative = dependent;
+  *out = q;
+  return LLVQ_OK;
+}
+
+static int seq_run(llvq_rt* rt, llvq_seq* q) {
+  q->args.run += 1;
+  SeqArgs a = q->args;
+  void* params[] = {&a};
+  const void* kernel = seq_kernel(q->tile, q->lean);
+  // a sequence with ordered items needs all of its workgroups resident: the cooperative launch refuses to start otherwise
+  if (q->cooperative) HIP_TRY(hipLaunchCooperativeKernel(kernel, dim3(q->grid), dim3(kWgThreads), params, (unsigned)q->lds, rt->stream));
+  else HIP_TRY(hipLaunchKernel(kernel, dim3(q->grid), dim3(kWgThreads), params, q->lds, rt->stream));
+  HIP_TRY(hipGetLastError());
+  q->args.hold_item = kSeqNoWait;
+  return LLVQ_OK;
+}
+
+int llvq_hip_sequence_create(llvq_rt* rt, const llvq_seq_item* items, int n_items, llvq_seq** out) {
+  if (!rt || !items || !out || n_items <= 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: bad argument");
+  *out = nullptr;
+  std::vector<SeqSpec> specs((size_t)n_items);
+  for (int i = 0; i < n_items; ++i) {
+    specs[(size_t)i].mats = items[i].mats;
+    specs[(size_t)i].n = items[i].n_mats;
+    specs[(size_t)i].x = items[i].x_f16_dev;
+    specs[(size_t)i].y = items[i].y_dev;
+    specs[(size_t)i].y_dtype = items[i].y_dtype;
+    specs[(size_t)i].after_previous = items[i].after_previous != 0;
+  }
+  return seq_create(rt, specs.data(), n_items, out);
+}
+
+int llvq_hip_sequence_run(llvq_rt* rt, llvq_seq* seq) {
+  if (!rt || !seq) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_run: null argument");
+  HIP_TRY(hipSetDevice(rt->device));
+  return seq_run(rt, seq);
+}
+
+int llvq_hip_sequence_status(llvq_rt* rt, llvq_seq* seq) {
+  if (!rt || !seq) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_status: null argument");
+  HIP_TRY(hipSetDevice(rt->device));
+  HIP_TRY(hipStreamSynchronize(rt->stream));
+  uint32_t st = 0;
+  HIP_TRY(hipMemcpy(&st, seq->args.status, sizeof st, hipMemcpyDeviceToHost));
+  if (!st) return LLVQ_OK;
+  // the counters of a run that gave up are short: start over from zero
+  HIP_TRY(hipMemset(seq->args.counters, 0, (size_t)((uint8_t*)seq->args.status - (uint8_t*)seq->args.counters) + 4));
+  seq->args.run = 0;
+  return fail(LLVQ_ERR_DEVICE, "sequence: a workgroup gave up waiting for an item; the run's outputs are incomplete");
+}
+
+int llvq_hip_sequence_tune(llvq_seq* seq, uint32_t spin_limit, int hold_item) {
+  if (!seq) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_tune: null sequence");
+  if (hold_item >= (int)seq->n_items) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_tune: no such item");
+  seq->args.spin_limit = spin_limit ? spin_limit : kSeqSpinLimit;
+  seq->args.hold_item = hold_item >= 0 ? (uint32_t)hold_item : kSeqNoWait;
+  return LLVQ_OK;
+}
+
+void llvq_hip_sequence_destroy(llvq_rt* rt, llvq_seq* seq) {
+  if (!seq) return;
+  if (rt) {
+    (void)hipSetDevice(rt->device);
+    (void)hipStreamSynchronize(rt->stream);
+  }
+  (void)hipFree(seq->blob);
+  delete seq;
 }
 
 // Grows a device buffer of the runtime to `need` bytes (contents are not kept).

@@ -100,6 +100,33 @@ class FusedProj:
         return self._rotation
 
 
+class FusedSequence:
+    """A bound list of group products that runs as one persistent kernel (no counterpart in the reference,
+    whose FusedOp launches per projection, fused_cuda.rs:758-900)."""
+
+    def __init__(self, rt, handle, outputs, keep):
+        self._rt, self.handle, self.outputs, self._keep = rt, handle, outputs, keep
+        self._run = _ffi.lib().llvq_hip_sequence_run
+
+    def run(self):
+        """Enqueues the whole list on the runtime's stream."""
+        rc = self._run(self._rt.handle, self.handle)
+        if rc:
+            _ffi.check(rc)
+
+    def status(self):
+        """Waits for the stream; raises LlvqError(Device) if a workgroup of an earlier run gave up waiting."""
+        _ffi.check(_ffi.lib().llvq_hip_sequence_status(self._rt.handle, self.handle))
+
+    def tune(self, spin_limit=0, hold_item=-1):
+        _ffi.check(_ffi.lib().llvq_hip_sequence_tune(self.handle, spin_limit, hold_item))
+
+    def close(self):
+        if self.handle:
+            _ffi.lib().llvq_hip_sequence_destroy(self._rt.handle, self.handle)
+            self.handle = None
+
+
 class FusedRuntime:
     """Tables and stream (fused_cuda.rs:145-180).  `FusedRuntime(model, device)`
     is `FusedRuntime::new`: it returns with every projection uploaded in `projs`."""
@@ -247,6 +274,36 @@ class FusedRuntime:
                 _ffi.check(rc)
 
         return launch, ys
+
+    def plan_sequence(self, items, out_dtype=None):
+        """Binds a list of group products as ONE launch (llvq_hip_sequence_create).  `items` is a list of
+        (projections, activation, after_previous[, outputs]): `activation` is an f16 device tensor of d_in
+        values; after_previous = True says the activation is (or depends on) an output of the item before it;
+        `outputs`, when given, are the caller's own result tensors of `out_dtype` (so that a later item can be
+        bound to them).  Returns a FusedSequence; its `outputs[i]` are item i's result tensors."""
+        torch = self._torch
+        out_dtype = out_dtype or torch.float16
+        code = self._out_code(out_dtype)
+        n = len(items)
+        arr = (_ffi.SeqItem * n)()
+        keep, outputs = [], []
+        for i, item in enumerate(items):
+            projs, x, after = item[0], item[1], item[2]
+            x = self._f16(x, projs[0])
+            ys = item[3] if len(item) > 3 and item[3] is not None else \
+                [torch.empty(list(x.shape[:-1]) + [p.d_out], dtype=out_dtype, device=x.device) for p in projs]
+            for y, p in zip(ys, projs):
+                if y.dtype != out_dtype or y.numel() != p.d_out or not y.is_contiguous():
+                    raise ValueError(f"{p.name}: output must be a contiguous {out_dtype} tensor of {p.d_out} values")
+            mats = (C.c_void_p * len(projs))(*[p.handle for p in projs])
+            outs = (C.c_void_p * len(projs))(*[y.data_ptr() for y in ys])
+            arr[i].mats, arr[i].n_mats, arr[i].x_f16_dev = mats, len(projs), x.data_ptr()
+            arr[i].y_dev, arr[i].y_dtype, arr[i].after_previous = outs, code, 1 if after else 0
+            keep.append((x, ys, mats, outs))
+            outputs.append(ys)
+        handle = C.c_void_p()
+        _ffi.check(_ffi.lib().llvq_hip_sequence_create(self.handle, arr, n, C.byref(handle)))
+        return FusedSequence(self, handle, outputs, keep)
 
     def forward_batched(self, proj: FusedProj, x, out_dtype=None):
         """Rows of `x` [M, d_in] through one projection (the row loop of model.rs:521-529)."""

@@ -182,6 +182,56 @@ class Qwen3Oracle:
         self.pos += 1
         return rnd(self.head @ x).astype(np.float32)
 
+    def prefill_rows(self, tokens, progress=None):
+        """The prompt's positions all at once, in matrix form (the reference's l > 1 path: every projection is
+        applied to all rows, model.rs:521-529; the causal mask of model.rs:985-994), from an empty cache.  Same
+        operators and the same roundings as forward_token — only the f64 summation order inside a product
+        differs — so the cache it leaves and the logits of its last row are those of a token-by-token run
+        (tests/test_oracle_runner.py compares the two).  Attention runs one query head at a time so that a long
+        prompt's score matrix stays one head's.  Returns the last row's logits."""
+        c = self.cfg
+        nh, nkv, hd = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+        eps, rnd = c.rms_norm_eps, self.rnd
+        assert self.pos == 0, "prefill_rows starts from an empty cache"
+        T = len(tokens)
+        h = self.embed[np.asarray(tokens, dtype=np.int64)].astype(np.float64)
+        cos, sin = self.cos[:T, None, :], self.sin[:T, None, :]
+        groups = nh // nkv
+        rows = np.arange(T)
+
+        def rope(t):
+            t1, t2 = t[..., : hd // 2], t[..., hd // 2:]
+            return rnd(np.concatenate([t1 * cos - t2 * sin, t1 * sin + t2 * cos], axis=-1))
+
+        for L in range(c.num_hidden_layers):
+            Wq, Wk, Wv, Wo, Wg, Wu, Wd = self.W[L]
+            x = rms_norm(h, self.ln1[L], eps, rnd)
+            q = rope(rms_norm(rnd(x @ Wq.T).reshape(T, nh, hd), self.qn[L], eps, rnd))
+            k = rope(rms_norm(rnd(x @ Wk.T).reshape(T, nkv, hd), self.kn[L], eps, rnd))
+            v = rnd(x @ Wv.T).reshape(T, nkv, hd)
+            if self.kv_mode == "q8":
+                k, v = quantize_dequantize(k), quantize_dequantize(v)
+            self.K[L] = [k[t] for t in range(T)]
+            self.V[L] = [v[t] for t in range(T)]
+            ctx = np.empty((T, nh, hd))
+            for head in range(nh):
+                kv = head // groups
+                s = (q[:, head, :] @ k[:, kv, :].T) / np.sqrt(float(hd))
+                s[rows[None, :] > rows[:, None]] = -np.inf
+                p = np.exp(s - s.max(-1, keepdims=True))
+                p /= p.sum(-1, keepdims=True)
+                ctx[:, head, :] = p @ v[:, kv, :]
+            ctx = rnd(ctx.reshape(T, nh * hd))
+            h = rnd(h + rnd(ctx @ Wo.T))
+            x = rms_norm(h, self.ln2[L], eps, rnd)
+            a = rnd(rnd(silu(rnd(x @ Wg.T))) * rnd(x @ Wu.T))
+            h = rnd(h + rnd(a @ Wd.T))
+            if progress:
+                progress(L)
+        self.pos = T
+        x = rms_norm(h[-1], self.fn, eps, rnd)
+        return rnd(self.head @ x).astype(np.float32)
+
     def generate(self, prompt, max_new):
         """model.rs:1041-1073; also returns the logits of every decoding step."""
         if max_new == 0:

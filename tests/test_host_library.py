@@ -285,14 +285,15 @@ def _c_type(decl):
     # drop the parameter name, if there is one
     known = {"void", "int", "char", "float", "double", "size_t", "uint8_t", "int8_t", "uint16_t", "uint32_t", "uint64_t",
              "llvq_rt", "llvq_mat", "llvq_decoder", "llvq_matrix_desc", "llvq_record_info", "llvq_raw_info", "llvq_blob_info",
-             "llvq_decoder_desc"}
+             "llvq_decoder_desc", "llvq_seq", "llvq_seq_item"}
     if len(words) > 1 and words[-1] not in known:
         words = words[:-1]
     ctype = " ".join(words)
     table = {"int": "c_int", "char": "c_char", "float": "f32", "double": "f64", "size_t": "usize", "uint8_t": "u8", "int8_t": "i8",
              "uint16_t": "u16", "uint32_t": "u32", "uint64_t": "u64", "void": "c_void", "llvq_rt": "LlvqRt", "llvq_mat": "LlvqMat",
              "llvq_decoder": "LlvqDecoder", "llvq_matrix_desc": "LlvqMatrixDesc", "llvq_record_info": "LlvqRecordInfo",
-             "llvq_raw_info": "LlvqRawInfo", "llvq_blob_info": "LlvqBlobInfo", "llvq_decoder_desc": "LlvqDecoderDesc"}
+             "llvq_raw_info": "LlvqRawInfo", "llvq_blob_info": "LlvqBlobInfo", "llvq_decoder_desc": "LlvqDecoderDesc",
+             "llvq_seq": "LlvqSeq", "llvq_seq_item": "LlvqSeqItem"}
     return table[ctype] + "*" * stars if stars else ("()" if ctype == "void" else table[ctype])
 
 

@@ -233,3 +233,32 @@ def test_reference_golden_tokens_of_the_tiny_model():
     assert got.tolist() == golden, (got.tolist(), [float(np.sort(t)[-1] - np.sort(t)[-2]) for t in trace])
     swapped, _ = _tiny_reference_model(swap_kv=True).generate(prompt, len(golden))
     assert swapped.tolist() != golden
+
+
+def test_matrix_form_prompt_pass_leaves_the_cache_of_a_token_by_token_run():
+    """prefill_rows (all prompt rows at once) against forward_token position by position: the cache
+    entries and the last row's logits agree up to what a different f64 summation order can move across a
+    binary16 rounding; the positions that follow, decoded over either cache, agree the same way."""
+    global CFG
+    saved = CFG
+    try:
+        for kv_mode, head_dim in (("f16", 16), ("q8", 64)):
+            CFG = SimpleNamespace(**{**vars(saved), "head_dim": head_dim})
+            _, W, w = _model(seed=7, tied=True)
+            ref = Q.Qwen3Oracle(CFG, W, w, kv_mode=kv_mode)
+            rows = Q.Qwen3Oracle(CFG, W, w, kv_mode=kv_mode)
+            tokens = np.random.default_rng(8).integers(0, CFG.vocab_size, size=13)
+            for t in tokens:
+                step = ref.forward_token(int(t))
+            last = rows.prefill_rows(tokens)
+            assert rows.pos == ref.pos == 13
+            assert np.abs(last - step).max() <= 2e-3 * np.abs(step).max() + 1e-6
+            for L in range(CFG.num_hidden_layers):
+                for a, b in ((ref.K[L], rows.K[L]), (ref.V[L], rows.V[L])):
+                    a, b = np.asarray(a), np.asarray(b)
+                    assert a.shape == b.shape and np.abs(a - b).max() <= 1e-2 * np.abs(a).max()
+            for t in (5, 1, 4):
+                x, y = ref.forward_token(t), rows.forward_token(t)
+                assert np.abs(x - y).max() <= 2e-3 * np.abs(x).max() + 1e-6
+    finally:
+        CFG = saved
