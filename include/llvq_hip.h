@@ -175,8 +175,10 @@ int llvq_hip_gemv_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
  * Results are those of the separate calls, bit for bit.
  *   after_previous = 0: the item's activation is complete before the run is enqueued.
  *   after_previous = 1: the activation is (or depends on) an output of the item before it in
- *     the list; the kernel orders the two on the device.  Such a sequence needs every
- *     workgroup resident at once and is launched cooperatively.
+ *     the list; the kernel orders the two on the device: a workgroup waits, a bounded time,
+ *     for the workgroups that store what it is about to read.  That needs every workgroup of the
+ *     launch resident at once (one per CU), which holds while nothing else occupies the device's
+ *     CUs for long; otherwise the run gives up and llvq_hip_sequence_status reports it.
  * Matrices stored in a rotated basis, and rows wider than 24 576 columns, are refused with
  * LLVQ_ERR_UNSUPPORTED (use the per-call entry points).  The pointers are captured at
  * creation; the matrices and buffers must outlive the sequence.  Runs of one sequence must
@@ -260,6 +262,17 @@ typedef struct llvq_quant_rows {
   const uint16_t* biases;
   uint32_t bits, group;     /* the kernels take 8 and 64 */
 } llvq_quant_rows;
+/* How llvq_hip_decoder_* launches the projection groups of a decoded position.  The results are the same bit for bit;
+ * the speed is not: a decode position is a chain of dependent products, and an ordered item of a sequence pays about
+ * what a launch boundary costs (measured on the Qwen3-4B shape: 245 / 226 / 220 tokens/s in the order below).
+ * Models a sequence cannot take (matrices in a rotated basis, hidden > 6144) use LLVQ_LAUNCH_PER_GROUP whatever is asked. */
+typedef enum llvq_launch_mode {
+  LLVQ_LAUNCH_PER_GROUP = 0,  /* one llvq_hip_gemv_group launch per group */
+  LLVQ_LAUNCH_SINGLE = 1,     /* one single-item sequence (llvq_hip_sequence_*) per group: the sequence kernel's tile loop */
+  LLVQ_LAUNCH_CHAINED = 2     /* o_proj, gate/up, down_proj and the next layer's q/k/v as one sequence of ordered items
+                                 between two attention launches */
+} llvq_launch_mode;
+
 typedef struct llvq_decoder_desc {
   uint32_t n_layers, hidden, n_heads, n_kv_heads, head_dim, intermediate, vocab;
   uint32_t max_positions;               /* KV-cache length, <= 8192 */
@@ -277,6 +290,7 @@ typedef struct llvq_decoder_desc {
   llvq_quant_rows lm_head_q8;           /* int8 head (Head::Q8, model.rs:569-575); absent and lm_head NULL = tied */
   uint32_t prefill_rows;                /* positions llvq_hip_decoder_prefill takes per pass (buffers for that many
                                            rows are allocated); 0 = the batched prompt path is not used */
+  uint32_t launch_mode;                 /* llvq_launch_mode: how a decoded position's projection groups are launched */
 } llvq_decoder_desc;
 /* Qwen3::new_with (model.rs:869): checks every projection's shape against the architecture. */
 int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* desc, llvq_decoder** out);

@@ -136,6 +136,7 @@ pub struct LlvqDecoderDesc {
     pub embed_q8: LlvqQuantRows,
     pub lm_head_q8: LlvqQuantRows,
     pub prefill_rows: u32,
+    pub launch_mode: u32,
 }
 
 pub const LLVQ_F32: c_int = 0;

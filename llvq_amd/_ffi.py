@@ -13,6 +13,7 @@ STATUS = {
     33: "Unsupported", 34: "Device",
 }
 F32, F16 = 0, 1
+LAUNCH_PER_GROUP, LAUNCH_SINGLE, LAUNCH_CHAINED = 0, 1, 2  # llvq_launch_mode
 STATIC_SCRATCH_BYTES = 64 << 20  # LLVQ_STATIC_SCRATCH_BYTES of include/llvq_hip.h
 FINGERPRINT = 0x338F420F11866319
 
@@ -75,7 +76,7 @@ class DecoderDesc(C.Structure):
         ("input_norm", C.c_void_p), ("post_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
         ("final_norm", C.c_void_p), ("embed", C.c_void_p), ("lm_head", C.c_void_p),
         ("kv_mode", C.c_uint32), ("embed_q8", QuantRows), ("lm_head_q8", QuantRows),
-        ("prefill_rows", C.c_uint32),
+        ("prefill_rows", C.c_uint32), ("launch_mode", C.c_uint32),
     ]
 
 

@@ -15,10 +15,11 @@
 //     behind the other wavefronts' arithmetic — and requests the code bytes of the tile after that;
 //   * two barriers per tile: [queue tile t, row sums of tile t - 1] | [unrank tile t, classify t + 1];
 //   * an item whose activation is produced by an earlier item of the list (`wait_item`) waits, just
-//     before it reads that activation, for a per-item counter that every workgroup bumps (release,
-//     device scope) when it has stored its last rows of the earlier item.  A workgroup only ever waits
+//     before it reads that activation, for a per-item counter that every workgroup bumps when its last
+//     rows of the earlier item have arrived in memory (outputs and activations are stored and loaded at
+//     device scope, past the XCDs' own L2s, so no cache is flushed).  A workgroup only ever waits
 //     for items below the one it is working on and takes its tiles in ascending order, so with every
-//     workgroup resident (grid <= CUs, one workgroup per CU, launched cooperatively) the waits end.
+//     workgroup resident (grid <= CUs, one workgroup per CU by its LDS, the device otherwise idle) the waits end.
 //     They are bounded all the same: a wait that reaches `spin_limit` polls sets `*status` and the
 //     workgroup returns, which makes every wait behind it give up in turn.
 //
@@ -57,7 +58,8 @@ struct SeqItem {
   uint32_t wait_item;     // kSeqNoWait, or the item that must be complete before the activation is read
   uint32_t expected;      // workgroups that take part in this item
   uint32_t signals;       // a later item waits for this one
-  uint32_t pad[2];
+  uint32_t wait_expected; // `expected` of wait_item
+  uint32_t pad;
 };
 static_assert(sizeof(SeqItem) == 80, "item records are read with scalar loads");
 
@@ -71,7 +73,22 @@ struct SeqArgs {
   uint32_t run;         // 1, 2, ...: item i is complete in this run at counters[i] == run * expected
   uint32_t spin_limit;
   uint32_t hold_item;  // kSeqNoWait, or an item this run must treat as never complete (tests of the give-up path)
+  unsigned long long* stamps;  // tuning builds (-DLLVQ_SEQ_STAMPS): [grid][kSeqStampTiles][8] realtime-counter readings, or null
 };
+
+// Phase timestamps of tuning builds: lane 0 of every workgroup stores the realtime counter (100 MHz) at the phase
+// boundaries of its first kSeqStampTiles tiles.  Slots: 0 round begins, 1 previous rows finished, 2 signalled,
+// 3 wait over, 4 activation staged, 5 queues and planes ready (barrier),
+// 6 unranked (this wavefront), 7 round ends (barrier).
+constexpr uint32_t kSeqStampTiles = 8;
+#ifdef LLVQ_SEQ_STAMPS
+#define LLVQ_SEQ_STAMP(k)                                                                                          \
+  do {                                                                                                             \
+    if (threadIdx.x == 0 && s.stamps && round < kSeqStampTiles) s.stamps[((size_t)blockIdx.x * kSeqStampTiles + round) * 8 + (k)] = wall_clock64(); \
+  } while (0)
+#else
+#define LLVQ_SEQ_STAMP(k) do {} while (0)
+#endif
 
 __host__ __device__ constexpr size_t gemv_seq_lds_bytes(uint32_t max_nb, uint32_t tile, size_t image_bytes) {
   return gemv_lds_bytes(max_nb, tile, image_bytes) + 2 * kCtrlWords * 4;  // a second set of counters and the wait's verdict
@@ -98,7 +115,9 @@ struct RowOperands {
   float rs[2], tl[2][2];
 };
 __device__ __forceinline__ void seq_request_row_operands(const SeqTile& t, uint32_t tail_w, RowOperands& o) {
-  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, sub = lane >> 4, l16 = lane & 15u;
+  uint32_t tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const uint32_t lane = tid & 63u, wave = tid >> 6, sub = lane >> 4, l16 = lane & 15u;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const uint32_t row = (wave * 4 + sub) + (uint32_t)j * (kWaves * 4);
@@ -113,7 +132,9 @@ __device__ __forceinline__ void seq_request_row_operands(const SeqTile& t, uint3
 // the row scale and the tail columns, and store y.
 __device__ __forceinline__ void seq_finish_rows(const SeqTile& t, const float* partial, const float* xtail, uint32_t nb, uint32_t tail_w,
                                                 uint32_t y_f16, const RowOperands& o) {
-  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, sub = lane >> 4, l16 = lane & 15u;
+  uint32_t tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));  // lane-derived values are formed per call, not carried around the loop over tiles
+  const uint32_t lane = tid & 63u, wave = tid >> 6, sub = lane >> 4, l16 = lane & 15u;
   for (uint32_t base = 0; base < t.rows; base += kWaves * 4) {
     const uint32_t j = base / (kWaves * 4);
     const uint32_t row = base + wave * 4 + sub;
@@ -136,9 +157,9 @@ __device__ __forceinline__ void seq_finish_rows(const SeqTile& t, const float* p
     v = fmaf(t1, l16 + 16 < tail_w ? xtail[l16 + 16] : 0.f, v);
 #pragma unroll
     for (int q = 8; q >= 1; q >>= 1) v += __shfl_xor(v, q, 16);  // fixed tree inside each group of 16 lanes
-    if (ok && l16 == 0) {
-      if (y_f16) store_out<__half>(t.y, row, v);
-      else store_out<float>(t.y, row, v);
+    if (ok && l16 == 0) {  // device scope: a later item of this launch may read it from another XCD
+      if (y_f16) store_half<true>(reinterpret_cast<__half*>(t.y) + row, __float2half_rn(v));
+      else __hip_atomic_store(reinterpret_cast<float*>(t.y) + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
@@ -177,6 +198,14 @@ __device__ __forceinline__ void carried_classified(const Carried<NB>& c, Classif
     cls.e1[i] = c.r[2 * i + 1];
   }
   cls.where = c.r[2 * NB];
+}
+
+// The lane's index in the workgroup as a value the compiler cannot see through: what is derived from it is formed
+// where it is used, not once before the loop over tiles and then carried around it in registers the decoders need.
+__device__ __forceinline__ uint32_t opaque_tid() {
+  uint32_t t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
 }
 
 template <int TILE, bool LEAN>
@@ -219,43 +248,76 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
   SeqTile prev{};            // its rows are finished at the top of the next round
   RowOperands ops{};
   uint32_t parity = 0;
-  // This workgroup has stored its last rows of item `it`: tell the items that wait for it.  Every
-  // wavefront first makes its own stores visible device-wide; one lane then counts the workgroup in.
+  // This workgroup has stored its last rows of item `it`: tell the items that wait for it.  The rows (and a
+  // new residual) went out as device-scope stores, which pass through this XCD's L2 to memory; every wavefront
+  // waits until its own have arrived, and one lane then counts the workgroup in.  No device-scope fence on either
+  // side: a release would write the whole L2 back and an acquire would empty it of the decode tables.
   auto signal_item = [&]() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_add(s.counters + it, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_fetch_add(s.counters + it, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
   __syncthreads();
+#ifdef LLVQ_SEQ_STAMPS
+  uint32_t round = 0;
+#endif
   for (;;) {
     // ---- the current tile's blocks join their queues; the previous tile's rows are finished
+    LLVQ_SEQ_STAMP(0);
     Q.ctrl = ctrl_sets + parity * kCtrlWords;
     Classified<kP1Blocks> cls;
     carried_classified(carried, cls);
-    queue_classified<kP1Blocks>(cls, TILE, Q);
+    queue_classified<kP1Blocks>(cls, TILE, Q, opaque_tid());
     const uint32_t origins = cls.where;
     seq_finish_rows(prev, Q.partial, xtail, nb, tail_w, y_f16, ops);
+    LLVQ_SEQ_STAMP(1);
+    // What a wavefront does for the NEXT tile in the gaps of a chunk loop: state 0 nothing done, 1 its code bytes
+    // requested (after the wavefront's first few chunks, a different number per wavefront of a SIMD), 2 classified
+    // (when the wavefront has no chunk left: the others are still on theirs).
+    const bool more = nxt < n_tiles;
+    const uint32_t request_after = wave >> 2;
+    auto classify_next = [&]() {
+      LaneRecords<kP1Blocks> rec;
+      carried_records(carried, rec);
+      Classified<kP1Blocks> c;
+      classify_records<kP1Blocks>(T, rec, next.nblk, c, opaque_tid());
+      carry_classified(c, carried);
+    };
+    auto for_next_tile = [&](uint32_t done, bool last, uint32_t state) {
+      if (!more) return 2u;
+      if (state == 0u && (last || done >= request_after)) {
+        LaneRecords<kP1Blocks> rec;
+#pragma unroll
+        for (int k = 0; k < kP1Blocks * 3 / 2; ++k) rec.w[k] = 0;
+        seq_request_records(next, opaque_tid(), rec);
+        carry_records(rec, carried);
+        return 1u;
+      }
+      return state;
+    };
     if (cur.item != it && cur.item != kSeqNoWait) {  // the same for every lane
       // the rows of the previous tile are finished with the old item's tail values before the new item's replace them
       if (it != kSeqNoWait && it_signals) signal_item();
       else __syncthreads();
+      LLVQ_SEQ_STAMP(2);
       const SeqItem I = s.items[cur.item];
       if (I.wait_item != kSeqNoWait) {
         if (tid == 0) {
-          const uint32_t target = s.run * s.items[I.wait_item].expected + (I.wait_item == s.hold_item ? 1u : 0u);
+          const uint32_t target = s.run * I.wait_expected + (I.wait_item == s.hold_item ? 1u : 0u);
           uint32_t ok = 0;
           for (uint32_t spins = 0; spins <= s.spin_limit; ++spins) {
             const uint32_t v = __hip_atomic_load(s.counters + I.wait_item, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if ((int32_t)(v - target) >= 0) { ok = 1; break; }
-            __builtin_amdgcn_s_sleep(2);
+            __builtin_amdgcn_s_sleep(1);
           }
           *verdict = ok;
           if (!ok) __hip_atomic_store(s.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __syncthreads();
         if (*verdict == 0) return;  // gave up: every lane leaves, and so will whoever waits for this workgroup
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        // what the awaited item stored is read below with device-scope loads, which do not stop at this XCD's L2
       }
+      LLVQ_SEQ_STAMP(3);
       // a derived activation is staged where the planes themselves go: the queues are already in use
       const ActivationSource src{I.x, nullptr, I.x2, I.norm_w, I.resid_out, I.eps, I.prologue, I.nb, I.tail_w,
                                  nullptr, nullptr, 1.f, 0u, 0u, nxt - G == I.first_tile};
@@ -266,40 +328,23 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
       inv_nb = I.inv_nb;
       y_f16 = I.y_f16;
       it_signals = I.signals;
+      LLVQ_SEQ_STAMP(4);
     }
     __syncthreads();
+    LLVQ_SEQ_STAMP(5);
 
-    // ---- the current tile is unranked; each wavefront, at a point of its own, requests and then classifies
-    // its share of the next tile
+    // ---- the current tile is unranked; each wavefront requests and classifies its share of the next tile on the way
     if (tid < (uint32_t)kCtrlWords) ctrl_sets[(parity ^ 1u) * kCtrlWords + tid] = 0;
-    settle_origins<kP1Blocks>(origins, Q.partial);
-    const bool more = nxt < n_tiles;
-    const uint32_t request_after = wave >> 2;
-    auto classify_next = [&]() {
-      LaneRecords<kP1Blocks> rec;
-      carried_records(carried, rec);
-      Classified<kP1Blocks> c;
-      classify_records<kP1Blocks>(T, rec, next.nblk, c);
-      carry_classified(c, carried);
-    };
-    // state: 0 nothing done, 1 the next tile's code bytes requested, 2 classified
-    const uint32_t state = unrank_tile<TILE, true>(T, Q, UnrankOperands{xplanes, xscale, nb, inv_nb, cur.g0, cur.g1},
-                                                   [&](uint32_t done, bool last, uint32_t state) {
-      if (!more) return 2u;
-      if (state == 0u && (last || done >= request_after)) {
-        LaneRecords<kP1Blocks> rec;
-#pragma unroll
-        for (int k = 0; k < kP1Blocks * 3 / 2; ++k) rec.w[k] = 0;
-        seq_request_records(next, tid, rec);
-        carry_records(rec, carried);
-        return 1u;
-      }
-      return state;
-    });
-    // a wavefront classifies when it has no chunk left: the others are still unranking theirs
+    settle_origins<kP1Blocks>(origins, Q.partial, opaque_tid());
+    const uint32_t state = unrank_tile<TILE, true>(T, Q, UnrankOperands{xplanes, xscale, nb, inv_nb, cur.g0, cur.g1}, for_next_tile);
     if (state == 1u) classify_next();
     seq_request_row_operands(cur, tail_w, ops);
+    LLVQ_SEQ_STAMP(6);
     __syncthreads();
+    LLVQ_SEQ_STAMP(7);
+#ifdef LLVQ_SEQ_STAMPS
+    ++round;
+#endif
     prev = cur;
     if (!more) break;
     cur = next;

@@ -359,8 +359,43 @@ __device__ __forceinline__ void store_out<__half>(void* y, uint32_t r, float v) 
   reinterpret_cast<__half*>(y)[r] = __float2half_rn(v);
 }
 
+// Loads and stores of values that another workgroup of the SAME launch produces or consumes (gemv_seq.h): device
+// scope, so that they meet in memory and not in an XCD's own L2, which the L2 of another XCD is not coherent with.
+// They replace the device-scope fences such an exchange would otherwise need — whose acquire side empties the
+// XCD's L2 of the decode tables every time.
+template <bool kDeviceScope>
+__device__ __forceinline__ __half load_half(const __half* p) {
+  if constexpr (kDeviceScope)
+    return __ushort_as_half(__hip_atomic_load(reinterpret_cast<const unsigned short*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  else
+    return *p;
+}
+template <bool kDeviceScope>
+__device__ __forceinline__ void store_half(__half* p, __half v) {
+  if constexpr (kDeviceScope)
+    __hip_atomic_store(reinterpret_cast<unsigned short*>(p), __half_as_ushort(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else
+    *p = v;
+}
+
 // One 24-column block of the activation -> scale and byte planes.
+template <bool kDeviceScope = false>
 __device__ __forceinline__ void load_block_f16(const __half* x, float (&v)[kDim]) {
+  if constexpr (kDeviceScope) {
+    if ((reinterpret_cast<uintptr_t>(x) & 3) == 0) {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(x);
+#pragma unroll
+      for (int k = 0; k < kDim / 2; ++k) {
+        const uint32_t w = __hip_atomic_load(src + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v[2 * k] = __half2float(__ushort_as_half((unsigned short)(w & 0xFFFFu)));
+        v[2 * k + 1] = __half2float(__ushort_as_half((unsigned short)(w >> 16)));
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kDim; ++j) v[j] = __half2float(load_half<true>(x + j));
+    }
+    return;
+  }
   if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
     const uint4* src = reinterpret_cast<const uint4*>(x);
 #pragma unroll
@@ -674,8 +709,8 @@ struct Classified {
 
 // First half of P1: table reads only, nothing is written — it may run while another tile's queues are in use.
 template <int NB>
-__device__ __forceinline__ void classify_records(const DecodeTables& T, const LaneRecords<NB>& rec, uint32_t nblk, Classified<NB>& c) {
-  const uint32_t tid = threadIdx.x;
+__device__ __forceinline__ void classify_records(const DecodeTables& T, const LaneRecords<NB>& rec, uint32_t nblk, Classified<NB>& c,
+                                                 uint32_t tid = threadIdx.x) {
   // Every LDS read below is unconditional, from a valid slot, so that the NB reads of a step go
   // out together (a guarded read is waited for where it is issued).  A lane past the tile's end
   // walks the tables with whatever bytes follow the tile and queues nothing.
@@ -720,8 +755,8 @@ __device__ __forceinline__ void classify_records(const DecodeTables& T, const La
 
 // Second half of P1: the lane's classified blocks go to the tile's queues (LDS writes and counters).
 template <int NB>
-__device__ __forceinline__ void queue_classified(Classified<NB>& c, uint32_t capacity, const GemvQueues& Q) {
-  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+__device__ __forceinline__ void queue_classified(Classified<NB>& c, uint32_t capacity, const GemvQueues& Q, uint32_t tid = threadIdx.x) {
+  const uint32_t lane = tid & 63u;
   uint32_t kq[NB];
 #pragma unroll
   for (int i = 0; i < NB; ++i) kq[i] = (c.where >> (2 * i)) & 3u;
@@ -791,11 +826,11 @@ __device__ __forceinline__ void queue_classified(Classified<NB>& c, uint32_t cap
 
 // The origin blocks of a lane's share decode to zero: their partial sums are written here.
 template <int NB>
-__device__ __forceinline__ void settle_origins(uint32_t where, float* partial) {
+__device__ __forceinline__ void settle_origins(uint32_t where, float* partial, uint32_t tid = threadIdx.x) {
   if (__any((where >> 8) & 15u)) {
 #pragma unroll
     for (int i = 0; i < NB; ++i)
-      if ((where >> (8 + i)) & 1u) partial[threadIdx.x * NB + (uint32_t)i] = 0.f;
+      if ((where >> (8 + i)) & 1u) partial[tid * NB + (uint32_t)i] = 0.f;
   }
 }
 
@@ -822,10 +857,14 @@ struct UnrankOperands {
   float inv_nb;             // 1 / nb, for the block -> column split
   float g0, g1;             // the matrix's gain centroids
 };
+
 template <int TILE, bool kHook, class Hook>
 __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const GemvQueues& Q, const UnrankOperands& op, Hook&& hook) {
   constexpr int kTileBlocks = TILE;
-  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  uint32_t tid = threadIdx.x;
+  // inside a persistent loop over tiles: lane-derived values are formed here, per call, not carried around that loop
+  if constexpr (kHook) asm volatile("" : "+v"(tid));
+  const uint32_t lane = tid & 63u;
   uint32_t* ctrl = Q.ctrl;
   float* partial = Q.partial;
   const uint32_t* xplanes = op.xplanes;
@@ -1019,9 +1058,9 @@ __device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint
 #pragma unroll
       for (int k = 0; k < kPer; ++k) {
         const uint32_t i = min(base + tid + (uint32_t)k * kWgThreads, d_in - 1u);
-        in0[k] = a.x[i];
-        in1[k] = src1[i];
-        in2[k] = src2[i];
+        in0[k] = load_half<kInPlace>(a.x + i);
+        in1[k] = load_half<kInPlace>(src1 + i);
+        in2[k] = src2[i];  // the norm's gains are constants (with SiLU this is x again, and unused)
       }
       request_first_tile();
       __builtin_amdgcn_sched_barrier(0);
@@ -1048,7 +1087,7 @@ __device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint
           if (i < d_in) {
             float r = __half2float(in0[k]);
             if (a.x2) r = __half2float(__float2half_rn(r + __half2float(in1[k])));
-            if (a.resid_out && a.writes_resid) a.resid_out[i] = __float2half_rn(r);
+            if (a.resid_out && a.writes_resid) store_half<kInPlace>(a.resid_out + i, __float2half_rn(r));
             v[k] = r;
             ss += r * r;
           }
@@ -1136,10 +1175,10 @@ __device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint
 #pragma unroll
         for (int j = 0; j < kDim; ++j) v[j] = a.x_f32[(size_t)c0 * kDim + j];
       } else {
-        load_block_f16(xsrc + (size_t)c0 * kDim, v);
+        load_block_f16<kInPlace>(xsrc + (size_t)c0 * kDim, v);
       }
     }
-    const float tail_v = tid < a.tail_w ? (a.x_f32 ? a.x_f32[(size_t)nb * kDim + tid] : __half2float(xsrc[(size_t)nb * kDim + tid])) : 0.f;
+    const float tail_v = tid < a.tail_w ? (a.x_f32 ? a.x_f32[(size_t)nb * kDim + tid] : __half2float(load_half<kInPlace>(xsrc + (size_t)nb * kDim + tid))) : 0.f;
     request_first_tile();
     __builtin_amdgcn_sched_barrier(0);
     if (tid < nb) quantize_values(v, xplanes + (size_t)tid * kPlaneDwords, xscale + tid);
@@ -1379,8 +1418,9 @@ struct llvq_seq {
   uint8_t* blob = nullptr;  // one device allocation: tiles | items | counters | status
   SeqArgs args{};
   uint32_t tile = 0, grid = 0, n_items = 0;
-  bool lean = false, cooperative = false;
+  bool lean = false;
   size_t lds = 0;
+  uint32_t* own_status = nullptr;  // the status word inside `blob` (args.status may point at a word several sequences share)
 };
 
 static thread_local std::string g_last_error;
@@ -2053,9 +2093,10 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
     const SeqSpec& sp = specs[i];
     const llvq_mat* m0 = sp.mats[0];
     const uint32_t nb = m0->nblocks;
-    // Ordered items are balanced one by one, like launches (everyone waits for an item's slowest workgroup);
-    // independent items fill their tiles, because the round-robin runs on across item boundaries.
-    uint32_t rpt = dependent ? pick_rows_per_tile(sp.mats, sp.n, nb, grid_cap, shape.tile) : (nb ? std::max(1u, shape.tile / nb) : 256u);
+    // Ordered items, and an item that is a launch by itself, are balanced one by one, like launches (everyone waits
+    // for an item's slowest workgroup); independent items fill their tiles, because the round-robin runs on across
+    // item boundaries.
+    uint32_t rpt = (dependent || n == 1) ? pick_rows_per_tile(sp.mats, sp.n, nb, grid_cap, shape.tile) : (nb ? std::max(1u, shape.tile / nb) : 256u);
     SeqItem& I = items[(size_t)i];
     std::memset(&I, 0, sizeof I);
     I.x = reinterpret_cast<const __half*>(sp.x);
@@ -2096,6 +2137,8 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
     const uint32_t t0 = items[(size_t)i].first_tile, t1 = i + 1 < n ? items[(size_t)i + 1].first_tile : n_tiles;
     items[(size_t)i].expected = std::min(t1 - t0, grid);
   }
+  for (int i = 0; i < n; ++i)
+    if (items[(size_t)i].wait_item != kSeqNoWait) items[(size_t)i].wait_expected = items[items[(size_t)i].wait_item].expected;
   HIP_TRY(hipSetDevice(rt->device));
   auto* q = new llvq_seq();
   const size_t off_items = tiles.size() * sizeof(SeqTile);
@@ -2118,15 +2161,16 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
   q->args.max_nb = max_nb;
   q->args.counters = reinterpret_cast<uint32_t*>(q->blob + off_counters);
   q->args.status = reinterpret_cast<uint32_t*>(q->blob + off_status);
+  q->own_status = q->args.status;
   q->args.run = 0;
   q->args.spin_limit = kSeqSpinLimit;
   q->args.hold_item = kSeqNoWait;
+  q->args.stamps = nullptr;
   q->tile = shape.tile;
   q->lean = shape.lean;
   q->lds = shape.lds;
   q->grid = grid;
   q->n_items = (uint32_t)n;
-  q->cooperative = dependent;
   *out = q;
   return LLVQ_OK;
 }
@@ -2136,11 +2180,21 @@ static int seq_run(llvq_rt* rt, llvq_seq* q) {
   SeqArgs a = q->args;
   void* params[] = {&a};
   const void* kernel = seq_kernel(q->tile, q->lean);
-  // a sequence with ordered items needs all of its workgroups resident: the cooperative launch refuses to start otherwise
-  if (q->cooperative) HIP_TRY(hipLaunchCooperativeKernel(kernel, dim3(q->grid), dim3(kWgThreads), params, (unsigned)q->lds, rt->stream));
-  else HIP_TRY(hipLaunchKernel(kernel, dim3(q->grid), dim3(kWgThreads), params, q->lds, rt->stream));
+  // An ordinary launch, also with ordered items: at most one workgroup per CU (by its LDS) and no more workgroups than
+  // CUs, so on a device this stream has to itself every workgroup is resident and the waits end.  (A cooperative launch
+  // would guarantee it, but costs some 200 us per launch here: 4B decode fell from 237 to 85 tokens/s with it.)  Should
+  // another queue hold CUs for longer than the bounded wait, the run gives up and says so; it cannot hang.
+  HIP_TRY(hipLaunchKernel(kernel, dim3(q->grid), dim3(kWgThreads), params, q->lds, rt->stream));
   HIP_TRY(hipGetLastError());
   q->args.hold_item = kSeqNoWait;
+  return LLVQ_OK;
+}
+
+// After a run that gave up: its counters are short, so the next run starts over from zero.
+static int seq_reset(llvq_seq* q) {
+  HIP_TRY(hipMemset(q->args.counters, 0, (size_t)q->n_items * 4));
+  HIP_TRY(hipMemset(q->args.status, 0, 4));
+  q->args.run = 0;
   return LLVQ_OK;
 }
 
@@ -2173,10 +2227,20 @@ int llvq_hip_sequence_status(llvq_rt* rt, llvq_seq* seq) {
   HIP_TRY(hipMemcpy(&st, seq->args.status, sizeof st, hipMemcpyDeviceToHost));
   if (!st) return LLVQ_OK;
   // the counters of a run that gave up are short: start over from zero
-  HIP_TRY(hipMemset(seq->args.counters, 0, (size_t)((uint8_t*)seq->args.status - (uint8_t*)seq->args.counters) + 4));
-  seq->args.run = 0;
+  const int rc = seq_reset(seq);
+  if (rc) return rc;
   return fail(LLVQ_ERR_DEVICE, "sequence: a workgroup gave up waiting for an item; the run's outputs are incomplete");
 }
+
+#ifdef LLVQ_SEQ_STAMPS
+// Tuning builds only: where the next runs of `seq` store their phase timestamps (device memory of
+// grid x kSeqStampTiles x 8 64-bit words, or null).
+extern "C" int llvq_hip_sequence_debug(llvq_seq* seq, void* stamps_dev, uint32_t* grid) {
+  seq->args.stamps = reinterpret_cast<unsigned long long*>(stamps_dev);
+  if (grid) *grid = seq->grid;
+  return LLVQ_OK;
+}
+#endif
 
 int llvq_hip_sequence_tune(llvq_seq* seq, uint32_t spin_limit, int hold_item) {
   if (!seq) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_tune: null sequence");
@@ -2519,6 +2583,14 @@ struct llvq_decoder {
   // llvq_hip_decoder_generate_phased: events recorded at the phase boundaries of a step (null otherwise)
   std::vector<hipEvent_t>* marks = nullptr;
   size_t next_mark = 0;
+  // A position's projections as sequences (empty: one launch of gemv_tiles_kernel per projection group).
+  //   chained: seqs[0] = layer 0's q/k/v, seqs[L + 1] = layer L's o_proj, gate/up, down_proj and layer L + 1's q/k/v,
+  //            each item ordered behind the one before it;
+  //   single:  seqs[4 L + j] = layer L's q/k/v, o_proj, gate/up, down_proj, one item each.
+  // They share one status word.
+  std::vector<llvq_seq*> seqs;
+  bool seq_chained = false;
+  uint32_t* seq_status = nullptr;
 };
 
 namespace {
@@ -2541,6 +2613,122 @@ void launch_head(llvq_decoder* d, uint32_t history_slot, bool record) {
   hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(1024), 0, st, d->best_val, d->best_idx,
                      d->head_grid * (kHeadThreads / 64), d->token, record ? d->history : (uint32_t*)nullptr, history_slot);
   phase_mark(d);
+}
+
+// Binds a position's projections as sequences (llvq_decoder::seqs), each item with the activation prologue its
+// launch would have.  The residual stream alternates between the decoder's two buffers exactly as decoder_step's
+// launches alternate them: layer 0's q/k/v reads h; every later prologue reads one buffer and stores the other.
+// A model a sequence cannot take (rotated matrices, rows too wide) leaves seqs empty: one launch per group then.
+int decoder_bind_sequences(llvq_decoder* d, bool chained) {
+  llvq_rt* rt = d->rt;
+  d->seq_chained = chained;
+  __half *h = d->h, *h_alt = d->h_alt;
+  auto give_up = [&](int rc) {
+    for (llvq_seq* q : d->seqs) llvq_hip_sequence_destroy(rt, q);
+    d->seqs.clear();
+    return rc == LLVQ_ERR_UNSUPPORTED ? (int)LLVQ_OK : rc;
+  };
+  void* qkv_out[3] = {d->q, d->k, d->v};
+  void* o_out[1] = {d->o};
+  void* gu_out[2] = {d->gate, d->up};
+  void* dn_out[1] = {d->down};
+  auto qkv_item = [&](uint32_t L, bool ordered) {
+    SeqSpec sp;
+    sp.mats = d->proj.data() + (size_t)L * 7;
+    sp.n = 3;
+    sp.x = h;
+    sp.y = qkv_out;
+    sp.after_previous = ordered;
+    sp.pro.kind = kPrologueAddRmsNorm;
+    sp.pro.norm_w = d->ln1 + (size_t)L * d->hidden;
+    sp.pro.eps = d->eps;
+    if (L) {  // the previous layer's MLP output joins the residual stream here
+      sp.pro.x2 = d->down;
+      sp.pro.resid_out = h_alt;
+      std::swap(h, h_alt);
+    }
+    return sp;
+  };
+  auto bind = [&](std::vector<SeqSpec>& items) {
+    llvq_seq* q = nullptr;
+    const int rc = seq_create(rt, items.data(), (int)items.size(), &q);
+    if (rc) return rc;
+    q->args.status = d->seq_status;
+    d->seqs.push_back(q);
+    return (int)LLVQ_OK;
+  };
+  if (!chained) {
+    for (uint32_t L = 0; L < d->n_layers; ++L) {
+      const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
+      std::vector<SeqSpec> one(1);
+      one[0] = qkv_item(L, false);
+      int rc = bind(one);
+      if (rc) return give_up(rc);
+      SeqSpec o;
+      o.mats = P + 3; o.n = 1; o.x = d->ctx; o.y = o_out;
+      one[0] = o;
+      if ((rc = bind(one))) return give_up(rc);
+      SeqSpec gu;
+      gu.mats = P + 4; gu.n = 2; gu.x = h; gu.y = gu_out;
+      gu.pro.kind = kPrologueAddRmsNorm;
+      gu.pro.norm_w = d->ln2 + (size_t)L * d->hidden;
+      gu.pro.eps = d->eps;
+      gu.pro.x2 = d->o;
+      gu.pro.resid_out = h_alt;
+      std::swap(h, h_alt);
+      one[0] = gu;
+      if ((rc = bind(one))) return give_up(rc);
+      SeqSpec dn;
+      dn.mats = P + 6; dn.n = 1; dn.x = d->up; dn.y = dn_out;
+      dn.pro.kind = kPrologueSiluMul;
+      dn.pro.x2 = d->gate;
+      one[0] = dn;
+      if ((rc = bind(one))) return give_up(rc);
+    }
+    return LLVQ_OK;
+  }
+  for (uint32_t L = 0; L <= d->n_layers; ++L) {
+    std::vector<SeqSpec> items;
+    if (L == 0) {
+      items.push_back(qkv_item(0, false));
+    } else {
+      const llvq_mat* const* P = d->proj.data() + (size_t)(L - 1) * 7;
+      SeqSpec o;
+      o.mats = P + 3; o.n = 1; o.x = d->ctx; o.y = o_out;
+      items.push_back(o);
+      SeqSpec gu;
+      gu.mats = P + 4; gu.n = 2; gu.x = h; gu.y = gu_out; gu.after_previous = true;
+      gu.pro.kind = kPrologueAddRmsNorm;
+      gu.pro.norm_w = d->ln2 + (size_t)(L - 1) * d->hidden;
+      gu.pro.eps = d->eps;
+      gu.pro.x2 = d->o;
+      gu.pro.resid_out = h_alt;
+      std::swap(h, h_alt);
+      items.push_back(gu);
+      SeqSpec dn;
+      dn.mats = P + 6; dn.n = 1; dn.x = d->up; dn.y = dn_out; dn.after_previous = true;
+      dn.pro.kind = kPrologueSiluMul;
+      dn.pro.x2 = d->gate;
+      items.push_back(dn);
+      if (L < d->n_layers) items.push_back(qkv_item(L, true));
+    }
+    const int rc = bind(items);
+    if (rc) return give_up(rc);
+  }
+  return LLVQ_OK;
+}
+
+// After the stream has drained: whether a workgroup of any sequence gave up waiting since the last check.
+int decoder_check_sequences(llvq_decoder* d) {
+  if (d->seqs.empty()) return LLVQ_OK;
+  uint32_t st = 0;
+  HIP_TRY(hipMemcpy(&st, d->seq_status, sizeof st, hipMemcpyDeviceToHost));
+  if (!st) return LLVQ_OK;
+  for (llvq_seq* q : d->seqs) {
+    const int rc = seq_reset(q);
+    if (rc) return rc;
+  }
+  return fail(LLVQ_ERR_DEVICE, "decoder: a workgroup gave up waiting for a projection of the same launch; the position's results are incomplete");
 }
 
 // Enqueues one position: embeds *dec->token, runs the layers at position dec->pos,
@@ -2592,23 +2780,8 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     }
     return forward_group(rt, mats, n, staged, outs, LLVQ_F16);
   };
-  // The residual stream alternates between two buffers: a projection launch whose
-  // prologue adds the previous branch reads one and (workgroup 0) writes the other.
-  for (uint32_t L = 0; L < d->n_layers; ++L) {
-    const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
-    // the previous layer's MLP output joins the residual stream in the q/k/v launch
-    Prologue ln1;
-    ln1.kind = kPrologueAddRmsNorm;
-    ln1.norm_w = d->ln1 + (size_t)L * d->hidden;
-    ln1.eps = d->eps;
-    if (L) {
-      ln1.x2 = d->down;
-      ln1.resid_out = h_alt;
-    }
-    void* qkv_out[3] = {d->q, d->k, d->v};
-    int rc = project(P, 3, h, qkv_out, ln1);
-    if (rc) return rc;
-    if (L) std::swap(h, h_alt);
+  // q/k norm, rope and the cache append of this position ride in the attention launch
+  auto attention = [&](uint32_t L) {
     KvQ8 lq8 = d->q8;
     if (d->kv_q8) {
       lq8.kq += L * cache_layer; lq8.vq += L * cache_layer;
@@ -2616,7 +2789,6 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     }
     __half* kc = d->kv_q8 ? nullptr : d->kcache + L * cache_layer;
     __half* vc = d->kv_q8 ? nullptr : d->vcache + L * cache_layer;
-    // q/k norm, rope and the cache append of this position ride in the attention launch
     AttnNew nw{};
     nw.q_raw = d->q;
     nw.k_raw = d->k;
@@ -2646,6 +2818,46 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     }
     if (!merge_inline)
       hipLaunchKernelGGL(attn_merge_kernel, dim3(d->n_heads), dim3(128), 0, st, d->attn_part, d->ctx, d->head_dim, n_splits);
+  };
+  if (!d->seqs.empty() && d->seq_chained) {
+    // the projections between two attention launches are one persistent launch each
+    int rc = seq_run(rt, d->seqs[0]);
+    if (rc) return rc;
+    for (uint32_t L = 0; L < d->n_layers; ++L) {
+      attention(L);
+      rc = seq_run(rt, d->seqs[(size_t)L + 1]);
+      if (rc) return rc;
+    }
+    h = d->n_layers ? d->h_alt : d->h;  // where the last post-attention residual went (decoder_bind_sequences)
+  } else if (!d->seqs.empty()) {
+    // one launch per projection group, through the sequence kernel's tile loop
+    for (uint32_t L = 0; L < d->n_layers; ++L) {
+      int rc = seq_run(rt, d->seqs[(size_t)L * 4]);
+      if (rc) return rc;
+      attention(L);
+      for (int j = 1; j < 4; ++j)
+        if ((rc = seq_run(rt, d->seqs[(size_t)L * 4 + j]))) return rc;
+    }
+    h = d->n_layers ? d->h_alt : d->h;
+  } else {
+  // The residual stream alternates between two buffers: a projection launch whose
+  // prologue adds the previous branch reads one and (workgroup 0) writes the other.
+  for (uint32_t L = 0; L < d->n_layers; ++L) {
+    const llvq_mat* const* P = d->proj.data() + (size_t)L * 7;
+    // the previous layer's MLP output joins the residual stream in the q/k/v launch
+    Prologue ln1;
+    ln1.kind = kPrologueAddRmsNorm;
+    ln1.norm_w = d->ln1 + (size_t)L * d->hidden;
+    ln1.eps = d->eps;
+    if (L) {
+      ln1.x2 = d->down;
+      ln1.resid_out = h_alt;
+    }
+    void* qkv_out[3] = {d->q, d->k, d->v};
+    int rc = project(P, 3, h, qkv_out, ln1);
+    if (rc) return rc;
+    if (L) std::swap(h, h_alt);
+    attention(L);
     void* o_out[1] = {d->o};
     rc = forward_group(rt, P + 3, 1, d->ctx, o_out, LLVQ_F16);
     if (rc) return rc;
@@ -2665,6 +2877,7 @@ int decoder_step(llvq_decoder* d, bool want_logits, uint32_t history_slot, bool 
     void* d_out[1] = {d->down};
     rc = project(P + 6, 1, d->up, d_out, act);
     if (rc) return rc;
+  }
   }
   phase_mark(d);
   if (want_logits) {
@@ -2879,6 +3092,7 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   const size_t o_bv = take(n_best * sizeof(float)), o_bi = take(n_best * sizeof(uint32_t));
   const size_t o_tok = take(sizeof(uint32_t)), o_hist = take((size_t)c->max_positions * sizeof(uint32_t));
   const size_t o_ap = take((size_t)c->n_heads * kAttnMaxSplits * (c->head_dim + 2) * sizeof(float)), o_ac = take((size_t)c->n_kv_heads * sizeof(uint32_t));
+  const size_t o_seqst = take(256);
   hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->blob), total);
   if (e != hipSuccess) { delete d; return hip_fail(e, "hipMalloc(decoder)"); }
   auto put = [&](size_t at, const void* src, size_t bytes) { return hipMemcpy(d->blob + at, src, bytes, hipMemcpyHostToDevice); };
@@ -2920,6 +3134,7 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
   d->history = reinterpret_cast<uint32_t*>(d->blob + o_hist);
   d->attn_part = reinterpret_cast<float*>(d->blob + o_ap);
   d->attn_counters = reinterpret_cast<uint32_t*>(d->blob + o_ac);
+  d->seq_status = reinterpret_cast<uint32_t*>(d->blob + o_seqst);
   if (c->prefill_rows) {
     // row buffers of the batched prompt path, one allocation
     const size_t R = c->prefill_rows;
@@ -2948,6 +3163,14 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
       if (rc) { (void)hipFree(d->pblob); (void)hipFree(d->blob); delete d; return rc; }
     }
   }
+  if (c->launch_mode > LLVQ_LAUNCH_CHAINED) {
+    (void)hipFree(d->pblob); (void)hipFree(d->blob); delete d;
+    return fail(LLVQ_ERR_INVALID_ARGUMENT, "decoder_create: unknown launch_mode");
+  }
+  if (c->launch_mode != LLVQ_LAUNCH_PER_GROUP) {
+    const int rc = decoder_bind_sequences(d, c->launch_mode == LLVQ_LAUNCH_CHAINED);
+    if (rc) { (void)hipFree(d->pblob); (void)hipFree(d->blob); delete d; return rc; }
+  }
   *out = d;
   return LLVQ_OK;
 }
@@ -2956,6 +3179,7 @@ void llvq_hip_decoder_destroy(llvq_decoder* d) {
   if (!d) return;
   (void)hipSetDevice(d->rt->device);
   (void)hipStreamSynchronize(d->rt->stream);
+  for (llvq_seq* q : d->seqs) llvq_hip_sequence_destroy(d->rt, q);
   (void)hipFree(d->pblob);
   (void)hipFree(d->blob);
   delete d;
@@ -2986,7 +3210,7 @@ int llvq_hip_decoder_forward_token(llvq_decoder* d, uint32_t token, float* logit
   if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, d->logits, (size_t)d->vocab * sizeof(float), hipMemcpyDeviceToHost, d->rt->stream));
   if (argmax_host) HIP_TRY(hipMemcpyAsync(argmax_host, d->token, sizeof(uint32_t), hipMemcpyDeviceToHost, d->rt->stream));
   HIP_TRY(hipStreamSynchronize(d->rt->stream));
-  return LLVQ_OK;
+  return decoder_check_sequences(d);
 }
 
 static int generate_impl(llvq_decoder* d, const uint32_t* prompt, size_t n_prompt, size_t max_new, uint32_t* out, bool batched,
@@ -3035,6 +3259,10 @@ static int generate_impl(llvq_decoder* d, const uint32_t* prompt, size_t n_promp
   }
   HIP_TRY(hipMemcpyAsync(out, d->history, max_new * sizeof(uint32_t), hipMemcpyDeviceToHost, d->rt->stream));
   HIP_TRY(hipStreamSynchronize(d->rt->stream));
+  {
+    const int rc = decoder_check_sequences(d);
+    if (rc) return rc;
+  }
   if (phase_ms) {
     auto between = [&](size_t a, size_t b, double* ms) -> int {
       float f = 0.f;
@@ -3082,5 +3310,11 @@ int llvq_hip_decoder_prefill(llvq_decoder* d, const uint32_t* tokens, size_t n, 
   HIP_TRY(hipStreamSynchronize(d->rt->stream));
   return LLVQ_OK;
 }
+
+#ifdef LLVQ_SEQ_STAMPS
+llvq_seq* llvq_hip_decoder_debug_sequence(llvq_decoder* d, int index) {
+  return d && index >= 0 && (size_t)index < d->seqs.size() ? d->seqs[(size_t)index] : nullptr;
+}
+#endif
 
 }  // extern "C"

@@ -99,8 +99,10 @@ class Decoder:
     """A Qwen3-architecture model on one GPU: projections uploaded through `rt`,
     the rest copied at construction."""
 
-    def __init__(self, rt: FusedRuntime, cfg: Qwen3Config, projections, weights: DecoderWeights, prefill_rows: int = 0):
-        """prefill_rows > 0 also allocates the row buffers of the batched prompt path (`prefill`)."""
+    def __init__(self, rt: FusedRuntime, cfg: Qwen3Config, projections, weights: DecoderWeights, prefill_rows: int = 0,
+                 launch_mode: int = _ffi.LAUNCH_PER_GROUP):
+        """prefill_rows > 0 also allocates the row buffers of the batched prompt path (`prefill`).
+        launch_mode: llvq_launch_mode of include/llvq_hip.h (how a position's projection groups are launched)."""
         self.rt, self.cfg = rt, cfg
         self.handle = None
         self._owned = []
@@ -150,7 +152,7 @@ class Decoder:
             cfg.max_positions, float(cfg.rope_theta), float(cfg.rms_norm_eps),
             C.cast(arr, C.POINTER(C.c_void_p)),
             keep[0].ctypes.data, keep[1].ctypes.data, keep[2].ctypes.data, keep[3].ctypes.data, keep[4].ctypes.data,
-            e_ptr, h_ptr, self._kv_mode(cfg.kv_mode), e_q, h_q, int(prefill_rows))
+            e_ptr, h_ptr, self._kv_mode(cfg.kv_mode), e_q, h_q, int(prefill_rows), int(launch_mode))
         self._alive = (keep, e_alive, h_alive)
         out = C.c_void_p()
         _ffi.check(_ffi.lib().llvq_hip_decoder_create(rt.handle, C.byref(desc), C.byref(out)))

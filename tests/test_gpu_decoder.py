@@ -476,3 +476,79 @@ def test_full_size_greedy_tokens_match_the_oracle_fixture(gpu_rt, fixture_name, 
                                f"oracle gap {fixture['top_two_gap'][int(np.argmin(same))]}"
     finally:
         dec.close()
+
+
+@pytest.mark.parametrize("cfg,seed", [(SMALL, 1), (RAGGED, 2), (Q8, 6)])
+def test_sequences_and_separate_launches_give_the_same_bits(gpu_rt, cfg, seed):
+    """The three ways a position's projection groups are launched (llvq_launch_mode: single-item sequences, one
+    llvq_hip_gemv_group launch per group, chains of ordered items between attention launches): the same arithmetic
+    in the same order, so logits and tokens must be identical bit for bit, position after position (30 positions;
+    the residual buffers alternate, the counters of the chained sequences count on)."""
+    from llvq_amd import _ffi
+
+    raws = decoder.synthetic_projections(cfg, seed)
+    weights = decoder.synthetic_weights(cfg, seed)
+    projs = [[gpu_rt.upload(m) for m in layer] for layer in raws]
+    decs = [decoder.Decoder(gpu_rt, cfg, projs, weights, launch_mode=m)
+            for m in (_ffi.LAUNCH_PER_GROUP, _ffi.LAUNCH_SINGLE, _ffi.LAUNCH_CHAINED)]
+    try:
+        tokens = np.random.default_rng(seed).integers(0, cfg.vocab_size, size=30)
+        for t in tokens:
+            outs = [d.forward_token(int(t)) for d in decs]
+            for l, tok in outs[1:]:
+                assert tok == outs[0][1] and np.array_equal(l, outs[0][0])
+        prompt = tokens[:9]
+        gens = [d.generate(prompt, 12) for d in decs]
+        assert np.array_equal(gens[0], gens[1]) and np.array_equal(gens[0], gens[2])
+    finally:
+        for d in decs:
+            d.close()
+        for layer in projs:
+            for p in layer:
+                gpu_rt.free(p)
+
+
+def test_config4_widths_and_context_against_the_oracle(gpu_rt):
+    """BASELINE config 4's regime in one piece, against the oracle: the Qwen3-14B widths (hidden 5120, 40 query
+    heads over 8 kv heads of 128, 17 408-wide down_proj rows — the lean-image kernel variant), int8 KV cache, 8192
+    cached positions; 2 layers and a vocabulary of 2048 so that the oracle can follow (its logits are the fixture
+    tests/golden/qwen3_14b_widths_q8kv_8192_logits.npz, written by make_config4_logits.py).  The device fills the
+    cache position by position (split-KV attention over 64 ranges and the merge kernel) and by the batched path
+    (512 rows a pass); the logits of the last prompt position and of six more are compared.  Bar: 1e-3 of the
+    largest logit, i.e. one binary16 step: logits are binary16 values on both sides, a step of the largest one is
+    between 4.9e-4 and 9.8e-4 of it, and a different summation order can move a logit across one rounding boundary
+    (observed position by position: 7.2e-4 — one step of a logit in [1, 2) under a largest logit of 1.36).  Two
+    steps fail."""
+    import importlib.util
+    import os
+
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_config4_logits", os.path.join(golden, "make_config4_logits.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)  # the model description and seeds the fixture was made with (runs nothing)
+    with np.load(os.path.join(golden, "qwen3_14b_widths_q8kv_8192_logits.npz")) as f:
+        want = f["logits"].astype(np.float64)
+        assert (int(f["model_seed"]), int(f["prompt_seed"]), int(f["more_seed"]), int(f["n_prompt"])) == \
+            (gen.MODEL_SEED, gen.PROMPT_SEED, gen.MORE_SEED, gen.N_PROMPT)
+    cfg = gen.CFG
+    assert (cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.kv_mode) == (5120, 17408, 40, 8, "q8")
+    dec = decoder.Decoder(gpu_rt, cfg, decoder.synthetic_projections(cfg, gen.MODEL_SEED), decoder.synthetic_weights(cfg, gen.MODEL_SEED),
+                          prefill_rows=512)
+    try:
+        tokens = np.random.default_rng(gen.PROMPT_SEED).integers(0, cfg.vocab_size, size=gen.N_PROMPT)
+        more = np.random.default_rng(gen.MORE_SEED).integers(0, cfg.vocab_size, size=gen.N_MORE)
+        for batched in (False, True):
+            dec.reset()
+            if batched:
+                got = [dec.prefill(tokens)[0]]
+            else:
+                for t in tokens[:-1]:
+                    dec.forward_token(int(t), want_logits=False)
+                got = [dec.forward_token(int(tokens[-1]))[0]]
+            got += [dec.forward_token(int(t))[0] for t in more]
+            assert dec.position == 8192
+            worst = max(float(np.abs(g - w).max() / np.abs(w).max()) for g, w in zip(got, want))
+            print(f"OBSERVED config4 widths, 8192 positions, batched={batched}: {worst:.3e}")
+            assert worst < 1e-3, f"batched={batched}: max |dlogit| / max|logit| = {worst:.3e}"
+    finally:
+        dec.close()
