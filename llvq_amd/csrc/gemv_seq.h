@@ -208,7 +208,7 @@ __device__ __forceinline__ uint32_t opaque_tid() {
   return t;
 }
 
-template <int TILE, bool LEAN>
+template <int TILE, bool LEAN, int PLANES>
 __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
   constexpr int kP1Blocks = TILE / kWgThreads;
   extern __shared__ __align__(16) uint8_t smem[];
@@ -293,6 +293,12 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
         carry_records(rec, carried);
         return 1u;
       }
+#ifdef LLVQ_EXP_CLASSIFY_MID
+      if (state == 1u && (last || done >= request_after + LLVQ_EXP_CLASSIFY_MID)) {
+        classify_next();
+        return 2u;
+      }
+#endif
       return state;
     };
     if (cur.item != it && cur.item != kSeqNoWait) {  // the same for every lane
@@ -320,8 +326,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
       LLVQ_SEQ_STAMP(3);
       // a derived activation is staged where the planes themselves go: the queues are already in use
       const ActivationSource src{I.x, nullptr, I.x2, I.norm_w, I.resid_out, I.eps, I.prologue, I.nb, I.tail_w,
-                                 nullptr, nullptr, 1.f, 0u, 0u, nxt - G == I.first_tile};
-      (void)stage_activation<TILE, false, true>(src, xplanes, xscale, xtail, reinterpret_cast<uint8_t*>(xplanes), Q.partial, [] {});
+                                 nullptr, nullptr, 1.f, 0u, 0u, nxt - G == I.first_tile, I.wait_item != kSeqNoWait};
+      (void)stage_activation<TILE, false, PLANES, true>(src, xplanes, xscale, xtail, reinterpret_cast<uint8_t*>(xplanes), Q.partial, [] {});
       it = cur.item;
       nb = I.nb;
       tail_w = I.tail_w;
@@ -336,7 +342,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     // ---- the current tile is unranked; each wavefront requests and classifies its share of the next tile on the way
     if (tid < (uint32_t)kCtrlWords) ctrl_sets[(parity ^ 1u) * kCtrlWords + tid] = 0;
     settle_origins<kP1Blocks>(origins, Q.partial, opaque_tid());
-    const uint32_t state = unrank_tile<TILE, true>(T, Q, UnrankOperands{xplanes, xscale, nb, inv_nb, cur.g0, cur.g1}, for_next_tile);
+    const uint32_t state = unrank_tile<TILE, true, PLANES>(T, Q, UnrankOperands{xplanes, xscale, nb, inv_nb, cur.g0, cur.g1}, for_next_tile);
     if (state == 1u) classify_next();
     seq_request_row_operands(cur, tail_w, ops);
     LLVQ_SEQ_STAMP(6);

@@ -414,23 +414,32 @@ __device__ __forceinline__ void load_block_f16(const __half* x, float (&v)[kDim]
   }
 }
 
+// PLANES = 3: x = scale (65536 d2 + 256 d1 + d0), |...| <= 2^22, for results stored as f32; PLANES = 2: x = scale (256 d1 + d0),
+// |...| <= 2^14, for results stored as binary16 — an activation is then rounded at 2^-15 of its block's largest value,
+// a sixteenth of the half ulp the stored result carries anyway, and a block costs a third fewer dot products.
+template <int PLANES>
 __device__ __forceinline__ void quantize_values(const float (&v)[kDim], uint32_t* planes, float* scale);
 
+template <int PLANES>
 __device__ __forceinline__ void quantize_block(const __half* x, uint32_t* planes, float* scale) {
   float v[kDim];
   load_block_f16(x, v);
-  quantize_values(v, planes, scale);
+  quantize_values<PLANES>(v, planes, scale);
 }
 
 // f32 activation (a rotated one, fused_cuda.rs:384): same block-scaled fixed point
+template <int PLANES>
 __device__ __forceinline__ void quantize_block_f32(const float* x, uint32_t* planes, float* scale) {
   float v[kDim];
 #pragma unroll
   for (int j = 0; j < kDim; ++j) v[j] = x[j];
-  quantize_values(v, planes, scale);
+  quantize_values<PLANES>(v, planes, scale);
 }
 
+template <int PLANES>
 __device__ __forceinline__ void quantize_values(const float (&v)[kDim], uint32_t* planes, float* scale) {
+  static_assert(PLANES == 2 || PLANES == 3, "two or three byte planes");
+  constexpr int kBits = PLANES == 3 ? 22 : 14;
   float amax = 0.f;
 #pragma unroll
   for (int j = 0; j < kDim; ++j) amax = fmaxf(amax, fabsf(v[j]));
@@ -439,18 +448,18 @@ __device__ __forceinline__ void quantize_values(const float (&v)[kDim], uint32_t
   for (int j = 0; j < kDim; ++j) bad |= !(fabsf(v[j]) <= 3.4028234e38f);  // inf or NaN
   int e = 0;
   (void)frexpf(amax, &e);  // amax = m 2^e, m in [0.5, 1)
-  const float up = ldexpf(1.f, 22 - e);
-  *scale = bad ? __builtin_nanf("") : (amax == 0.f ? 0.f : ldexpf(1.f, e - 22));
+  const float up = ldexpf(1.f, kBits - e);
+  *scale = bad ? __builtin_nanf("") : (amax == 0.f ? 0.f : ldexpf(1.f, e - kBits));
   uint32_t p0[6], p1[6], p2[6];
 #pragma unroll
   for (int q = 0; q < 6; ++q) p0[q] = p1[q] = p2[q] = 0;
 #pragma unroll
   for (int j = 0; j < kDim; ++j) {
-    const int xq = (amax == 0.f || bad) ? 0 : (int)rintf(v[j] * up);  // |xq| <= 2^22
+    const int xq = (amax == 0.f || bad) ? 0 : (int)rintf(v[j] * up);  // |xq| <= 2^kBits
     const int d0 = (int)(int8_t)(xq & 0xFF);
     const int x1 = (xq - d0) >> 8;
     const int d1 = (int)(int8_t)(x1 & 0xFF);
-    const int d2 = (x1 - d1) >> 8;
+    const int d2 = (x1 - d1) >> 8;  // zero with two planes: |x1| <= 64
     p0[j >> 2] |= (uint32_t)(d0 & 0xFF) << (8 * (j & 3));
     p1[j >> 2] |= (uint32_t)(d1 & 0xFF) << (8 * (j & 3));
     p2[j >> 2] |= (uint32_t)(d2 & 0xFF) << (8 * (j & 3));
@@ -459,11 +468,13 @@ __device__ __forceinline__ void quantize_values(const float (&v)[kDim], uint32_t
   for (int q = 0; q < 6; ++q) {
     planes[q] = p0[q];
     planes[6 + q] = p1[q];
-    planes[12 + q] = p2[q];
+    if (PLANES == 3) planes[12 + q] = p2[q];
   }
 }
 
+template <int PLANES>
 __device__ __forceinline__ float planes_to_float(int d0, int d1, int d2) {
+  if (PLANES == 2) return fmaf((float)d1, 256.f, (float)d0);
   return fmaf((float)d2, 65536.f, fmaf((float)d1, 256.f, (float)d0));
 }
 
@@ -858,7 +869,7 @@ struct UnrankOperands {
   float g0, g1;             // the matrix's gain centroids
 };
 
-template <int TILE, bool kHook, class Hook>
+template <int TILE, bool kHook, int PLANES, class Hook>
 __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const GemvQueues& Q, const UnrankOperands& op, Hook&& hook) {
   constexpr int kTileBlocks = TILE;
   uint32_t tid = threadIdx.x;
@@ -910,9 +921,9 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
     for (int q = 0; q < 6; ++q) {
       d0 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[q], d0, false);
       d1 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[6 + q], d1, false);
-      d2 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[12 + q], d2, false);
+      if (PLANES == 3) d2 = __builtin_amdgcn_sdot4((int)w[q], (int)xp[12 + q], d2, false);
     }
-    partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (c.inv_norm * b.g);
+    partial[b.f] = planes_to_float<PLANES>(d0, d1, d2) * xscale[b.col] * (c.inv_norm * b.g);
   };
   auto odd_block = [&](uint2 e, uint32_t f) {
     const Block b = open_block(e, f);
@@ -923,9 +934,9 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
       const int w = (int)__builtin_amdgcn_perm(fc.tab_hi, fc.tab_lo, sel);
       d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
       d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-      d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+      if (PLANES == 3) d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
     });
-    partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
+    partial[b.f] = planes_to_float<PLANES>(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
   };
   auto even_block = [&](uint2 e, uint32_t f, auto second) {
     constexpr bool kSecond = decltype(second)::value;
@@ -940,9 +951,9 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
       if (kSecond) w |= (int)__builtin_amdgcn_perm(tab2_hi, tab2_lo, sel2);
       d0 = __builtin_amdgcn_sdot4(w, (int)xp[q], d0, false);
       d1 = __builtin_amdgcn_sdot4(w, (int)xp[6 + q], d1, false);
-      d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
+      if (PLANES == 3) d2 = __builtin_amdgcn_sdot4(w, (int)xp[12 + q], d2, false);
     });
-    partial[b.f] = planes_to_float(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
+    partial[b.f] = planes_to_float<PLANES>(d0, d1, d2) * xscale[b.col] * (fc.inv_norm * b.g);
   };
   uint32_t chunk = ticket();
   // the generic chunks, kept out of the loop below: their code and registers are not the hot path's
@@ -1013,6 +1024,7 @@ struct ActivationSource {
   float rot_inv;
   uint32_t rot_m, rot_k;
   bool writes_resid;   // this workgroup is the one that stores the new residual
+  bool device_scope = false;  // a finished activation is read at device scope (another workgroup of this launch stored it)
 };
 
 // Fills the activation planes, scales and tail values in LDS from `a`, by every lane of the workgroup.
@@ -1021,7 +1033,7 @@ struct ActivationSource {
 // activation's operands (the caller's first code bytes go out there).  Returns whether the staging
 // area was used: the caller then needs a barrier before the area becomes queues again.  kInPlace: `raw` is the
 // planes' own memory (rows of at most as many blocks as the workgroup has lanes, natural basis only).
-template <int TILE, bool ROT, bool kInPlace = false, class Request>
+template <int TILE, bool ROT, int PLANES, bool kInPlace = false, class Request>
 __device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint32_t* xplanes, float* xscale, float* xtail, uint8_t* raw,
                                                  float* partial, Request&& request_first_tile) {
   constexpr int kTileBlocks = TILE;
@@ -1147,7 +1159,7 @@ __device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint
     rotate_lds(xf, d_in, a.rot_m, a.rot_k, a.rot_inv, a.rot_small);
     __syncthreads();
     for (uint32_t col = tid; col < nb; col += kWgThreads)
-      quantize_block_f32(xf + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+      quantize_block_f32<PLANES>(xf + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     if (tid < a.tail_w) xtail[tid] = xf[(size_t)nb * kDim + tid];
   } else if (a.prologue != kPrologueNone) {
     if constexpr (kInPlace) {
@@ -1156,11 +1168,11 @@ __device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint
       load_block_f16(xsrc + (size_t)min(tid, nb ? nb - 1u : 0u) * kDim, v);
       const float tail_v = tid < a.tail_w ? __half2float(xsrc[(size_t)nb * kDim + tid]) : 0.f;
       __syncthreads();
-      if (tid < nb) quantize_values(v, xplanes + (size_t)tid * kPlaneDwords, xscale + tid);
+      if (tid < nb) quantize_values<PLANES>(v, xplanes + (size_t)tid * kPlaneDwords, xscale + tid);
       if (tid < a.tail_w) xtail[tid] = tail_v;
     } else {
       for (uint32_t col = tid; col < nb; col += kWgThreads)
-        quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+        quantize_block<PLANES>(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
       if (tid < a.tail_w) xtail[tid] = __half2float(xsrc[(size_t)nb * kDim + tid]);
     }
   } else {
@@ -1175,17 +1187,24 @@ __device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint
 #pragma unroll
         for (int j = 0; j < kDim; ++j) v[j] = a.x_f32[(size_t)c0 * kDim + j];
       } else {
-        load_block_f16<kInPlace>(xsrc + (size_t)c0 * kDim, v);
+        // (an activation another workgroup of this launch stored is read at device scope; any other through the caches)
+        if (kInPlace && a.device_scope) load_block_f16<true>(xsrc + (size_t)c0 * kDim, v);
+        else load_block_f16<false>(xsrc + (size_t)c0 * kDim, v);
       }
     }
-    const float tail_v = tid < a.tail_w ? (a.x_f32 ? a.x_f32[(size_t)nb * kDim + tid] : __half2float(load_half<kInPlace>(xsrc + (size_t)nb * kDim + tid))) : 0.f;
+    float tail_v = 0.f;
+    if (tid < a.tail_w) {
+      if (a.x_f32) tail_v = a.x_f32[(size_t)nb * kDim + tid];
+      else if (kInPlace && a.device_scope) tail_v = __half2float(load_half<true>(xsrc + (size_t)nb * kDim + tid));
+      else tail_v = __half2float(xsrc[(size_t)nb * kDim + tid]);
+    }
     request_first_tile();
     __builtin_amdgcn_sched_barrier(0);
-    if (tid < nb) quantize_values(v, xplanes + (size_t)tid * kPlaneDwords, xscale + tid);
+    if (tid < nb) quantize_values<PLANES>(v, xplanes + (size_t)tid * kPlaneDwords, xscale + tid);
     if (tid < a.tail_w) xtail[tid] = tail_v;
     for (uint32_t col = tid + kWgThreads; col < nb; col += kWgThreads) {
-      if (a.x_f32) quantize_block_f32(a.x_f32 + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
-      else quantize_block(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+      if (a.x_f32) quantize_block_f32<PLANES>(a.x_f32 + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
+      else quantize_block<PLANES>(xsrc + (size_t)col * kDim, xplanes + (size_t)col * kPlaneDwords, xscale + col);
     }
   }
   return a.prologue != kPrologueNone || rotated;
@@ -1200,6 +1219,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   // the tile capacity of this instantiation (these shadow the namespace-level defaults)
   constexpr int kTileBlocks = TILE;
   constexpr int kP1Blocks = TILE / kWgThreads;
+  constexpr int kPlanes = std::is_same<OutT, __half>::value ? 2 : 3;  // byte planes of the activation (quantize_values)
   extern __shared__ __align__(16) uint8_t smem[];
 #ifdef LLVQ_PHASE_TIMING
   if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 3] = wall_clock64();
@@ -1232,7 +1252,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const ActivationSource src{a.x, a.x_f32, a.x2, a.norm_w, a.resid_out, a.eps, a.prologue, nb, a.tail_w,
                              a.rot_signbits, a.rot_small, a.rot_inv, a.rot_m, a.rot_k, blockIdx.x == 0};
-  if (stage_activation<kTileBlocks, ROT>(src, xplanes, xscale, xtail, raw, partial, request_first_tile))
+  if (stage_activation<kTileBlocks, ROT, kPlanes>(src, xplanes, xscale, xtail, raw, partial, request_first_tile))
     __syncthreads();  // the staging area becomes the tile's queues
 
 #ifdef LLVQ_PHASE_TIMING
@@ -1268,7 +1288,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
     prefetch_records(a, tile + gridDim.x, tid, pre);
 
     // P2: unrank and reduce
-    unrank_tile<kTileBlocks, false>(T, Q, UnrankOperands{xplanes, xscale, nb, a.inv_nblocks, M.g0, M.g1}, [](uint32_t, bool, uint32_t) { return 0u; });
+    unrank_tile<kTileBlocks, false, kPlanes>(T, Q, UnrankOperands{xplanes, xscale, nb, a.inv_nblocks, M.g0, M.g1}, [](uint32_t, bool, uint32_t) { return 0u; });
     LLVQ_STAMP(4);
     __syncthreads();
     LLVQ_STAMP(5);
@@ -1418,7 +1438,7 @@ struct llvq_seq {
   uint8_t* blob = nullptr;  // one device allocation: tiles | items | counters | status
   SeqArgs args{};
   uint32_t tile = 0, grid = 0, n_items = 0;
-  bool lean = false;
+  bool lean = false, f32 = false;
   size_t lds = 0;
   uint32_t* own_status = nullptr;  // the status word inside `blob` (args.status may point at a word several sequences share)
 };
@@ -2045,10 +2065,16 @@ struct SeqSpec {
   Prologue pro{};
 };
 
-static const void* seq_kernel(uint32_t tile, bool lean) {
-  if (lean) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, true>);
-  if (tile == (uint32_t)kTileBlocks) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, false>);
-  return reinterpret_cast<const void*>(gemv_seq_kernel<kSmallTileBlocks, false>);
+// three byte planes of the activation for f32 results, two for binary16 results, as gemv_tiles_kernel
+static const void* seq_kernel(uint32_t tile, bool lean, bool f32) {
+  if (f32) {
+    if (lean) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, true, 3>);
+    if (tile == (uint32_t)kTileBlocks) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, false, 3>);
+    return reinterpret_cast<const void*>(gemv_seq_kernel<kSmallTileBlocks, false, 3>);
+  }
+  if (lean) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, true, 2>);
+  if (tile == (uint32_t)kTileBlocks) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, false, 2>);
+  return reinterpret_cast<const void*>(gemv_seq_kernel<kSmallTileBlocks, false, 2>);
 }
 
 // The kernel variant for a sequence whose widest rows have max_nb blocks (as pick_gemv_shape).
@@ -2071,6 +2097,7 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
     if (!sp.mats || sp.n <= 0 || !sp.x || !sp.y) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: item " + std::to_string(i) + " has a null or empty field");
     if (sp.y_dtype != LLVQ_F32 && sp.y_dtype != LLVQ_F16) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: unknown output dtype");
     if (sp.after_previous && i == 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: the first item has no item before it");
+    if (sp.y_dtype != specs[0].y_dtype) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: the items of a sequence share one output dtype");
     for (int j = 0; j < sp.n; ++j) {
       const llvq_mat* m = sp.mats[j];
       if (!m || !sp.y[j]) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: null matrix or output in item " + std::to_string(i));
@@ -2168,6 +2195,9 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
   q->args.stamps = nullptr;
   q->tile = shape.tile;
   q->lean = shape.lean;
+  q->f32 = specs[0].y_dtype == LLVQ_F32;
+  // the activation planes of a wide row push dynamic LDS past the 64 KB default
+  (void)hipFuncSetAttribute(seq_kernel(shape.tile, shape.lean, q->f32), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
   q->lds = shape.lds;
   q->grid = grid;
   q->n_items = (uint32_t)n;
@@ -2179,7 +2209,7 @@ static int seq_run(llvq_rt* rt, llvq_seq* q) {
   q->args.run += 1;
   SeqArgs a = q->args;
   void* params[] = {&a};
-  const void* kernel = seq_kernel(q->tile, q->lean);
+  const void* kernel = seq_kernel(q->tile, q->lean, q->f32);
   // An ordinary launch, also with ordered items: at most one workgroup per CU (by its LDS) and no more workgroups than
   // CUs, so on a device this stream has to itself every workgroup is resident and the waits end.  (A cooperative launch
   // would guarantee it, but costs some 200 us per launch here: 4B decode fell from 237 to 85 tokens/s with it.)  Should
