@@ -74,6 +74,7 @@ struct SeqArgs {
   uint32_t spin_limit;
   uint32_t hold_item;  // kSeqNoWait, or an item this run must treat as never complete (tests of the give-up path)
   unsigned long long* stamps;  // tuning builds (-DLLVQ_SEQ_STAMPS): [grid][kSeqStampTiles][8] realtime-counter readings, or null
+  SeqItem item0;        // items[0] again, as a kernel argument: most workgroups start there, and need not wait for the table
 };
 
 // Phase timestamps of tuning builds: lane 0 of every workgroup stores the realtime counter (100 MHz) at the phase
@@ -257,6 +258,31 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     __syncthreads();
     if (tid == 0) __hip_atomic_fetch_add(s.counters + it, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
+  // A first item that waits for nothing is staged right away, as a launch of its own would: the loads of its
+  // operands go out behind the table image's, the first tile's code bytes behind those (the memory counter retires
+  // in order, and the code bytes are needed last).
+  uint32_t first_state = 0;  // 1: the first tile's code bytes are requested
+  {
+    SeqItem I = s.item0;
+    if (next.item != 0) I = s.items[next.item];
+    if (I.wait_item == kSeqNoWait) {
+      LaneRecords<kP1Blocks> rec;
+#pragma unroll
+      for (int r = 0; r < kP1Blocks * 3 / 2; ++r) rec.w[r] = 0;
+      const ActivationSource src{I.x, nullptr, I.x2, I.norm_w, I.resid_out, I.eps, I.prologue, I.nb, I.tail_w,
+                                 nullptr, nullptr, 1.f, 0u, 0u, nxt == I.first_tile, false};
+      (void)stage_activation<TILE, false, PLANES, true>(src, xplanes, xscale, xtail, reinterpret_cast<uint8_t*>(xplanes), Q.partial,
+                                                        [&] { seq_request_records(next, tid, rec); });
+      carry_records(rec, carried);
+      first_state = 1;
+      it = next.item;
+      nb = I.nb;
+      tail_w = I.tail_w;
+      inv_nb = I.inv_nb;
+      y_f16 = I.y_f16;
+      it_signals = I.signals;
+    }
+  }
   __syncthreads();
 #ifdef LLVQ_SEQ_STAMPS
   uint32_t round = 0;
@@ -342,7 +368,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     // ---- the current tile is unranked; each wavefront requests and classifies its share of the next tile on the way
     if (tid < (uint32_t)kCtrlWords) ctrl_sets[(parity ^ 1u) * kCtrlWords + tid] = 0;
     settle_origins<kP1Blocks>(origins, Q.partial, opaque_tid());
-    const uint32_t state = unrank_tile<TILE, true, PLANES>(T, Q, UnrankOperands{xplanes, xscale, nb, inv_nb, cur.g0, cur.g1}, for_next_tile);
+    const uint32_t state = unrank_tile<TILE, true, PLANES>(T, Q, UnrankOperands{xplanes, xscale, nb, inv_nb, cur.g0, cur.g1, first_state}, for_next_tile);
+    first_state = 0;
     if (state == 1u) classify_next();
     seq_request_row_operands(cur, tail_w, ops);
     LLVQ_SEQ_STAMP(6);

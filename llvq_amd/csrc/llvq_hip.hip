@@ -867,6 +867,7 @@ struct UnrankOperands {
   uint32_t nb;              // blocks per row
   float inv_nb;             // 1 / nb, for the block -> column split
   float g0, g1;             // the matrix's gain centroids
+  uint32_t hook_state = 0;  // the state the hook is first called with
 };
 
 template <int TILE, bool kHook, int PLANES, class Hook>
@@ -967,7 +968,7 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
   // The chunks of the small even queue come first (their queue ends in a partial chunk as well).
   const uint32_t c_pair = min(c_odd, c_even);
   const uint32_t c_all = c_gen + c_sec + c_odd + c_even;
-  uint32_t done = 0, hook_state = 0;
+  uint32_t done = 0, hook_state = op.hook_state;
   for (;; ++done, chunk = ticket()) {
     if constexpr (kHook) hook_state = hook(done, chunk >= c_all, hook_state);
     if (chunk >= c_all) break;
@@ -2193,6 +2194,7 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
   q->args.spin_limit = kSeqSpinLimit;
   q->args.hold_item = kSeqNoWait;
   q->args.stamps = nullptr;
+  q->args.item0 = items[0];
   q->tile = shape.tile;
   q->lean = shape.lean;
   q->f32 = specs[0].y_dtype == LLVQ_F32;
