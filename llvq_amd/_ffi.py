@@ -4,8 +4,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# LLVQ_HIP_LIB points at another build of the same library (tuning builds)
-_LIB = os.environ.get("LLVQ_HIP_LIB") or os.path.join(_HERE, "csrc", "libllvq_hip.so")
+_LIB = os.path.join(_HERE, "csrc", "libllvq_hip.so")
 
 STATUS = {
     0: "Ok", 1: "NotAnArtifact", 2: "Truncated", 3: "BadName", 5: "Inconsistent", 7: "IndexTooWide",

@@ -203,13 +203,19 @@ struct SliceWalk {
   uint32_t piece;               // which of the band's partial sums this workgroup's run of slices feeds
 };
 
+// Stage timestamps of tuning builds (-DLLVQ_PHASE_TIMING): lane 0 of EVERY wavefront stores the realtime counter at
+// the boundaries of the workgroup's stage kGemmStampStage.  Producers: 0 stage begins, 1 its share of the slice
+// unranked, 2 its share of the next slice classified, 3 through the barrier.  Consumers: 0 stage begins, 1 its K-steps
+// multiplied, 3 through the barrier.
 #ifdef LLVQ_PHASE_TIMING
-#define LLVQ_GSTAMP(base, k)                                                                                          \
-  do {                                                                                                                \
-    if (tid == ((base) ? (uint32_t)PW * 64u : 0u) && stage_no == 3) g_phase_stamps[((base) + blockIdx.x) * 8 + (k)] = wall_clock64(); \
+constexpr uint32_t kGemmStampStage = 3;
+__device__ unsigned long long g_gemm_stamps[1024 * 16 * 4];
+#define LLVQ_GSTAMP(k)                                                                                                 \
+  do {                                                                                                                 \
+    if (lane == 0 && stage_no == kGemmStampStage) g_gemm_stamps[((size_t)blockIdx.x * 16 + wave) * 4 + (k)] = wall_clock64(); \
   } while (0)
 #else
-#define LLVQ_GSTAMP(base, k) do {} while (0)
+#define LLVQ_GSTAMP(k) do {} while (0)
 #endif
 
 // A launch covers up to four matrices that share their activations (q/k/v, gate/up): their
@@ -400,15 +406,15 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 #ifdef LLVQ_PHASE_TIMING
       ++stage_no;
 #endif
-      LLVQ_GSTAMP(0, 0);
+      LLVQ_GSTAMP(0);
       if (live(w2)) stage_raw((g + 2u) % 3u, pre);
       prefetch(w3, pre);
       unrank(view(w0, g));
-      LLVQ_GSTAMP(0, 1);
+      LLVQ_GSTAMP(1);
       if (live(w1)) classify(view(w1, g + 1u));
-      LLVQ_GSTAMP(0, 2);
+      LLVQ_GSTAMP(2);
       wg_barrier();
-      LLVQ_GSTAMP(0, 3);
+      LLVQ_GSTAMP(3);
       ++g;
       w0 = w1;
       w1 = w2;
@@ -481,7 +487,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 #ifdef LLVQ_PHASE_TIMING
       ++stage_no;
 #endif
-      LLVQ_GSTAMP(256, 0);
+      LLVQ_GSTAMP(0);
       const bool last_of_unit = w.si + 1 == w.run_len;  // the band ends, or this workgroup's share of it
       // The loads run ahead into the unit's next slice.  At the unit's end they re-read this
       // slice (the ring starts afresh behind the epilogue, which needs the registers).
@@ -515,9 +521,9 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 #pragma unroll
           for (int f = 0; f < 2; ++f) ring[0][ct][f] = ring[1][ct][f];
       }
-      LLVQ_GSTAMP(256, 3);
+      LLVQ_GSTAMP(1);
       consumer_barrier();
-      LLVQ_GSTAMP(256, 4);
+      LLVQ_GSTAMP(3);
 
       const SliceWalk done = w;
       w = ahead;

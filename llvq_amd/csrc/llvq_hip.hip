@@ -1574,8 +1574,13 @@ void llvq_hip_runtime_destroy(llvq_rt* rt) {
 }
 
 #ifdef LLVQ_PHASE_TIMING
+// Tuning builds only: the phase timestamps of the last gemv_tiles_kernel launch ([workgroup][8]) and the stage
+// timestamps of the last gemm_tiles_kernel launch ([workgroup][wavefront][4]).
 int llvq_hip_debug_phase_stamps(unsigned long long* out, size_t n) {
   return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_phase_stamps), n * sizeof(unsigned long long));
+}
+int llvq_hip_debug_gemm_stamps(unsigned long long* out, size_t n) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_gemm_stamps), n * sizeof(unsigned long long));
 }
 #endif
 
