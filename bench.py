@@ -190,7 +190,7 @@ def bench_decode14b(args, torch, llvq_amd):
     log(f"[bench] decoder built in {time.time() - t0:.1f}s")
     n_new = max(8, args.steps)
     start = max(0, min(cfg.max_positions - n_new - args.warmup - 2, args.context - n_new))
-    results = {}
+    results, tokens_seen = {}, {}
     for name, pos in (("short", 0), ("long", start)):
         dec.seek(pos)
         tok = 1
@@ -203,6 +203,18 @@ def bench_decode14b(args, torch, llvq_amd):
         dt = (time.perf_counter() - t1) / n_new
         results[name] = dt
         log(f"[bench] {name} context ({pos}+): {dt * 1e3:.3f} ms/token")
+        # the same positions again from the same state must give the same tokens (the loop holds no hidden state
+        # besides the cache entries it rewrites here)
+        first = []
+        for rerun in range(2):
+            dec.seek(pos)
+            tok, got = 1, []
+            for _ in range(4):
+                _, tok = dec.forward_token(tok, want_logits=False)
+                got.append(int(tok))
+            first.append(got)
+        assert first[0] == first[1], f"decode14b: {name} context gave {first[0]} and then {first[1]} from the same state"
+        tokens_seen[name] = first[0]
     dec.close()
     step = results["long"]
     kv_bytes = 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * (1 + 4 / 64) * (start + n_new)
@@ -227,6 +239,7 @@ def bench_decode14b(args, torch, llvq_amd):
         "attention_ms_per_token": round((results["long"] - results["short"]) * 1e3, 4),
         "kv_cache_bytes_read_per_token": int(kv_bytes),
         "encoded_weight_GBps": round(enc_bytes / step / 1e9, 2),
+        "first_tokens": tokens_seen,
     }
     rt.close()
     print(json.dumps(out), flush=True)

@@ -240,7 +240,10 @@ int llvq_hip_gemm_static(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, 
 
 /* Parity probe (the role of decode_probe, llvq-cuda/kernels/preflight.cu:39):
  * unrank packed 6-byte records on the device.  points: 24 int8 per block;
- * gains: one byte per block; shells (may be NULL): one byte per block. */
+ * gains: one byte per block; shells (may be NULL): one byte per block.
+ * codes_dev holds exactly 6 * nblocks bytes and needs no slack behind them: no byte past
+ * the last record is read (that record is fetched byte by byte).  codes_dev starts on a
+ * 4-byte boundary (records are read as dwords); LLVQ_ERR_INVALID_ARGUMENT otherwise. */
 int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks,
                            int8_t* points_dev, uint8_t* gains_dev, uint8_t* shells_dev);
 

@@ -594,7 +594,9 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
 #pragma unroll
                 for (int ct = 0; ct < 2; ++ct) acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[rt], bv[ct], acc[rt][ct], 0, 0, 0);
             }
-            const bool vec = (mt.d_out & 3u) == 0;
+            // four results go out as one store where rows of y keep a vector's alignment: d_out a multiple of four and
+            // y itself on a 4-element boundary (a view into a caller's buffer need not be)
+            const bool vec = (mt.d_out & 3u) == 0 && (reinterpret_cast<uintptr_t>(mt.y) & (a.y_f32 ? 15u : 7u)) == 0;
 #pragma unroll
             for (int ct = 0; ct < 2; ++ct) {
               const uint32_t my_m = lane_m + 32u * ct;
@@ -718,7 +720,7 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmReduceArgs a) {
     v[i] = fmaf(sum[i], mt.rscale[r0 + r], ts);
   }
   const size_t at = (size_t)m * mt.d_out + r0 + row;
-  if ((mt.d_out & 3u) == 0 && row + 3 < rows) {
+  if ((mt.d_out & 3u) == 0 && (reinterpret_cast<uintptr_t>(mt.y) & (4 * sizeof(OutT) - 1)) == 0 && row + 3 < rows) {
     if constexpr (sizeof(OutT) == 4) {
       *reinterpret_cast<float4*>(reinterpret_cast<float*>(mt.y) + at) = make_float4(v[0], v[1], v[2], v[3]);
     } else {

@@ -319,12 +319,6 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
         carry_records(rec, carried);
         return 1u;
       }
-#ifdef LLVQ_EXP_CLASSIFY_MID
-      if (state == 1u && (last || done >= request_after + LLVQ_EXP_CLASSIFY_MID)) {
-        classify_next();
-        return 2u;
-      }
-#endif
       return state;
     };
     if (cur.item != it && cur.item != kSeqNoWait) {  // the same for every lane

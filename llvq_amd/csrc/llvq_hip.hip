@@ -2489,6 +2489,26 @@ static int gemm_same_basis(llvq_rt* rt, const llvq_mat* const* mats, int n, cons
       }
     return LLVQ_OK;
   }
+  if (wsp && wsp->fixed) {
+    // a caller-provided region is never outgrown part-way: every launch's carvings (released once it is enqueued)
+    // are sized before the first launch, since a short last chunk can need more than a full one, and a call
+    // that does not fit is refused whole
+    auto after = [](size_t used, size_t bytes) { return ((used + 255) & ~(size_t)255) + bytes; };
+    const size_t base = m0->has_rotation ? after(wsp->used, (size_t)M * m0->d_in * sizeof(__half)) : wsp->used;
+    size_t need = base;
+    for (int m_lo = 0; m_lo < M; m_lo += kGemmMaxM) {
+      const uint32_t mc = (uint32_t)(M - m_lo < kGemmMaxM ? M - m_lo : kGemmMaxM);
+      for (int i0 = 0; i0 < n; i0 += kGemmMaxGroup) {
+        size_t ws = 0, xt = 0;
+        gemm_workspace_bytes(rt, mats + i0, n - i0 < kGemmMaxGroup ? n - i0 : kGemmMaxGroup, mc, &ws, &xt);
+        const size_t top = after(ws ? after(base, ws) : base, xt);
+        if (top > need) need = top;
+      }
+    }
+    if (need > wsp->fixed_bytes)
+      return fail(LLVQ_ERR_UNSUPPORTED, "gemm_static: this shape needs " + std::to_string(need) +
+                                            " bytes of workspace, the static one holds " + std::to_string(wsp->fixed_bytes));
+  }
   if (m0->has_rotation) {
     // rows are rotated (f32 inside) and narrowed to the binary16 the matrix cores take
     void* rows = nullptr;
@@ -2572,6 +2592,7 @@ int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks
   if (!rt) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decode_blocks: runtime is null");
   if (nblocks == 0) return LLVQ_OK;  // an empty stream is valid and writes nothing
   if (!points_dev || !codes_dev) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decode_blocks: null argument");
+  if (reinterpret_cast<uintptr_t>(codes_dev) & 3) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decode_blocks: codes must start on a 4-byte boundary");
   HIP_TRY(hipSetDevice(rt->device));
   size_t grid = (nblocks + 255) / 256;
   const size_t cap = (size_t)(rt->cu_count > 0 ? rt->cu_count : 256) * 2;

@@ -71,20 +71,24 @@ def synthetic_weights(cfg: Qwen3Config, seed: int = 0) -> DecoderWeights:
 
 
 def quantize_rows_q8(name: str, table, group: int = 64) -> artifact.RawTensor:
-    """A [rows, d] table as the int8 tensor of the sealed sections (llvq-artifact/src/sealed.rs:64-78, written by
-    the reference's embedq tool, llvq-llm/src/embedquant.rs:22-92): per group of `group` along a row,
-    scale = f16((max - min) / 255), bias = f16(min), code = round((w - bias) / scale) against the rounded
-    scale and bias; a constant group codes as zeros."""
-    w = np.asarray(table, dtype=np.float32)
+    """A [rows, d] binary16 table as the int8 tensor of the sealed sections (llvq-artifact/src/sealed.rs:64-78), with the
+    bytes the reference's embedq tool writes (llvq-llm/src/embedquant.rs:22-92, f32 arithmetic throughout): per group
+    of `group` along a row, scale = f16((max - min) / 255), bias = f16(min), code = the quotient (w - bias) / scale
+    against the rounded scale and bias, rounded half away from zero and clamped to [0, 255]; a group whose scale
+    rounds to zero stores scale 1.0 and codes 0, the bias carrying the value."""
+    w = np.asarray(table, dtype=np.float16).astype(np.float32)
     rows, d = w.shape
     if d % group:
         raise ValueError(f"{name}: row length {d} is not a multiple of the group {group}")
     g = w.reshape(rows, d // group, group)
     mn, mx = g.min(-1, keepdims=True), g.max(-1, keepdims=True)
-    s = ((mx - mn) / 255.0).astype(np.float16)
+    s = ((mx - mn) / np.float32(255.0)).astype(np.float16)
     b = mn.astype(np.float16)
-    safe = np.where(s.astype(np.float32) > 0, s.astype(np.float32), 1.0)
-    q = np.clip(np.rint((g - b.astype(np.float32)) / safe), 0, 255).astype(np.uint8)
+    graded = s.astype(np.float32) > 0
+    s = np.where(graded, s, np.float16(1.0)).astype(np.float16)
+    t = ((g - b.astype(np.float32)) / s.astype(np.float32)).astype(np.float64)  # f32 quotient; the half is added exactly
+    t = np.sign(t) * np.floor(np.abs(t) + 0.5)
+    q = np.where(graded, np.clip(t, 0, 255), 0).astype(np.uint8)
     return artifact.RawTensor(name, [rows, d], bits=8, group=group, packed=q.reshape(-1), scales=s.reshape(-1).view(np.uint16),
                               biases=b.reshape(-1).view(np.uint16))
 

@@ -153,6 +153,30 @@ def test_gemm_matches_gemv_rows(gpu_rt):
     assert (Y - rows).abs().max().item() < 2e-3 * scale
 
 
+@pytest.mark.parametrize("M", [48, 512])
+def test_gemm_into_an_output_that_is_only_element_aligned(gpu_rt, M):
+    """y as a view one element into a larger buffer (2 bytes off for binary16, 4 for f32): the kernels
+    group four results into one store only where y keeps that alignment, and the bits are those of an
+    aligned output either way.  48 rows finish through the partial sums, 512 also inside the launch."""
+    import torch
+
+    raw = synth.make_matrix("model.layers.3.self_attn.v_proj.weight", 1024, 2560, seed=4)
+    proj = gpu_rt.upload(raw)
+    try:
+        X = _x16(synth.make_activation(2560, seed=6, rows=M))
+        for dt in (torch.float16, torch.float32):
+            want = gpu_rt.forward_batched(proj, X, out_dtype=dt)
+            buf = torch.full((M * 1024 + 8,), float("nan"), dtype=dt, device="cuda")
+            y = buf[1:1 + M * 1024].view(M, 1024)
+            assert y.data_ptr() % 8 != 0
+            gpu_rt.forward_batched_into(proj, X, y)
+            gpu_rt.synchronize()
+            assert torch.equal(y, want)
+            assert bool(torch.isnan(buf[0])) and bool(torch.isnan(buf[1 + M * 1024:]).all())
+    finally:
+        gpu_rt.free(proj)
+
+
 @pytest.mark.parametrize("site,d_out,d_in,M", [
     ("self_attn.k_proj", 1024, 4096, 64),     # few bands: the block range is split over units
     ("mlp.down_proj", 4096, 12288, 16),
@@ -306,6 +330,15 @@ def test_reserved_workspaces_change_nothing(gpu_rt):
         few = [gpu_rt.forward_batched(p, X[:40].contiguous(), out_dtype=torch.float32) for p in projs]
         for b, y in zip(before, few):
             assert torch.equal(b[:40], y) or float((b[:40] - y).abs().max()) < 1e-3 * float(b.abs().max())
+        # and what it promises: calls up to the reserved row count take no device memory
+        X6 = _x16(synth.make_activation(1000, seed=6, rows=600))
+        y6 = [torch.empty((600, p.d_out), dtype=torch.float32, device="cuda") for p in projs]
+        gpu_rt.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        for M in (600, 300, 100, 40):
+            gpu_rt.forward_batched_group_into(projs, X6[:M], [y[:M] for y in y6])
+        gpu_rt.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
         with pytest.raises(Exception):
             gpu_rt.reserve_batched(projs, -1)
     finally:

@@ -111,3 +111,20 @@ def test_sealed_file_round_trip():
     cut = buf[: len(artifact.write_header(4, 1)) + len(artifact.write_matrix_raw(m))]
     with pytest.raises(artifact.Truncated):
         artifact.read_sealed(cut)
+
+
+def test_int8_writer_follows_the_reference_writer_on_hand_computed_groups():  # embedquant.rs:22-92
+    """Four groups of four whose bytes can be worked out by hand.  (1) min -8, max 55.75: the scale is exactly
+    0.25, so -7.375 sits at quotient 2.5 and must code as 3 (half away from zero; half-to-even would say 2),
+    -7.125 at 3.5 codes as 4.  (2) a constant group: scale 1.0, codes 0, the bias carries the value.  (3) a
+    range that rounds to zero in binary16 (two neighbouring subnormals): ungraded like the constant one.
+    (4) min 0, max 255: scale 1, codes are the values."""
+    from llvq_amd import decoder
+
+    rows = np.array([[-8.0, -7.375, -7.125, 55.75, 3.0, 3.0, 3.0, 3.0, 0.0, 2.0 ** -24, 0.0, 2.0 ** -24, 0.0, 7.0, 255.0, 100.0]],
+                    dtype=np.float16)
+    t = decoder.quantize_rows_q8("model.embed_tokens.weight", rows, group=4)
+    assert (t.bits, t.group, list(t.dims)) == (8, 4, [1, 16])
+    assert np.asarray(t.packed).tolist() == [0, 3, 4, 255, 0, 0, 0, 0, 0, 0, 0, 0, 0, 7, 255, 100]
+    assert np.asarray(t.scales).tolist() == [0x3400, 0x3C00, 0x3C00, 0x3C00]  # 0.25, 1, 1, 1
+    assert np.asarray(t.biases).tolist() == [0xC800, 0x4200, 0x0000, 0x0000]  # -8, 3, 0, 0

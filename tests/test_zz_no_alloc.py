@@ -48,6 +48,15 @@ def test_static_workspace_matches_the_allocating_entry_point(gpu_rt, rotated):
                 want, got = _both(gpu_rt, proj, X, dtype)
                 assert np.isfinite(want.astype(np.float64)).all()
                 assert np.array_equal(want.view(np.uint8), got.view(np.uint8)), f"{proj.name} M={M} {dtype}"
+        # the defining property: with inputs and outputs in place, the calls take no device memory
+        x = _x16(synth.make_activation(p_big.d_in, seed=4, rows=130))
+        y = torch.empty((130, p_big.d_out), dtype=torch.float16, device="cuda")
+        gpu_rt.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        for M in (130, 64, 2):
+            gpu_rt.forward_batched_static_into(p_big, x[:M], y[:M])
+        gpu_rt.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
     finally:
         gpu_rt.free(p_big)
         gpu_rt.free(p_small)
@@ -70,5 +79,28 @@ def test_static_workspace_refuses_what_does_not_fit(gpu_rt):
         gpu_rt.forward_batched_static_into(proj, x[:16].contiguous(), y2)
         gpu_rt.synchronize()
         assert torch.isfinite(y2).all()
+    finally:
+        gpu_rt.free(proj)
+
+
+def test_static_workspace_refuses_the_whole_call(gpu_rt):
+    """Rows beyond 512 go out as further launches, and a short last one can need more partial sums than a
+    full one (its consumers split the K-steps): 17000 x 4096 at 576 rows fits its first 512 and not its last
+    64.  The call is refused before anything is enqueued, so no row of y is written."""
+    import torch
+
+    raw = synth.make_matrix("model.layers.0.static.uneven.weight", 17000, 4096, seed=14)
+    proj = gpu_rt.upload(raw)
+    try:
+        x = _x16(synth.make_activation(4096, seed=5, rows=576))
+        y = torch.full((576, 17000), float("nan"), dtype=torch.float16, device="cuda")
+        with pytest.raises(_ffi.LlvqError) as err:
+            gpu_rt.forward_batched_static_into(proj, x, y)
+        assert err.value.kind == "Unsupported" and "static" in str(err.value)
+        gpu_rt.synchronize()
+        assert bool(torch.isnan(y).all())
+        gpu_rt.forward_batched_static_into(proj, x[:512], y[:512])  # the part that does fit, by itself
+        gpu_rt.synchronize()
+        assert bool(torch.isfinite(y[:512]).all()) and bool(torch.isnan(y[512:]).all())
     finally:
         gpu_rt.free(proj)
