@@ -23,7 +23,8 @@
 //                                rows x 64 activation rows (64 accumulator
 //                                registers, live across a band's slices), A
 //                                fragments from LDS, B fragments from global
-//                                memory / L2, two K-steps in flight.
+//                                memory / L2 through a buffer descriptor, each
+//                                16-byte piece in flight for most of two K-steps.
 // The unranking is integer and f64 VALU work and the contraction runs on the
 // matrix cores, so the two overlap on every SIMD.  Because the roles are separate
 // branches of one kernel, the accumulators and the decode state are never live
@@ -427,42 +428,56 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
     // Consumer c owns activation rows [64 ctile, +64) on the K-steps p = kpart (mod kparts) of
     // every slice: 12 / kparts steps, whatever the slice's length (past a short last slice's end
     // the activations are zero and the W buffer holds finite leftovers).  The loop is
-    // branch-free, and the B fragments of three K-steps are in flight at any time, across
-    // barriers and from one slice into the next: step i of the sequence lives in ring slot i mod 3.
+    // branch-free, and the B fragments of two K-steps are in flight at any time, across
+    // barriers and from one slice into the next: step i of the sequence lives in ring slot i mod 2.
     const uint32_t c = wave - (uint32_t)PW;
     const uint32_t ctn = 1u << a.ct_shift, kparts = (uint32_t)kConsumers >> a.ct_shift;
     const uint32_t ctile = c & (ctn - 1u), kpart = c >> a.ct_shift;
-    const uint32_t l32 = lane & 31u, lh = lane >> 5;
     const uint32_t m0 = ctile * kGemmColTile;
     const bool tile_live = m0 < a.M;  // a consumer past the batch's last tile multiplies that tile again and stores nothing
-    // K-step p of the matrix: 32 binary16 values per activation row, rows 64 bytes apart.  A load
-    // address is a wavefront-uniform base (slice, K-step) plus this lane's byte offset in the step.
-    const uint32_t lane_off = (min(m0, a.m_pad - kGemmColTile) + l32) * 64u + lh * 32u;
-    const size_t step_bytes = (size_t)a.m_pad * 64u;
-    const size_t own_bytes = (size_t)kparts * step_bytes;  // between two of this consumer's K-steps
-    const uint32_t n_own = (uint32_t)(kGemmKb * 24 / 32) / kparts;  // 12, 6 or 3 K-steps
-    auto slice_base = [&](const SliceWalk& w) {  // twelve K-steps per slice
-      return reinterpret_cast<const uint8_t*>(a.xt) + (size_t)(w.j * (uint32_t)(kGemmKb * 24 / 32) + kpart) * step_bytes;
+    // K-step p of the matrix: 32 binary16 values per activation row, rows 64 bytes apart.  The loads go through a
+    // buffer descriptor over the tiled copy: a 32-bit lane offset in a vector register, the K-step's offset (the same
+    // in every lane) in a scalar one, the place inside the step in the instruction.  No 64-bit address arithmetic, and
+    // the loads are counted in order (vmcnt), which generic-pointer loads are not: with those every wait drains them all.
+    // This lane's byte offset in a K-step of the tiled copy, from a lane number asked for on the spot: it is worked
+    // out again at every stage's start and behind every epilogue, because kept alive through an epilogue it would be
+    // a register the epilogue does not have.
+    auto lane_offset = [&]() {
+      uint32_t ln;
+      asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+      return (min(m0, a.m_pad - kGemmColTile) + (ln & 31u)) * 64u + (ln >> 5) * 32u;
     };
+    const uint32_t step_bytes = a.m_pad * 64u;
+    const uint32_t own_bytes = kparts * step_bytes;  // between two of this consumer's K-steps
+    const uint32_t n_own = (uint32_t)(kGemmKb * 24 / 32) / kparts;  // 12, 6 or 3 K-steps
+    const __amdgpu_buffer_rsrc_t xt_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<__half*>(a.xt), 0, a.spb * (uint32_t)(kGemmKb * 24 / 32) * step_bytes, 0x00020000);
+    auto slice_base = [&](const SliceWalk& w) {  // twelve K-steps per slice; byte offset of this consumer's first
+      return (w.j * (uint32_t)(kGemmKb * 24 / 32) + kpart) * step_bytes;
+    };
+    auto piece = [&](uint32_t lane_off, uint32_t step_off, int ct, int f) {
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(xt_rsrc, (int)lane_off,
+                                                            __builtin_amdgcn_readfirstlane((int)step_off) + (ct * 32 * 64 + f * 16), 0);
+      return __builtin_bit_cast(half8_t, v);
+    };
+    // B fragments of two K-steps: slot s holds the steps of parity s, as four 16-byte pieces [column half][K half]
     half8_t ring[2][2][2];
-    auto fetch = [&](const uint8_t* step_any, half8_t (&dst)[2][2]) {
-      // the step's address is the same in every lane: said so, it stays in scalar registers and the
-      // loads take it with a 32-bit lane offset
-      const uint64_t bits = reinterpret_cast<uint64_t>(step_any);
-      const uint8_t* step = reinterpret_cast<const uint8_t*>(
-          ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(bits >> 32)) << 32) | (uint32_t)__builtin_amdgcn_readfirstlane((int)bits));
+    auto fetch = [&](uint32_t lane_off, uint32_t step_off, half8_t (&dst)[2][2]) {
 #pragma unroll
-      for (int ct = 0; ct < 2; ++ct)
+      for (int f = 0; f < 2; ++f)
 #pragma unroll
-        for (int f = 0; f < 2; ++f) dst[ct][f] = *reinterpret_cast<const half8_t*>(step + lane_off + ct * 32 * 64 + f * 16);
+        for (int ct = 0; ct < 2; ++ct) dst[ct][f] = piece(lane_off, step_off, ct, f);
     };
 
-    SliceWalk w, ahead;
+    SliceWalk w;
     start_walk(w);
-    ahead = w;
-    advance(ahead);
-    const uint8_t* xs = slice_base(w);
-    fetch(xs, ring[0]);
+    uint32_t xs = slice_base(w);
+    {
+      const uint32_t lane_off = lane_offset();
+      fetch(lane_off, xs, ring[0]);
+      fetch(lane_off, xs + own_bytes, ring[1]);
+    }
 
     consumer_barrier();  // the table image (unused here) and slice 0's code bytes
     consumer_barrier();  // slice 0 classified
@@ -479,7 +494,6 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
           for (int j = 0; j < 16; ++j) acc[rt][ct][j] = 0.f;
     };
     clear_acc();
-    const uint32_t a_lane = (l32 * kGemmWStride + lh * 16u + kpart * 32u) * 2u;  // this lane's byte offset in a W buffer
 #ifdef LLVQ_PHASE_TIMING
     uint32_t stage_no = 1;
 #endif
@@ -491,10 +505,28 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
       const bool last_of_unit = w.si + 1 == w.run_len;  // the band ends, or this workgroup's share of it
       // The loads run ahead into the unit's next slice.  At the unit's end they re-read this
       // slice (the ring starts afresh behind the epilogue, which needs the registers).
-      const uint8_t* xs_next = last_of_unit ? xs : slice_base(ahead);
+      // (the slice after this one is worked out here and again at the stage's end: kept, its ten fields would be
+      // live through the products, and this kernel has no register to spare)
+      uint32_t xs_next = xs;
+      if (!last_of_unit) {
+        SliceWalk nx = w;
+        advance(nx);
+        xs_next = slice_base(nx);
+      }
       const uint8_t* wbuf = reinterpret_cast<const uint8_t*>(W0 + buf * kWBuf);
-      auto multiply = [&](uint32_t i, const half8_t (&b)[2][2]) {
-        const uint8_t* ap = wbuf + a_lane + i * kparts * 64u;
+      const uint32_t lane_off = lane_offset();
+      uint32_t a_lane;  // this lane's byte offset in a W buffer, per stage for the same reason
+      {
+        uint32_t ln;
+        asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+        a_lane = ((ln & 31u) * kGemmWStride + (ln >> 5) * 16u + kpart * 32u) * 2u;
+      }
+      auto step_src = [&](uint32_t i) { return i < n_own ? xs + i * own_bytes : xs_next + (i - n_own) * own_bytes; };
+      // K-step k from its slot; every 16-byte piece of the slot is asked for again, for the step two on, as soon as
+      // the products that read it are issued: a piece is in flight for most of two K-steps
+      auto multiply = [&](uint32_t k, half8_t (&b)[2][2]) {
+        const uint8_t* ap = wbuf + a_lane + k * kparts * 64u;
+        const uint32_t nx = step_src(k + 2);
 #pragma unroll
         for (int f = 0; f < 2; ++f) {
 #pragma unroll
@@ -503,31 +535,32 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
             acc[rt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, b[0][f], acc[rt][0], 0, 0, 0);
             acc[rt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, b[1][f], acc[rt][1], 0, 0, 0);
           }
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct) b[ct][f] = piece(lane_off, nx, ct, f);
         }
       };
-      auto step_src = [&](uint32_t i) { return i < n_own ? xs + i * own_bytes : xs_next + (i - n_own) * own_bytes; };
       uint32_t i = 0;
       for (; i + 1 < n_own; i += 2) {
-        fetch(step_src(i + 1), ring[1]);
         multiply(i, ring[0]);
-        fetch(step_src(i + 2), ring[0]);
         multiply(i + 1, ring[1]);
       }
-      if (i < n_own) {  // an odd count (three K-steps): the last one
-        fetch(step_src(i + 1), ring[1]);
+      if (i < n_own) {  // an odd count (three K-steps): the slots change places
         multiply(i, ring[0]);
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-          for (int f = 0; f < 2; ++f) ring[0][ct][f] = ring[1][ct][f];
+          for (int f = 0; f < 2; ++f) {
+            const half8_t t = ring[0][ct][f];
+            ring[0][ct][f] = ring[1][ct][f];
+            ring[1][ct][f] = t;
+          }
       }
       LLVQ_GSTAMP(1);
       consumer_barrier();
       LLVQ_GSTAMP(3);
 
       const SliceWalk done = w;
-      w = ahead;
-      advance(ahead);
+      advance(w);
       xs = slice_base(w);  // past the last slice: an address that is not read
       buf ^= 1u;
       if (last_of_unit) {
@@ -597,6 +630,9 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
             // four results go out as one store where rows of y keep a vector's alignment: d_out a multiple of four and
             // y itself on a 4-element boundary (a view into a caller's buffer need not be)
             const bool vec = (mt.d_out & 3u) == 0 && (reinterpret_cast<uintptr_t>(mt.y) & (a.y_f32 ? 15u : 7u)) == 0;
+            uint32_t ln_again;  // asked for once more: the row offset does not stay alive through the tail products
+            asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln_again));
+            const uint32_t store_r = 4u * (ln_again >> 5);
 #pragma unroll
             for (int ct = 0; ct < 2; ++ct) {
               const uint32_t my_m = lane_m + 32u * ct;
@@ -605,7 +641,7 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
                 for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
                   for (int j4 = 0; j4 < 4; ++j4) {
-                    const uint32_t row = 32u * rt + 8u * j4 + lane_r;
+                    const uint32_t row = 32u * rt + 8u * j4 + store_r;
                     const size_t at = (size_t)my_m * mt.d_out + done.r0 + row;
                     const float v0 = acc[rt][ct][4 * j4], v1 = acc[rt][ct][4 * j4 + 1], v2 = acc[rt][ct][4 * j4 + 2], v3 = acc[rt][ct][4 * j4 + 3];
                     if (vec && row + 3u < done.rows) {
@@ -633,7 +669,11 @@ __global__ __launch_bounds__(kWgThreads) void gemm_tiles_kernel(GemmArgs a) {
           }
         }
         clear_acc();
-        if (live(w)) fetch(xs, ring[0]);
+        if (live(w)) {
+          const uint32_t lane_off = lane_offset();
+          fetch(lane_off, xs, ring[0]);
+          fetch(lane_off, xs + own_bytes, ring[1]);
+        }
       }
     }
   }

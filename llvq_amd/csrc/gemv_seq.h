@@ -95,6 +95,34 @@ __host__ __device__ constexpr size_t gemv_seq_lds_bytes(uint32_t max_nb, uint32_
   return gemv_lds_bytes(max_nb, tile, image_bytes) + 2 * kCtrlWords * 4;  // a second set of counters and the wait's verdict
 }
 
+// Pointers that a kernel reads out of a table in memory carry no address space, and loads through them would be
+// generic ("flat") ones: those count on two wait counters out of order, so every wait after one — an LDS read's
+// included — has to drain all loads in flight, among them the code bytes requested for the next tile.  The tables'
+// pointers are the same in every lane and point into device memory: said so (made scalar, typed global), loads
+// through them are global ones with a scalar base, counted in order.
+template <typename T>
+__device__ __forceinline__ T* uniform_global(T* p) {
+  typedef T __attribute__((address_space(1))) global_t;
+  const uint64_t bits = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)bits), hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(bits >> 32));
+  return (T*)reinterpret_cast<global_t*>(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ SeqTile seq_tile_at(const SeqTile* tiles, uint32_t i) {
+  SeqTile t = tiles[i];
+  t.codes = uniform_global(t.codes);
+  t.rscale = uniform_global(t.rscale);
+  t.tail = uniform_global(t.tail);
+  t.y = uniform_global(t.y);
+  return t;
+}
+__device__ __forceinline__ SeqItem seq_item_of(SeqItem I) {
+  I.x = uniform_global(I.x);
+  I.x2 = uniform_global(I.x2);
+  I.norm_w = uniform_global(I.norm_w);
+  I.resid_out = uniform_global(I.resid_out);
+  return I;
+}
+
 template <int NB>
 __device__ __forceinline__ void seq_request_records(const SeqTile& t, uint32_t tid, LaneRecords<NB>& r) {
   if (t.nblk == 0) return;  // rows of tail columns only have no code bytes
@@ -237,7 +265,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
   SeqTile cur{};
   cur.item = kSeqNoWait;
   uint32_t nxt = blockIdx.x;  // the tile after `cur`
-  SeqTile next = s.tiles[nxt];
+  SeqTile next = seq_tile_at(s.tiles, nxt);
   Carried<kP1Blocks> carried;
 #pragma unroll
   for (int k = 0; k < 2 * kP1Blocks + 1; ++k) carried.r[k] = 0;
@@ -265,6 +293,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
   {
     SeqItem I = s.item0;
     if (next.item != 0) I = s.items[next.item];
+    I = seq_item_of(I);
     if (I.wait_item == kSeqNoWait) {
       LaneRecords<kP1Blocks> rec;
 #pragma unroll
@@ -326,7 +355,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
       if (it != kSeqNoWait && it_signals) signal_item();
       else __syncthreads();
       LLVQ_SEQ_STAMP(2);
-      const SeqItem I = s.items[cur.item];
+      const SeqItem I = seq_item_of(s.items[cur.item]);
       if (I.wait_item != kSeqNoWait) {
         if (tid == 0) {
           const uint32_t target = s.run * I.wait_expected + (I.wait_item == s.hold_item ? 1u : 0u);
@@ -376,7 +405,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     if (!more) break;
     cur = next;
     nxt += G;
-    next = s.tiles[min(nxt, n_tiles - 1u)];
+    next = seq_tile_at(s.tiles, min(nxt, n_tiles - 1u));
     parity ^= 1u;
   }
   seq_finish_rows(prev, Q.partial, xtail, nb, tail_w, y_f16, ops);

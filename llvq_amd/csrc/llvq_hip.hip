@@ -696,7 +696,7 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
 // three are different straight-line programs.  Blocks of the rare generic classes go to two small
 // queues, by coset; what does not fit rides in the odd queue, flagged.
 constexpr uint32_t kQaClassShift = 13, kQaGainShift = 22;
-constexpr uint32_t kQaSecond = 0x40000000u, kQaGeneric = 0x80000000u;
+constexpr uint32_t kQaSecond = 0x40000000u;
 enum : uint32_t { kCtrlOdd = 0, kCtrlEven = 1, kCtrlGenOdd = 2, kCtrlTicket = 3, kCtrlSec = 4, kCtrlGenEven = 5, kCtrlWords = 8 };
 
 struct GemvQueues {
@@ -2442,6 +2442,8 @@ static int launch_gemm(llvq_rt* rt, const llvq_mat* const* mats, int n, const vo
   // every slice has all its twelve K-steps in the tiled copy, zeros past the matrix's last block
   const uint32_t n_steps = (m0->nblocks + kGemmKb - 1) / kGemmKb * (kGemmKb * 24 / 32);
   if (xt_bytes != (size_t)n_steps * a.m_pad * 64) return fail(LLVQ_ERR_DEVICE, "gemm: activation-copy sizing disagrees with the launch");
+  // the kernel reads the copy through a buffer descriptor: 32-bit offsets
+  if (xt_bytes >= (1ull << 32)) return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": rows too wide for the batched launch's 32-bit activation offsets");
   rc = workspace_take(rt, wsp, reinterpret_cast<void**>(&rt->gemm_xt), &rt->gemm_xt_bytes, xt_bytes, &xt_buf);
   if (rc) return rc;
   if (wsp) wsp->used = mark;
