@@ -53,16 +53,22 @@ typedef struct llvq_mat llvq_mat; /* replaces FusedProj     (fused_cuda.rs:119-1
 /* One projection as the file stores it: the fields of RawMatrix
  * (llvq-artifact/src/format.rs:215-229) with the code stream left packed
  * (format.rs:185-203: per block index_bits(cap) bits of index then the gain
- * bit, MSB first — 6 bytes per block at cap 12). All pointers are host memory. */
+ * bit, MSB first — 6 bytes per block at cap 12, 49 bits per block in a dense
+ * stream at cap 13, format.rs:87-89). All pointers are host memory.
+ * Cap 12 and cap 13 are accepted; other caps are refused by name
+ * (LLVQ_ERR_UNSUPPORTED).  A cap-13 matrix is served by llvq_hip_gemv,
+ * llvq_hip_gemv_group (matrices of one call share their cap), llvq_hip_rotate /
+ * llvq_hip_gemv_rotated and, as a loop over its rows, by llvq_hip_gemm /
+ * llvq_hip_gemm_group; sequences and the decode loop refuse it by name. */
 typedef struct llvq_matrix_desc {
   const char* name;          /* may be NULL */
   uint32_t d_out, d_in;
-  uint32_t shell_cap;        /* 12 is the only cap with a 6-byte record */
+  uint32_t shell_cap;        /* 12 (6-byte records) or 13 (49-bit blocks, dense) */
   uint32_t n_centroids;      /* must be 2 */
   const double* centroids;   /* [n_centroids] */
   const double* row_scales;  /* [d_out] */
   const float* tail;         /* [d_out * (d_in % 24)], row-major; may be NULL when d_in % 24 == 0 */
-  const uint8_t* codes;      /* packed stream, >= 6 * d_out * (d_in / 24) bytes */
+  const uint8_t* codes;      /* packed stream, >= ceil(bits per block * d_out * (d_in / 24) / 8) bytes */
   size_t code_bytes;
   uint64_t rotation_seed;
   uint32_t has_rotation;     /* stored as W Q^T: the activation is rotated by Q(d_in, rotation_seed) first */
@@ -245,6 +251,12 @@ int llvq_hip_gemm_static(llvq_rt* rt, const llvq_mat* m, const void* x_f16_dev, 
  * the last record is read (that record is fetched byte by byte).  codes_dev starts on a
  * 4-byte boundary (records are read as dwords); LLVQ_ERR_INVALID_ARGUMENT otherwise. */
 int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks,
+                           int8_t* points_dev, uint8_t* gains_dev, uint8_t* shells_dev);
+/* The same for the code stream of a matrix of any accepted shell cap (pack.rs:48-82): cap 12 is
+ * llvq_hip_decode_blocks; at cap 13 block b is the 49 bits from bit 49 b on, codes_dev holds
+ * ceil(49 * nblocks / 8) bytes, no byte past them is read and no alignment is asked.  An index
+ * past N(13) decodes to zeros with shell 0xFF. */
+int llvq_hip_decode_stream(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks, uint32_t shell_cap,
                            int8_t* points_dev, uint8_t* gains_dev, uint8_t* shells_dev);
 
 /* ---- batch-1 decode loop ---------------------------------------------------

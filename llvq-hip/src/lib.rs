@@ -176,6 +176,7 @@ extern "C" {
     pub fn llvq_hip_reserve_batched(rt: *mut LlvqRt, mats: *const *const LlvqMat, n: c_int, max_rows: c_int) -> c_int;
     pub fn llvq_hip_gemm_static(rt: *mut LlvqRt, m: *const LlvqMat, x_f16_dev: *const c_void, rows: c_int, y_dev: *mut c_void, y_dtype: c_int) -> c_int;
     pub fn llvq_hip_decode_blocks(rt: *mut LlvqRt, codes_dev: *const u8, nblocks: usize, points_dev: *mut i8, gains_dev: *mut u8, shells_dev: *mut u8) -> c_int;
+    pub fn llvq_hip_decode_stream(rt: *mut LlvqRt, codes_dev: *const u8, nblocks: usize, shell_cap: u32, points_dev: *mut i8, gains_dev: *mut u8, shells_dev: *mut u8) -> c_int;
     pub fn llvq_hip_decoder_create(rt: *mut LlvqRt, desc: *const LlvqDecoderDesc, out: *mut *mut LlvqDecoder) -> c_int;
     pub fn llvq_hip_decoder_destroy(dec: *mut LlvqDecoder);
     pub fn llvq_hip_decoder_reset(dec: *mut LlvqDecoder) -> c_int;

@@ -137,6 +137,7 @@ def lib():
     L.llvq_hip_gemm_static.argtypes = [vp, vp, vp, C.c_int, vp, C.c_int]
     L.llvq_hip_gemm_group.argtypes = [vp, C.POINTER(vp), C.c_int, vp, C.c_int, C.POINTER(vp), C.c_int]
     L.llvq_hip_decode_blocks.argtypes = [vp, vp, sz, vp, vp, vp]
+    L.llvq_hip_decode_stream.argtypes = [vp, vp, sz, C.c_uint32, vp, vp, vp]
     L.llvq_hip_synchronize.argtypes = [vp]
     L.llvq_hip_decoder_create.argtypes = [vp, C.POINTER(DecoderDesc), C.POINTER(vp)]
     L.llvq_hip_decoder_destroy.argtypes = [vp]
@@ -165,7 +166,7 @@ EXPORTS = [
     "llvq_hip_matrix_from_record", "llvq_hip_parse_raw_tensor", "llvq_hip_parse_blob",
     "llvq_hip_matrix_free", "llvq_hip_matrix_info", "llvq_hip_matrix_name", "llvq_hip_gemv",
     "llvq_hip_gemv_group", "llvq_hip_sequence_create", "llvq_hip_sequence_run", "llvq_hip_sequence_status", "llvq_hip_sequence_tune",
-    "llvq_hip_sequence_destroy", "llvq_hip_gemm", "llvq_hip_gemm_static", "llvq_hip_reserve_batched", "llvq_hip_decoder_generate_phased", "llvq_hip_gemm_group", "llvq_hip_decode_blocks", "llvq_hip_synchronize",
+    "llvq_hip_sequence_destroy", "llvq_hip_gemm", "llvq_hip_gemm_static", "llvq_hip_reserve_batched", "llvq_hip_decoder_generate_phased", "llvq_hip_gemm_group", "llvq_hip_decode_blocks", "llvq_hip_decode_stream", "llvq_hip_synchronize",
     "llvq_hip_last_error", "llvq_hip_version",
     "llvq_hip_host_rotate", "llvq_hip_rotate", "llvq_hip_gemv_rotated", "llvq_hip_matrix_rotation",
     "llvq_hip_decoder_create", "llvq_hip_decoder_destroy", "llvq_hip_decoder_reset", "llvq_hip_decoder_position", "llvq_hip_decoder_seek",

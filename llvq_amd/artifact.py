@@ -105,30 +105,43 @@ class RawMatrix:
         return int(self.codes.size + 4 * self.tail.size + 8 * self.row_scales.size + 8 * self.centroids.size)
 
     def unpack(self):
-        """(indices u64, gains u8) of a 48-bit-per-block stream (cap 12, two centroids)."""
+        """(indices u64, gains u8) of the code stream: per block index_bits(cap) bits of index, then the gain bits,
+        most significant first, blocks back to back (6 bytes per block at cap 12, 49 bits at cap 13)."""
         ib, gb = index_bits(self.shell_cap), gain_bits(self.centroids.size)
-        if ib + gb != 48:
-            raise Inconsistent(f"{self.name}: {ib}+{gb} bits per block is not a 6-byte record")
         n = self.d_out * self.nblocks
-        b = self.codes[: 6 * n].reshape(n, 6).astype(np.uint64)
-        v = np.zeros(n, np.uint64)
-        for k in range(6):
-            v = (v << np.uint64(8)) | b[:, k]
+        if ib + gb == 48:
+            b = self.codes[: 6 * n].reshape(n, 6).astype(np.uint64)
+            v = np.zeros(n, np.uint64)
+            for k in range(6):
+                v = (v << np.uint64(8)) | b[:, k]
+        else:
+            w = ib + gb
+            if w > 64:
+                raise Inconsistent(f"{self.name}: {w} bits per block")
+            bits = np.unpackbits(self.codes[: (n * w + 7) // 8])[: n * w].reshape(n, w)
+            v = np.zeros(n, np.uint64)
+            for k in range(w):
+                v = (v << np.uint64(1)) | bits[:, k].astype(np.uint64)
         return v >> np.uint64(gb), (v & np.uint64((1 << gb) - 1)).astype(np.uint8)
 
 
 def pack_codes(indices, gains, index_width=47):
-    """Per block `index_width` bits of index then one gain bit, MSB first
-    (llvq-search/src/pack.rs:10-18, format.rs:185-203) — 6 bytes at cap 12."""
+    """Per block `index_width` bits of index then one gain bit, MSB first, blocks back to back
+    (llvq-search/src/pack.rs:10-18, :48-82, format.rs:185-203) — 6 bytes per block at cap 12 (47 bits of
+    index), 49 bits per block at cap 13 (48), the stream's last byte zero-padded."""
     idx = np.ascontiguousarray(indices, dtype=np.uint64)
     g = np.ascontiguousarray(gains, dtype=np.uint64)
-    if index_width != 47:
-        raise Inconsistent("only 47-bit indices pack into 6-byte records")
+    if not 1 <= index_width <= 62:
+        raise Inconsistent(f"{index_width}-bit indices")
     if idx.size and int(idx.max()) >= (1 << index_width):
         raise IndexTooWide(f"index {int(idx.max())} does not fit in {index_width} bits")
     v = (idx << np.uint64(1)) | (g & np.uint64(1))
     be = v.astype(">u8").view(np.uint8).reshape(-1, 8)
-    return np.ascontiguousarray(be[:, 2:]).reshape(-1)
+    if index_width == 47:
+        return np.ascontiguousarray(be[:, 2:]).reshape(-1)
+    w = index_width + 1
+    bits = np.unpackbits(be, axis=1)[:, 64 - w:]
+    return np.packbits(np.ascontiguousarray(bits).reshape(-1))
 
 
 def write_header(version, n_matrices):

@@ -51,6 +51,11 @@ struct GlobalTables {
   const uint32_t* off_lut;
   const uint32_t* expand;
   const uint64_t* tail_codes;
+  // what a 48-bit index (shell cap 13) can reach and the LDS image leaves out: every fast-path class record,
+  // the whole first level of the class-find table and all its second-level tables
+  const FastClass* wide_fast;
+  const uint16_t* wide_lut;
+  const uint16_t* wide_lut2;
 };
 
 constexpr size_t kLdsImageBytesLean = offsetof(TableImage, golay);  // without the Golay words and the support-arrangement table
@@ -61,7 +66,9 @@ static_assert(kLdsImageBytesLeanest % 16 == 0, "LDS part of the table image is c
 // kFull: the whole image goes to LDS; otherwise its last two tables (33 KB) are
 // read through L2, for a kernel that needs the LDS for something else.  kLut = false
 // leaves the 4 KB class lookup table (one read per block) in L2 as well.
-template <bool kFull = true, bool kLut = true>
+// kWide: for 48-bit indices the class records, class starts and class-find tables are the full ones in device
+// memory (read through L2); the LDS copies cover what a 47-bit index reaches.
+template <bool kFull = true, bool kLut = true, bool kWide = false>
 __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const GlobalTables& g) {
   static_assert(kLut || !kFull, "the tables that stay in L2 are the image's last ones");
   const uint4* src = reinterpret_cast<const uint4*>(g.image);
@@ -83,6 +90,9 @@ __device__ __forceinline__ DecodeTables stage_tables(uint8_t* smem, const Global
   }
   const TableImage* s = reinterpret_cast<const TableImage*>(smem);
   const TableImage* far = kFull ? s : g.image;
+  if constexpr (kWide)
+    return DecodeTables{far->golay, g.cls, g.wide_fast, g.starts, g.starts, g.wide_lut, g.wide_lut2, s->rcp, far->on_lut, g.off_lut,
+                        g.expand, s->pdep4, s->step - kTailSlots * 25 * 2, s->tail_meta, g.tail_codes};
   return DecodeTables{far->golay, g.cls, s->fast, s->starts, g.starts, kLut ? s->lut : g.image->lut, kLut ? s->lut2 : g.image->lut2, s->rcp, far->on_lut, g.off_lut,
                       g.expand, s->pdep4, s->step - kTailSlots * 25 * 2, s->tail_meta, g.tail_codes};
 }
@@ -130,14 +140,33 @@ __device__ __forceinline__ uint32_t wave_prefix_sum(uint32_t v) {
   return v;
 }
 
+constexpr uint32_t kDenseBits = 49;  // bits per block at shell cap 13: a 48-bit index and the gain bit
+
 // ---- parity probe: unrank records to points -----------------------------------
+template <bool WIDE>
 __global__ __launch_bounds__(256) void decode_blocks_kernel(GlobalTables g, const uint8_t* __restrict__ codes,
                                                             size_t nblocks, int8_t* __restrict__ points,
                                                             uint8_t* __restrict__ gains,
                                                             uint8_t* __restrict__ shells) {
   extern __shared__ __align__(16) uint8_t smem[];
-  const DecodeTables T = stage_tables(smem, g);
+  const DecodeTables T = stage_tables<true, true, WIDE>(smem, g);
   __syncthreads();
+  if constexpr (WIDE) {
+    // 49-bit blocks of a dense stream (shell cap 13): block b is the 49 bits from bit 49 b on, read byte by byte
+    // (at most seven bytes hold it), so that no byte past the stream's ceil(49 nblocks / 8) is touched
+    for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < nblocks; b += (size_t)gridDim.x * blockDim.x) {
+      const uint64_t bit = (uint64_t)b * kDenseBits;
+      const uint32_t sh = (uint32_t)(bit & 7u), nbytes = (sh + kDenseBits + 7u) >> 3;
+      uint64_t acc = 0;
+      for (uint32_t k = 0; k < 7u; ++k) acc = (acc << 8) | (k < nbytes ? codes[(bit >> 3) + k] : 0u);
+      const uint64_t rec = (acc >> (56u - sh - kDenseBits)) & ((1ULL << kDenseBits) - 1u);  // index << 1 | gain
+      int8_t* out = points + b * kDim;
+      const int ci = decode_index(T, rec >> 1, [&](int p, int v) { out[p] = (int8_t)v; });
+      if (gains) gains[b] = (uint8_t)(rec & 1);
+      if (shells) shells[b] = ci >= 0 ? (uint8_t)T.cls[ci].shell : (ci == -1 ? 0 : 0xFF);
+    }
+    return;
+  }
   for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < nblocks;
        b += (size_t)gridDim.x * blockDim.x) {
     // the stream's last record is read byte by byte: the two-dword read would touch up to two
@@ -539,6 +568,75 @@ __device__ __forceinline__ void lane_record(const LaneRecords<NB>& r, int j, uin
   }
 }
 
+// ---- records of the cap-13 ball: 49 bits per block in a dense stream -------------------------------
+// At shell cap 13 an index takes 48 bits (N(13) < 2^48), so a block is 49 bits — index, then the gain bit,
+// most significant bit first — and blocks follow one another without padding (llvq-search/src/pack.rs:48-82,
+// llvq-artifact/src/format.rs:87-89): block b of a matrix starts at bit 49 b of its code stream.  A lane takes
+// four consecutive blocks, 196 bits, from the eight dwords that hold them: the stream position of its first
+// block, cut to a dword boundary, plus the bits `s0` left over.  Unconditional loads, as for the 6-byte records:
+// a lane past the tile's end reads the tile's first blocks again; every byte read lies inside the tile or within
+// 32 bytes behind it, which the slack behind a matrix's code stream covers.
+struct DenseRecords {
+  uint32_t w[8];
+  uint32_t s0;  // bits of w[0] ahead of the lane's first block (0..31)
+};
+typedef uint32_t dwords4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+__device__ __forceinline__ void prefetch_records(const GroupArgs& a, uint32_t tile, uint32_t tid, DenseRecords& r) {
+  if (tile >= a.n_tiles || a.nblocks == 0) return;
+  MatArg M;
+  uint32_t r0, rows;
+  tile_of(a, tile, M, r0, rows);
+  const uint64_t tile_bit = (uint64_t)r0 * a.nblocks * kDenseBits;    // the tile's first bit in the matrix's stream
+  const uint64_t tile_base = (tile_bit >> 3) & ~(uint64_t)3;           // ... cut to a dword
+  const uint32_t rem = (uint32_t)(tile_bit - 8u * tile_base);           // 0..31
+  const uint32_t first = tid * 4u < rows * a.nblocks ? tid * 4u : 0u;  // the lane's first block in the tile
+  const uint32_t lane_bit = rem + first * kDenseBits;
+  const uint8_t* src = M.codes + tile_base + (size_t)(lane_bit >> 5) * 4;
+  const dwords4_a4 lo = __builtin_nontemporal_load(reinterpret_cast<const dwords4_a4*>(src));
+  const dwords4_a4 hi = __builtin_nontemporal_load(reinterpret_cast<const dwords4_a4*>(src + 16));
+  r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w; r.w[4] = hi.x; r.w[5] = hi.y; r.w[6] = hi.z; r.w[7] = hi.w;
+  r.s0 = lane_bit & 31u;
+}
+
+// The index (ilo, ihi) and gain bit of record i of a lane's share.  6-byte records: 47 bits of index.
+template <int NB>
+__device__ __forceinline__ const LaneRecords<NB>& prepared_records(const LaneRecords<NB>& rec) { return rec; }
+template <int NB>
+__device__ __forceinline__ void record_index(const LaneRecords<NB>& rec, int i, uint32_t& ilo, uint32_t& ihi, uint32_t& gain) {
+  uint32_t lo32, hi16;
+  lane_record(rec, i, lo32, hi16);
+  gain = lo32 & 1u;
+  ilo = __builtin_amdgcn_alignbit(hi16, lo32, 1);
+  ihi = hi16 >> 1;
+}
+// 49-bit blocks: the dwords become big-endian words and the lane's bits are moved to the front of them, once;
+// block j is then the 49 bits from bit 49 j on.  48 bits of index.
+struct DenseWords {
+  uint32_t n[7];
+};
+__device__ __forceinline__ DenseWords prepared_records(const DenseRecords& rec) {
+  uint32_t be[8];
+  DenseWords d;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) be[i] = __builtin_bswap32(rec.w[i]);
+#pragma unroll
+  for (int i = 0; i < 7; ++i) d.n[i] = (uint32_t)((((uint64_t)be[i] << 32) | be[i + 1]) >> (32u - rec.s0));
+  return d;
+}
+__device__ __forceinline__ void record_index(const DenseWords& r, int j, uint32_t& ilo, uint32_t& ihi, uint32_t& gain) {
+  constexpr uint32_t kW = kDenseBits;
+  const int d = (int)(kW * (uint32_t)j) >> 5;
+  const uint32_t sh = (kW * (uint32_t)j) & 31u;
+  const uint64_t top = (((uint64_t)r.n[d] << 32) | r.n[d + 1]);
+  const uint64_t x = sh ? (top << sh) | (uint64_t)(r.n[d + 2 > 6 ? 6 : d + 2] >> (32u - sh)) : top;  // 64 bits from the block's first
+  const uint64_t v = x >> (64u - kW);                                                                  // the block: index << 1 | gain
+  gain = (uint32_t)v & 1u;
+  ilo = (uint32_t)(v >> 1);
+  ihi = (uint32_t)(v >> 33);
+}
+template <class Rec> struct RecordTraits { static constexpr bool kWide = false; };
+template <> struct RecordTraits<DenseRecords> { static constexpr bool kWide = true; };
+
 // Phase timestamps for tuning builds (-DLLVQ_PHASE_TIMING): wave 0 of each
 // workgroup stores the realtime counter at every phase boundary of its first tile.
 #ifdef LLVQ_PHASE_TIMING
@@ -555,12 +653,13 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 // (kLutKind*).  Two table probes and one comparison each, every read unconditional so that the NB
 // reads of a step go out together; the indices whose bucket meets several class starts (0.09 % of
 // uniform draws) take the halving search afterwards, under a wavefront-wide test.
-template <int NB>
+template <int NB, bool WIDE = false>
 __device__ __forceinline__ void find_classes(const DecodeTables& T, const uint32_t (&zlo)[NB], const uint32_t (&zhi)[NB],
                                              uint32_t (&ci)[NB], uint64_t (&start)[NB], uint32_t (&kind)[NB]) {
   uint32_t e[NB], e2[NB];
+  // (48-bit indices reach the whole first-level table; T's class-find tables are then the full ones, in device memory)
 #pragma unroll
-  for (int i = 0; i < NB; ++i) e[i] = T.lut[(zhi[i] >> (kLutShift - 32)) & 2047u];
+  for (int i = 0; i < NB; ++i) e[i] = T.lut[(zhi[i] >> (kLutShift - 32)) & (WIDE ? (uint32_t)kLutSize - 1u : 2047u)];
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     const uint32_t sub = __builtin_amdgcn_alignbit(zhi[i], zlo[i], kLut2Shift) & (uint32_t)(kLut2Span - 1);
@@ -719,9 +818,10 @@ struct Classified {
 };
 
 // First half of P1: table reads only, nothing is written — it may run while another tile's queues are in use.
-template <int NB>
-__device__ __forceinline__ void classify_records(const DecodeTables& T, const LaneRecords<NB>& rec, uint32_t nblk, Classified<NB>& c,
+template <int NB, class Rec>
+__device__ __forceinline__ void classify_records(const DecodeTables& T, const Rec& rec, uint32_t nblk, Classified<NB>& c,
                                                  uint32_t tid = threadIdx.x) {
+  constexpr bool kWide = RecordTraits<Rec>::kWide;
   // Every LDS read below is unconditional, from a valid slot, so that the NB reads of a step go
   // out together (a guarded read is waited for where it is issued).  A lane past the tile's end
   // walks the tables with whatever bytes follow the tile and queues nothing.
@@ -729,21 +829,23 @@ __device__ __forceinline__ void classify_records(const DecodeTables& T, const La
   uint64_t start[NB];
   bool live[NB];  // a block of the tile that is not the origin (which decodes to zero whatever the gain, index.rs:335-337)
   uint32_t where = 0;
+  const auto& records = prepared_records(rec);
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     const uint32_t f = tid * NB + (uint32_t)i;
-    uint32_t lo32, hi16;
-    lane_record(rec, i, lo32, hi16);
-    gain[i] = lo32 & 1u;
-    const uint32_t ilo = __builtin_amdgcn_alignbit(hi16, lo32, 1), ihi = hi16 >> 1;  // the 47-bit index
+    uint32_t ilo, ihi;  // the 47-bit (48-bit) index
+    record_index(records, i, ilo, ihi, gain[i]);
     const bool origin = (ilo | ihi) == 0u;
     live[i] = f < nblk && !origin;
     where |= (f < nblk && origin) ? 1u << (8 + i) : 0u;
-    const uint64_t z = (((uint64_t)ihi << 32) | ilo) - 1u;  // zero-based
+    uint64_t z = (((uint64_t)ihi << 32) | ilo) - 1u;  // zero-based
+    // a 48-bit field can hold numbers past N(13): the host refuses such a matrix, and a lane past the tile's
+    // end, which reads whatever bits follow, must still walk the tables inside them
+    if (kWide) z = z < kN13 ? z : 0u;
     zlo[i] = (uint32_t)z;
-    zhi[i] = (uint32_t)(z >> 32) & 0x7FFFu;  // an origin wraps to all ones: keep it a 47-bit index
+    zhi[i] = (uint32_t)(z >> 32) & (kWide ? 0xFFFFu : 0x7FFFu);  // an origin wraps to all ones: keep it inside the field
   }
-  find_classes<NB>(T, zlo, zhi, ci, start, kind);
+  find_classes<NB, kWide>(T, zlo, zhi, ci, start, kind);
   // Which queue a block joins.  A generic block rides in the odd queue, flagged, unless its coset's small
   // queue has room (settled when the block is queued).
   uint32_t any_generic = 0;
@@ -845,8 +947,8 @@ __device__ __forceinline__ void settle_origins(uint32_t where, float* partial, u
   }
 }
 
-template <int NB>
-__device__ __forceinline__ void classify_stream(const DecodeTables& T, const LaneRecords<NB>& rec, uint32_t nblk, uint32_t capacity,
+template <int NB, class Rec>
+__device__ __forceinline__ void classify_stream(const DecodeTables& T, const Rec& rec, uint32_t nblk, uint32_t capacity,
                                                 const GemvQueues& Q) {
   Classified<NB> c;
   classify_records<NB>(T, rec, nblk, c);
@@ -1215,8 +1317,11 @@ __device__ __forceinline__ bool stage_activation(const ActivationSource& a, uint
 // room for the full tile beside the activation planes of a very wide row.
 // ROT: the launch can rotate its own activation (GroupArgs::rot_m); kept out of the other
 // instantiations, whose hot loop it would otherwise cost registers and a few per cent.
-template <typename OutT, int TILE = kTileBlocks, bool LEAN = false, bool ROT = false>
+// WIDE: the matrices are cap-13 ones (49-bit blocks in a dense stream, 48-bit indices): a lane extracts its blocks
+// from the stream, and the class tables a 47-bit index cannot reach are read from device memory.
+template <typename OutT, int TILE = kTileBlocks, bool LEAN = false, bool ROT = false, bool WIDE = false>
 __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
+  static_assert(!WIDE || (TILE == 4 * kWgThreads && !ROT), "the dense-stream variant takes four blocks per lane and no in-launch rotation");
   // the tile capacity of this instantiation (these shadow the namespace-level defaults)
   constexpr int kTileBlocks = TILE;
   constexpr int kP1Blocks = TILE / kWgThreads;
@@ -1225,14 +1330,15 @@ __global__ __launch_bounds__(kWgThreads) void gemv_tiles_kernel(GroupArgs a) {
 #ifdef LLVQ_PHASE_TIMING
   if (threadIdx.x == 0) g_phase_stamps[blockIdx.x * 8 + 3] = wall_clock64();
 #endif
-  const DecodeTables T = stage_tables<!LEAN>(smem, a.tables);
+  const DecodeTables T = stage_tables<!LEAN, true, WIDE>(smem, a.tables);
   // A lane loads the records it classifies itself, HBM -> registers; the next tile's loads are
   // issued while the current one is being decoded.  The first tile's are issued right behind the
   // loads of the activation: the memory counter retires in order, so whatever is requested
   // after them would wait for HBM with them, and they are not needed before the activation is.
-  LaneRecords<kP1Blocks> pre;
+  typename std::conditional<WIDE, DenseRecords, LaneRecords<kP1Blocks>>::type pre;
 #pragma unroll
-  for (int k = 0; k < kP1Blocks * 3 / 2; ++k) pre.w[k] = 0;
+  for (int k = 0; k < (int)(sizeof(pre.w) / sizeof(pre.w[0])); ++k) pre.w[k] = 0;
+  if constexpr (WIDE) pre.s0 = 0;
   auto request_first_tile = [&]() { prefetch_records(a, blockIdx.x, threadIdx.x, pre); };
   const uint32_t nb = a.nblocks;
   uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + (LEAN ? kLdsImageBytesLean : kLdsImageBytes));
@@ -1335,14 +1441,24 @@ __host__ const void* gemv_kernel(bool f32, uint32_t tile, bool lean, bool rot) {
   if (f32) return rot ? gemv_kernel_of<float, true>(tile, lean) : gemv_kernel_of<float, false>(tile, lean);
   return rot ? gemv_kernel_of<__half, true>(tile, lean) : gemv_kernel_of<__half, false>(tile, lean);
 }
+// ... and for cap-13 matrices (full tile only, with the whole or the lean table image, no in-launch rotation)
+__host__ const void* gemv_kernel_wide(bool f32, bool lean) {
+  if (f32) return lean ? reinterpret_cast<const void*>(gemv_tiles_kernel<float, kTileBlocks, true, false, true>)
+                       : reinterpret_cast<const void*>(gemv_tiles_kernel<float, kTileBlocks, false, false, true>);
+  return lean ? reinterpret_cast<const void*>(gemv_tiles_kernel<__half, kTileBlocks, true, false, true>)
+              : reinterpret_cast<const void*>(gemv_tiles_kernel<__half, kTileBlocks, false, false, true>);
+}
 template <class Fn>
 __host__ void for_each_gemv_kernel(Fn&& fn) {
-  for (int f32 = 0; f32 < 2; ++f32)
+  for (int f32 = 0; f32 < 2; ++f32) {
     for (int rot = 0; rot < 2; ++rot) {
       fn(gemv_kernel(f32, kTileBlocks, false, rot));
       fn(gemv_kernel(f32, kSmallTileBlocks, false, rot));
       fn(gemv_kernel(f32, kTileBlocks, true, rot));
     }
+    fn(gemv_kernel_wide(f32, false));
+    fn(gemv_kernel_wide(f32, true));
+  }
 }
 
 // ---- incoherence rotation of an activation ----------------------------------------
@@ -1424,6 +1540,7 @@ struct llvq_rt {
 struct llvq_mat {
   std::string name;
   uint32_t d_out = 0, d_in = 0, nblocks = 0, tail_w = 0;
+  uint32_t record_bits = 48;  // 48: 6-byte records (shell cap 12); 49: the dense stream of shell cap 13
   float g[2] = {0, 0};
   uint8_t* codes = nullptr;  // device
   float* rscale = nullptr;   // device
@@ -1510,7 +1627,11 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   const size_t off_exp = (off_lut + cb.off_lut.size() * 4 + 15) & ~(size_t)15;
   const size_t off_tail = off_exp + sizeof(cb.expand);
   static_assert(sizeof(cb.expand) % 16 == 0, "the walk-tail codes are read as 8-byte units");
-  const size_t total = off_tail + cb.tail_codes.size() * 8;
+  // ... | every fast-path class record | the whole class-find table, both levels (for 48-bit indices)
+  const size_t off_wfast = (off_tail + cb.tail_codes.size() * 8 + 15) & ~(size_t)15;
+  const size_t off_wlut = off_wfast + sizeof(cb.fast);
+  const size_t off_wlut2 = off_wlut + sizeof(cb.lut);
+  const size_t total = off_wlut2 + cb.lut2.size() * 2;
   std::vector<uint8_t> host(total, 0);
   auto* img = reinterpret_cast<TableImage*>(host.data());
   std::memcpy(img->golay, cb.golay, sizeof img->golay);
@@ -1536,6 +1657,9 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   std::memcpy(host.data() + off_lut, cb.off_lut.data(), cb.off_lut.size() * 4);
   std::memcpy(host.data() + off_exp, cb.expand, sizeof(cb.expand));
   std::memcpy(host.data() + off_tail, cb.tail_codes.data(), cb.tail_codes.size() * 8);
+  std::memcpy(host.data() + off_wfast, cb.fast, sizeof(cb.fast));
+  std::memcpy(host.data() + off_wlut, cb.lut, sizeof(cb.lut));
+  std::memcpy(host.data() + off_wlut2, cb.lut2.data(), cb.lut2.size() * 2);
   e = hipMalloc(reinterpret_cast<void**>(&rt->blob), total);
   if (e != hipSuccess) { delete rt; return hip_fail(e, "hipMalloc(tables)"); }
   e = hipMemcpy(rt->blob, host.data(), total, hipMemcpyHostToDevice);
@@ -1546,6 +1670,9 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   rt->tables.off_lut = reinterpret_cast<const uint32_t*>(rt->blob + off_lut);
   rt->tables.expand = reinterpret_cast<const uint32_t*>(rt->blob + off_exp);
   rt->tables.tail_codes = reinterpret_cast<const uint64_t*>(rt->blob + off_tail);
+  rt->tables.wide_fast = reinterpret_cast<const FastClass*>(rt->blob + off_wfast);
+  rt->tables.wide_lut = reinterpret_cast<const uint16_t*>(rt->blob + off_wlut);
+  rt->tables.wide_lut2 = reinterpret_cast<const uint16_t*>(rt->blob + off_wlut2);
   // the activation tile of a wide matrix pushes dynamic LDS past the 64 KB default
   const int max_lds = 160 * 1024;
   for_each_gemv_kernel([&](const void* kernel) { (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds); });
@@ -1636,13 +1763,14 @@ static int upload_impl(llvq_rt* rt, const std::string& name, uint32_t d_out, uin
     return fail(LLVQ_ERR_UNSUPPORTED, name + ": " + std::to_string(n_centroids) +
                                           " centroids, but the kernels hard-code 1 gain bit");
   const int ib = index_bits(shell_cap);
-  if (ib + 1 != 48)
+  if (ib + 1 != 48 && ib + 1 != (int)kDenseBits)
     return fail(LLVQ_ERR_UNSUPPORTED, name + ": shell cap " + std::to_string(shell_cap) + " packs " +
                                           std::to_string(ib + 1) +
-                                          " bits per block; the kernels read 6-byte records (cap 12)");
+                                          " bits per block; the kernels read 6-byte records (cap 12) and the 49-bit stream of cap 13");
+  const uint32_t record_bits = (uint32_t)ib + 1u;
   const uint32_t nblocks = d_in / kDim, tail_w = d_in % kDim;
   const uint64_t total_blocks = (uint64_t)d_out * nblocks;
-  if ((unsigned __int128)total_blocks * 48 > (unsigned __int128)code_bytes * 8)
+  if ((unsigned __int128)total_blocks * record_bits > (unsigned __int128)code_bytes * 8)
     return fail(LLVQ_ERR_TRUNCATED, "file ends mid-code stream");
   if (d_out == 0 || d_in == 0) return fail(LLVQ_ERR_INVALID_ARGUMENT, name + ": empty matrix");
   if ((total_blocks && !codes) || !centroids || !row_scales || (tail_w && !tail))
@@ -1650,10 +1778,13 @@ static int upload_impl(llvq_rt* rt, const std::string& name, uint32_t d_out, uin
   // Index range (format.rs:389-392).  The bound is N(13) whatever the cap; a
   // 47-bit field cannot exceed it (2^47 < N(13)), so at cap 12 this never fires.
   if (ib < 64 && ((1ULL << ib) - 1) > kN13) {
+    // (only the 48-bit field of cap 13 can: block b is the record_bits bits from bit record_bits * b on)
     for (uint64_t b = 0; b < total_blocks; ++b) {
-      const uint8_t* p = codes + 6 * b;
-      const uint64_t v = ((uint64_t)p[0] << 40) | ((uint64_t)p[1] << 32) | ((uint64_t)p[2] << 24) |
-                         ((uint64_t)p[3] << 16) | ((uint64_t)p[4] << 8) | p[5];
+      const uint64_t bit = b * record_bits;
+      const uint32_t sh = (uint32_t)(bit & 7u), nbytes = (sh + record_bits + 7u) >> 3;
+      uint64_t acc = 0;
+      for (uint32_t k = 0; k < 7u; ++k) acc = (acc << 8) | (k < nbytes ? codes[(bit >> 3) + k] : 0u);
+      const uint64_t v = (acc >> (56u - sh - record_bits)) & ((1ULL << record_bits) - 1u);
       if ((v >> 1) > kN13)
         return fail(LLVQ_ERR_INDEX_OUT_OF_RANGE,
                     name + ": index " + std::to_string(v >> 1) + " is not a codebook member");
@@ -1675,12 +1806,13 @@ static int upload_impl(llvq_rt* rt, const std::string& name, uint32_t d_out, uin
   m->d_in = d_in;
   m->nblocks = nblocks;
   m->tail_w = tail_w;
+  m->record_bits = record_bits;
   m->g[0] = (float)centroids[0];  // fused.rs:1209
   m->g[1] = (float)centroids[1];
   std::vector<float> rs(d_out);
   for (uint32_t r = 0; r < d_out; ++r) rs[r] = (float)row_scales[r];  // fused.rs:1210
-  const size_t code_len = (size_t)total_blocks * 6;
-  const size_t code_alloc = code_len + 64;  // slack so wide loads may run past the last record
+  const size_t code_len = (size_t)((total_blocks * record_bits + 7) / 8);
+  const size_t code_alloc = ((code_len + 3) & ~(size_t)3) + 64;  // slack so wide loads may run past the last record
   const size_t tail_len = (size_t)d_out * tail_w * sizeof(float);
   auto cleanup = [&](hipError_t e, const char* what) {
     (void)hipFree(m->codes);
@@ -1880,6 +2012,7 @@ static bool prologue_fits(const llvq_mat* m0) {
 // Whether a launch over rows of this width can rotate its own activation: the f32
 // values take the place of the first tile's queues and partial sums.
 static bool rotation_fits(const llvq_mat* m0) {
+  if (m0->record_bits != 48) return false;  // the dense-stream kernels have no in-launch rotation: a kernel of its own rotates
   const size_t tile = pick_gemv_shape(m0->nblocks).tile;
   return (size_t)m0->d_in * 4 + 64 <= tile * 6 + 32 + tile * 8;
 }
@@ -1941,7 +2074,13 @@ static int launch_group(llvq_rt* rt, const llvq_mat* const* mats, int n, const v
   }
   a.n_tiles = tiles;
   const uint32_t grid = tiles < grid_cap ? tiles : grid_cap;
-  const void* kernel = gemv_kernel(y_dtype == LLVQ_F32, tile, shape.lean, rot != nullptr);
+  const bool wide = m0->record_bits != 48;
+  for (int i = 1; i < n; ++i)
+    if (mats[i]->record_bits != m0->record_bits)
+      return fail(LLVQ_ERR_INVALID_ARGUMENT, mats[i]->name + ": matrices of one launch must share their shell cap");
+  if (wide && (tile != (uint32_t)kTileBlocks || rot))
+    return fail(LLVQ_ERR_UNSUPPORTED, m0->name + ": rows too wide for the cap-13 kernels");
+  const void* kernel = wide ? gemv_kernel_wide(y_dtype == LLVQ_F32, shape.lean) : gemv_kernel(y_dtype == LLVQ_F32, tile, shape.lean, rot != nullptr);
   void* params[] = {&a};
   HIP_TRY(hipLaunchKernel(kernel, dim3(grid), dim3(kWgThreads), params, lds, rt->stream));
   HIP_TRY(hipGetLastError());
@@ -1968,7 +2107,7 @@ static int launch_rotate(llvq_rt* rt, const llvq_rt::DevRotation* rot, const voi
 }
 
 static bool same_basis(const llvq_mat* a, const llvq_mat* b) {
-  return a->has_rotation == b->has_rotation && (!a->has_rotation || a->rotation_seed == b->rotation_seed);
+  return a->record_bits == b->record_bits && a->has_rotation == b->has_rotation && (!a->has_rotation || a->rotation_seed == b->rotation_seed);
 }
 
 // One activation through projections that share it: consecutive matrices in the
@@ -2109,6 +2248,7 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
       if (!m || !sp.y[j]) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: null matrix or output in item " + std::to_string(i));
       if (m->d_in != sp.mats[0]->d_in) return fail(LLVQ_ERR_INVALID_ARGUMENT, m->name + ": projections of one item must share d_in");
       if (m->has_rotation) return fail(LLVQ_ERR_UNSUPPORTED, m->name + ": a sequence takes natural-basis matrices only");
+      if (m->record_bits != 48) return fail(LLVQ_ERR_UNSUPPORTED, m->name + ": a sequence takes 6-byte records (shell cap 12) only");
     }
     if (sp.mats[0]->nblocks > 1024u) return fail(LLVQ_ERR_UNSUPPORTED, sp.mats[0]->name + ": rows wider than 24 576 columns do not fit a sequence");
     max_nb = std::max(max_nb, sp.mats[0]->nblocks);
@@ -2367,7 +2507,9 @@ static int reserve_batched(llvq_rt* rt, const llvq_mat* const* mats, int n, uint
     while (i1 < n && i1 - i0 < kGemmMaxGroup && mats[i1]->has_rotation == mats[i0]->has_rotation &&
            (!mats[i0]->has_rotation || mats[i1]->rot == mats[i0]->rot))
       ++i1;
-    if (mats[i0]->nblocks) {
+    bool six_byte = true;
+    for (int i = i0; i < i1; ++i) six_byte &= mats[i]->record_bits == 48;
+    if (mats[i0]->nblocks && six_byte) {  // (cap-13 matrices take the row loop, which has no workspace)
       // every row count up to the chunk: the partial-sum layout is not monotone in M where the consumers' split changes
       for (uint32_t M : {chunk, (uint32_t)64, (uint32_t)128, (uint32_t)256}) {
         if (M > chunk) continue;
@@ -2482,7 +2624,9 @@ static int gemm_same_basis(llvq_rt* rt, const llvq_mat* const* mats, int n, cons
   const llvq_mat* m0 = mats[0];
   const size_t esz = y_dtype == LLVQ_F32 ? 4 : 2;
   const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
-  const bool mfma_ok = M >= 2 && m0->d_in % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && m0->nblocks > 0;
+  bool six_byte = true;  // the matrix-core kernel's producers read 6-byte records: cap-13 matrices take the row loop
+  for (int i = 0; i < n; ++i) six_byte &= mats[i]->record_bits == 48;
+  const bool mfma_ok = M >= 2 && m0->d_in % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && m0->nblocks > 0 && six_byte;
   if (!mfma_ok) {
     for (int i = 0; i < n; ++i)
       for (int r = 0; r < M; ++r) {
@@ -2599,7 +2743,28 @@ int llvq_hip_decode_blocks(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks
   size_t grid = (nblocks + 255) / 256;
   const size_t cap = (size_t)(rt->cu_count > 0 ? rt->cu_count : 256) * 2;
   if (grid > cap) grid = cap;
-  hipLaunchKernelGGL(decode_blocks_kernel, dim3((uint32_t)grid), dim3(256), kLdsImageBytes, rt->stream,
+  hipLaunchKernelGGL(decode_blocks_kernel<false>, dim3((uint32_t)grid), dim3(256), kLdsImageBytes, rt->stream,
+                     rt->tables, codes_dev, nblocks, points_dev, gains_dev, shells_dev);
+  HIP_TRY(hipGetLastError());
+  return LLVQ_OK;
+}
+
+int llvq_hip_decode_stream(llvq_rt* rt, const uint8_t* codes_dev, size_t nblocks, uint32_t shell_cap, int8_t* points_dev,
+                           uint8_t* gains_dev, uint8_t* shells_dev) {
+  if (!rt) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decode_stream: runtime is null");
+  if (shell_cap > (uint32_t)kMaxShell) return fail(LLVQ_ERR_INCONSISTENT, "decode_stream: shell cap " + std::to_string(shell_cap) + " exceeds the supported ball (m <= 13)");
+  const int bits = index_bits(shell_cap) + 1;
+  if (bits == 48) return llvq_hip_decode_blocks(rt, codes_dev, nblocks, points_dev, gains_dev, shells_dev);
+  if (bits != (int)kDenseBits)
+    return fail(LLVQ_ERR_UNSUPPORTED, "decode_stream: shell cap " + std::to_string(shell_cap) + " packs " + std::to_string(bits) +
+                                          " bits per block; the kernels read 6-byte records (cap 12) and the 49-bit stream of cap 13");
+  if (nblocks == 0) return LLVQ_OK;
+  if (!points_dev || !codes_dev) return fail(LLVQ_ERR_INVALID_ARGUMENT, "decode_stream: null argument");
+  HIP_TRY(hipSetDevice(rt->device));
+  size_t grid = (nblocks + 255) / 256;
+  const size_t cap = (size_t)(rt->cu_count > 0 ? rt->cu_count : 256) * 2;
+  if (grid > cap) grid = cap;
+  hipLaunchKernelGGL(decode_blocks_kernel<true>, dim3((uint32_t)grid), dim3(256), kLdsImageBytes, rt->stream,
                      rt->tables, codes_dev, nblocks, points_dev, gains_dev, shells_dev);
   HIP_TRY(hipGetLastError());
   return LLVQ_OK;
@@ -3098,6 +3263,9 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
         return fail(LLVQ_ERR_INCONSISTENT, "decoder_create: layer " + std::to_string(L) + " " + kSite[j] + " is " +
                                                std::to_string(m->d_out) + "x" + std::to_string(m->d_in) + ", the architecture needs " +
                                                std::to_string(want_out[j]) + "x" + std::to_string(want_in[j]));
+      if (m->record_bits != 48)
+        return fail(LLVQ_ERR_UNSUPPORTED, "decoder_create: layer " + std::to_string(L) + " " + kSite[j] +
+                                              " is a cap-13 matrix; the decode loop takes 6-byte records (shell cap 12), cap-13 matrices are served by llvq_hip_gemv / _gemv_group / _gemm");
     }
   HIP_TRY(hipSetDevice(rt->device));
   auto* d = new llvq_decoder();

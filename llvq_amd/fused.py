@@ -378,6 +378,17 @@ class FusedRuntime:
                                                       gains.data_ptr(), shells.data_ptr()))
         return pts, gains, shells
 
+    def decode_stream(self, codes, nblocks: int, shell_cap: int):
+        """`decode_blocks` for the code stream of any accepted shell cap (cap 13: 49 bits per block, dense)."""
+        torch = self._torch
+        n = int(nblocks)
+        pts = torch.empty((n, 24), dtype=torch.int8, device=codes.device)
+        gains = torch.empty(n, dtype=torch.uint8, device=codes.device)
+        shells = torch.empty(n, dtype=torch.uint8, device=codes.device)
+        _ffi.check(_ffi.lib().llvq_hip_decode_stream(self.handle, codes.data_ptr(), n, int(shell_cap), pts.data_ptr(),
+                                                      gains.data_ptr(), shells.data_ptr()))
+        return pts, gains, shells
+
     def synchronize(self):
         _ffi.check(_ffi.lib().llvq_hip_synchronize(self.handle))
 

@@ -10,7 +10,7 @@ f32).  Gain centroids are {0.8, 1.25}.  An activation is its own stream.
 """
 import numpy as np
 
-from .artifact import DIM, N12, RawMatrix, pack_codes
+from .artifact import DIM, N12, N13, RawMatrix, pack_codes
 
 _GAMMA = 0x9E3779B97F4A7C15
 _M1 = 0xBF58476D1CE4E5B9
@@ -56,8 +56,11 @@ def matrix_seed(seed: int, name: str) -> int:
     return (seed ^ fnv1a64(name.encode())) & _MASK
 
 
-def make_matrix(name: str, d_out: int, d_in: int, seed: int = 0, index_bound: int = N12 + 1,
-                centroids=(0.8, 1.25)) -> RawMatrix:
+def make_matrix(name: str, d_out: int, d_in: int, seed: int = 0, index_bound: int = None,
+                centroids=(0.8, 1.25), shell_cap: int = 12) -> RawMatrix:
+    """Indices uniform below `index_bound` (default: the whole ball of the cap, origin included)."""
+    if index_bound is None:
+        index_bound = {12: N12, 13: N13}[shell_cap] + 1
     rng = SplitMix64(matrix_seed(seed, name))
     nb = d_out * (d_in // DIM)
     draws = rng.take(2 * nb)
@@ -65,8 +68,8 @@ def make_matrix(name: str, d_out: int, d_in: int, seed: int = 0, index_bound: in
     gain = draws[1::2] & np.uint64(1)
     row_scales = np.exp(-4.0 + 0.3 * rng.gaussian(d_out))
     tail = (0.02 * rng.gaussian(d_out * (d_in % DIM))).astype(np.float32)
-    return RawMatrix(name, d_out, d_in, 12, np.array(centroids, np.float64), row_scales, tail,
-                     pack_codes(idx, gain))
+    return RawMatrix(name, d_out, d_in, shell_cap, np.array(centroids, np.float64), row_scales, tail,
+                     pack_codes(idx, gain, index_width={12: 47, 13: 48}[shell_cap]))
 
 
 def make_activation(d_in: int, seed: int = 0, rows: int = 1) -> np.ndarray:

@@ -218,3 +218,30 @@ def test_splitmix_vectors(orc):
     g_np = synth.SplitMix64(0xA4C0DE).gaussian(1000)
     assert np.allclose(g_c, g_np, rtol=1e-12, atol=1e-14)
     assert abs(g_np.mean()) < 0.1 and abs(g_np.std() - 1) < 0.1
+
+
+def test_host_packer_follows_the_bit_writer_at_every_block_width(orc):
+    """llvq_amd.artifact.pack_codes / RawMatrix.unpack against the oracle's bit writer (pack.rs:48-82) for blocks of
+    3 bits (the reference's own known answer, g6_pack.rs:17-27: 101 011 110 -> AF 00), 48 bits (cap 12) and 49 bits
+    (cap 13, the dense stream: 48 bits of index, format.rs:87-89), and a cap-13 record through both readers."""
+    from llvq_amd import synth
+
+    assert artifact.pack_codes([0b10, 0b01, 0b11], [1, 1, 0], index_width=2).tobytes() == bytes([0b10101111, 0])
+    rng = np.random.default_rng(49)
+    for width, bound in ((47, orc.N12 + 1), (48, orc.N13 + 1)):
+        idx = rng.integers(0, bound, size=1001, dtype=np.uint64)
+        idx[:3] = [0, bound - 1, 1]
+        gains = rng.integers(0, 2, size=idx.size).astype(np.uint8)
+        want = orc.pack_bits([f for i, g in zip(idx.tolist(), gains.tolist()) for f in ((i, width), (g, 1))])
+        got = artifact.pack_codes(idx, gains, index_width=width)
+        assert got.tobytes() == want and got.size == (idx.size * (width + 1) + 7) // 8
+    assert artifact.index_bits(13) == 48 and orc.lib().orc_index_bits(13) == 48
+    raw = synth.make_matrix("model.layers.0.cap13.weight", 9, 24 * 5 + 3, seed=2, shell_cap=13)
+    assert raw.codes.size == (9 * 5 * 49 + 7) // 8
+    blob = artifact.write_matrix_raw(raw)
+    om, _ = orc.read_matrix_raw(blob)
+    back, _ = artifact.read_matrix_raw(blob)
+    idx, gains = back.unpack()
+    assert np.array_equal(idx, om.indices().astype(np.uint64)) and np.array_equal(gains, om.gains().astype(np.uint8))
+    assert int(idx.max()) <= orc.N13 and int(idx.max()) >= (1 << 47)  # the draw reaches shell 13's upper half
+    assert om.write() == blob
