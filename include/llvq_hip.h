@@ -57,9 +57,10 @@ typedef struct llvq_mat llvq_mat; /* replaces FusedProj     (fused_cuda.rs:119-1
  * stream at cap 13, format.rs:87-89). All pointers are host memory.
  * Cap 12 and cap 13 are accepted; other caps are refused by name
  * (LLVQ_ERR_UNSUPPORTED).  A cap-13 matrix is served by llvq_hip_gemv,
- * llvq_hip_gemv_group (matrices of one call share their cap), llvq_hip_rotate /
- * llvq_hip_gemv_rotated and, as a loop over its rows, by llvq_hip_gemm /
- * llvq_hip_gemm_group; sequences and the decode loop refuse it by name. */
+ * llvq_hip_gemv_group (a call may mix caps: one launch per cap), llvq_hip_rotate /
+ * llvq_hip_gemv_rotated, the decode loop (per-group launches) and, as a loop over
+ * its rows, by llvq_hip_gemm / llvq_hip_gemm_group and the batched prompt path;
+ * llvq_hip_sequence_create refuses it by name. */
 typedef struct llvq_matrix_desc {
   const char* name;          /* may be NULL */
   uint32_t d_out, d_in;
@@ -280,7 +281,8 @@ typedef struct llvq_quant_rows {
 /* How llvq_hip_decoder_* launches the projection groups of a decoded position.  The results are the same bit for bit;
  * the speed is not: a decode position is a chain of dependent products, and an ordered item of a sequence pays about
  * what a launch boundary costs (measured on the Qwen3-4B shape: 245 / 226 / 220 tokens/s in the order below).
- * Models a sequence cannot take (matrices in a rotated basis, hidden > 6144) use LLVQ_LAUNCH_PER_GROUP whatever is asked. */
+ * Models a sequence cannot take (matrices in a rotated basis or of shell cap 13, hidden > 6144) use LLVQ_LAUNCH_PER_GROUP
+ * whatever is asked. */
 typedef enum llvq_launch_mode {
   LLVQ_LAUNCH_PER_GROUP = 0,  /* one llvq_hip_gemv_group launch per group */
   LLVQ_LAUNCH_SINGLE = 1,     /* one single-item sequence (llvq_hip_sequence_*) per group: the sequence kernel's tile loop */

@@ -3263,9 +3263,6 @@ int llvq_hip_decoder_create(llvq_rt* rt, const llvq_decoder_desc* c, llvq_decode
         return fail(LLVQ_ERR_INCONSISTENT, "decoder_create: layer " + std::to_string(L) + " " + kSite[j] + " is " +
                                                std::to_string(m->d_out) + "x" + std::to_string(m->d_in) + ", the architecture needs " +
                                                std::to_string(want_out[j]) + "x" + std::to_string(want_in[j]));
-      if (m->record_bits != 48)
-        return fail(LLVQ_ERR_UNSUPPORTED, "decoder_create: layer " + std::to_string(L) + " " + kSite[j] +
-                                              " is a cap-13 matrix; the decode loop takes 6-byte records (shell cap 12), cap-13 matrices are served by llvq_hip_gemv / _gemv_group / _gemm");
     }
   HIP_TRY(hipSetDevice(rt->device));
   auto* d = new llvq_decoder();

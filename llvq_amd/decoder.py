@@ -93,10 +93,10 @@ def quantize_rows_q8(name: str, table, group: int = 64) -> artifact.RawTensor:
                               biases=b.reshape(-1).view(np.uint16))
 
 
-def synthetic_projections(cfg: Qwen3Config, seed: int = 0):
+def synthetic_projections(cfg: Qwen3Config, seed: int = 0, shell_cap: int = 12):
     """Random LLVQ codes for every projection, drawn as the single-matrix benchmark draws them."""
-    return [[synth.make_matrix(f"model.layers.{layer}.{site}.weight", do, di, seed) for site, do, di in cfg.shapes()]
-            for layer in range(cfg.num_hidden_layers)]
+    return [[synth.make_matrix(f"model.layers.{layer}.{site}.weight", do, di, seed, shell_cap=shell_cap)
+             for site, do, di in cfg.shapes()] for layer in range(cfg.num_hidden_layers)]
 
 
 class Decoder:

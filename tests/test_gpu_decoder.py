@@ -45,10 +45,10 @@ Q8 = decoder.Qwen3Config(num_hidden_layers=2, hidden_size=256, num_attention_hea
                          max_positions=80, tie_word_embeddings=True, kv_mode="q8")  # 5 query heads per kv head, as at 14B
 
 
-def _build(gpu_rt, orc, cfg, seed, rotate=False, prefill_rows=0):
+def _build(gpu_rt, orc, cfg, seed, rotate=False, prefill_rows=0, shell_cap=12):
     from oracle import qwen3_oracle
 
-    raws = decoder.synthetic_projections(cfg, seed)
+    raws = decoder.synthetic_projections(cfg, seed, shell_cap=shell_cap)
     if rotate:
         # stored as W Q^T (format.rs:435-437): q/k/v share a basis, gate/up another, o and down have their own;
         # layer 1 keeps k and v in the natural basis, so one group call spans two bases
@@ -90,6 +90,27 @@ def test_teacher_forced_logits(gpu_rt, orc, cfg, seed, n):
         assert worst < _bar(cfg), f"max |dlogit| / max|logit| = {worst:.3e}"
         assert agree >= len(tokens) - 2
         assert dec.position == len(tokens)
+    finally:
+        dec.close()
+
+
+def test_cap13_projections_in_the_loop(gpu_rt, orc):
+    """Every projection a cap-13 matrix (49-bit blocks in a dense stream, llvq-llm/src/fused.rs:1166-1180): the prompt
+    through the batched path (a row loop for such matrices), then position by position, against the oracle."""
+    dec, ref = _build(gpu_rt, orc, SMALL, 9, prefill_rows=16, shell_cap=13)
+    try:
+        tokens = np.random.default_rng(9).integers(0, SMALL.vocab_size, size=20)
+        for t in tokens[:-1]:
+            ref.forward_token(int(t))
+        want = ref.forward_token(int(tokens[-1]))
+        got, _ = dec.prefill(tokens)
+        worst = float(np.abs(got - want).max() / np.abs(want).max())
+        for t in np.random.default_rng(109).integers(0, SMALL.vocab_size, size=12):
+            want = ref.forward_token(int(t))
+            got, _ = dec.forward_token(int(t))
+            worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
+        print(f"OBSERVED cap13_loop: {worst:.3e}")
+        assert worst < BAR_SMALL, f"max |dlogit| / max|logit| = {worst:.3e}"
     finally:
         dec.close()
 
