@@ -280,7 +280,7 @@ typedef struct llvq_quant_rows {
 } llvq_quant_rows;
 /* How llvq_hip_decoder_* launches the projection groups of a decoded position.  The results are the same bit for bit;
  * the speed is not: a decode position is a chain of dependent products, and an ordered item of a sequence pays about
- * what a launch boundary costs (measured on the Qwen3-4B shape: 245 / 226 / 220 tokens/s in the order below).
+ * what a launch boundary costs (measured on the Qwen3-4B shape: 248 / 235 / 227 tokens/s in the order below).
  * Models a sequence cannot take (matrices in a rotated basis or of shell cap 13, hidden > 6144) use LLVQ_LAUNCH_PER_GROUP
  * whatever is asked. */
 typedef enum llvq_launch_mode {
