@@ -23,20 +23,21 @@ constexpr int kClassSlots = 384;   // 383 classes + one sentinel, a power-of-two
 constexpr int kStartsPadded = 512; // class starts, padded with UINT64_MAX past N(13)
 constexpr int kStartsLds = 320;    // what a 47-bit index can reach (class <= 317) plus its upper neighbour; the rare wide search reads the padded table
 constexpr int kFastLds = 320;      // fast-path class records a 47-bit index can reach
-constexpr int kLutShift = 36;      // class-find table is keyed on the zero-based index >> 36
+constexpr int kLutShift = 36;      // class-find table is keyed on the index as a record holds it (1 .. N) >> 36
 constexpr int kOnLutSlots = 4352;  // LDS slots for the support-arrangement table (4322 entries used)
-constexpr int kLutSize = 4096;     // covers every zero-based index < N(13) < 2^48 (a 47-bit field uses the lower half)
+constexpr int kLutSize = 4096;     // covers every index <= N(13) < 2^48 (a 47-bit field uses the lower half)
 constexpr int kLut2Shift = 31;     // second-level buckets of the class-find table
 constexpr int kLut2Span = 1 << (kLutShift - kLut2Shift);  // entries of a second-level table
 constexpr int kLut2Lds = 54 * kLut2Span;  // second-level entries the lower half of the first level refers to (53 tables)
-// Class-find table entries (16 bits).  First level, keyed on the zero-based index >> kLutShift:
-//   bit 15 set: bits 0..14 = a second-level table, keyed on (index >> kLut2Shift) % kLut2Span;
-//   else a final entry.  Final entry (either level): bits 0..8 = class c0 holding the bucket's first
+// Class-find table entries (16 bits).  First level, keyed on the index as a record holds it >> kLutShift:
+//   bit 15 clear: the entry is where a second-level table begins in lut2 (a multiple of kLut2Span), that table
+//   keyed on (index >> kLut2Shift) % kLut2Span; bit 15 set (kLutFinal): a final entry.  Every second-level entry is
+//   final, with or without the bit.  Final entry (either level): bits 0..8 = class c0 holding the bucket's first
 //   index; bit 13 clear: the bucket meets at most one class start, so the class is c0 or c0 + 1
 //   (one comparison with starts[c0 + 1]) and bits 9..10 / 11..12 are the decoders of c0 / c0 + 1
 //   (kLutKind*); bit 13 set: the bucket meets several class starts, bits 9..11 = k with the class
 //   at most 2^k - 1 further, found by a halving search.
-constexpr uint32_t kLutRedirect = 0x8000u, kLutWide = 0x2000u;
+constexpr uint32_t kLutFinal = 0x8000u, kLutWide = 0x2000u;
 enum : uint32_t { kLutKindOdd = 0, kLutKindEven = 1, kLutKindEvenSecond = 2, kLutKindGeneric = 3 };
 
 struct KindCount {
@@ -118,8 +119,8 @@ struct Codebook {
   std::vector<ClassDef> classes;          // 383, format order
   // device-shaped tables
   DevClass dev_classes[kClassSlots];
-  uint64_t starts[kStartsPadded];         // starts[c] = offset of class c, starts[383] = N(13), then UINT64_MAX
-  uint16_t lut[kLutSize];                 // first level of the class-find table (see kLutRedirect)
+  uint64_t starts[kStartsPadded];         // starts[c] = offset of class c + 1 (the first index of class c as a record holds it), starts[383] = N(13) + 1, then UINT64_MAX
+  uint16_t lut[kLutSize];                 // first level of the class-find table (see kLutFinal)
   std::vector<uint16_t> lut2;             // its second-level tables, those of the lowest keys first
   double rcp[32];                         // rcp[c] = 1/c, rcp[0] unused
   // step[(m * 25 + c) * 2 + {0,1}] = {m / c, 1 - m / c}: the odd-coset walk's per-slot

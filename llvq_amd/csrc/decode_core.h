@@ -56,9 +56,9 @@ struct DecodeTables {
   const uint32_t* golay;    // 4096 codewords, canonical order
   const DevClass* cls;      // generic-walk class records
   const FastClass* fast;    // fast-path class records
-  const uint64_t* starts;   // starts[c] = first zero-based index of class c; starts[383] = N(13) (a kernel's copy may end at kStartsLds)
+  const uint64_t* starts;   // starts[c] = first index of class c as a record holds it (class 0 begins at 1); starts[383] = N(13) + 1 (a kernel's copy may end at kStartsLds)
   const uint64_t* starts_far;  // the whole padded table, for the wide search
-  const uint16_t* lut;      // class-find table, first level (kLutRedirect in codebook.hpp)
+  const uint16_t* lut;      // class-find table, first level (kLutFinal in codebook.hpp)
   const uint16_t* lut2;     // its second-level tables
   const double* rcp;        // rcp[c] = 1/c for c in 1..24
   const uint32_t* on_lut;   // even coset, support arrangements
@@ -127,11 +127,11 @@ LLVQ_HD uint32_t walk_step(double& rho, uint32_t& tg, uint32_t n, const double* 
   return jj;
 }
 
-// Final class-find entry of the zero-based index i < N(13): one table probe on the top bits and,
+// Final class-find entry of the index 1 <= i <= N(13), as a record holds it: one table probe on the top bits and,
 // where that bucket meets several class starts, one on the bits below.
 LLVQ_HD uint32_t class_entry(const DecodeTables& T, uint64_t i) {
   uint32_t e = T.lut[(uint32_t)(i >> kLutShift)];
-  if (e & kLutRedirect) e = T.lut2[(e & 0x7FFFu) * (uint32_t)kLut2Span + ((uint32_t)(i >> kLut2Shift) & (uint32_t)(kLut2Span - 1))];
+  if (!(e & kLutFinal)) e = T.lut2[e + ((uint32_t)(i >> kLut2Shift) & (uint32_t)(kLut2Span - 1))];
   return e;
 }
 // The class from its entry: one comparison, or (0.09 % of uniformly drawn indices) a halving
@@ -340,9 +340,8 @@ LLVQ_HD int decode_index(const DecodeTables& T, uint64_t idx, Emit&& emit) {
     for (int p = 0; p < kDim; ++p) emit(p, 0);
     return idx == 0 ? -1 : -2;
   }
-  const uint64_t i = idx - 1;
-  const uint32_t ci = find_class(T, i);
-  const uint64_t li = i - T.starts[ci];
+  const uint32_t ci = find_class(T, idx);
+  const uint64_t li = idx - T.starts[ci];
   const FastClass f = T.fast[ci];
   const uint32_t path = (f.meta >> kMetaPathShift) & 3u;
   if (path == kPathOdd) {

@@ -111,7 +111,7 @@ __device__ __forceinline__ void unrank_queues_to_slice(const DecodeTables& T, co
       const uint32_t f = entry & 0xFFFu, ci = (entry >> 16) & 0x1FFu;
       const uint32_t row = (f * inv_kb) >> 16, b = f - row * kb;
       const uint64_t rec = record_at(row, b);
-      const uint64_t li = (rec >> 1) - 1 - T.starts[ci];
+      const uint64_t li = (rec >> 1) - T.starts[ci];
       const float g = (entry >> 25) & 1u ? g1 : g0;
       _Float16* wrow = W + (size_t)row * WSTRIDE + b * 24u;
       if (entry & kEntryOrigin) {

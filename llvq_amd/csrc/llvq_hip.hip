@@ -29,8 +29,8 @@ namespace llvq {
 // What every workgroup copies into LDS.  The rarely used generic class records
 // and the large even-coset tables stay in HBM (they live in L2).
 struct TableImage {
+  uint64_t starts[kStartsLds];  // first: read twice per block, its offset then needs no add of its own
   FastClass fast[kFastLds];
-  uint64_t starts[kStartsLds];
   double rcp[32];
   double step[(24 - kTailSlots) * 25 * 2];  // rows m >= kTailSlots: the walk's last slots are looked up
   uint8_t pdep4[256];
@@ -649,7 +649,19 @@ __device__ unsigned long long g_phase_stamps[1024 * 8];
 #define LLVQ_STAMP(k) do {} while (0)
 #endif
 
-// Classes of NB zero-based indices (< 2^47) side by side: the class, its first index and its decoder
+// The same number as one the compiler can relate to nothing it knows.  Used where what it would derive costs
+// more than the plain form: the address of an element of a second array with the same index (formed from the
+// first element's address by a 64-bit multiply-add), a table key re-shaped into three instructions, a 16-bit
+// entry zero-extended again.
+__device__ __forceinline__ uint32_t detached(uint32_t v) {
+  asm("" : "+v"(v));
+  return v;
+}
+
+static_assert(kLutFinal == 0x8000u, "the final flag is the top bit of a 16-bit entry");
+
+// Classes of NB indices as records hold them (1 .. N, below 2^47; 0 walks the tables harmlessly) side by side:
+// the class, its first index and its decoder
 // (kLutKind*).  Two table probes and one comparison each, every read unconditional so that the NB
 // reads of a step go out together; the indices whose bucket meets several class starts (0.09 % of
 // uniform draws) take the halving search afterwards, under a wavefront-wide test.
@@ -659,17 +671,21 @@ __device__ __forceinline__ void find_classes(const DecodeTables& T, const uint32
   uint32_t e[NB], e2[NB];
   // (48-bit indices reach the whole first-level table; T's class-find tables are then the full ones, in device memory)
 #pragma unroll
-  for (int i = 0; i < NB; ++i) e[i] = T.lut[(zhi[i] >> (kLutShift - 32)) & (WIDE ? (uint32_t)kLutSize - 1u : 2047u)];
+  for (int i = 0; i < NB; ++i) {
+    // a bit-field extract and a scaled add; the entry as the 32-bit word the load returns (upper half zero)
+    const uint32_t key = detached(__builtin_amdgcn_ubfe(zhi[i], kLutShift - 32, WIDE ? 12 : 11));
+    e[i] = detached(T.lut[key]);
+  }
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    const uint32_t sub = __builtin_amdgcn_alignbit(zhi[i], zlo[i], kLut2Shift) & (uint32_t)(kLut2Span - 1);
-    const uint32_t at = (e[i] & 0x7FFFu) * (uint32_t)kLut2Span + sub;
-    e2[i] = T.lut2[(e[i] & kLutRedirect) ? at : 0u];
+    // a first-level entry that is not final is where its second-level table begins, a multiple of the span
+    const uint32_t at = (__builtin_amdgcn_alignbit(zhi[i], zlo[i], kLut2Shift) & (uint32_t)(kLut2Span - 1)) | e[i];
+    e2[i] = T.lut2[e[i] < kLutFinal ? at : 0u];  // the flag is the entry's top bit: one comparison
   }
   uint64_t s0[NB], s1[NB];
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    e[i] = (e[i] & kLutRedirect) ? e2[i] : e[i];
+    e[i] = e[i] < kLutFinal ? e2[i] : e[i];
     s0[i] = T.starts[e[i] & 511u];
     s1[i] = T.starts[(e[i] & 511u) + 1u];
   }
@@ -716,7 +732,7 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
                                                  uint32_t first = threadIdx.x) {
   const uint32_t tid = first, lane = threadIdx.x & 63u;
   uint32_t entry[NB], ci[NB];
-  uint64_t zi[NB];  // zero-based index, ~0 when the lane has no block / an origin
+  uint64_t zi[NB];  // the record's index, ~0 when the lane has no block / an origin
   bool queued_origin[NB];
   // Every LDS read of this phase is unconditional (a lane without a block reads a valid slot and
   // ignores it), so that the NB reads of a step go out together: a guarded read is waited for
@@ -738,7 +754,7 @@ __device__ __forceinline__ void classify_and_bin(const DecodeTables& T, uint32_t
         queued_origin[i] = origin(f);
         if (queued_origin[i]) entry[i] |= kEntryOrigin;
       } else {
-        zi[i] = (rec >> 1) - 1;
+        zi[i] = rec >> 1;
       }
     }
   }
@@ -829,39 +845,50 @@ __device__ __forceinline__ void classify_records(const DecodeTables& T, const Re
   uint64_t start[NB];
   bool live[NB];  // a block of the tile that is not the origin (which decodes to zero whatever the gain, index.rs:335-337)
   uint32_t where = 0;
+  bool any_origin = false;
   const auto& records = prepared_records(rec);
+  const uint32_t share = nblk > tid * NB ? nblk - tid * NB : 0u;  // this lane's blocks are its first `share` (NB or more: all)
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    const uint32_t f = tid * NB + (uint32_t)i;
     uint32_t ilo, ihi;  // the 47-bit (48-bit) index
     record_index(records, i, ilo, ihi, gain[i]);
-    const bool origin = (ilo | ihi) == 0u;
-    live[i] = f < nblk && !origin;
-    where |= (f < nblk && origin) ? 1u << (8 + i) : 0u;
-    uint64_t z = (((uint64_t)ihi << 32) | ilo) - 1u;  // zero-based
-    // a 48-bit field can hold numbers past N(13): the host refuses such a matrix, and a lane past the tile's
-    // end, which reads whatever bits follow, must still walk the tables inside them
-    if (kWide) z = z < kN13 ? z : 0u;
-    zlo[i] = (uint32_t)z;
-    zhi[i] = (uint32_t)(z >> 32) & (kWide ? 0xFFFFu : 0x7FFFu);  // an origin wraps to all ones: keep it inside the field
+    // The tables are keyed on the index as the record holds it.  A 48-bit field can hold numbers past N(13):
+    // the host refuses such a matrix, and a lane past the tile's end, which reads whatever bits follow, must
+    // still walk the tables inside them: such a number counts as the origin
+    if (kWide) {
+      const uint64_t v = ((uint64_t)ihi << 32) | ilo;
+      const bool inside = v <= kN13;
+      ilo = inside ? ilo : 0u;
+      ihi = inside ? ihi : 0u;
+    }
+    const bool origin = (ilo | ihi) == 0u, mine = (uint32_t)i < share;
+    live[i] = mine && !origin;
+    any_origin |= mine && origin;
+    zlo[i] = ilo;
+    zhi[i] = ihi;
+  }
+  if (__any(any_origin)) {  // rare: a block at the origin is flagged for settle_origins
+    asm volatile("");       // (a branch, not selects on the common path)
+#pragma unroll
+    for (int i = 0; i < NB; ++i) where |= ((uint32_t)i < share && (zlo[i] | zhi[i]) == 0u) ? 1u << (8 + i) : 0u;
   }
   find_classes<NB, kWide>(T, zlo, zhi, ci, start, kind);
-  // Which queue a block joins.  A generic block rides in the odd queue, flagged, unless its coset's small
-  // queue has room (settled when the block is queued).
-  uint32_t any_generic = 0;
+  // Which queue a block joins.  A generic block (rare) joins none here: it is settled when the block is queued
+  // (its coset's small queue, or the odd queue, flagged, when that one is full).
+  bool any_generic = false;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     const uint64_t li = (((uint64_t)zhi[i] << 32) | zlo[i]) - start[i];
-    const uint32_t generic = kind[i] == kLutKindGeneric ? 1u : 0u;
     c.e0[i] = (uint32_t)li;
-    c.e1[i] = (uint32_t)(li >> 32) | (ci[i] << kQaClassShift) | (gain[i] << kQaGainShift) | (generic << 31);
-    where |= (live[i] ? (generic ? 0u : kind[i]) : 3u) << (2 * i);
-    any_generic |= live[i] ? generic : 0u;
+    c.e1[i] = (uint32_t)(li >> 32) | (ci[i] << kQaClassShift) | (gain[i] << kQaGainShift);
+    where |= (live[i] ? kind[i] : 3u) << (2 * i);
+    any_generic |= live[i] && kind[i] == kLutKindGeneric;
   }
-  if (__any(any_generic != 0u)) {
+  static_assert(kLutKindGeneric == 3u, "a generic block and a block that joins no queue share the code 3");
+  if (__any(any_generic)) {
 #pragma unroll
     for (int i = 0; i < NB; ++i)
-      if (((where >> (2 * i)) & 3u) == 0u && (c.e1[i] >> 31) && !(T.fast[ci[i]].meta & kMetaOdd)) where |= 1u << (12 + i);
+      if (live[i] && kind[i] == kLutKindGeneric) where |= (1u << (16 + i)) | ((T.fast[ci[i]].meta & kMetaOdd) ? 0u : 1u << (12 + i));
   }
   c.where = where;
 }
@@ -873,19 +900,18 @@ __device__ __forceinline__ void queue_classified(Classified<NB>& c, uint32_t cap
   uint32_t kq[NB];
 #pragma unroll
   for (int i = 0; i < NB; ++i) kq[i] = (c.where >> (2 * i)) & 3u;
-  uint32_t any_generic = 0;
-#pragma unroll
-  for (int i = 0; i < NB; ++i) any_generic |= (kq[i] == 0u) ? c.e1[i] >> 31 : 0u;
-  if (__any(any_generic != 0u)) {
+  if (__any((c.where >> 16) & 15u)) {  // generic blocks: to the small queue of their coset while it has room
 #pragma unroll
     for (int i = 0; i < NB; ++i)
-      if (kq[i] == 0u && (c.e1[i] >> 31)) {
+      if ((c.where >> (16 + i)) & 1u) {
         const uint32_t even = (c.where >> (12 + i)) & 1u;
         const uint32_t slot = atomicAdd(&Q.ctrl[even ? kCtrlGenEven : kCtrlGenOdd], 1u);
+        c.e1[i] |= 0x80000000u;  // the walk, not a fast decoder
         if (slot < (uint32_t)kGenericSlots) {
           Q.gqa[even * kGenericSlots + slot] = make_uint2(c.e0[i], c.e1[i]);
           Q.gqf[even * kGenericSlots + slot] = (uint16_t)(tid * NB + (uint32_t)i);
-          kq[i] = 3u;  // placed
+        } else {
+          kq[i] = 0u;  // rides in the odd queue, flagged
         }
       }
   }
@@ -895,9 +921,9 @@ __device__ __forceinline__ void queue_classified(Classified<NB>& c, uint32_t cap
   uint32_t sh[NB], running[NB], total = 0;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    sh[i] = kq[i] * 10u;
+    sh[i] = __umul24(kq[i], 10u);
     running[i] = total;
-    total += kq[i] < 3u ? 1u << sh[i] : 0u;
+    total += (1u << sh[i]) & 0x3FFFFFFFu;  // a block that joins no queue (3) counts nowhere
   }
   const uint32_t through = wave_prefix_sum(total);  // this lane's blocks included
   const uint32_t below = through - total;
@@ -917,22 +943,32 @@ __device__ __forceinline__ void queue_classified(Classified<NB>& c, uint32_t cap
   // odd from the bottom, even from the top, the small queue behind both
   const uint32_t top = capacity - 1u - base_e, small = capacity + base_s;
   const bool spills = base_s + n_s > (uint32_t)kSecSlots;  // wavefront-uniform, rare
-  const uint32_t fits = base_s >= (uint32_t)kSecSlots ? 0u : (uint32_t)kSecSlots - base_s;  // small-queue ranks below this fit
-#pragma unroll
-  for (int i = 0; i < NB; ++i) {
-    const uint32_t rank = ((below + running[i]) >> sh[i]) & 1023u;
-    const uint32_t up = base_o + rank, down = top - rank, behind = small + rank;
-    uint32_t pos = kq[i] == 1u ? down : up;
-    pos = kq[i] == 2u ? behind : pos;
-    uint32_t e1 = c.e1[i];
-    if (spills) {
-      const bool out = kq[i] == 2u && rank >= fits;
-      pos = out ? top - (n_e + (rank - fits)) : pos;
-      e1 |= out ? kQaSecond : 0u;
-    }
+  auto place = [&](int i, uint32_t pos, uint32_t e1) {
     if (kq[i] != 3u) {
       Q.qa[pos] = make_uint2(c.e0[i], e1);
-      Q.qf[pos] = (uint16_t)(tid * NB + (uint32_t)i);
+      Q.qf[detached(pos)] = (uint16_t)(tid * NB + (uint32_t)i);
+    }
+  };
+  if (!spills) {  // a branch of its own: the rare case's arithmetic stays out of the common one
+    // the three queues' first slots in vector registers, formed once, and a signed step: the even queue runs down
+    const uint32_t v_odd = detached(base_o), v_top = detached(top), v_small = detached(small);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const uint32_t rank = __builtin_amdgcn_ubfe(below + running[i], sh[i], 10);
+      const uint32_t first = kq[i] == 1u ? v_top : (kq[i] == 2u ? v_small : v_odd);
+      const int step = kq[i] == 1u ? -1 : 1;
+      place(i, (uint32_t)__mul24((int)rank, step) + first, c.e1[i]);
+    }
+  } else {
+    const uint32_t fits = base_s >= (uint32_t)kSecSlots ? 0u : (uint32_t)kSecSlots - base_s;  // small-queue ranks below this fit
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const uint32_t rank = __builtin_amdgcn_ubfe(below + running[i], sh[i], 10);
+      const uint32_t up = base_o + rank, down = top - rank, behind = small + rank;
+      uint32_t pos = kq[i] == 1u ? down : up;
+      pos = kq[i] == 2u ? behind : pos;
+      const bool out = kq[i] == 2u && rank >= fits;
+      place(i, out ? top - (n_e + (rank - fits)) : pos, c.e1[i] | (out ? kQaSecond : 0u));
     }
   }
 }
@@ -1005,7 +1041,7 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
     b.ci = (e.y >> kQaClassShift) & 0x1FFu;
     b.f = f;
     const uint32_t row = (uint32_t)(((float)f + 0.5f) * op.inv_nb);
-    b.col = f - row * nb;
+    b.col = f - __umul24(row, nb);  // both below 2^24: the full-rate multiply
     b.g = (e.y >> kQaGainShift) & 1u ? op.g1 : op.g0;
     return b;
   };
@@ -1013,7 +1049,7 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
   // the same integer dot products as the fast paths
   auto generic_block = [&](uint2 e, uint32_t f) {
     const Block b = open_block(e, f);
-    const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+    const uint32_t* xp = xplanes + __umul24(b.col, (uint32_t)kPlaneDwords);
     const DevClass c = T.cls[b.ci];
     uint32_t w[6] = {0, 0, 0, 0, 0, 0};
     auto emit = [&](int p, int v) { w[p >> 2] |= ((uint32_t)v & 0xFFu) << (8 * (p & 3)); };
@@ -1030,7 +1066,7 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
   };
   auto odd_block = [&](uint2 e, uint32_t f) {
     const Block b = open_block(e, f);
-    const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+    const uint32_t* xp = xplanes + __umul24(b.col, (uint32_t)kPlaneDwords);
     const FastClass fc = T.fast[b.ci];
     int d0 = 0, d1 = 0, d2 = 0;
     odd_codes(T, fc, b.li, [&](int q, uint32_t sel) {
@@ -1044,7 +1080,7 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
   auto even_block = [&](uint2 e, uint32_t f, auto second) {
     constexpr bool kSecond = decltype(second)::value;
     const Block b = open_block(e, f);
-    const uint32_t* xp = xplanes + (size_t)b.col * kPlaneDwords;
+    const uint32_t* xp = xplanes + __umul24(b.col, (uint32_t)kPlaneDwords);
     const FastClass fc = T.fast[b.ci];
     const uint32_t fv1 = fc.u0 >> 16;
     const uint32_t tab2_lo = fv1 << 8, tab2_hi = ((0u - fv1) & 0xFFu) << 8;
@@ -1077,7 +1113,7 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
     const uint32_t ts = chunk - c_gen;
     if (ts < c_sec) {
       const uint32_t k = ts * 64u + lane;
-      if (k < n_sec) even_block(Q.qa[kTileBlocks + k], Q.qf[kTileBlocks + k], std::true_type{});
+      if (k < n_sec) even_block(Q.qa[kTileBlocks + k], Q.qf[detached(kTileBlocks + k)], std::true_type{});
       continue;
     }
     const uint32_t t = ts - c_sec;
@@ -1089,7 +1125,7 @@ __device__ __forceinline__ uint32_t unrank_tile(const DecodeTables& T, const Gem
       const uint32_t at = min(k, (uint32_t)kTileBlocks - 1u);
       const uint2 e = Q.qa[at];
       // generic blocks that found their small queue full wait for the pass below
-      if (k < n_odd && !(e.y >> 31)) odd_block(e, Q.qf[at]);
+      if (k < n_odd && !(e.y >> 31)) odd_block(e, Q.qf[detached(at)]);
     } else {
       const uint32_t at = kTileBlocks - 1 - min(k, (uint32_t)kTileBlocks - 1u);
       const uint2 e = Q.qa[at];
@@ -1641,7 +1677,7 @@ int llvq_hip_runtime_create(int device, void* hip_stream, llvq_rt** out) {
   // a 47-bit index reaches no class past kFastLds - 2 and no second-level table past kLut2Lds
   uint32_t lut2_used = 0;
   for (uint16_t e : img->lut)
-    if (e & kLutRedirect) lut2_used = std::max<uint32_t>(lut2_used, ((e & 0x7FFFu) + 1u) * kLut2Span);
+    if (!(e & kLutFinal)) lut2_used = std::max<uint32_t>(lut2_used, (uint32_t)e + (uint32_t)kLut2Span);
   if (lut2_used > (uint32_t)kLut2Lds || lut2_used > cb.lut2.size() || cb.starts[kFastLds - 1] < (1ULL << 47)) {
     delete rt;
     return fail(LLVQ_ERR_UNSUPPORTED, "class-find tables outgrew their LDS slots");
