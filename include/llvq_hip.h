@@ -58,9 +58,9 @@ typedef struct llvq_mat llvq_mat; /* replaces FusedProj     (fused_cuda.rs:119-1
  * Cap 12 and cap 13 are accepted; other caps are refused by name
  * (LLVQ_ERR_UNSUPPORTED).  A cap-13 matrix is served by llvq_hip_gemv,
  * llvq_hip_gemv_group (a call may mix caps: one launch per cap), llvq_hip_rotate /
- * llvq_hip_gemv_rotated, the decode loop (per-group launches) and, as a loop over
- * its rows, by llvq_hip_gemm / llvq_hip_gemm_group and the batched prompt path;
- * llvq_hip_sequence_create refuses it by name. */
+ * llvq_hip_gemv_rotated, llvq_hip_sequence_* (the matrices of one sequence share
+ * their cap), the decode loop and, as a loop over its rows, by llvq_hip_gemm /
+ * llvq_hip_gemm_group and the batched prompt path. */
 typedef struct llvq_matrix_desc {
   const char* name;          /* may be NULL */
   uint32_t d_out, d_in;
@@ -280,8 +280,8 @@ typedef struct llvq_quant_rows {
 } llvq_quant_rows;
 /* How llvq_hip_decoder_* launches the projection groups of a decoded position.  The results are the same bit for bit;
  * the speed is not: a decode position is a chain of dependent products, and an ordered item of a sequence pays about
- * what a launch boundary costs (measured on the Qwen3-4B shape: 248 / 235 / 227 tokens/s in the order below).
- * Models a sequence cannot take (matrices in a rotated basis or of shell cap 13, hidden > 6144) use LLVQ_LAUNCH_PER_GROUP
+ * what a launch boundary costs (measured on the Qwen3-4B shape: 251 / 235 / 227 tokens/s in the order below).
+ * Models a sequence cannot take (matrices in a rotated basis or of mixed shell caps, hidden > 6144) use LLVQ_LAUNCH_PER_GROUP
  * whatever is asked. */
 typedef enum llvq_launch_mode {
   LLVQ_LAUNCH_PER_GROUP = 0,  /* one llvq_hip_gemv_group launch per group */

@@ -40,7 +40,8 @@ struct SeqTile {          // one tile of the sequence: whole rows of one matrix,
   uint32_t rows;
   uint32_t nblk;          // rows x blocks per row
   uint32_t item;
-  uint32_t pad[3];
+  uint32_t bit0;          // dense 49-bit blocks: bits of the byte at `codes` ahead of the tile's first block (0..7); 0 for 6-byte records
+  uint32_t pad[2];
 };
 static_assert(sizeof(SeqTile) == 64, "a tile descriptor is one 64-byte scalar load");
 
@@ -139,6 +140,25 @@ __device__ __forceinline__ void seq_request_records(const SeqTile& t, uint32_t t
   }
 }
 
+// The same for the dense 49-bit blocks of a cap-13 matrix (prefetch_records): eight dwords from the dword that
+// holds the lane's first block.  seq_dense_bit: where that block begins, in bits from the dword boundary at or
+// below the tile's first byte.
+__device__ __forceinline__ uint32_t seq_dense_bit(const SeqTile& t, uint32_t tid) {
+  const uint32_t first = tid * 4u < t.nblk ? tid * 4u : 0u;
+  const uint32_t skew = (uint32_t)reinterpret_cast<uintptr_t>(t.codes) & 3u;  // `codes` is a byte address: back to its dword
+  return skew * 8u + t.bit0 + first * kDenseBits;
+}
+__device__ __forceinline__ void seq_request_records(const SeqTile& t, uint32_t tid, DenseRecords& r) {
+  if (t.nblk == 0) return;
+  const uint32_t skew = (uint32_t)reinterpret_cast<uintptr_t>(t.codes) & 3u;
+  const uint32_t lane_bit = seq_dense_bit(t, tid);
+  const uint8_t* src = t.codes - skew + (size_t)(lane_bit >> 5) * 4;
+  const dwords4_a4 lo = __builtin_nontemporal_load(reinterpret_cast<const dwords4_a4*>(src));
+  const dwords4_a4 hi = __builtin_nontemporal_load(reinterpret_cast<const dwords4_a4*>(src + 16));
+  r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w; r.w[4] = hi.x; r.w[5] = hi.y; r.w[6] = hi.z; r.w[7] = hi.w;
+  r.s0 = lane_bit & 31u;
+}
+
 // Row scales and tail weights of a tile's first 128 rows, requested ahead of the row sums.
 struct RowOperands {
   float rs[2], tl[2][2];
@@ -210,6 +230,29 @@ __device__ __forceinline__ void carry_records(const LaneRecords<NB>& rec, Carrie
 #pragma unroll
   for (int k = 0; k < NB * 3 / 2; ++k) c.r[k] = rec.w[k];
 }
+// Dense blocks take the eight words in front; the ninth stays what it is (the `where` word of a classified share:
+// before a workgroup's first tile it says "nothing to queue", and must go on saying so while records are carried).
+// The bit offset of the lane's first block is worked out again where the records are classified (seq_dense_bit).
+static_assert(sizeof(DenseRecords) == sizeof(Carried<4>), "a lane's dense blocks fit the carried registers");
+__device__ __forceinline__ void carried_records(const Carried<4>& c, DenseRecords& rec) {
+#pragma unroll
+  for (int k = 0; k < 8; ++k) rec.w[k] = c.r[k];
+}
+__device__ __forceinline__ void carry_records(const DenseRecords& rec, Carried<4>& c) {
+#pragma unroll
+  for (int k = 0; k < 8; ++k) c.r[k] = rec.w[k];
+}
+template <class Rec>
+__device__ __forceinline__ void clear_records(Rec& rec) {
+  if constexpr (RecordTraits<Rec>::kWide) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) rec.w[k] = 0;
+    rec.s0 = 0;
+  } else {
+#pragma unroll
+    for (size_t k = 0; k < sizeof(rec.w) / sizeof(rec.w[0]); ++k) rec.w[k] = 0;
+  }
+}
 template <int NB>
 __device__ __forceinline__ void carry_classified(const Classified<NB>& cls, Carried<NB>& c) {
 #pragma unroll
@@ -237,14 +280,17 @@ __device__ __forceinline__ uint32_t opaque_tid() {
   return t;
 }
 
-template <int TILE, bool LEAN, int PLANES>
+// WIDE: every matrix of the sequence is a cap-13 one (49-bit blocks in a dense stream, as in gemv_tiles_kernel).
+template <int TILE, bool LEAN, int PLANES, bool WIDE = false>
 __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
   constexpr int kP1Blocks = TILE / kWgThreads;
+  static_assert(!WIDE || TILE == 4 * kWgThreads, "the dense-stream variant takes four blocks per lane");
+  using Records = typename std::conditional<WIDE, DenseRecords, LaneRecords<kP1Blocks>>::type;
   extern __shared__ __align__(16) uint8_t smem[];
   const uint32_t tid = threadIdx.x, wave = tid >> 6;
   const uint32_t G = gridDim.x, n_tiles = s.n_tiles;
   if (blockIdx.x >= n_tiles) return;
-  const DecodeTables T = stage_tables<!LEAN>(smem, s.tables);
+  const DecodeTables T = stage_tables<!LEAN, true, WIDE>(smem, s.tables);
   const uint32_t max_nb = s.max_nb;
   uint32_t* xplanes = reinterpret_cast<uint32_t*>(smem + (LEAN ? kLdsImageBytesLean : kLdsImageBytes));
   float* xscale = reinterpret_cast<float*>(xplanes + (size_t)max_nb * kPlaneDwords);
@@ -295,9 +341,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     if (next.item != 0) I = s.items[next.item];
     I = seq_item_of(I);
     if (I.wait_item == kSeqNoWait) {
-      LaneRecords<kP1Blocks> rec;
-#pragma unroll
-      for (int r = 0; r < kP1Blocks * 3 / 2; ++r) rec.w[r] = 0;
+      Records rec;
+      clear_records(rec);
       const ActivationSource src{I.x, nullptr, I.x2, I.norm_w, I.resid_out, I.eps, I.prologue, I.nb, I.tail_w,
                                  nullptr, nullptr, 1.f, 0u, 0u, nxt == I.first_tile, false};
       (void)stage_activation<TILE, false, PLANES, true>(src, xplanes, xscale, xtail, reinterpret_cast<uint8_t*>(xplanes), Q.partial,
@@ -332,8 +377,9 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     const bool more = nxt < n_tiles;
     const uint32_t request_after = wave >> 2;
     auto classify_next = [&]() {
-      LaneRecords<kP1Blocks> rec;
+      Records rec;
       carried_records(carried, rec);
+      if constexpr (WIDE) rec.s0 = seq_dense_bit(next, opaque_tid()) & 31u;
       Classified<kP1Blocks> c;
       classify_records<kP1Blocks>(T, rec, next.nblk, c, opaque_tid());
       carry_classified(c, carried);
@@ -341,9 +387,8 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     auto for_next_tile = [&](uint32_t done, bool last, uint32_t state) {
       if (!more) return 2u;
       if (state == 0u && (last || done >= request_after)) {
-        LaneRecords<kP1Blocks> rec;
-#pragma unroll
-        for (int k = 0; k < kP1Blocks * 3 / 2; ++k) rec.w[k] = 0;
+        Records rec;
+        clear_records(rec);
         seq_request_records(next, opaque_tid(), rec);
         carry_records(rec, carried);
         return 1u;

@@ -1592,7 +1592,7 @@ struct llvq_seq {
   uint8_t* blob = nullptr;  // one device allocation: tiles | items | counters | status
   SeqArgs args{};
   uint32_t tile = 0, grid = 0, n_items = 0;
-  bool lean = false, f32 = false;
+  bool lean = false, f32 = false, wide = false;
   size_t lds = 0;
   uint32_t* own_status = nullptr;  // the status word inside `blob` (args.status may point at a word several sequences share)
 };
@@ -2247,7 +2247,11 @@ struct SeqSpec {
 };
 
 // three byte planes of the activation for f32 results, two for binary16 results, as gemv_tiles_kernel
-static const void* seq_kernel(uint32_t tile, bool lean, bool f32) {
+static const void* seq_kernel(uint32_t tile, bool lean, bool f32, bool wide) {
+  if (wide) {  // cap-13 matrices: full tiles only
+    if (f32) return lean ? reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, true, 3, true>) : reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, false, 3, true>);
+    return lean ? reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, true, 2, true>) : reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, false, 2, true>);
+  }
   if (f32) {
     if (lean) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, true, 3>);
     if (tile == (uint32_t)kTileBlocks) return reinterpret_cast<const void*>(gemv_seq_kernel<kTileBlocks, false, 3>);
@@ -2284,7 +2288,7 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
       if (!m || !sp.y[j]) return fail(LLVQ_ERR_INVALID_ARGUMENT, "sequence_create: null matrix or output in item " + std::to_string(i));
       if (m->d_in != sp.mats[0]->d_in) return fail(LLVQ_ERR_INVALID_ARGUMENT, m->name + ": projections of one item must share d_in");
       if (m->has_rotation) return fail(LLVQ_ERR_UNSUPPORTED, m->name + ": a sequence takes natural-basis matrices only");
-      if (m->record_bits != 48) return fail(LLVQ_ERR_UNSUPPORTED, m->name + ": a sequence takes 6-byte records (shell cap 12) only");
+      if (m->record_bits != specs[0].mats[0]->record_bits) return fail(LLVQ_ERR_UNSUPPORTED, m->name + ": the matrices of a sequence share one shell cap");
     }
     if (sp.mats[0]->nblocks > 1024u) return fail(LLVQ_ERR_UNSUPPORTED, sp.mats[0]->name + ": rows wider than 24 576 columns do not fit a sequence");
     max_nb = std::max(max_nb, sp.mats[0]->nblocks);
@@ -2292,6 +2296,8 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
   }
   const GemvShape shape = pick_seq_shape(max_nb);
   if (shape.lds > 160 * 1024 || max_nb > shape.tile) return fail(LLVQ_ERR_UNSUPPORTED, "sequence_create: the widest rows do not fit the LDS activation tile");
+  const bool wide = specs[0].mats[0]->record_bits != 48;
+  if (wide && shape.tile != (uint32_t)kTileBlocks) return fail(LLVQ_ERR_UNSUPPORTED, "sequence_create: rows this wide do not fit a sequence of cap-13 matrices");
   for (int i = 0; i < n; ++i)
     if (specs[i].pro.kind == kPrologueAddRmsNorm && specs[i].mats[0]->d_in > 6u * kWgThreads)
       return fail(LLVQ_ERR_UNSUPPORTED, specs[i].mats[0]->name + ": d_in too wide for a fused norm inside a sequence");
@@ -2328,7 +2334,9 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
         SeqTile t{};
         t.rows = std::min(rpt, m->d_out - r0);
         t.nblk = t.rows * nb;
-        t.codes = m->codes + (size_t)r0 * nb * 6;
+        const uint64_t first_bit = (uint64_t)r0 * nb * m->record_bits;  // 6-byte records begin on a byte; dense 49-bit blocks need not
+        t.codes = m->codes + (first_bit >> 3);
+        t.bit0 = (uint32_t)(first_bit & 7u);
         t.rscale = m->rscale + r0;
         t.tail = m->tail + (size_t)r0 * m->tail_w;
         t.y = reinterpret_cast<uint8_t*>(sp.y[j]) + (size_t)r0 * ysz;
@@ -2379,8 +2387,9 @@ static int seq_create(llvq_rt* rt, const SeqSpec* specs, int n, llvq_seq** out) 
   q->tile = shape.tile;
   q->lean = shape.lean;
   q->f32 = specs[0].y_dtype == LLVQ_F32;
+  q->wide = wide;
   // the activation planes of a wide row push dynamic LDS past the 64 KB default
-  (void)hipFuncSetAttribute(seq_kernel(shape.tile, shape.lean, q->f32), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  (void)hipFuncSetAttribute(seq_kernel(shape.tile, shape.lean, q->f32, q->wide), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
   q->lds = shape.lds;
   q->grid = grid;
   q->n_items = (uint32_t)n;
@@ -2392,7 +2401,7 @@ static int seq_run(llvq_rt* rt, llvq_seq* q) {
   q->args.run += 1;
   SeqArgs a = q->args;
   void* params[] = {&a};
-  const void* kernel = seq_kernel(q->tile, q->lean, q->f32);
+  const void* kernel = seq_kernel(q->tile, q->lean, q->f32, q->wide);
   // An ordinary launch, also with ordered items: at most one workgroup per CU (by its LDS) and no more workgroups than
   // CUs, so on a device this stream has to itself every workgroup is resident and the waits end.  (A cooperative launch
   // would guarantee it, but costs some 200 us per launch here: 4B decode fell from 237 to 85 tokens/s with it.)  Should

@@ -127,7 +127,7 @@ def test_cap13_groups_rotation_and_batched_rows(gpu_rt, orc):
 
 def test_cap13_refusals(gpu_rt, orc):
     """Named refusals, nothing enqueued: an index past N(13) in the stream, a cap whose blocks are neither 48 nor 49
-    bits, a cap-13 matrix in a sequence."""
+    bits, a sequence that mixes caps."""
     import torch
 
     idx = np.array([5, orc.N13 + 1, 7], np.uint64)
@@ -142,10 +142,77 @@ def test_cap13_refusals(gpu_rt, orc):
     with pytest.raises(LlvqError) as err:
         gpu_rt.upload(cap11)
     assert err.value.kind == "Unsupported" and "cap 11" in str(err.value)
-    p = gpu_rt.upload(synth.make_matrix("model.layers.0.seq13.weight", 64, 512, seed=1, shell_cap=13))
+    p13 = gpu_rt.upload(synth.make_matrix("model.layers.0.seq13.weight", 64, 512, seed=1, shell_cap=13))
+    p12 = gpu_rt.upload(synth.make_matrix("model.layers.0.seq12.weight", 64, 512, seed=1, shell_cap=12))
     try:
-        with pytest.raises(LlvqError) as err:
-            gpu_rt.plan_sequence([([p], torch.zeros(512, dtype=torch.float16, device="cuda"), False)])
-        assert err.value.kind == "Unsupported"
+        x = torch.zeros(512, dtype=torch.float16, device="cuda")
+        with pytest.raises(LlvqError) as err:  # one record width per sequence
+            gpu_rt.plan_sequence([([p13], x, False), ([p12], x, False)])
+        assert err.value.kind == "Unsupported" and "one shell cap" in str(err.value)
     finally:
-        gpu_rt.free(p)
+        gpu_rt.free(p13)
+        gpu_rt.free(p12)
+
+
+@pytest.mark.parametrize("out", ["f16", "f32"])
+def test_cap13_sequence_matches_the_separate_calls(gpu_rt, orc, out):
+    """Cap-13 matrices through the sequence kernel: items of several widths (tiles that begin inside a byte of the
+    dense stream, rows of one block, tail columns only, more tiles than workgroups), independent and ordered,
+    against llvq_hip_gemv_group item by item, bit for bit, on two runs; one item against the CPU oracle."""
+    import torch
+
+    dt = torch.float16 if out == "f16" else torch.float32
+    groups = [[(1024, 2560), (256, 2560)], [(640, 4096)], [(2432, 2560), (2432, 2560)], [(320, 9728)], [(40, 17)],
+              [(5000, 48)], [(7, 24 * 700 + 5)], [(333, 2560)]]
+    uploaded, items, xs = [], [], {}
+    try:
+        for gi, shapes in enumerate(groups):
+            raws = [synth.make_matrix(f"model.layers.{gi}.s{j}.weight", do, di, seed=40 + gi, shell_cap=13) for j, (do, di) in enumerate(shapes)]
+            projs = [gpu_rt.upload(m) for m in raws]
+            uploaded.append((raws, projs))
+            d_in = shapes[0][1]
+            if d_in not in xs:
+                xs[d_in] = synth.make_activation(d_in, seed=d_in)[0]
+            items.append((projs, _x16(xs[d_in]), False))
+        seq = gpu_rt.plan_sequence(items, out_dtype=dt)
+        try:
+            want = [gpu_rt.forward_group(projs, x, out_dtype=dt) for projs, x, _ in items]
+            for run in range(2):
+                for ys in seq.outputs:
+                    for y in ys:
+                        y.fill_(float("nan"))
+                seq.run()
+                seq.status()
+                for gi, (ys, ws) in enumerate(zip(seq.outputs, want)):
+                    for y, w in zip(ys, ws):
+                        assert torch.equal(y.view(torch.int16 if out == "f16" else torch.int32), w.view(torch.int16 if out == "f16" else torch.int32)), \
+                            f"run {run}, item {gi}: outputs differ from the separate call"
+            if out == "f32":
+                raw, x = uploaded[7][0][0], xs[2560]
+                y_ref, a_ref = _oracle_matrix(orc, raw).fused_product(x.astype(np.float64))
+                assert (np.abs(seq.outputs[7][0].cpu().numpy().reshape(-1) - y_ref) / np.maximum(a_ref, 1e-30)).max() < 1e-5
+        finally:
+            seq.close()
+        # ordered: the second item reads what the first one wrote
+        a = gpu_rt.upload(synth.make_matrix("model.layers.9.a.weight", 2560, 2560, seed=77, shell_cap=13))
+        b = gpu_rt.upload(synth.make_matrix("model.layers.9.b.weight", 1000, 2560, seed=78, shell_cap=13))
+        try:
+            x = _x16(xs[2560])
+            mid = gpu_rt.forward(a, x, out_dtype=torch.float16).reshape(-1)
+            want_b = gpu_rt.forward(b, mid, out_dtype=torch.float16).reshape(-1)
+            ya = torch.empty(2560, dtype=torch.float16, device="cuda")
+            chain = gpu_rt.plan_sequence([([a], x, False, [ya]), ([b], ya, True)], out_dtype=torch.float16)
+            try:
+                chain.run()
+                chain.status()
+                assert torch.equal(chain.outputs[0][0].view(torch.int16), mid.view(torch.int16))
+                assert torch.equal(chain.outputs[1][0].view(torch.int16), want_b.view(torch.int16))
+            finally:
+                chain.close()
+        finally:
+            gpu_rt.free(a)
+            gpu_rt.free(b)
+    finally:
+        for _, projs in uploaded:
+            for p in projs:
+                gpu_rt.free(p)

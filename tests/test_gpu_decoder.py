@@ -499,15 +499,16 @@ def test_full_size_greedy_tokens_match_the_oracle_fixture(gpu_rt, fixture_name, 
         dec.close()
 
 
-@pytest.mark.parametrize("cfg,seed", [(SMALL, 1), (RAGGED, 2), (Q8, 6)])
-def test_sequences_and_separate_launches_give_the_same_bits(gpu_rt, cfg, seed):
+@pytest.mark.parametrize("cfg,seed,cap", [(SMALL, 1, 12), (RAGGED, 2, 12), (Q8, 6, 12), (SMALL, 3, 13)])
+def test_sequences_and_separate_launches_give_the_same_bits(gpu_rt, cfg, seed, cap):
     """The three ways a position's projection groups are launched (llvq_launch_mode: single-item sequences, one
     llvq_hip_gemv_group launch per group, chains of ordered items between attention launches): the same arithmetic
     in the same order, so logits and tokens must be identical bit for bit, position after position (30 positions;
-    the residual buffers alternate, the counters of the chained sequences count on)."""
+    the residual buffers alternate, the counters of the chained sequences count on).  Once with cap-13 matrices
+    (the dense 49-bit blocks through the sequence kernel, with the fused prologues of the loop)."""
     from llvq_amd import _ffi
 
-    raws = decoder.synthetic_projections(cfg, seed)
+    raws = decoder.synthetic_projections(cfg, seed, shell_cap=cap)
     weights = decoder.synthetic_weights(cfg, seed)
     projs = [[gpu_rt.upload(m) for m in layer] for layer in raws]
     decs = [decoder.Decoder(gpu_rt, cfg, projs, weights, launch_mode=m)

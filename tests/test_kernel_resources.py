@@ -42,7 +42,7 @@ def test_no_kernel_spills(usage):
     # 2 output types x ((full tile, half tile, lean image) x (natural, rotated basis) + cap-13 stream x (whole, lean image))
     assert len(gemv) == 16
     seq = {k: v for k, v in usage.items() if "gemv_seq_kernel" in k}
-    assert len(seq) == 6  # (full tile, lean image, half tile) x (two, three activation planes)
+    assert len(seq) == 10  # (full tile, lean image, half tile; full and lean again for the dense 49-bit blocks) x (two, three activation planes)
     gemv.update(seq)
     for name, u in usage.items():
         assert u["ScratchSize"] == 0, f"{name} spills {u['ScratchSize']} bytes per lane"
