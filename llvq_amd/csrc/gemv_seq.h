@@ -367,8 +367,7 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     Q.ctrl = ctrl_sets + parity * kCtrlWords;
     Classified<kP1Blocks> cls;
     carried_classified(carried, cls);
-    // (a wavefront none of whose lanes holds a block of the tile has nothing to queue)
-    if ((opaque_tid() & ~63u) * (uint32_t)kP1Blocks < cur.nblk) queue_classified<kP1Blocks>(cls, TILE, Q, opaque_tid());
+    queue_classified<kP1Blocks>(cls, TILE, Q, opaque_tid());
     const uint32_t origins = cls.where;
     seq_finish_rows(prev, Q.partial, xtail, nb, tail_w, y_f16, ops);
     LLVQ_SEQ_STAMP(1);
@@ -378,10 +377,6 @@ __global__ __launch_bounds__(kWgThreads) void gemv_seq_kernel(SeqArgs s) {
     const bool more = nxt < n_tiles;
     const uint32_t request_after = wave >> 2;
     auto classify_next = [&]() {
-      if ((opaque_tid() & ~63u) * (uint32_t)kP1Blocks >= next.nblk) {  // no block of the next tile in this wavefront
-        carried.r[2 * kP1Blocks] = 0xFFu;
-        return;
-      }
       Records rec;
       carried_records(carried, rec);
       if constexpr (WIDE) rec.s0 = seq_dense_bit(next, opaque_tid()) & 31u;

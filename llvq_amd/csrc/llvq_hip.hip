@@ -986,10 +986,6 @@ __device__ __forceinline__ void settle_origins(uint32_t where, float* partial, u
 template <int NB, class Rec>
 __device__ __forceinline__ void classify_stream(const DecodeTables& T, const Rec& rec, uint32_t nblk, uint32_t capacity,
                                                 const GemvQueues& Q) {
-  // A wavefront none of whose lanes holds a block of the tile has nothing to classify or queue (the launches of a
-  // decode position often leave a workgroup one tile that is a quarter or a half full): P1 is bound by instruction
-  // issue, so the wavefronts that do hold blocks get the SIMDs to themselves.
-  if ((threadIdx.x & ~63u) * (uint32_t)NB >= nblk) return;
   Classified<NB> c;
   classify_records<NB>(T, rec, nblk, c);
   settle_origins<NB>(c.where, Q.partial);
